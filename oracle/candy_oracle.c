@@ -1,0 +1,531 @@
+/*
+ * candy_oracle.c -- CPU restatement of candy's quantized-matmul path.
+ *
+ * TEST INFRASTRUCTURE ONLY: used by tests/, the smoke check and the CPU-baseline
+ * leg of the benchmark as the checker.  The shipped HIP library never links it.
+ *
+ * Build with -ffp-contract=off: every f32 expression below is meant to round
+ * once per operation, exactly as written.
+ *
+ * Reference files are cited relative to the candy checkout:
+ *   QGO  = tensor/internal/cpu/kernels/quantized.go
+ *   QCU  = tensor/internal/cuda/kernels/quantized.cu
+ *   CONV = tensor/internal/cpu/kernels/conv.go
+ *   RED  = tensor/internal/cpu/kernels/reduce.go
+ *   UNA  = tensor/internal/cpu/kernels/unary.go
+ *   IDX  = tensor/internal/cpu/kernels/indexing.go
+ *
+ * Pinning status (what fixes each function besides this restatement itself;
+ * the checks live in tests/test_oracle_*.py):
+ *   co_fp16_to_f32        QGO:149-173. Pinned: all 65536 inputs against numpy's IEEE
+ *                         float16->float32 (bit patterns, NaN payloads included).
+ *   co_f32_to_fp16        no reference implementation (candy never narrows to fp16 on
+ *                         the CPU; QCU:3556 relies on the hardware conversion). Pinned:
+ *                         round-to-nearest-even against numpy's float32->float16 on all
+ *                         fp16 values, all midpoints and a random sweep.
+ *   co_dequantize Q4_0    QGO:85-93 (interleaved order). Pinned: exact rational values
+ *                         with Python Fractions; order relation to the ggml order QCU:862-866.
+ *   co_dequantize Q8_0    QGO:131-136. Pinned: exact rational values.
+ *   co_get_scale_min_k4   QCU:993-1005. Pinned: against an independent reading of the
+ *                         16-bit masked unpack QCU:2600-2612 over random and exhaustive
+ *                         byte-pair patterns.
+ *   co_dequantize Q4_K    QCU:1008-1041. Pinned: exact value (one rounding) in Fractions.
+ *   co_dequantize Q6_K    QCU:1103-1128. Pinned: exact value in Fractions.
+ *   co_quantize_q8_0      QCU:3521-3558 without the `sum` half. Pinned: float64 evaluation
+ *                         of round-half-away(x/d) with numpy float32 division; invariants.
+ *   co_vec_dot_q8_0       QCU:2058-2073, 2239-2263, 2367-2389 (shape of the float
+ *                         combination); integer parts pinned with Python ints, the float
+ *                         result against exact-arithmetic sum of dequantized products.
+ *   co_qmatmul            authored here (candy has no CPU QMatMul); pinned as above.
+ *   co_matmul_dequant_f32 CONV:373-389 applied to dequantized weights.
+ *   co_naive_batched_*    CONV:251-267, 373-389. Pinned: reference fixtures of
+ *                         conv_test.go:11-65.
+ *   co_fast_rms_norm_f32  RED:3071-3092. Pinned: reduce_test.go:1909-1971 fixtures.
+ *   co_rope_f32           RED:3987-4006. Pinned: reduce_test.go:2775-2832 fixtures.
+ *   co_fast_softmax_f32   RED:2855-2879. Pinned: reduce_test.go:1665-1717 fixtures.
+ *   co_silu_f32           UNA:3353-3366. Pinned: unary_test.go:4199-4241 closed form.
+ *   co_fast_argmax_f32    RED:846-862. Pinned: reduce_test.go:1063-1113 fixtures.
+ *   co_index_select_f32   IDX:8-26. Pinned: gather identity against numpy take.
+ *   co_attention_decode_f32  authored here as a composition of the ops above (candy has
+ *                         no attention on the CPU); pinned against a float64 numpy evaluation.
+ */
+#include "candy_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---- block layouts: QGO:8-11, 34-37, 55-59, 70-75; sizes asserted at QCU:305,347,410,444 ---- */
+#pragma pack(push, 1)
+typedef struct { uint16_t d; uint8_t qs[16]; } co_block_q4_0;
+typedef struct { uint16_t d; int8_t qs[32]; } co_block_q8_0;
+typedef struct { uint16_t dm[2]; uint8_t scales[12]; uint8_t qs[128]; } co_block_q4_k;
+typedef struct { uint8_t ql[128]; uint8_t qh[64]; int8_t scales[16]; uint16_t d; } co_block_q6_k;
+#pragma pack(pop)
+
+_Static_assert(sizeof(co_block_q4_0) == 18, "q4_0");
+_Static_assert(sizeof(co_block_q8_0) == 34, "q8_0");
+_Static_assert(sizeof(co_block_q4_k) == 144, "q4_K");
+_Static_assert(sizeof(co_block_q6_k) == 210, "q6_K");
+
+int co_block_elems(int fmt) {
+    switch (fmt) {
+    case CO_Q4_0: case CO_Q4_0_GGML: case CO_Q8_0: return 32;
+    case CO_Q4_K: case CO_Q6_K: return 256;
+    default: return 0;
+    }
+}
+
+int co_block_bytes(int fmt) {
+    switch (fmt) {
+    case CO_Q4_0: case CO_Q4_0_GGML: return 18;
+    case CO_Q8_0: return 34;
+    case CO_Q4_K: return 144;
+    case CO_Q6_K: return 210;
+    default: return 0;
+    }
+}
+
+static float bits_to_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static uint32_t f32_to_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+/* QGO:149-173 */
+float co_fp16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (uint32_t)(h & 0x7C00u);
+    uint32_t mant = (uint32_t)(h & 0x03FFu);
+    if (exp == 0x7C00u) /* inf / NaN keeps the payload shifted up: QGO:156 */
+        return bits_to_f32(sign | 0x7F800000u | (mant << 13));
+    if (exp == 0) {
+        if (mant == 0) return bits_to_f32(sign);
+        exp = (127u - 14u) << 23; /* QGO:162-168: normalise the subnormal */
+        while ((mant & 0x400u) == 0) { mant <<= 1; exp -= 1u << 23; }
+        mant &= 0x3FFu;
+        return bits_to_f32(sign | exp | (mant << 13));
+    }
+    return bits_to_f32(sign | ((((exp >> 10) - 15u + 127u) << 23)) | (mant << 13));
+}
+
+/* IEEE-754 binary32 -> binary16, round to nearest even (what QCU:3556 gets from the
+ * hardware conversion when it stores `d` into a half). */
+uint16_t co_f32_to_fp16(float f) {
+    uint32_t x = f32_to_bits(f);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t ax = x & 0x7FFFFFFFu;
+    if (ax >= 0x7F800000u) { /* inf / NaN */
+        if (ax == 0x7F800000u) return (uint16_t)(sign | 0x7C00u);
+        uint16_t payload = (uint16_t)((ax >> 13) & 0x3FFu);
+        return (uint16_t)(sign | 0x7C00u | 0x200u | payload); /* quiet NaN, keep top payload bits */
+    }
+    if (ax >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u); /* >= 65520 rounds to inf */
+    if (ax < 0x33000001u) return sign;                          /* <= 2^-25 rounds to zero */
+    int32_t e = (int32_t)(ax >> 23) - 127;
+    uint32_t m = (ax & 0x7FFFFFu) | 0x800000u; /* 24-bit significand */
+    uint32_t shift, half_e;
+    if (e < -14) { shift = (uint32_t)(13 + (-14 - e)); half_e = 0; }
+    else { shift = 13; half_e = (uint32_t)(e + 15); }
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (q & 1u))) q++;
+    /* for normals q carries the implicit bit (0x400); adding the exponent field on top
+     * lets a mantissa overflow carry into the exponent naturally */
+    uint32_t out = (half_e == 0) ? q : ((half_e - 1u) << 10) + q;
+    return (uint16_t)(sign | out);
+}
+
+/* QCU:993-1005 */
+void co_get_scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* QGO:85-93: interleaved element order */
+static void dequant_q4_0(const co_block_q4_0 *b, float *y) {
+    float d = co_fp16_to_f32(b->d);
+    for (int i = 0; i < 32; i += 2) {
+        int q1 = b->qs[i / 2] & 0xF;
+        int q2 = b->qs[i / 2] >> 4;
+        y[i] = d * ((float)q1 - 8.0f);
+        y[i + 1] = d * ((float)q2 - 8.0f);
+    }
+}
+
+/* QCU:862-866: low nibbles first, then high nibbles; d*q + (-8d) */
+static void dequant_q4_0_ggml(const co_block_q4_0 *b, float *y) {
+    float d = co_fp16_to_f32(b->d);
+    float dm = -8.0f * d;
+    for (int l = 0; l < 16; ++l) {
+        y[l] = d * (float)(b->qs[l] & 0xF) + dm;
+        y[l + 16] = d * (float)(b->qs[l] >> 4) + dm;
+    }
+}
+
+/* QGO:131-136 */
+static void dequant_q8_0(const co_block_q8_0 *b, float *y) {
+    float d = co_fp16_to_f32(b->d);
+    for (int i = 0; i < 32; ++i) y[i] = d * (float)b->qs[i];
+}
+
+/* QCU:1008-1041: group il of 64 values; low nibbles use scale 2il, high use 2il+1 */
+static void dequant_q4_k(const co_block_q4_k *b, float *y) {
+    float dall = co_fp16_to_f32(b->dm[0]);
+    float dmin = co_fp16_to_f32(b->dm[1]);
+    for (int il = 0; il < 4; ++il) {
+        uint8_t sc, m;
+        co_get_scale_min_k4(2 * il, b->scales, &sc, &m);
+        float d1 = dall * (float)sc, m1 = dmin * (float)m;
+        co_get_scale_min_k4(2 * il + 1, b->scales, &sc, &m);
+        float d2 = dall * (float)sc, m2 = dmin * (float)m;
+        const uint8_t *q = b->qs + 32 * il;
+        for (int l = 0; l < 32; ++l) {
+            y[64 * il + l] = d1 * (float)(q[l] & 0xF) - m1;
+            y[64 * il + 32 + l] = d2 * (float)(q[l] >> 4) - m2;
+        }
+    }
+}
+
+/* QCU:1103-1128 */
+static void dequant_q6_k(const co_block_q6_k *b, float *y) {
+    float d = co_fp16_to_f32(b->d);
+    for (int ip = 0; ip < 2; ++ip) {
+        for (int il = 0; il < 32; ++il) {
+            int is = 8 * ip + il / 16;
+            const uint8_t *ql = b->ql + 64 * ip + il;
+            uint8_t qh = b->qh[32 * ip + il];
+            const int8_t *sc = b->scales + is;
+            float *yy = y + 128 * ip + il;
+            yy[0] = d * (float)sc[0] * (float)((int8_t)((ql[0] & 0xF) | (((qh >> 0) & 3) << 4)) - 32);
+            yy[32] = d * (float)sc[2] * (float)((int8_t)((ql[32] & 0xF) | (((qh >> 2) & 3) << 4)) - 32);
+            yy[64] = d * (float)sc[4] * (float)((int8_t)((ql[0] >> 4) | (((qh >> 4) & 3) << 4)) - 32);
+            yy[96] = d * (float)sc[6] * (float)((int8_t)((ql[32] >> 4) | (((qh >> 6) & 3) << 4)) - 32);
+        }
+    }
+}
+
+int co_dequantize(int fmt, const void *blocks, int64_t n_blocks, float *y) {
+    switch (fmt) {
+    case CO_Q4_0:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q4_0((const co_block_q4_0 *)blocks + i, y + 32 * i);
+        return 0;
+    case CO_Q4_0_GGML:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q4_0_ggml((const co_block_q4_0 *)blocks + i, y + 32 * i);
+        return 0;
+    case CO_Q8_0:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q8_0((const co_block_q8_0 *)blocks + i, y + 32 * i);
+        return 0;
+    case CO_Q4_K:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q4_k((const co_block_q4_k *)blocks + i, y + 256 * i);
+        return 0;
+    case CO_Q6_K:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q6_k((const co_block_q6_k *)blocks + i, y + 256 * i);
+        return 0;
+    default:
+        return -1;
+    }
+}
+
+/* QCU:3521-3558 with the `sum` half dropped (Q8_0 instead of Q8_1).
+ * amax is a NaN-ignoring maximum (fmaxf, as warp_reduce_max uses); d = amax/127 in f32;
+ * q = amax == 0 ? 0 : roundf(x/d) with the UNROUNDED d; the stored scale is fp16(d). */
+int co_quantize_q8_0(const float *x, int64_t rows, int64_t cols, void *out_blocks) {
+    if (cols % 32 != 0 || rows < 0 || cols < 0) return -1;
+    co_block_q8_0 *out = (co_block_q8_0 *)out_blocks;
+    int64_t nb = rows * cols / 32;
+    for (int64_t b = 0; b < nb; ++b) {
+        const float *xb = x + 32 * b;
+        float amax = 0.0f;
+        for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(xb[i]));
+        const float d = amax / 127.0f;
+        for (int i = 0; i < 32; ++i)
+            out[b].qs[i] = (amax == 0.0f) ? 0 : (int8_t)roundf(xb[i] / d);
+        out[b].d = co_f32_to_fp16(d);
+    }
+    return 0;
+}
+
+/* ---- integer vec-dots against Q8_0 activation blocks ---- */
+
+/* QGO:85-93 element order: even elements pair with low nibbles, odd with high. */
+static float vec_dot_q4_0(const co_block_q4_0 *w, const co_block_q8_0 *x, int64_t nb) {
+    float acc = 0.0f;
+    for (int64_t b = 0; b < nb; ++b) {
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; ++j) {
+            sumi += ((int)(w[b].qs[j] & 0xF) - 8) * (int)x[b].qs[2 * j];
+            sumi += ((int)(w[b].qs[j] >> 4) - 8) * (int)x[b].qs[2 * j + 1];
+        }
+        acc += (co_fp16_to_f32(w[b].d) * co_fp16_to_f32(x[b].d)) * (float)sumi;
+    }
+    return acc;
+}
+
+/* ggml order (QCU:2426-2433 pairs low nibbles with q8[0..15], high with q8[16..31]) */
+static float vec_dot_q4_0_ggml(const co_block_q4_0 *w, const co_block_q8_0 *x, int64_t nb) {
+    float acc = 0.0f;
+    for (int64_t b = 0; b < nb; ++b) {
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; ++j) {
+            sumi += ((int)(w[b].qs[j] & 0xF) - 8) * (int)x[b].qs[j];
+            sumi += ((int)(w[b].qs[j] >> 4) - 8) * (int)x[b].qs[j + 16];
+        }
+        acc += (co_fp16_to_f32(w[b].d) * co_fp16_to_f32(x[b].d)) * (float)sumi;
+    }
+    return acc;
+}
+
+/* QCU:2058-2073: d8_0 * d8_1 * sumi */
+static float vec_dot_q8_0(const co_block_q8_0 *w, const co_block_q8_0 *x, int64_t nb) {
+    float acc = 0.0f;
+    for (int64_t b = 0; b < nb; ++b) {
+        int32_t sumi = 0;
+        for (int i = 0; i < 32; ++i) sumi += (int)w[b].qs[i] * (int)x[b].qs[i];
+        acc += (co_fp16_to_f32(w[b].d) * co_fp16_to_f32(x[b].d)) * (float)sumi;
+    }
+    return acc;
+}
+
+/* QCU:2239-2263: sumf_d += d8*(dot1*sc); sumf_m += d8*(dot2*m); dm.x*sumf_d - dm.y*sumf_m,
+ * taken over the eight 32-value sub-blocks of one super-block in ascending order. */
+static float vec_dot_q4_k(const co_block_q4_k *w, const co_block_q8_0 *x, int64_t nsb) {
+    float acc = 0.0f;
+    for (int64_t s = 0; s < nsb; ++s) {
+        float sumf_d = 0.0f, sumf_m = 0.0f;
+        for (int t = 0; t < 8; ++t) {
+            const co_block_q8_0 *xb = x + 8 * s + t;
+            const uint8_t *q = w[s].qs + 32 * (t / 2);
+            int32_t dot1 = 0, dot2 = 0;
+            for (int l = 0; l < 32; ++l) {
+                int q4 = (t & 1) ? (q[l] >> 4) : (q[l] & 0xF);
+                dot1 += q4 * (int)xb->qs[l];
+                dot2 += (int)xb->qs[l];
+            }
+            uint8_t sc, m;
+            co_get_scale_min_k4(t, w[s].scales, &sc, &m);
+            float d8 = co_fp16_to_f32(xb->d);
+            sumf_d += d8 * (float)(dot1 * (int)sc);
+            sumf_m += d8 * (float)(dot2 * (int)m);
+        }
+        acc += co_fp16_to_f32(w[s].dm[0]) * sumf_d - co_fp16_to_f32(w[s].dm[1]) * sumf_m;
+    }
+    return acc;
+}
+
+/* QCU:2367-2389: sumf += d8 * (dot * sc) per 16-value group; d * sumf per super-block. */
+static float vec_dot_q6_k(const co_block_q6_k *w, const co_block_q8_0 *x, int64_t nsb) {
+    float acc = 0.0f;
+    for (int64_t s = 0; s < nsb; ++s) {
+        float sumf = 0.0f;
+        for (int g = 0; g < 16; ++g) {
+            const co_block_q8_0 *xb = x + 8 * s + g / 2;
+            int32_t dot = 0;
+            for (int l = 0; l < 16; ++l) {
+                int e = 16 * g + l;
+                int ip = e / 128, quarter = (e % 128) / 32, il = e % 32;
+                uint8_t qlb = w[s].ql[64 * ip + il + 32 * (quarter & 1)];
+                int lo4 = (quarter < 2) ? (qlb & 0xF) : (qlb >> 4);
+                int hi2 = (w[s].qh[32 * ip + il] >> (2 * quarter)) & 3;
+                int q6 = (lo4 | (hi2 << 4)) - 32;
+                dot += q6 * (int)xb->qs[(e % 32)];
+            }
+            sumf += co_fp16_to_f32(xb->d) * (float)(dot * (int)w[s].scales[g]);
+        }
+        acc += co_fp16_to_f32(w[s].d) * sumf;
+    }
+    return acc;
+}
+
+float co_vec_dot_q8_0(int fmt, const void *w_row, const void *x_q8_0, int64_t k) {
+    const co_block_q8_0 *x = (const co_block_q8_0 *)x_q8_0;
+    switch (fmt) {
+    case CO_Q4_0: return vec_dot_q4_0((const co_block_q4_0 *)w_row, x, k / 32);
+    case CO_Q4_0_GGML: return vec_dot_q4_0_ggml((const co_block_q4_0 *)w_row, x, k / 32);
+    case CO_Q8_0: return vec_dot_q8_0((const co_block_q8_0 *)w_row, x, k / 32);
+    case CO_Q4_K: return vec_dot_q4_k((const co_block_q4_k *)w_row, x, k / 256);
+    case CO_Q6_K: return vec_dot_q6_k((const co_block_q6_k *)w_row, x, k / 256);
+    default: return NAN;
+    }
+}
+
+int co_qmatmul(int fmt, const void *w_blocks, int64_t rows, int64_t cols,
+               const float *x, int64_t m, float *y) {
+    int qk = co_block_elems(fmt), bs = co_block_bytes(fmt);
+    if (qk == 0 || cols % qk != 0 || rows < 0 || m < 0) return -1;
+    size_t xq_bytes = (size_t)(m * cols / 32) * 34;
+    void *xq = malloc(xq_bytes ? xq_bytes : 1);
+    if (!xq) return -2;
+    co_quantize_q8_0(x, m, cols, xq);
+    size_t row_bytes = (size_t)(cols / qk) * (size_t)bs;
+    size_t xrow_bytes = (size_t)(cols / 32) * 34;
+    for (int64_t i = 0; i < m; ++i)
+        for (int64_t n = 0; n < rows; ++n)
+            y[i * rows + n] = co_vec_dot_q8_0(fmt, (const uint8_t *)w_blocks + (size_t)n * row_bytes,
+                                              (const uint8_t *)xq + (size_t)i * xrow_bytes, cols);
+    free(xq);
+    return 0;
+}
+
+/* CONV:251-267 */
+void co_naive_batched_matmul_f32(int64_t bsz, int64_t m, int64_t n, int64_t k,
+                                 const float *a, const float *b, float *c) {
+    for (int64_t bb = 0; bb < bsz; ++bb) {
+        int64_t a_base = bb * m * k, b_base = bb * k * n, c_base = bb * m * n;
+        for (int64_t i = 0; i < m; ++i)
+            for (int64_t j = 0; j < n; ++j) {
+                float sum = 0.0f;
+                for (int64_t l = 0; l < k; ++l) sum += a[a_base + i * k + l] * b[b_base + l * n + j];
+                c[c_base + i * n + j] = sum;
+            }
+    }
+}
+
+/* CONV:373-389 */
+void co_naive_batched_matmul_strided_f32(int64_t bsz, int64_t m, int64_t n, int64_t k,
+                                         const float *a, const float *b, float *c,
+                                         const int64_t as[3], const int64_t bs[3], const int64_t cs[3]) {
+    for (int64_t bb = 0; bb < bsz; ++bb)
+        for (int64_t i = 0; i < m; ++i)
+            for (int64_t j = 0; j < n; ++j) {
+                float sum = 0.0f;
+                for (int64_t l = 0; l < k; ++l)
+                    sum += a[bb * as[0] + i * as[1] + l * as[2]] * b[bb * bs[0] + l * bs[1] + j * bs[2]];
+                c[bb * cs[0] + i * cs[1] + j * cs[2]] = sum;
+            }
+}
+
+/* What nn.Linear does on candy's CPU backend (nn/linear.go:58-112 -> cpu/storage.go:889-909):
+ * the weight is a [rows, cols] tensor viewed transposed with strides {1, cols}. */
+int co_matmul_dequant_f32(int fmt, const void *w_blocks, int64_t rows, int64_t cols,
+                          const float *x, int64_t m, float *y) {
+    int qk = co_block_elems(fmt);
+    if (qk == 0 || cols % qk != 0) return -1;
+    int64_t nel = rows * cols;
+    float *wf = (float *)malloc((size_t)(nel > 0 ? nel : 1) * sizeof(float));
+    if (!wf) return -2;
+    co_dequantize(fmt, w_blocks, rows * cols / qk, wf);
+    const int64_t as[3] = {0, cols, 1}, bs[3] = {0, 1, cols}, cs[3] = {0, rows, 1};
+    co_naive_batched_matmul_strided_f32(1, m, rows, cols, x, wf, y, as, bs, cs);
+    free(wf);
+    return 0;
+}
+
+/* RED:3071-3092 */
+void co_fast_rms_norm_f32(int64_t numel, int64_t ncols, float eps, const float *alpha,
+                          const float *x, float *dst) {
+    if (ncols <= 0) return;
+    int64_t rows = numel / ncols;
+    for (int64_t r = 0; r < rows; ++r) {
+        float sum = 0.0f;
+        for (int64_t c = 0; c < ncols; ++c) { float xi = x[r * ncols + c]; sum += xi * xi; }
+        float mean = sum / (float)ncols;
+        float scale = 1.0f / (float)sqrt((double)(mean + eps));
+        for (int64_t c = 0; c < ncols; ++c) {
+            int64_t i = r * ncols + c;
+            dst[i] = alpha ? scale * x[i] * alpha[c] : scale * x[i];
+        }
+    }
+}
+
+/* RED:3987-4006 */
+void co_rope_f32(int64_t bh, int64_t td, int64_t d, int64_t stride_b, const float *src,
+                 const float *cos_t, const float *sin_t, float *dst) {
+    int64_t num_pairs = bh * td / 2;
+    for (int64_t idx = 0; idx < num_pairs; ++idx) {
+        int64_t i_bh = idx / (td / 2);
+        int64_t i_td = idx - (td / 2) * i_bh;
+        int64_t i_t = i_td / (d / 2);
+        int64_t i_d = i_td - (d / 2) * i_t;
+        int64_t i1 = i_bh * td + i_t * d + i_d;
+        int64_t i2 = i1 + d / 2;
+        int64_t i_cs = i_t * (d / 2) + i_d;
+        if (stride_b > 0) i_cs += ((2 * idx) / stride_b) * (td / 2);
+        float c = cos_t[i_cs], s = sin_t[i_cs];
+        float a = src[i1], b = src[i2];
+        dst[i1] = a * c - b * s;
+        dst[i2] = a * s + b * c;
+    }
+}
+
+/* RED:2855-2879 */
+void co_fast_softmax_f32(int64_t numel, int64_t ncols, const float *src, float *dst) {
+    if (ncols <= 0) return;
+    int64_t rows = numel / ncols;
+    for (int64_t r = 0; r < rows; ++r) {
+        float max_val = -3.40282346638528859811704183484516925440e+38f;
+        for (int64_t c = 0; c < ncols; ++c) if (src[r * ncols + c] > max_val) max_val = src[r * ncols + c];
+        float sum = 0.0f;
+        for (int64_t c = 0; c < ncols; ++c) {
+            float v = (float)exp((double)(src[r * ncols + c] - max_val));
+            dst[r * ncols + c] = v;
+            sum += v;
+        }
+        float inv = 1.0f / sum;
+        for (int64_t c = 0; c < ncols; ++c) dst[r * ncols + c] *= inv;
+    }
+}
+
+/* UNA:3353-3366 */
+void co_silu_f32(int64_t numel, const float *inp, float *out) {
+    const float *s = inp ? inp : out;
+    for (int64_t i = 0; i < numel; ++i) { double x = (double)s[i]; out[i] = (float)(x / (1.0 + exp(-x))); }
+}
+
+/* RED:846-862 */
+void co_fast_argmax_f32(int64_t numel, int64_t ncols, const float *src, uint32_t *dst) {
+    if (ncols <= 0) return;
+    int64_t n = numel / ncols;
+    for (int64_t i = 0; i < n; ++i) {
+        float max_val = -3.40282346638528859811704183484516925440e+38f;
+        uint32_t max_idx = 0;
+        for (int64_t j = 0; j < ncols; ++j)
+            if (src[i * ncols + j] > max_val) { max_val = src[i * ncols + j]; max_idx = (uint32_t)j; }
+        dst[i] = max_idx;
+    }
+}
+
+/* IDX:8-26 (ids equal to MaxInt64 select zero) */
+void co_index_select_f32(int64_t numel, const int64_t *ids, const float *inp, float *out,
+                         int64_t left, int64_t src_dim, int64_t ids_dim, int64_t right) {
+    (void)left;
+    for (int64_t i = 0; i < numel; ++i) {
+        int64_t left_i = i / (ids_dim * right);
+        int64_t id_i = (i / right) % ids_dim;
+        int64_t right_i = i % right;
+        int64_t idx = ids[id_i];
+        if (idx == INT64_MAX) { out[i] = 0.0f; continue; }
+        out[i] = inp[left_i * src_dim * right + idx * right + right_i];
+    }
+}
+
+/* binary.go BAddF32 / BMulF32: plain elementwise loops */
+void co_add_f32(int64_t n, const float *a, const float *b, float *out) { for (int64_t i = 0; i < n; ++i) out[i] = a[i] + b[i]; }
+void co_mul_f32(int64_t n, const float *a, const float *b, float *out) { for (int64_t i = 0; i < n; ++i) out[i] = a[i] * b[i]; }
+
+void co_attention_decode_f32(const float *q, const float *k_cache, const float *v_cache,
+                             int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,
+                             int64_t n_pos, int64_t cache_stride, float scale, float *out) {
+    float *s = (float *)malloc((size_t)(n_pos ? n_pos : 1) * sizeof(float));
+    int64_t group = n_heads / n_kv_heads;
+    for (int64_t h = 0; h < n_heads; ++h) {
+        const float *kh = k_cache + (h / group) * cache_stride;
+        const float *vh = v_cache + (h / group) * cache_stride;
+        const float *qh = q + h * head_dim;
+        for (int64_t p = 0; p < n_pos; ++p) { /* q . K^T: CONV:251-267 with m=1 */
+            float sum = 0.0f;
+            for (int64_t d = 0; d < head_dim; ++d) sum += qh[d] * kh[p * head_dim + d];
+            s[p] = sum * scale;
+        }
+        co_fast_softmax_f32(n_pos, n_pos, s, s);
+        for (int64_t d = 0; d < head_dim; ++d) { /* p . V */
+            float sum = 0.0f;
+            for (int64_t p = 0; p < n_pos; ++p) sum += s[p] * vh[p * head_dim + d];
+            out[h * head_dim + d] = sum;
+        }
+    }
+    free(s);
+}
