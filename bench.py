@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+`python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line.
+
+Workload (the one the headline metric is quoted on): Q4_K weight 4096 x 11008
+(N outputs x K contraction, 25 362 432 bytes of blocks), batch 1, f32 activation in, f32
+output out.  A "step" is one pass of that path: quantize the activation to Q8_0 on the
+device, then the matvec.  Steps rotate over enough distinct copies of the weight (>= 512 MB)
+that none of it is still in the 256 MB last-level cache when it is read again, so `value` is
+an HBM figure.  Inputs are resident in HBM before the timed region starts.
+
+Extra objects on the same line:
+  roofline     the matvec kernel alone (activations quantized before the timed region), timed
+               with HIP events on the library's stream over the same rotation.
+  cpu_baseline candy's literal CPU composition (dequantize, then the naive f32 matmul loops)
+               restated in C, single thread, on a bounded sample of the same workload.
+  sweep        the other shapes / formats of the batch-1 sweep (GB/s of the matvec kernel).
+  decode       random-init 7B Q4_K decode step, tokens/s.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+ROTATE_BYTES = 640 << 20  # distinct weight bytes cycled through (last-level cache is 256 MB)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def algorithmic_bytes(fmt, rows, cols, m=1):
+    from candy_amd import synth
+    return synth.weight_nbytes(fmt, rows, cols) + 4 * m * cols + 4 * m * rows
+
+
+def make_rotation(dev, fmt, rows, cols, seed):
+    """Distinct device copies of one random weight shape, >= ROTATE_BYTES in total."""
+    from candy_amd import synth
+    nbytes = synth.weight_nbytes(fmt, rows, cols)
+    n = max(2, -(-ROTATE_BYTES // nbytes))
+    base = synth.random_weight(fmt, rows, cols, seed=seed)
+    ws = []
+    for i in range(n):
+        # cheap distinct contents: rotate the block array (still valid blocks, still random)
+        blk = synth.BLOCK_BYTES[fmt]
+        ws.append(dev.qtensor(fmt, rows, cols, np.roll(base.reshape(-1, blk), i, axis=0).reshape(-1)))
+    return ws, nbytes
+
+
+def time_matvec(dev, fmt, rows, cols, steps, warmup, quantize_each, seed=1, m=1):
+    from candy_amd import synth
+    ws, nbytes = make_rotation(dev, fmt, rows, cols, seed)
+    x = dev.from_numpy(synth.random_activations(m, cols, seed=seed + 1))
+    y = dev.alloc(4 * m * rows)
+    dev.qmatmul_sweep(ws, x, m, y, warmup, quantize_each)
+    ms = dev.qmatmul_sweep(ws, x, m, y, steps, quantize_each)
+    for w in ws:
+        w.free()
+    return ms / steps, len(ws)
+
+
+def cpu_baseline(rows, cols, budget_s=12.0):
+    """candy's CPU path (dequantize + naive f32 loops), C restatement, one thread."""
+    from candy_amd import synth
+    from oracle import oracle as o
+    fmt = synth.Q4_K
+    sample_rows = 512  # a slice of the same weight keeps one call short
+    w = synth.random_weight(fmt, sample_rows, cols, seed=77)
+    x = synth.random_activations(1, cols, seed=78)
+    o.matmul_dequant_f32(fmt, w, sample_rows, cols, x)  # warm
+    t0 = time.perf_counter()
+    calls = 0
+    while time.perf_counter() - t0 < budget_s:
+        o.matmul_dequant_f32(fmt, w, sample_rows, cols, x)
+        calls += 1
+    dt = time.perf_counter() - t0
+    per_full = dt / calls * (rows / sample_rows)
+    gbps = algorithmic_bytes(fmt, rows, cols) / per_full / 1e9
+    return {"value": round(gbps, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{calls} calls of dequantize+naive-f32-matmul on a {sample_rows}x{cols} Q4_K slice "
+                      f"({dt:.1f} s), scaled to {rows} rows; host has {os.cpu_count()} logical CPUs",
+            "ms_per_step": round(per_full * 1e3, 3)}
+
+
+def build_7b(dev, n_layers=32, max_pos=2176, seed=4000):
+    """Random-init Llama-7B-shaped decoder: Q4_K linears, Q6_K head, Q8_0 embedding rows."""
+    from candy_amd import hip, synth
+    cfg = dict(n_layers=n_layers, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=11008, vocab=32000,
+               max_pos=max_pos, rms_eps=1e-5, rope_base=10000.0)
+    model = hip.Llama(dev, **cfg)
+    shapes = [(hip.W_Q, 4096, 4096), (hip.W_K, 4096, 4096), (hip.W_V, 4096, 4096), (hip.W_O, 4096, 4096),
+              (hip.W_GATE, 11008, 4096), (hip.W_UP, 11008, 4096), (hip.W_DOWN, 4096, 11008)]
+    ones = np.ones(4096, np.float32)
+    sc = synth.unit_scale(synth.Q4_K)
+    t0 = time.perf_counter()
+    for l in range(n_layers):
+        for kind, r, k in shapes:
+            seed += 1
+            model.set_qweight(kind, l, dev.qtensor(synth.Q4_K, r, k, synth.random_weight(synth.Q4_K, r, k, seed, sc)))
+        model.set_norm(hip.W_ATTN_NORM, l, ones)
+        model.set_norm(hip.W_FFN_NORM, l, ones)
+        if l % 8 == 7:
+            log(f"  built layer {l + 1}/{n_layers} ({time.perf_counter() - t0:.0f} s)")
+    model.set_norm(hip.W_OUT_NORM, -1, ones)
+    model.set_qweight(hip.W_HEAD, -1, dev.qtensor(synth.Q6_K, 32000, 4096, synth.random_weight(
+        synth.Q6_K, 32000, 4096, seed + 1, synth.unit_scale(synth.Q6_K))))
+    model.set_qweight(hip.W_EMBED, -1, dev.qtensor(synth.Q8_0, 32000, 4096, synth.random_weight(
+        synth.Q8_0, 32000, 4096, seed + 2, synth.unit_scale(synth.Q8_0))))
+    return cfg, model
+
+
+def prefill_kv(dev, model, cfg, n_pos, seed=9):
+    """KV cache positions [0, n_pos) <- N(0,1) f32."""
+    from candy_amd import hip
+    kptr, vptr, nbytes = model.kv_cache()
+    rng = np.random.Generator(np.random.Philox(seed))
+    per_head = cfg["max_pos"] * cfg["head_dim"]
+    rows = cfg["n_layers"] * cfg["n_kv_heads"]
+    chunk = np.empty((cfg["n_kv_heads"], n_pos, cfg["head_dim"]), np.float32)
+    for base in (kptr, vptr):
+        for l in range(cfg["n_layers"]):
+            rng.standard_normal(chunk.shape, dtype=np.float32, out=chunk)
+            for h in range(cfg["n_kv_heads"]):
+                off = ((l * cfg["n_kv_heads"] + h) * per_head) * 4
+                hip._check(hip.lib().candy_hip_h2d(dev.handle, base + off, chunk[h].ctypes.data, chunk[h].nbytes))
+    del rows
+
+
+def decode_leg(dev, steps, warmup):
+    from candy_amd import synth
+    log("building random-init 7B (Q4_K, Q6_K head) ...")
+    n_pos = 2048
+    cfg, model = build_7b(dev, max_pos=n_pos + steps + warmup + 8)
+    prefill_kv(dev, model, cfg, n_pos)
+    rng = np.random.default_rng(1234)
+    prompt = rng.integers(0, cfg["vocab"], 128)
+    tok = int(prompt[-1])
+    pos = n_pos
+    for _ in range(warmup):
+        tok, _ = model.decode(tok, pos, want_logits=False)
+        pos += 1
+    dev.synchronize()
+    t0 = time.perf_counter()
+    toks = []
+    for _ in range(steps):
+        tok, _ = model.decode(tok, pos, want_logits=False)
+        toks.append(tok)
+        pos += 1
+    dev.synchronize()
+    dt = time.perf_counter() - t0
+    layer_bytes = 4 * synth.weight_nbytes(synth.Q4_K, 4096, 4096) + 3 * synth.weight_nbytes(synth.Q4_K, 11008, 4096)
+    kv_bytes = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * n_pos * cfg["head_dim"] * 4
+    bpt = cfg["n_layers"] * layer_bytes + synth.weight_nbytes(synth.Q6_K, 32000, 4096) + kv_bytes
+    ms = dt / steps * 1e3
+    model.free()
+    return {"tok_s": round(steps / dt, 2), "ms_per_token": round(ms, 4), "steps": steps, "kv_positions": n_pos,
+            "bytes_per_token": bpt, "hbm_GBps": round(bpt / (ms * 1e-3) / 1e9, 1),
+            "hbm_frac": round(bpt / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "tokens": toks[:8]}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the other shapes of the batch-1 sweep")
+    ap.add_argument("--no-decode", action="store_true", help="skip the 7B decode leg")
+    ap.add_argument("--decode-steps", type=int, default=32)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE MI355X; --gpus must be 1 (no collectives, no sharding)")
+
+    from candy_amd import hip, synth
+    dev = hip.Device(0)
+    log("device:", dev.name)
+    fmt, rows, cols = synth.Q4_K, 4096, 11008
+    alg = algorithmic_bytes(fmt, rows, cols)
+
+    # headline: whole f32-in -> f32-out path
+    ms_step, n_copies = time_matvec(dev, fmt, rows, cols, args.steps, args.warmup, quantize_each=True)
+    value = alg / (ms_step * 1e-3) / 1e9
+    # dominant kernel alone
+    ms_kernel, _ = time_matvec(dev, fmt, rows, cols, args.steps, args.warmup, quantize_each=False)
+    achieved = alg / (ms_kernel * 1e-3) / 1e9
+    log(f"Q4_K {rows}x{cols}: path {ms_step * 1e3:.2f} us/step = {value:.0f} GB/s; "
+        f"matvec kernel {ms_kernel * 1e3:.2f} us = {achieved:.0f} GB/s ({achieved / HBM_PEAK_GBPS:.1%} of 8 TB/s)")
+
+    out = {
+        "metric": "Q4_K matvec GB/s (batch 1, 4096x11008, f32 in -> f32 out)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8", "data": "synthetic",
+        "config": {"workload": "configs[1]: Q4_K 4096x11008 (N x K) batch-1 matvec, activation quantized to Q8_0 "
+                               "on device each step", "weight_bytes": synth.weight_nbytes(fmt, rows, cols),
+                   "algorithmic_bytes_per_step": alg, "distinct_weight_copies": n_copies,
+                   "device": dev.name},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "k_matvec<UnitQ4K>", "us_per_launch": round(ms_kernel * 1e3, 3)},
+    }
+
+    if not args.no_sweep:
+        sweep = []
+        s_steps, s_warm = max(200, args.steps // 4), max(20, args.warmup // 4)
+        for f, name in ((synth.Q4_K, "q4_k"), (synth.Q8_0, "q8_0")):
+            for r, k in ((4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)):
+                ms, _ = time_matvec(dev, f, r, k, s_steps, s_warm, quantize_each=False, seed=r + k)
+                gb = algorithmic_bytes(f, r, k) / (ms * 1e-3) / 1e9
+                sweep.append({"fmt": name, "rows": r, "cols": k, "us": round(ms * 1e3, 3), "GBps": round(gb, 1),
+                              "frac": round(gb / HBM_PEAK_GBPS, 4)})
+                log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
+        for f, name, r, k in ((synth.Q6_K, "q6_k", 32000, 4096), (synth.Q4_0, "q4_0", 4096, 4096)):
+            ms, _ = time_matvec(dev, f, r, k, s_steps, s_warm, quantize_each=False, seed=r + k + f)
+            gb = algorithmic_bytes(f, r, k) / (ms * 1e-3) / 1e9
+            sweep.append({"fmt": name, "rows": r, "cols": k, "us": round(ms * 1e3, 3), "GBps": round(gb, 1),
+                          "frac": round(gb / HBM_PEAK_GBPS, 4)})
+            log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
+        out["sweep"] = sweep
+
+    if not args.no_decode:
+        out["decode"] = decode_leg(dev, args.decode_steps, 4)
+        log("decode:", out["decode"])
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(rows, cols)
+        log("cpu baseline:", out["cpu_baseline"])
+    else:
+        out["cpu_baseline"] = None
+
+    dev.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

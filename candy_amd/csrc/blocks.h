@@ -1,0 +1,78 @@
+// Device-side view of candy's block formats
+// (tensor/internal/cpu/kernels/quantized.go:8-11, 34-37, 55-59, 70-75; little-endian, packed).
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace candy {
+
+struct __attribute__((packed)) BlockQ4_0 {
+    uint16_t d;
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ8_0 {
+    uint16_t d;
+    int8_t qs[32];
+};
+struct __attribute__((packed)) BlockQ4K {
+    uint16_t d, dmin;
+    uint8_t scales[12];
+    uint8_t qs[128];
+};
+struct __attribute__((packed)) BlockQ6K {
+    uint8_t ql[128];
+    uint8_t qh[64];
+    int8_t scales[16];
+    uint16_t d;
+};
+static_assert(sizeof(BlockQ4_0) == 18 && sizeof(BlockQ8_0) == 34, "block size");
+static_assert(sizeof(BlockQ4K) == 144 && sizeof(BlockQ6K) == 210, "block size");
+
+// Vector types whose loads may sit on 2-byte boundaries (Q8_0 / Q4_0 / Q6_K blocks are only
+// 2-byte aligned); gfx950 global loads accept unaligned addresses.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+typedef uint32_t u32_a2 __attribute__((aligned(2)));
+
+// IEEE half -> single; exact for every input including subnormals
+// (same mapping as fp16ToFloat32, quantized.go:149-173).
+__device__ __forceinline__ float half_bits_to_float(uint16_t h) {
+    return __half2float(__ushort_as_half(h));
+}
+
+// The 6-bit (scale, min) pairs of sub-blocks 2*pair and 2*pair+1 of a Q4_K super-block,
+// unpacked on 16-bit lanes (get_scale_min_k4, quantized.cu:993-1005).
+// s0, s1, s2 are scales[0..3], scales[4..7], scales[8..11] as little-endian words.
+// Returns sc in bytes 0,1 of `sc2` and m in bytes 0,1 of `m2`.
+__device__ __forceinline__ void q4k_scale_min_pair(uint32_t s0, uint32_t s1, uint32_t s2, int pair,
+                                                   uint32_t &sc2, uint32_t &m2) {
+    const int sh = (pair & 1) * 16;
+    const uint32_t a = (s0 >> sh) & 0xFFFFu, b = (s1 >> sh) & 0xFFFFu, c = (s2 >> sh) & 0xFFFFu;
+    const uint32_t sc_lo = a & 0x3F3Fu, m_lo = b & 0x3F3Fu;
+    const uint32_t sc_hi = (c & 0x0F0Fu) | ((a & 0xC0C0u) >> 2);
+    const uint32_t m_hi = ((c >> 4) & 0x0F0Fu) | ((b & 0xC0C0u) >> 2);
+    sc2 = pair < 2 ? sc_lo : sc_hi;
+    m2 = pair < 2 ? m_lo : m_hi;
+}
+
+__device__ __forceinline__ int dot4_i8(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// Sum over the 64 lanes of a wavefront; every lane gets the total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+}  // namespace candy

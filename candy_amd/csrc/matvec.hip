@@ -1,0 +1,421 @@
+// Batch-1 (and small-batch, m < 16) quantized matvec: y[m, N] = x[m, K] . W^T with W in candy's
+// block formats and x pre-quantized to planar Q8_0.  Bandwidth-bound: the weights are read
+// exactly once, 16 bytes per load, straight from the original block layout.
+//
+// Arithmetic follows the integer vec-dots of tensor/internal/cuda/kernels/quantized.cu
+// (vec_dot_q4_0_q8_1 :1919-1941, vec_dot_q8_0_q8_1 :2058-2073, vec_dot_q4_K_q8_1 :2239-2263,
+// vec_dot_q6_K_q8_1 :2367-2389) with Q8_0 activations; the launch shape replaces
+// mul_mat_vec_q (:2787-2871), which is laid out for 32-wide warps.
+//
+// Work split: a workgroup of WAVES wavefronts stages the quantized activations in LDS once,
+// then every wavefront owns R consecutive weight rows.  A lane owns one "unit" of the row
+// (64 weights of a Q4_K super-block, 32 weights otherwise) per step, so consecutive lanes read
+// consecutive bytes of the row; the R rows' loads are issued together to keep many bytes in
+// flight per wavefront.  Per-row partial sums are reduced across the 64 lanes at the end.
+#include "blocks.h"
+#include "internal.h"
+
+namespace candy {
+
+// LDS image of the activations: quants with 16 bytes of skew per 256 bytes (keeps 16-byte
+// reads of lanes that are 32 or 64 bytes apart on distinct banks), then the scales.
+__device__ __forceinline__ int skewed(int byte_off) { return byte_off + ((byte_off >> 8) << 4); }
+
+template <int NB, int THREADS>
+__device__ __forceinline__ void stage_activations(const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs,
+                                                  int K, uint8_t *smem, int8_t *&sq, Q8Scale *&ss) {
+    const int q_bytes = skewed(K);  // per activation row, a multiple of 16
+    sq = (int8_t *)smem;
+    ss = (Q8Scale *)(smem + NB * q_bytes);
+    const int chunks = K >> 4;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const uint4 *src = (const uint4 *)(xq + (size_t)nb * K);
+        uint4 *dst = (uint4 *)(sq + nb * q_bytes);
+        for (int c = threadIdx.x; c < chunks; c += THREADS) dst[c + (c >> 4)] = src[c];
+    }
+    const uint2 *s2 = (const uint2 *)xs;
+    uint2 *d2 = (uint2 *)ss;
+    for (int i = threadIdx.x; i < NB * (K >> 5); i += THREADS) d2[i] = s2[i];
+    __syncthreads();
+}
+
+// ------------------------------------------------------------------ per-format units
+
+struct UnitQ4K {
+    static constexpr int ELEMS = 64;        // two 32-value sub-blocks sharing 32 bytes of nibbles
+    static constexpr int ROW_ALIGN = 16;
+    struct W { uint4 hdr, q0, q1; };
+    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 144; }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const uint8_t *blk = row + (size_t)(u >> 2) * 144;
+        w.hdr = *(const uint4 *)blk;
+        const uint4 *q = (const uint4 *)(blk + 16 + (u & 3) * 32);
+        w.q0 = q[0];
+        w.q1 = q[1];
+    }
+    // sum over the unit of w*x, with x = d_x * q_x: quantized.cu:2239-2263
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        const uint4 *xa = (const uint4 *)(sq + skewed(u * 64));
+        const uint4 x0 = xa[0], x1 = xa[1], x2 = xa[2], x3 = xa[3];
+        const Q8Scale s0 = ss[2 * u], s1 = ss[2 * u + 1];
+        uint32_t sc2, m2;
+        q4k_scale_min_pair(w.hdr.y, w.hdr.z, w.hdr.w, u & 3, sc2, m2);
+        const uint32_t M = 0x0F0F0F0Fu;
+        int lo = 0, hi = 0;
+        lo = dot4_i8(w.q0.x & M, x0.x, lo); hi = dot4_i8((w.q0.x >> 4) & M, x2.x, hi);
+        lo = dot4_i8(w.q0.y & M, x0.y, lo); hi = dot4_i8((w.q0.y >> 4) & M, x2.y, hi);
+        lo = dot4_i8(w.q0.z & M, x0.z, lo); hi = dot4_i8((w.q0.z >> 4) & M, x2.z, hi);
+        lo = dot4_i8(w.q0.w & M, x0.w, lo); hi = dot4_i8((w.q0.w >> 4) & M, x2.w, hi);
+        lo = dot4_i8(w.q1.x & M, x1.x, lo); hi = dot4_i8((w.q1.x >> 4) & M, x3.x, hi);
+        lo = dot4_i8(w.q1.y & M, x1.y, lo); hi = dot4_i8((w.q1.y >> 4) & M, x3.y, hi);
+        lo = dot4_i8(w.q1.z & M, x1.z, lo); hi = dot4_i8((w.q1.z >> 4) & M, x3.z, hi);
+        lo = dot4_i8(w.q1.w & M, x1.w, lo); hi = dot4_i8((w.q1.w >> 4) & M, x3.w, hi);
+        const float d = half_bits_to_float((uint16_t)(w.hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_float((uint16_t)(w.hdr.x >> 16));
+        const float sd = s0.d * (float)(lo * (int)(sc2 & 0xFF)) + s1.d * (float)(hi * (int)(sc2 >> 8));
+        const float sm = s0.d * (float)(s0.bsum * (int)(m2 & 0xFF)) + s1.d * (float)(s1.bsum * (int)(m2 >> 8));
+        return d * sd - dmin * sm;
+    }
+};
+
+struct UnitQ8_0 {
+    static constexpr int ELEMS = 32;
+    static constexpr int ROW_ALIGN = 2;
+    struct W { u32x4 q0, q1; uint16_t d; };
+    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 34; }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const BlockQ8_0 *blk = (const BlockQ8_0 *)row + u;
+        w.d = blk->d;
+        w.q0 = *(const u32x4_a2 *)(blk->qs);
+        w.q1 = *(const u32x4_a2 *)(blk->qs + 16);
+    }
+    // quantized.cu:2058-2073
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        const uint4 *xa = (const uint4 *)(sq + skewed(u * 32));
+        const uint4 x0 = xa[0], x1 = xa[1];
+        int s = 0;
+        s = dot4_i8(w.q0.x, x0.x, s); s = dot4_i8(w.q0.y, x0.y, s); s = dot4_i8(w.q0.z, x0.z, s); s = dot4_i8(w.q0.w, x0.w, s);
+        s = dot4_i8(w.q1.x, x1.x, s); s = dot4_i8(w.q1.y, x1.y, s); s = dot4_i8(w.q1.z, x1.z, s); s = dot4_i8(w.q1.w, x1.w, s);
+        return (half_bits_to_float(w.d) * ss[u].d) * (float)s;
+    }
+};
+
+template <bool GGML_ORDER>
+struct UnitQ4_0 {
+    static constexpr int ELEMS = 32;
+    static constexpr int ROW_ALIGN = 2;
+    struct W { u32x4 q; uint16_t d; };
+    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 18; }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const BlockQ4_0 *blk = (const BlockQ4_0 *)row + u;
+        w.d = blk->d;
+        w.q = *(const u32x4_a2 *)(blk->qs);
+    }
+    // Sum (q-8)*x = sum q*x - 8*sum x, all in integers. quantized.cu:1919-1941 gets the
+    // second term from the Q8_1 block's float sum; with Q8_0 activations it is the exact integer.
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        const uint4 *xa = (const uint4 *)(sq + skewed(u * 32));
+        const uint4 x0 = xa[0], x1 = xa[1];
+        const Q8Scale sx = ss[u];
+        const uint32_t M = 0x0F0F0F0Fu;
+        int s = 0;
+        if (GGML_ORDER) {
+            // low nibble of byte j pairs with x[j], high nibble with x[j+16] (quantized.cu:2426-2433)
+            s = dot4_i8(w.q.x & M, x0.x, s); s = dot4_i8((w.q.x >> 4) & M, x1.x, s);
+            s = dot4_i8(w.q.y & M, x0.y, s); s = dot4_i8((w.q.y >> 4) & M, x1.y, s);
+            s = dot4_i8(w.q.z & M, x0.z, s); s = dot4_i8((w.q.z >> 4) & M, x1.z, s);
+            s = dot4_i8(w.q.w & M, x0.w, s); s = dot4_i8((w.q.w >> 4) & M, x1.w, s);
+        } else {
+            // candy CPU order (quantized.go:87-92): byte j holds elements 2j (low) and 2j+1 (high);
+            // gather the even and odd activation bytes of each 8-element run
+            const uint32_t xs8[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            const uint32_t qw[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t even = __builtin_amdgcn_perm(xs8[2 * j + 1], xs8[2 * j], 0x06040200u);
+                const uint32_t odd = __builtin_amdgcn_perm(xs8[2 * j + 1], xs8[2 * j], 0x07050301u);
+                s = dot4_i8(qw[j] & M, even, s);
+                s = dot4_i8((qw[j] >> 4) & M, odd, s);
+            }
+        }
+        s -= 8 * sx.bsum;
+        return (half_bits_to_float(w.d) * sx.d) * (float)s;
+    }
+};
+
+struct UnitQ6K {
+    static constexpr int ELEMS = 32;   // 8 values from each 32-value quarter of one 128-value half
+    static constexpr int ROW_ALIGN = 2;
+    struct W { u32x2 ql0, ql1, qh; uint32_t sc; uint16_t d; };
+    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 210; }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const BlockQ6K *blk = (const BlockQ6K *)row + (u >> 3);
+        const int ip = (u >> 2) & 1, j = u & 3;
+        w.ql0 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 8 * j);
+        w.ql1 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 32 + 8 * j);
+        w.qh = *(const u32x2_a2 *)(blk->qh + 32 * ip + 8 * j);
+        const int8_t *sc = blk->scales + 8 * ip + (j >> 1);
+        w.sc = (uint32_t)(uint8_t)sc[0] | ((uint32_t)(uint8_t)sc[2] << 8) | ((uint32_t)(uint8_t)sc[4] << 16) |
+               ((uint32_t)(uint8_t)sc[6] << 24);
+        w.d = blk->d;
+    }
+    // quantized.cu:2367-2389: d * sum over 16-value groups of d8 * (dot * scale); the -32 offset is
+    // applied as dot(q,x) - 32*sum(x) in integers.
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        const int sb = u >> 3, ip = (u >> 2) & 1, j = u & 3;
+        const int blk0 = sb * 8 + ip * 4;  // first of the four 32-value activation blocks
+        float sumf = 0.0f;
+        const uint32_t M = 0x0F0F0F0Fu, H = 0x30303030u, ones = 0x01010101u;
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            const uint2 x = *(const uint2 *)(sq + skewed((blk0 + qd) * 32 + 8 * j));
+            const u32x2 ql = (qd & 1) ? w.ql1 : w.ql0;
+            const uint32_t lx = (qd < 2) ? (ql.x & M) : ((ql.x >> 4) & M);
+            const uint32_t ly = (qd < 2) ? (ql.y & M) : ((ql.y >> 4) & M);
+            const uint32_t vx = lx | (((w.qh.x >> (2 * qd)) << 4) & H);
+            const uint32_t vy = ly | (((w.qh.y >> (2 * qd)) << 4) & H);
+            int dq = dot4_i8(vy, x.y, dot4_i8(vx, x.x, 0));
+            const int sx = dot4_i8(ones, x.y, dot4_i8(ones, x.x, 0));
+            dq -= 32 * sx;
+            const int scale = (int)(int8_t)((w.sc >> (8 * qd)) & 0xFF);
+            sumf += ss[blk0 + qd].d * (float)(dq * scale);
+        }
+        return half_bits_to_float(w.d) * sumf;
+    }
+};
+
+// ------------------------------------------------------------------ kernel
+
+template <class U, int NB, int R, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
+                                                       const Q8Scale *__restrict__ xs, float *__restrict__ y,
+                                                       int N, int K) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    int8_t *sq;
+    Q8Scale *ss;
+    stage_activations<NB, WAVES * 64>(xq, xs, K, smem, sq, ss);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row0 = (blockIdx.x * WAVES + wave) * R;
+    if (row0 >= N) return;
+    const int units = K / U::ELEMS;
+    const size_t rb = U::row_bytes(K);
+    const int q_bytes = skewed(K);
+    const int blocks_per_row = K >> 5;
+
+    float acc[R][NB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.0f;
+
+    for (int u = lane; u < units; u += 64) {
+        typename U::W w[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int row = min(row0 + r, N - 1);  // tail rows recompute the last row, never stored
+            U::load(W + (size_t)row * rb, u, w[r]);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][nb] += U::dot(w[r], u, sq + nb * q_bytes, ss + nb * blocks_per_row);
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const float v = wave_sum(acc[r][nb]);
+            if (lane == 0 && row0 + r < N) y[(size_t)nb * N + row0 + r] = v;
+        }
+}
+
+template <class U, int NB, int R, int WAVES>
+static int launch_one(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                      float *y) {
+    const int N = (int)w->rows, K = (int)w->cols;
+    const size_t q_bytes = (size_t)K + (((size_t)K >> 8) << 4);
+    const size_t smem = NB * (q_bytes + (size_t)(K >> 5) * sizeof(Q8Scale));
+    CANDY_REQUIRE(smem <= 64 * 1024, "contraction dim %d too large for the matvec kernel (%zu bytes of LDS)", K, smem);
+    const int rows_per_wg = R * WAVES;
+    const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
+    hipLaunchKernelGGL((k_matvec<U, NB, R, WAVES>), dim3(grid), dim3(WAVES * 64), smem, dev->stream,
+                       (const uint8_t *)w->data, qs, scales, y, N, K);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+template <class U>
+static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                      int64_t m, float *y) {
+    const int64_t K = w->cols, N = w->rows;
+    const int64_t sstride = K >> 5;
+    int64_t done = 0;
+    while (done < m) {
+        const int64_t left = m - done;
+        const int8_t *q = qs + done * K;
+        const Q8Scale *s = scales + done * sstride;
+        float *yo = y + done * N;
+        int rc;
+        // LDS holds NB activation rows; keep the workgroup's share under 64 KB
+        if (left >= 4 && K <= 8192) { rc = launch_one<U, 4, 2, 4>(dev, w, q, s, yo); done += 4; }
+        else if (left >= 2 && K <= 16384) { rc = launch_one<U, 2, 2, 4>(dev, w, q, s, yo); done += 2; }
+        else { rc = launch_one<U, 1, 2, 4>(dev, w, q, s, yo); done += 1; }
+        if (rc) return rc;
+    }
+    return CANDY_HIP_OK;
+}
+
+int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                  int64_t m, float *y) {
+    CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && w->cols <= 0x7FFFFFFF, "matrix too large");
+    switch (w->fmt) {
+    case CANDY_HIP_Q4_K: return launch_fmt<UnitQ4K>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q8_0: return launch_fmt<UnitQ8_0>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q4_0: return launch_fmt<UnitQ4_0<false>>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q4_0_GGML: return launch_fmt<UnitQ4_0<true>>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q6_K: return launch_fmt<UnitQ6K>(dev, w, qs, scales, m, y);
+    default: return fail(CANDY_HIP_ERR_INVALID, "unknown quantized format %d", w->fmt);
+    }
+}
+
+}  // namespace candy
+
+using namespace candy;
+
+extern "C" {
+
+static int qmatmul_common(candy_hip_device *dev, const candy_hip_qtensor *w, int64_t m, float *dev_y,
+                          size_t *q_off, size_t *s_off, size_t *total) {
+    CANDY_REQUIRE(w, "rhs qtensor is nil");
+    CANDY_REQUIRE(dev && w->dev == dev, "rhs storage must live on the same HIP device");
+    CANDY_REQUIRE(m >= 0, "invalid matrix dimensions");
+    CANDY_REQUIRE(m == 0 || dev_y, "output is nil");
+    const size_t qb = (size_t)m * (size_t)w->cols;
+    *q_off = 0;
+    *s_off = (qb + 255) & ~(size_t)255;
+    *total = *s_off + (size_t)m * (size_t)(w->cols >> 5) * sizeof(Q8Scale);
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m, float *dev_y) {
+    size_t q_off, s_off, total;
+    if (int rc = qmatmul_common(dev, w, m, dev_y, &q_off, &s_off, &total)) return rc;
+    if (m == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dev_x, "lhs is nil");
+    CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "lhs must be 16-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    void *ws = nullptr;
+    if (int rc = workspace(dev, total, &ws)) return rc;
+    int8_t *qs = (int8_t *)ws + q_off;
+    Q8Scale *sc = (Q8Scale *)((uint8_t *)ws + s_off);
+    if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, qs, sc, nullptr)) return rc;
+    return m < 16 ? launch_matvec(dev, w, qs, sc, m, dev_y) : launch_mmq(dev, w, qs, sc, m, dev_y);
+}
+
+int candy_hip_qmatmul_q8(candy_hip_device *dev, const candy_hip_qtensor *w, const void *dev_x_q8_0, int64_t m,
+                         float *dev_y) {
+    size_t q_off, s_off, total;
+    if (int rc = qmatmul_common(dev, w, m, dev_y, &q_off, &s_off, &total)) return rc;
+    if (m == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dev_x_q8_0, "lhs is nil");
+    CANDY_REQUIRE(((uintptr_t)dev_x_q8_0 & 1) == 0, "lhs blocks must be 2-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    void *ws = nullptr;
+    if (int rc = workspace(dev, total, &ws)) return rc;
+    int8_t *qs = (int8_t *)ws + q_off;
+    Q8Scale *sc = (Q8Scale *)((uint8_t *)ws + s_off);
+    if (int rc = launch_q8_blocks_to_planar(dev, dev_x_q8_0, m * (w->cols >> 5), qs, sc)) return rc;
+    return m < 16 ? launch_matvec(dev, w, qs, sc, m, dev_y) : launch_mmq(dev, w, qs, sc, m, dev_y);
+}
+
+int candy_hip_qact_create(candy_hip_device *dev, int64_t max_m, int64_t max_cols, candy_hip_qact **out) {
+    CANDY_REQUIRE(out, "out is nil");
+    *out = nullptr;
+    CANDY_REQUIRE(max_m > 0 && max_cols > 0 && max_cols % 32 == 0, "invalid capacity %lld x %lld", (long long)max_m,
+                  (long long)max_cols);
+    if (int rc = use_device(dev)) return rc;
+    candy_hip_qact *a = new candy_hip_qact();
+    a->dev = dev;
+    a->max_m = max_m;
+    a->max_cols = max_cols;
+    void *q = nullptr, *s = nullptr;
+    int rc = candy_hip_alloc(dev, (size_t)(max_m * max_cols), &q);
+    if (!rc) rc = candy_hip_alloc(dev, (size_t)(max_m * (max_cols >> 5)) * sizeof(Q8Scale), &s);
+    if (rc) {
+        if (q) (void)candy_hip_free(dev, q);
+        delete a;
+        return rc;
+    }
+    a->qs = (int8_t *)q;
+    a->scales = (Q8Scale *)s;
+    *out = a;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_qact_free(candy_hip_qact *a) {
+    if (!a) return CANDY_HIP_OK;
+    int rc = candy_hip_free(a->dev, a->qs);
+    int rc2 = candy_hip_free(a->dev, a->scales);
+    delete a;
+    return rc ? rc : rc2;
+}
+
+int candy_hip_qact_quantize(candy_hip_qact *a, const float *dev_x, int64_t m, int64_t cols) {
+    CANDY_REQUIRE(a, "qact is nil");
+    CANDY_REQUIRE(m > 0 && cols > 0, "invalid matrix dimensions");
+    CANDY_REQUIRE(cols % 32 == 0, "cols %lld is not a multiple of the block size 32", (long long)cols);
+    CANDY_REQUIRE(m * cols <= a->max_m * a->max_cols, "%lld x %lld exceeds the capacity %lld x %lld", (long long)m,
+                  (long long)cols, (long long)a->max_m, (long long)a->max_cols);
+    CANDY_REQUIRE(dev_x && ((uintptr_t)dev_x & 15) == 0, "input must be non-nil and 16-byte aligned");
+    if (int rc = use_device(a->dev)) return rc;
+    a->m = m;
+    a->cols = cols;
+    return launch_quantize_q8(a->dev, dev_x, m, cols, a->qs, a->scales, nullptr);
+}
+
+int candy_hip_qmatmul_qact(candy_hip_device *dev, const candy_hip_qtensor *w, const candy_hip_qact *a, float *dev_y) {
+    CANDY_REQUIRE(w && a, "nil argument");
+    CANDY_REQUIRE(dev && w->dev == dev && a->dev == dev, "operands must live on the same HIP device");
+    CANDY_REQUIRE(a->m > 0, "activations have not been quantized yet");
+    CANDY_REQUIRE(a->cols == w->cols, "activation width %lld does not match the weight's contraction dim %lld",
+                  (long long)a->cols, (long long)w->cols);
+    CANDY_REQUIRE(dev_y, "output is nil");
+    if (int rc = use_device(dev)) return rc;
+    return a->m < 16 ? launch_matvec(dev, w, a->qs, a->scales, a->m, dev_y)
+                     : launch_mmq(dev, w, a->qs, a->scales, a->m, dev_y);
+}
+
+int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws, const float *dev_x,
+                            int64_t m, float *dev_y, int iters, int quantize_each, float *elapsed_ms) {
+    CANDY_REQUIRE(dev && ws && n_ws > 0 && dev_x && dev_y && elapsed_ms, "nil argument");
+    CANDY_REQUIRE(m > 0 && iters > 0, "invalid iteration count or batch");
+    for (int i = 0; i < n_ws; ++i) {
+        CANDY_REQUIRE(ws[i] && ws[i]->dev == dev, "weight %d is nil or on another device", i);
+        CANDY_REQUIRE(ws[i]->cols == ws[0]->cols && ws[i]->rows == ws[0]->rows, "weights must share one shape");
+    }
+    CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "lhs must be 16-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    const int64_t K = ws[0]->cols;
+    const size_t s_off = ((size_t)(m * K) + 255) & ~(size_t)255;
+    void *wsp = nullptr;
+    if (int rc = workspace(dev, s_off + (size_t)(m * (K >> 5)) * sizeof(Q8Scale), &wsp)) return rc;
+    int8_t *qs = (int8_t *)wsp;
+    Q8Scale *sc = (Q8Scale *)((uint8_t *)wsp + s_off);
+    if (int rc = launch_quantize_q8(dev, dev_x, m, K, qs, sc, nullptr)) return rc;
+    CANDY_HIP_TRY(hipEventRecord(dev->ev_start, dev->stream));
+    for (int i = 0; i < iters; ++i) {
+        if (quantize_each)
+            if (int rc = launch_quantize_q8(dev, dev_x, m, K, qs, sc, nullptr)) return rc;
+        const candy_hip_qtensor *w = ws[i % n_ws];
+        if (int rc = m < 16 ? launch_matvec(dev, w, qs, sc, m, dev_y) : launch_mmq(dev, w, qs, sc, m, dev_y)) return rc;
+    }
+    CANDY_HIP_TRY(hipEventRecord(dev->ev_stop, dev->stream));
+    CANDY_HIP_TRY(hipEventSynchronize(dev->ev_stop));
+    CANDY_HIP_TRY(hipEventElapsedTime(elapsed_ms, dev->ev_start, dev->ev_stop));
+    return CANDY_HIP_OK;
+}
+
+}  // extern "C"

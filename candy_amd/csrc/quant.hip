@@ -1,0 +1,293 @@
+// Activation quantization to Q8_0 and block dequantization. Both are bit-exact with candy's
+// definitions: every product in the dequantizers is exact in f32 (fp16 scale times small
+// integers), so instruction selection cannot change a result.
+#include "blocks.h"
+#include "internal.h"
+
+namespace candy {
+
+// ------------------------------------------------------------------ quantize_q8_0
+// quantize_q8_1 (quantized.cu:3521-3558) without its `sum` half: per 32 values
+//   amax = max|x|, d = amax / 127 (IEEE f32 division), q = amax == 0 ? 0 : roundf(x / d),
+// the stored scale is fp16(d) while q uses the unrounded d.
+// One lane owns 4 consecutive values; the 8 lanes of a block reduce with cross-lane xor.
+__global__ __launch_bounds__(256) void k_quantize_q8_0(const float4 *__restrict__ x, int64_t n4,
+                                                       uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
+                                                       uint8_t *__restrict__ blocks) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool active = i < n4;  // n4 is a multiple of 8, so a block's 8 lanes agree
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (active) v = x[i];
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    const float d = amax / 127.0f;
+    int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+    if (amax != 0.0f) {
+        q0 = (int)roundf(v.x / d);
+        q1 = (int)roundf(v.y / d);
+        q2 = (int)roundf(v.z / d);
+        q3 = (int)roundf(v.w / d);
+    }
+    int s = q0 + q1 + q2 + q3;
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    s += __shfl_xor(s, 4, 64);
+    if (!active) return;
+    const uint32_t packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
+                            ((uint32_t)(q3 & 0xFF) << 24);
+    const int64_t b = i >> 3;
+    const int part = (int)(i & 7);
+    const __half h = __float2half_rn(d);
+    if (qs) qs[i] = packed;
+    if (scales && part == 0) {
+        Q8Scale sc;
+        sc.d = __half2float(h);
+        sc.bsum = s;
+        scales[b] = sc;
+    }
+    if (blocks) {
+        uint8_t *blk = blocks + b * 34;  // 2-byte aligned only
+        if (part == 0) *(uint16_t *)blk = __half_as_ushort(h);
+        uint16_t *p = (uint16_t *)(blk + 2 + part * 4);
+        p[0] = (uint16_t)(packed & 0xFFFFu);
+        p[1] = (uint16_t)(packed >> 16);
+    }
+}
+
+// Q8_0 blocks (34 B) -> planar quants + scales, one lane per block.
+__global__ __launch_bounds__(256) void k_q8_blocks_to_planar(const BlockQ8_0 *__restrict__ blocks, int64_t nb,
+                                                             uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales) {
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= nb) return;
+    const BlockQ8_0 *blk = blocks + b;
+    const u32x4 a = *(const u32x4_a2 *)(blk->qs);
+    const u32x4 c = *(const u32x4_a2 *)(blk->qs + 16);
+    int s = 0;
+    const uint32_t ones = 0x01010101u;
+    s = dot4_i8(a.x, ones, s); s = dot4_i8(a.y, ones, s); s = dot4_i8(a.z, ones, s); s = dot4_i8(a.w, ones, s);
+    s = dot4_i8(c.x, ones, s); s = dot4_i8(c.y, ones, s); s = dot4_i8(c.z, ones, s); s = dot4_i8(c.w, ones, s);
+    u32x4 *out = (u32x4 *)(qs + b * 8);
+    out[0] = a;
+    out[1] = c;
+    Q8Scale sc;
+    sc.d = half_bits_to_float(blk->d);
+    sc.bsum = s;
+    scales[b] = sc;
+}
+
+int launch_quantize_q8(candy_hip_device *dev, const float *x, int64_t rows, int64_t cols, int8_t *qs, Q8Scale *scales,
+                       void *blocks) {
+    const int64_t n4 = rows * cols / 4;
+    if (n4 == 0) return CANDY_HIP_OK;
+    const int64_t grid = (n4 + 255) / 256;
+    CANDY_REQUIRE(grid <= 0x7FFFFFFF, "activation too large");
+    hipLaunchKernelGGL(k_quantize_q8_0, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const float4 *)x, n4,
+                       (uint32_t *)qs, scales, (uint8_t *)blocks);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+int launch_q8_blocks_to_planar(candy_hip_device *dev, const void *blocks, int64_t nb, int8_t *qs, Q8Scale *scales) {
+    if (nb == 0) return CANDY_HIP_OK;
+    const int64_t grid = (nb + 255) / 256;
+    CANDY_REQUIRE(grid <= 0x7FFFFFFF, "activation too large");
+    hipLaunchKernelGGL(k_q8_blocks_to_planar, dim3((unsigned)grid), dim3(256), 0, dev->stream,
+                       (const BlockQ8_0 *)blocks, nb, (uint32_t *)qs, scales);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+// ------------------------------------------------------------------ dequantize
+// Each lane writes whole float4 vectors so the (dominant) output stream is coalesced.
+// With `ids` set the kernels gather rows: output block b comes from row ids[b / bpr] of a
+// table with bpr blocks per row (embedding lookup, indexing.go:8-26 on a quantized table).
+__device__ __forceinline__ int64_t src_block(int64_t b, const int64_t *__restrict__ ids, int64_t bpr) {
+    return ids ? ids[b / bpr] * bpr + b % bpr : b;
+}
+
+// quantized.go:85-93: y[2j] = d*(lo(qs[j])-8), y[2j+1] = d*(hi(qs[j])-8). 4 lanes per block.
+__global__ __launch_bounds__(256) void k_dequant_q4_0(const BlockQ4_0 *__restrict__ blocks, int64_t nb,
+        const int64_t *__restrict__ ids, int64_t bpr,
+                                                      float4 *__restrict__ y, int ggml_order) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = t >> 2;
+    if (b >= nb) return;
+    const int j = (int)(t & 3);  // bytes 4j..4j+3
+    const BlockQ4_0 *blk = blocks + src_block(b, ids, bpr);
+    const float d = half_bits_to_float(blk->d);
+    const uint32_t q = *(const u32_a2 *)(blk->qs + 4 * j);
+    float lo[4], hi[4];
+    const float dm = -8.0f * d;
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        const float ql = (float)((q >> (8 * l)) & 0xF), qh = (float)((q >> (8 * l + 4)) & 0xF);
+        // the two reference forms agree everywhere except the sign of a zero result
+        lo[l] = ggml_order ? d * ql + dm : d * (ql - 8.0f);
+        hi[l] = ggml_order ? d * qh + dm : d * (qh - 8.0f);
+    }
+    float4 *out = y + b * 8;
+    if (ggml_order) {  // quantized.cu:862-866: low nibbles fill y[0..15], high nibbles y[16..31]
+        out[j] = make_float4(lo[0], lo[1], lo[2], lo[3]);
+        out[4 + j] = make_float4(hi[0], hi[1], hi[2], hi[3]);
+    } else {
+        out[2 * j] = make_float4(lo[0], hi[0], lo[1], hi[1]);
+        out[2 * j + 1] = make_float4(lo[2], hi[2], lo[3], hi[3]);
+    }
+}
+
+// quantized.go:131-136: y[i] = d*qs[i]. 8 lanes per block.
+__global__ __launch_bounds__(256) void k_dequant_q8_0(const BlockQ8_0 *__restrict__ blocks, int64_t nb,
+        const int64_t *__restrict__ ids, int64_t bpr,
+                                                      float4 *__restrict__ y) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = t >> 3;
+    if (b >= nb) return;
+    const int j = (int)(t & 7);
+    const BlockQ8_0 *blk = blocks + src_block(b, ids, bpr);
+    const float d = half_bits_to_float(blk->d);
+    const uint32_t q = *(const u32_a2 *)(blk->qs + 4 * j);
+    y[t] = make_float4(d * (float)(int8_t)(q & 0xFF), d * (float)(int8_t)((q >> 8) & 0xFF),
+                       d * (float)(int8_t)((q >> 16) & 0xFF), d * (float)(int8_t)(q >> 24));
+}
+
+// quantized.cu:1008-1041: group il of 64 values, low nibbles with (sc, m) of sub-block 2il,
+// high nibbles with those of 2il+1; y = (d*sc)*q - (dmin*m). 32 lanes per super-block.
+__global__ __launch_bounds__(256) void k_dequant_q4_k(const BlockQ4K *__restrict__ blocks, int64_t nb,
+        const int64_t *__restrict__ ids, int64_t bpr,
+                                                      float4 *__restrict__ y) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = t >> 5;
+    if (b >= nb) return;
+    const int il = (int)(t & 31) >> 3;  // 64-value group
+    const int ir = (int)(t & 7);        // 4 bytes within the group's 32
+    const uint32_t *w = (const uint32_t *)(blocks + src_block(b, ids, bpr));  // 144-byte blocks keep 16-byte alignment
+    const uint32_t dm = w[0];
+    const float dall = half_bits_to_float((uint16_t)(dm & 0xFFFF));
+    const float dmin = half_bits_to_float((uint16_t)(dm >> 16));
+    uint32_t sc2, m2;
+    q4k_scale_min_pair(w[1], w[2], w[3], il, sc2, m2);
+    const float d1 = dall * (float)(sc2 & 0xFF), m1 = dmin * (float)(m2 & 0xFF);
+    const float d2 = dall * (float)(sc2 >> 8), m2f = dmin * (float)(m2 >> 8);
+    const uint32_t q = w[4 + il * 8 + ir];
+    float lo[4], hi[4];
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        lo[l] = d1 * (float)((q >> (8 * l)) & 0xF) - m1;
+        hi[l] = d2 * (float)((q >> (8 * l + 4)) & 0xF) - m2f;
+    }
+    float4 *out = y + b * 64 + il * 16 + ir;
+    out[0] = make_float4(lo[0], lo[1], lo[2], lo[3]);
+    out[8] = make_float4(hi[0], hi[1], hi[2], hi[3]);
+}
+
+// quantized.cu:1103-1128. 16 lanes per super-block, each 4 consecutive `il` of one half.
+__global__ __launch_bounds__(256) void k_dequant_q6_k(const BlockQ6K *__restrict__ blocks, int64_t nb,
+        const int64_t *__restrict__ ids, int64_t bpr,
+                                                      float4 *__restrict__ y) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = t >> 4;
+    if (b >= nb) return;
+    const int ip = (int)(t & 15) >> 3;
+    const int il0 = ((int)(t & 7)) * 4;
+    const BlockQ6K *blk = blocks + src_block(b, ids, bpr);
+    const float d = half_bits_to_float(blk->d);
+    const uint32_t ql0 = *(const u32_a2 *)(blk->ql + 64 * ip + il0);
+    const uint32_t ql1 = *(const u32_a2 *)(blk->ql + 64 * ip + 32 + il0);
+    const uint32_t qh = *(const u32_a2 *)(blk->qh + 32 * ip + il0);
+    const int is = 8 * ip + il0 / 16;
+    const float s0 = d * (float)blk->scales[is], s1 = d * (float)blk->scales[is + 2];
+    const float s2 = d * (float)blk->scales[is + 4], s3 = d * (float)blk->scales[is + 6];
+    float o[4][4];
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        const uint32_t a = (ql0 >> (8 * l)) & 0xFF, c = (ql1 >> (8 * l)) & 0xFF, h = (qh >> (8 * l)) & 0xFF;
+        o[0][l] = s0 * (float)((int)((a & 0xF) | (((h >> 0) & 3) << 4)) - 32);
+        o[1][l] = s1 * (float)((int)((c & 0xF) | (((h >> 2) & 3) << 4)) - 32);
+        o[2][l] = s2 * (float)((int)((a >> 4) | (((h >> 4) & 3) << 4)) - 32);
+        o[3][l] = s3 * (float)((int)((c >> 4) | (((h >> 6) & 3) << 4)) - 32);
+    }
+    float4 *out = y + b * 64 + ip * 32 + il0 / 4;
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) out[8 * qd] = make_float4(o[qd][0], o[qd][1], o[qd][2], o[qd][3]);
+}
+
+}  // namespace candy
+
+using namespace candy;
+
+extern "C" {
+
+static int dequantize_impl(candy_hip_device *dev, int fmt, const void *dev_blocks, int64_t n_blocks,
+                           const int64_t *ids, int64_t bpr, float *dev_out) {
+    FormatInfo fi = format_info(fmt);
+    CANDY_REQUIRE(fi.elems != 0, "unknown quantized format %d", fmt);
+    CANDY_REQUIRE(n_blocks >= 0, "negative block count");
+    if (n_blocks == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dev_blocks && dev_out, "nil pointer");
+    CANDY_REQUIRE(((uintptr_t)dev_out & 15) == 0, "output must be 16-byte aligned");
+    CANDY_REQUIRE(((uintptr_t)dev_blocks & (fmt == CANDY_HIP_Q4_K ? 15 : 1)) == 0, "blocks are misaligned");
+    if (int rc = use_device(dev)) return rc;
+    const int lanes_per_block = fmt == CANDY_HIP_Q4_K ? 32 : fmt == CANDY_HIP_Q6_K ? 16 : fmt == CANDY_HIP_Q8_0 ? 8 : 4;
+    const int64_t grid = (n_blocks * lanes_per_block + 255) / 256;
+    CANDY_REQUIRE(grid <= 0x7FFFFFFF, "too many blocks");
+    dim3 g((unsigned)grid), blk(256);
+    switch (fmt) {
+    case CANDY_HIP_Q4_0:
+    case CANDY_HIP_Q4_0_GGML:
+        hipLaunchKernelGGL(k_dequant_q4_0, g, blk, 0, dev->stream, (const BlockQ4_0 *)dev_blocks, n_blocks, ids, bpr,
+                           (float4 *)dev_out, fmt == CANDY_HIP_Q4_0_GGML ? 1 : 0);
+        break;
+    case CANDY_HIP_Q8_0:
+        hipLaunchKernelGGL(k_dequant_q8_0, g, blk, 0, dev->stream, (const BlockQ8_0 *)dev_blocks, n_blocks, ids, bpr,
+                           (float4 *)dev_out);
+        break;
+    case CANDY_HIP_Q4_K:
+        hipLaunchKernelGGL(k_dequant_q4_k, g, blk, 0, dev->stream, (const BlockQ4K *)dev_blocks, n_blocks, ids, bpr,
+                           (float4 *)dev_out);
+        break;
+    case CANDY_HIP_Q6_K:
+        hipLaunchKernelGGL(k_dequant_q6_k, g, blk, 0, dev->stream, (const BlockQ6K *)dev_blocks, n_blocks, ids, bpr,
+                           (float4 *)dev_out);
+        break;
+    }
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_dequantize_blocks(candy_hip_device *dev, int fmt, const void *dev_blocks, int64_t n_blocks,
+                                float *dev_out) {
+    return dequantize_impl(dev, fmt, dev_blocks, n_blocks, nullptr, 1, dev_out);
+}
+
+int candy_hip_qindex_select(candy_hip_device *dev, const candy_hip_qtensor *q, const int64_t *dev_ids, int64_t n_ids,
+                            float *out) {
+    CANDY_REQUIRE(q, "qtensor is nil");
+    CANDY_REQUIRE(q->dev == dev, "qtensor lives on another device");
+    CANDY_REQUIRE(n_ids >= 0, "negative id count");
+    if (n_ids == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dev_ids, "ids is nil");
+    const int64_t bpr = q->cols / format_info(q->fmt).elems;
+    return dequantize_impl(dev, q->fmt, q->data, n_ids * bpr, dev_ids, bpr, out);
+}
+
+int candy_hip_dequantize(candy_hip_device *dev, const candy_hip_qtensor *q, float *dev_out) {
+    CANDY_REQUIRE(q, "qtensor is nil");
+    CANDY_REQUIRE(q->dev == dev, "qtensor lives on another device");
+    return candy_hip_dequantize_blocks(dev, q->fmt, q->data, q->rows * (q->cols / format_info(q->fmt).elems), dev_out);
+}
+
+int candy_hip_quantize_q8_0(candy_hip_device *dev, const float *dev_x, int64_t rows, int64_t cols,
+                            void *dev_out_blocks) {
+    CANDY_REQUIRE(rows >= 0 && cols >= 0, "invalid matrix dimensions");
+    CANDY_REQUIRE(cols % 32 == 0, "cols %lld is not a multiple of the block size 32", (long long)cols);
+    if (rows * cols == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dev_x && dev_out_blocks, "nil pointer");
+    CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "input must be 16-byte aligned");
+    CANDY_REQUIRE(((uintptr_t)dev_out_blocks & 1) == 0, "output blocks must be 2-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    return launch_quantize_q8(dev, dev_x, rows, cols, nullptr, nullptr, dev_out_blocks);
+}
+
+}  // extern "C"

@@ -1,0 +1,282 @@
+// Library runtime: error text, device handles, raw memory, timing.
+// Stands behind candy.BackendDevice (device.go:49-82) and the storage plumbing of
+// candy.BackendStorage (backend.go:4-16).
+#include <cstring>
+
+#include "internal.h"
+
+namespace candy {
+
+static thread_local std::string g_last_error;
+
+void set_error(const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+}
+
+int fail(int status, const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return status;
+}
+
+FormatInfo format_info(int fmt) {
+    switch (fmt) {
+    case CANDY_HIP_Q4_0:
+    case CANDY_HIP_Q4_0_GGML: return {32, 18};
+    case CANDY_HIP_Q8_0: return {32, 34};
+    case CANDY_HIP_Q4_K: return {256, 144};
+    case CANDY_HIP_Q6_K: return {256, 210};
+    default: return {0, 0};
+    }
+}
+
+int use_device(const candy_hip_device *dev) {
+    if (!dev) return fail(CANDY_HIP_ERR_INVALID, "device handle is nil");
+    CANDY_HIP_TRY(hipSetDevice(dev->ordinal));
+    return CANDY_HIP_OK;
+}
+
+int workspace(candy_hip_device *dev, size_t bytes, void **out) {
+    if (bytes > dev->ws_bytes) {
+        // Work already enqueued may still read the old buffer.
+        CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
+        if (dev->ws) CANDY_HIP_TRY(hipFree(dev->ws));
+        dev->ws = nullptr;
+        dev->ws_bytes = 0;
+        size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        CANDY_HIP_TRY(hipMalloc(&dev->ws, want));
+        dev->ws_bytes = want;
+    }
+    *out = dev->ws;
+    return CANDY_HIP_OK;
+}
+
+}  // namespace candy
+
+using namespace candy;
+
+extern "C" {
+
+const char *candy_hip_last_error(void) { return g_last_error.c_str(); }
+
+const char *candy_hip_version(void) { return "candy-hip 0.1 (gfx950)"; }
+
+int candy_hip_device_count(int *count) {
+    CANDY_REQUIRE(count, "count is nil");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *count = 0;
+        return fail(CANDY_HIP_ERR_HIP, "hipGetDeviceCount failed: %s", hipGetErrorString(e));
+    }
+    *count = n;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_open(int ordinal, candy_hip_device **out) {
+    CANDY_REQUIRE(out, "out is nil");
+    *out = nullptr;
+    int n = 0;
+    CANDY_HIP_TRY(hipGetDeviceCount(&n));
+    CANDY_REQUIRE(ordinal >= 0 && ordinal < n, "device ordinal %d out of range (have %d)", ordinal, n);
+    CANDY_HIP_TRY(hipSetDevice(ordinal));
+    hipDeviceProp_t props;
+    CANDY_HIP_TRY(hipGetDeviceProperties(&props, ordinal));
+    if (strncmp(props.gcnArchName, "gfx950", 6) != 0)
+        return fail(CANDY_HIP_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", ordinal,
+                    props.gcnArchName);
+    candy_hip_device *dev = new candy_hip_device();
+    dev->ordinal = ordinal;
+    dev->num_cus = props.multiProcessorCount;
+    snprintf(dev->name, sizeof(dev->name), "%s (%s)", props.name, props.gcnArchName);
+    hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&dev->ev_start);
+    if (e == hipSuccess) e = hipEventCreate(&dev->ev_stop);
+    if (e != hipSuccess) {
+        candy_hip_close(dev);
+        return fail(CANDY_HIP_ERR_HIP, "creating stream/events failed: %s", hipGetErrorString(e));
+    }
+    *out = dev;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_close(candy_hip_device *dev) {
+    if (!dev) return CANDY_HIP_OK;
+    (void)hipSetDevice(dev->ordinal);
+    if (dev->stream) (void)hipStreamSynchronize(dev->stream);
+    if (dev->ws) (void)hipFree(dev->ws);
+    if (dev->ev_start) (void)hipEventDestroy(dev->ev_start);
+    if (dev->ev_stop) (void)hipEventDestroy(dev->ev_stop);
+    if (dev->stream) (void)hipStreamDestroy(dev->stream);
+    delete dev;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_device_ordinal(const candy_hip_device *dev, int *ordinal) {
+    CANDY_REQUIRE(dev && ordinal, "nil argument");
+    *ordinal = dev->ordinal;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_device_name(const candy_hip_device *dev, char *buf, size_t buf_len) {
+    CANDY_REQUIRE(dev && buf && buf_len > 0, "nil argument");
+    snprintf(buf, buf_len, "%s", dev->name);
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_synchronize(candy_hip_device *dev) {
+    if (int rc = use_device(dev)) return rc;
+    CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_alloc(candy_hip_device *dev, size_t bytes, void **dptr) {
+    CANDY_REQUIRE(dptr, "dptr is nil");
+    *dptr = nullptr;
+    if (int rc = use_device(dev)) return rc;
+    if (bytes == 0) bytes = 1;  // a zero-length storage still gets a distinct address
+    CANDY_HIP_TRY(hipMalloc(dptr, bytes));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_free(candy_hip_device *dev, void *dptr) {
+    if (!dptr) return CANDY_HIP_OK;
+    if (int rc = use_device(dev)) return rc;
+    CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));  // kernels in flight may still use it
+    CANDY_HIP_TRY(hipFree(dptr));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_zero(candy_hip_device *dev, void *dptr, size_t bytes) {
+    if (bytes == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dptr, "dptr is nil");
+    if (int rc = use_device(dev)) return rc;
+    CANDY_HIP_TRY(hipMemsetAsync(dptr, 0, bytes, dev->stream));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_h2d(candy_hip_device *dev, void *dst_dev, const void *src_host, size_t bytes) {
+    if (bytes == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dst_dev && src_host, "nil pointer");
+    if (int rc = use_device(dev)) return rc;
+    // Pageable host memory: the copy is complete (staged) when this returns, so the caller's
+    // buffer is not referenced afterwards.
+    CANDY_HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, dev->stream));
+    CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_d2h(candy_hip_device *dev, void *dst_host, const void *src_dev, size_t bytes) {
+    if (bytes == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dst_host && src_dev, "nil pointer");
+    if (int rc = use_device(dev)) return rc;
+    CANDY_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, dev->stream));
+    CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_d2d(candy_hip_device *dev, void *dst_dev, const void *src_dev, size_t bytes) {
+    if (bytes == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dst_dev && src_dev, "nil pointer");
+    if (int rc = use_device(dev)) return rc;
+    CANDY_HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, dev->stream));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_block_elems(int fmt) { return format_info(fmt).elems; }
+int candy_hip_block_bytes(int fmt) { return format_info(fmt).bytes; }
+
+size_t candy_hip_qweight_bytes(int fmt, int64_t rows, int64_t cols) {
+    FormatInfo fi = format_info(fmt);
+    if (fi.elems == 0 || rows < 0 || cols < 0 || cols % fi.elems != 0) return 0;
+    return (size_t)rows * (size_t)(cols / fi.elems) * (size_t)fi.bytes;
+}
+
+static int qtensor_check(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols, size_t nbytes) {
+    FormatInfo fi = format_info(fmt);
+    CANDY_REQUIRE(dev, "device handle is nil");
+    CANDY_REQUIRE(fi.elems != 0, "unknown quantized format %d", fmt);
+    CANDY_REQUIRE(rows > 0 && cols > 0, "invalid matrix dimensions %lld x %lld", (long long)rows, (long long)cols);
+    CANDY_REQUIRE(cols % fi.elems == 0, "cols %lld is not a multiple of the block size %d", (long long)cols, fi.elems);
+    size_t want = candy_hip_qweight_bytes(fmt, rows, cols);
+    CANDY_REQUIRE(nbytes == want, "weight has %zu bytes, %lld x %lld blocks of format %d need %zu", nbytes,
+                  (long long)rows, (long long)cols, fmt, want);
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_qtensor_upload(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols, const void *host_blocks,
+                             size_t nbytes, candy_hip_qtensor **out) {
+    CANDY_REQUIRE(out, "out is nil");
+    *out = nullptr;
+    if (int rc = qtensor_check(dev, fmt, rows, cols, nbytes)) return rc;
+    CANDY_REQUIRE(host_blocks, "host_blocks is nil");
+    void *d = nullptr;
+    // 64 bytes of slack after the last block: the matvec kernels read whole 16-byte vectors.
+    if (int rc = candy_hip_alloc(dev, nbytes + 64, &d)) return rc;
+    if (int rc = candy_hip_h2d(dev, d, host_blocks, nbytes)) {
+        (void)hipFree(d);
+        return rc;
+    }
+    candy_hip_qtensor *q = new candy_hip_qtensor();
+    q->dev = dev; q->fmt = fmt; q->rows = rows; q->cols = cols; q->nbytes = nbytes; q->data = d; q->owned = true;
+    *out = q;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_qtensor_wrap(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols, void *dev_blocks,
+                           size_t nbytes, candy_hip_qtensor **out) {
+    CANDY_REQUIRE(out, "out is nil");
+    *out = nullptr;
+    if (int rc = qtensor_check(dev, fmt, rows, cols, nbytes)) return rc;
+    CANDY_REQUIRE(dev_blocks, "dev_blocks is nil");
+    CANDY_REQUIRE(((uintptr_t)dev_blocks & 15) == 0, "device blocks must be 16-byte aligned");
+    candy_hip_qtensor *q = new candy_hip_qtensor();
+    q->dev = dev; q->fmt = fmt; q->rows = rows; q->cols = cols; q->nbytes = nbytes; q->data = dev_blocks; q->owned = false;
+    *out = q;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_qtensor_free(candy_hip_qtensor *q) {
+    if (!q) return CANDY_HIP_OK;
+    int rc = CANDY_HIP_OK;
+    if (q->owned && q->data) rc = candy_hip_free(q->dev, q->data);
+    delete q;
+    return rc;
+}
+
+int candy_hip_qtensor_info(const candy_hip_qtensor *q, int *fmt, int64_t *rows, int64_t *cols, size_t *nbytes,
+                           void **dev_blocks) {
+    CANDY_REQUIRE(q, "qtensor is nil");
+    if (fmt) *fmt = q->fmt;
+    if (rows) *rows = q->rows;
+    if (cols) *cols = q->cols;
+    if (nbytes) *nbytes = q->nbytes;
+    if (dev_blocks) *dev_blocks = q->data;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_timer_start(candy_hip_device *dev) {
+    if (int rc = use_device(dev)) return rc;
+    CANDY_HIP_TRY(hipEventRecord(dev->ev_start, dev->stream));
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_timer_stop(candy_hip_device *dev, float *elapsed_ms) {
+    CANDY_REQUIRE(elapsed_ms, "elapsed_ms is nil");
+    if (int rc = use_device(dev)) return rc;
+    CANDY_HIP_TRY(hipEventRecord(dev->ev_stop, dev->stream));
+    CANDY_HIP_TRY(hipEventSynchronize(dev->ev_stop));
+    CANDY_HIP_TRY(hipEventElapsedTime(elapsed_ms, dev->ev_start, dev->ev_stop));
+    return CANDY_HIP_OK;
+}
+
+}  // extern "C"

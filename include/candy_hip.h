@@ -1,0 +1,216 @@
+/*
+ * candy_hip.h -- C ABI of libcandy_hip.so: candy's quantized-matmul path on one MI355X.
+ *
+ * This is the boundary a cgo shim binds (the way llm/internal/flashattn/flashattn.go:3-13
+ * binds flash_api.h:71-117): plain C, opaque handles, raw device pointers, sizes by value.
+ * Unlike that precedent every call returns a status and the failure text is retrievable
+ * (candy's Go convention is `(value, error)` on every fallible call, tensor/ops.go:88-90).
+ *
+ * Each declaration names the reference interface it stands behind.  "QCU" is
+ * tensor/internal/cuda/kernels/quantized.cu, "QGO" is tensor/internal/cpu/kernels/quantized.go.
+ *
+ * Threading: handles may be used from any OS thread (cgo migrates goroutines between
+ * threads); every call selects its device itself.  Calls on one device handle are
+ * enqueued on that handle's stream in call order; two threads using the same handle at
+ * the same time must serialise themselves, as candy's tensors do (no locks anywhere in
+ * the reference).  No host pointer passed in is retained after the call returns.
+ */
+#ifndef CANDY_HIP_H
+#define CANDY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct candy_hip_device candy_hip_device;     /* one GPU + its stream + its workspace   */
+typedef struct candy_hip_qtensor candy_hip_qtensor;   /* device-resident quantized weight matrix */
+typedef struct candy_hip_qact candy_hip_qact;         /* activations quantized once, reusable     */
+typedef struct candy_hip_llama candy_hip_llama;       /* Llama-style decoder built on the ops    */
+
+enum candy_hip_status {
+    CANDY_HIP_OK = 0,
+    CANDY_HIP_ERR_INVALID = 1,     /* bad argument: nil pointer, shape, unknown format        */
+    CANDY_HIP_ERR_HIP = 2,         /* a HIP runtime call failed; text has hipGetErrorString   */
+    CANDY_HIP_ERR_OOM = 3,         /* device allocation failed                                 */
+    CANDY_HIP_ERR_UNSUPPORTED = 4  /* valid request this build has no kernel for               */
+};
+
+/* Block formats; values are the GGML type ids (what a GGUF file stores).
+ * Layouts: QGO:8-11 (Q4_0, 18 B / 32), QGO:34-37 (Q8_0, 34 B / 32),
+ * QGO:55-59 (Q4_K, 144 B / 256), QGO:70-75 (Q6_K, 210 B / 256). */
+enum candy_hip_qformat {
+    CANDY_HIP_Q4_0 = 2,        /* element order of candy's CPU dequantize, QGO:85-93 (interleaved) */
+    CANDY_HIP_Q8_0 = 8,
+    CANDY_HIP_Q4_K = 12,
+    CANDY_HIP_Q6_K = 14,
+    CANDY_HIP_Q4_0_GGML = 102  /* element order of QCU:862-866 / GGUF files (low half, high half)   */
+};
+
+/* ------------------------------------------------------------------ library / device
+ * Stands behind candy.BackendDevice (device.go:49-82): Location/IsSame -> ordinal,
+ * Synchronize -> candy_hip_synchronize, StorageFromSlice -> alloc + h2d, Alloc/Zeros -> alloc + zero. */
+const char *candy_hip_last_error(void);                 /* thread-local text of the last failure   */
+const char *candy_hip_version(void);
+int candy_hip_device_count(int *count);
+int candy_hip_open(int ordinal, candy_hip_device **out);
+int candy_hip_close(candy_hip_device *dev);
+int candy_hip_device_ordinal(const candy_hip_device *dev, int *ordinal);
+int candy_hip_device_name(const candy_hip_device *dev, char *buf, size_t buf_len);
+int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchronize                */
+
+/* ------------------------------------------------------------------ raw device memory
+ * Backs BackendStorage[T] (backend.go:4-16): Data() is a d2h copy, Clone() a d2d copy. */
+int candy_hip_alloc(candy_hip_device *dev, size_t bytes, void **dptr);
+int candy_hip_free(candy_hip_device *dev, void *dptr);
+int candy_hip_zero(candy_hip_device *dev, void *dptr, size_t bytes);
+int candy_hip_h2d(candy_hip_device *dev, void *dst_dev, const void *src_host, size_t bytes);
+int candy_hip_d2h(candy_hip_device *dev, void *dst_host, const void *src_dev, size_t bytes); /* synchronises */
+int candy_hip_d2d(candy_hip_device *dev, void *dst_dev, const void *src_dev, size_t bytes);
+
+/* ------------------------------------------------------------------ block formats */
+int candy_hip_block_elems(int fmt);   /* 32 / 256, 0 if unknown                                   */
+int candy_hip_block_bytes(int fmt);   /* 18 / 34 / 144 / 210, 0 if unknown                        */
+/* bytes of a [rows, cols] weight, 0 if fmt is unknown or cols is not a multiple of the block */
+size_t candy_hip_qweight_bytes(int fmt, int64_t rows, int64_t cols);
+
+/* Quantized weight [rows, cols] (cols = contraction dim) kept on the device in the ORIGINAL
+ * block layout, row-major blocks, as QCU:2827 indexes them (`x[kbx + row*blocks_per_row]`).
+ * upload copies host blocks; wrap adopts device memory the caller keeps owning. */
+int candy_hip_qtensor_upload(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols,
+                             const void *host_blocks, size_t nbytes, candy_hip_qtensor **out);
+int candy_hip_qtensor_wrap(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols,
+                           void *dev_blocks, size_t nbytes, candy_hip_qtensor **out);
+int candy_hip_qtensor_free(candy_hip_qtensor *q);
+int candy_hip_qtensor_info(const candy_hip_qtensor *q, int *fmt, int64_t *rows, int64_t *cols,
+                           size_t *nbytes, void **dev_blocks);
+
+/* Dequantize n_blocks blocks to f32 (device -> device).
+ * QGO:85-93 DequantizeBlockQ4_0F32, QGO:131-136 DequantizeBlockQ8_0F32,
+ * QCU:1008-1041 dequantize_block_q4_K, QCU:1103-1128 dequantize_block_q6_K.  Bit-exact. */
+int candy_hip_dequantize_blocks(candy_hip_device *dev, int fmt, const void *dev_blocks,
+                                int64_t n_blocks, float *dev_out);
+int candy_hip_dequantize(candy_hip_device *dev, const candy_hip_qtensor *q, float *dev_out);
+
+/* f32 [rows, cols] -> Q8_0 blocks (34 B each, rows*cols/32 of them), cols % 32 == 0.
+ * QCU:3521-3558 quantize_q8_1 without its `sum` half.  Bit-exact. */
+int candy_hip_quantize_q8_0(candy_hip_device *dev, const float *dev_x, int64_t rows, int64_t cols,
+                            void *dev_out_blocks);
+
+/* y[m, rows] = x[m, cols] . W^T, activations quantized to Q8_0 on the device first.
+ * m < 16 runs the bandwidth-bound matvec family (QCU:2787-2871 mul_mat_vec_q and its entry
+ * points :2874, :2906, :2930, :2946); m >= 16 the MFMA tile kernel (QCU:455-578 mul_mat_q).
+ * y is row-major [m, rows] (candy's result layout, tensor/ops.go:1264). */
+int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x,
+                      int64_t m, float *dev_y);
+
+/* Same contraction, activations already in Q8_0 blocks on the device ([m, cols/32] blocks). */
+int candy_hip_qmatmul_q8(candy_hip_device *dev, const candy_hip_qtensor *w, const void *dev_x_q8_0,
+                         int64_t m, float *dev_y);
+
+/* Activations quantized once and contracted against several weights (q/k/v share one input,
+ * gate/up another): QCU's host flow quantizes with quantize_q8_1 (:3521) and then launches
+ * mul_mat_vec_q (:2787) per weight.  The handle owns its device memory; quantize may be called
+ * again on the same handle with any shape up to the capacity it was created with. */
+int candy_hip_qact_create(candy_hip_device *dev, int64_t max_m, int64_t max_cols, candy_hip_qact **out);
+int candy_hip_qact_free(candy_hip_qact *a);
+int candy_hip_qact_quantize(candy_hip_qact *a, const float *dev_x, int64_t m, int64_t cols);
+int candy_hip_qmatmul_qact(candy_hip_device *dev, const candy_hip_qtensor *w, const candy_hip_qact *a,
+                           float *dev_y);
+
+/* ------------------------------------------------------------------ f32 ops of the decode step
+ * One-to-one with the BackendStorage methods a Llama block calls (backend.go). */
+/* backend.go:78 MatMul on contiguous f32: c[b,m,n] = a[b,m,k] . b[b,k,n]; if rhs_transposed the
+ * rhs is [b,n,k] (the strided W^T view nn/linear.go:65 creates).  CONV:251-267 / :373-389. */
+int candy_hip_matmul_f32(candy_hip_device *dev, const float *a, const float *b, float *c,
+                         int64_t batch, int64_t m, int64_t n, int64_t k, int rhs_transposed);
+/* backend.go:150 FastRmsNorm; reduce.go:3071-3092.  alpha may be NULL. */
+int candy_hip_rms_norm(candy_hip_device *dev, const float *x, const float *alpha, float eps,
+                       int64_t rows, int64_t cols, float *out);
+/* backend.go:159 Rope; reduce.go:3987-4006 (pairs (i, i+d/2)). */
+int candy_hip_rope(candy_hip_device *dev, const float *src, const float *cos_t, const float *sin_t,
+                   int64_t bh, int64_t td, int64_t d, int64_t stride_b, float *dst);
+/* backend.go:147 FastSoftmax; reduce.go:2855-2879. */
+int candy_hip_softmax(candy_hip_device *dev, const float *src, int64_t rows, int64_t cols, float *dst);
+/* backend.go:228 Silu; unary.go:3353-3366. */
+int candy_hip_silu(candy_hip_device *dev, const float *x, int64_t n, float *out);
+/* backend.go:21 Add, :27 Mul on contiguous same-shape operands. */
+int candy_hip_add(candy_hip_device *dev, const float *a, const float *b, int64_t n, float *out);
+int candy_hip_mul(candy_hip_device *dev, const float *a, const float *b, int64_t n, float *out);
+/* silu(gate) * up in one pass (Silu then Mul). */
+int candy_hip_silu_mul(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *out);
+/* backend.go:129 FastArgmax; reduce.go:846-862 (first maximum wins). */
+int candy_hip_argmax(candy_hip_device *dev, const float *src, int64_t rows, int64_t cols, uint32_t *out);
+/* IndexSelect along dim 0 of a [n_src, width] f32 table; indexing.go:8-26. ids are int64 on the device. */
+int candy_hip_index_select(candy_hip_device *dev, const float *table, int64_t n_src, int64_t width,
+                           const int64_t *dev_ids, int64_t n_ids, float *out);
+/* Row gather from a quantized table (embedding lookup): dequantizes rows ids[i] of q. */
+int candy_hip_qindex_select(candy_hip_device *dev, const candy_hip_qtensor *q, const int64_t *dev_ids,
+                            int64_t n_ids, float *out);
+/* Batch-1 attention of one new token over an f32 KV cache: softmax(q.K^T * scale).V per head,
+ * the MatMul / FastSoftmax / MatMul sequence a candy Llama block would issue.
+ * q, out: [n_heads, head_dim]; k_cache, v_cache: [n_kv_heads, *, head_dim] with cache_stride
+ * elements between kv heads; positions 0..n_pos-1 are attended. */
+int candy_hip_attention_decode(candy_hip_device *dev, const float *q, const float *k_cache,
+                               const float *v_cache, int64_t n_heads, int64_t n_kv_heads,
+                               int64_t head_dim, int64_t n_pos, int64_t cache_stride, float scale,
+                               float *out);
+
+/* ------------------------------------------------------------------ Llama-style decoder
+ * A decoder assembled from the ops above (candy has no model code; the layer order is the
+ * standard Llama block: RMSNorm, q/k/v, RoPE, attention over the cache, o, residual,
+ * RMSNorm, SwiGLU, residual; final RMSNorm, head, argmax). */
+typedef struct candy_hip_llama_config {
+    int32_t n_layers, d_model, n_heads, n_kv_heads, head_dim, d_ffn, vocab, max_pos;
+    float rms_eps, rope_base;
+} candy_hip_llama_config;
+
+enum candy_hip_llama_weight {
+    CANDY_HIP_W_ATTN_NORM = 0,  /* f32 [d_model]                 */
+    CANDY_HIP_W_Q = 1,          /* q  [n_heads*head_dim, d_model]    */
+    CANDY_HIP_W_K = 2,          /* q  [n_kv_heads*head_dim, d_model] */
+    CANDY_HIP_W_V = 3,
+    CANDY_HIP_W_O = 4,          /* q  [d_model, n_heads*head_dim]    */
+    CANDY_HIP_W_FFN_NORM = 5,   /* f32 [d_model]                 */
+    CANDY_HIP_W_GATE = 6,       /* q  [d_ffn, d_model]           */
+    CANDY_HIP_W_UP = 7,
+    CANDY_HIP_W_DOWN = 8,       /* q  [d_model, d_ffn]           */
+    CANDY_HIP_W_OUT_NORM = 9,   /* f32 [d_model], layer = -1     */
+    CANDY_HIP_W_HEAD = 10,      /* q  [vocab, d_model], layer = -1 */
+    CANDY_HIP_W_EMBED = 11      /* q  [vocab, d_model], layer = -1 (row gather) */
+};
+
+int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *cfg, candy_hip_llama **out);
+int candy_hip_llama_free(candy_hip_llama *m);
+/* The model borrows the tensors; they must outlive it. */
+int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const candy_hip_qtensor *w);
+int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const float *dev_alpha);
+/* f32 KV cache, [n_layers][n_kv_heads][max_pos][head_dim] for K and the same for V. */
+int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, size_t *bytes_each);
+/* One decode step: token id at position pos -> logits [vocab] (device pointer owned by the
+ * model, valid until the next step) and the greedy next token.  Either output may be NULL. */
+int candy_hip_llama_decode(candy_hip_llama *m, int32_t token, int32_t pos, const float **dev_logits,
+                           int32_t *next_token);
+/* Same step with the hidden state of the token given directly instead of an embedding row. */
+int candy_hip_llama_decode_hidden(candy_hip_llama *m, const float *dev_hidden, int32_t pos,
+                                  const float **dev_logits, int32_t *next_token);
+
+/* ------------------------------------------------------------------ timing (HIP events on the handle's stream) */
+/* Runs `iters` contractions back to back, iteration i using weight ws[i % n_ws] (all the same
+ * shape), and returns the elapsed time between HIP events recorded on the handle's stream
+ * around the loop.  Rotating over more distinct weights than the last-level cache holds makes
+ * every iteration stream from HBM.  quantize_each != 0: each iteration is the whole f32-in ->
+ * f32-out path (activation quantization + contraction); 0: the activations are quantized once
+ * before the timed region and each iteration is the contraction kernel alone. */
+int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws,
+                            const float *dev_x, int64_t m, float *dev_y, int iters, int quantize_each,
+                            float *elapsed_ms);
+int candy_hip_timer_start(candy_hip_device *dev);
+int candy_hip_timer_stop(candy_hip_device *dev, float *elapsed_ms);   /* synchronises */
+
+#ifdef __cplusplus
+}
+#endif
+#endif

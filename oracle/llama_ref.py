@@ -1,0 +1,69 @@
+"""CPU composition of one Llama-style decode step from the oracle's ops.
+
+TEST INFRASTRUCTURE ONLY (see oracle/candy_oracle.c). candy holds no model code, so this
+is the sequence of candy CPU kernels a candy Llama block would run, with the quantized
+Linear (oracle.qmatmul) in place of MatMul:
+  RMSNorm (reduce.go:3071-3092) -> q/k/v -> Rope (reduce.go:3987-4006) -> append to the f32 KV
+  cache -> MatMul/FastSoftmax/MatMul attention -> o -> Add -> RMSNorm -> gate/up -> Silu*Mul
+  (unary.go:3353-3366) -> down -> Add; final RMSNorm -> head -> FastArgmax (reduce.go:846-862).
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+from . import oracle as o
+
+
+def rope_tables(max_pos: int, head_dim: int, base: float):
+    """cos/sin [max_pos, head_dim/2]: angle(p, i) = p * base^(-2i/d) in float64, stored as f32."""
+    i = np.arange(head_dim // 2, dtype=np.float64)
+    inv = np.power(np.float64(base), -2.0 * i / head_dim)
+    ang = np.arange(max_pos, dtype=np.float64)[:, None] * inv[None, :]
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+class LlamaRef:
+    def __init__(self, cfg: dict, weights: dict):
+        """weights: {(kind, layer): (fmt, blocks) | f32 array}; kinds as in candy_hip.h."""
+        self.c = cfg
+        self.w = weights
+        c = cfg
+        self.k_cache = np.zeros((c["n_layers"], c["n_kv_heads"], c["max_pos"], c["head_dim"]), np.float32)
+        self.v_cache = np.zeros_like(self.k_cache)
+        self.cos, self.sin = rope_tables(c["max_pos"], c["head_dim"], c["rope_base"])
+
+    def _lin(self, kind, layer, x, rows, cols):
+        fmt, blocks = self.w[(kind, layer)]
+        return o.qmatmul(fmt, blocks, rows, cols, x).reshape(-1)
+
+    def embed(self, token: int) -> np.ndarray:
+        fmt, blocks = self.w[("embed", -1)]
+        rb = o.block_bytes(fmt) * (self.c["d_model"] // o.block_elems(fmt))
+        return o.dequantize(fmt, blocks[token * rb:(token + 1) * rb])
+
+    def step(self, h: np.ndarray, pos: int):
+        c = self.c
+        d, hd, nh, nkv, ffn = c["d_model"], c["head_dim"], c["n_heads"], c["n_kv_heads"], c["d_ffn"]
+        h = np.ascontiguousarray(h, np.float32).copy()
+        for l in range(c["n_layers"]):
+            xn = o.fast_rms_norm(h, d, c["rms_eps"], self.w[("attn_norm", l)])
+            q = self._lin("q", l, xn, nh * hd, d)
+            k = self._lin("k", l, xn, nkv * hd, d)
+            v = self._lin("v", l, xn, nkv * hd, d)
+            q = o.rope(q, self.cos[pos], self.sin[pos], nh, hd, hd)
+            k = o.rope(k, self.cos[pos], self.sin[pos], nkv, hd, hd)
+            self.k_cache[l, :, pos, :] = k.reshape(nkv, hd)
+            self.v_cache[l, :, pos, :] = v.reshape(nkv, hd)
+            att = o.attention_decode(q, self.k_cache[l], self.v_cache[l], nh, nkv, hd, pos + 1,
+                                     c["max_pos"] * hd, 1.0 / math.sqrt(hd))
+            h = o.add(h, self._lin("o", l, att, d, nh * hd))
+            xn = o.fast_rms_norm(h, d, c["rms_eps"], self.w[("ffn_norm", l)])
+            g = self._lin("gate", l, xn, ffn, d)
+            u = self._lin("up", l, xn, ffn, d)
+            act = o.mul(o.silu(g), u)
+            h = o.add(h, self._lin("down", l, act, d, ffn))
+        xn = o.fast_rms_norm(h, d, c["rms_eps"], self.w[("out_norm", -1)])
+        logits = self._lin("head", -1, xn, c["vocab"], d)
+        return int(o.fast_argmax(logits, c["vocab"])[0]), logits, h

@@ -1,0 +1,103 @@
+"""Decode-step parity: the device decoder against the CPU composition of oracle ops on a
+reduced-depth Llama with full-width layers, plus properties at the full 7B shape."""
+import numpy as np
+import pytest
+
+from candy_amd import hip, synth
+from oracle import llama_ref
+
+pytestmark = pytest.mark.gpu
+
+KINDS = {"q": hip.W_Q, "k": hip.W_K, "v": hip.W_V, "o": hip.W_O, "gate": hip.W_GATE, "up": hip.W_UP,
+         "down": hip.W_DOWN, "head": hip.W_HEAD, "embed": hip.W_EMBED,
+         "attn_norm": hip.W_ATTN_NORM, "ffn_norm": hip.W_FFN_NORM, "out_norm": hip.W_OUT_NORM}
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = hip.Device(0)
+    yield d
+    d.close()
+
+
+def build(dev, cfg, fmts, seed=0):
+    """Random-init weights in the given formats, on the host (for the oracle) and the device."""
+    c = cfg
+    qd, kvd = c["n_heads"] * c["head_dim"], c["n_kv_heads"] * c["head_dim"]
+    shapes = {"q": (qd, c["d_model"]), "k": (kvd, c["d_model"]), "v": (kvd, c["d_model"]), "o": (c["d_model"], qd),
+              "gate": (c["d_ffn"], c["d_model"]), "up": (c["d_ffn"], c["d_model"]), "down": (c["d_model"], c["d_ffn"])}
+    rng = np.random.default_rng(seed)
+    host, model = {}, hip.Llama(dev, **c)
+    s = seed * 1000
+    for l in range(c["n_layers"]):
+        for kind, (r, k) in shapes.items():
+            fmt = fmts.get(kind, fmts["default"])
+            blocks = synth.random_weight(fmt, r, k, seed=(s := s + 1), scale=synth.unit_scale(fmt))
+            host[(kind, l)] = (fmt, blocks)
+            model.set_qweight(KINDS[kind], l, dev.qtensor(fmt, r, k, blocks))
+        for kind in ("attn_norm", "ffn_norm"):
+            a = (1 + 0.1 * rng.standard_normal(c["d_model"])).astype(np.float32)
+            host[(kind, l)] = a
+            model.set_norm(KINDS[kind], l, a)
+    a = (1 + 0.1 * rng.standard_normal(c["d_model"])).astype(np.float32)
+    host[("out_norm", -1)] = a
+    model.set_norm(hip.W_OUT_NORM, -1, a)
+    for kind in ("head", "embed"):
+        fmt = fmts.get(kind, fmts["default"])
+        blocks = synth.random_weight(fmt, c["vocab"], c["d_model"], seed=(s := s + 1), scale=synth.unit_scale(fmt))
+        host[(kind, -1)] = (fmt, blocks)
+        model.set_qweight(KINDS[kind], -1, dev.qtensor(fmt, c["vocab"], c["d_model"], blocks))
+    return host, model
+
+
+def rel(got, want):
+    return float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want)))
+
+
+@pytest.mark.parametrize("name,cfg,fmts", [
+    ("7b-shaped", dict(n_layers=2, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=11008, vocab=2048,
+                       max_pos=48, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}),
+    ("8b-shaped-gqa", dict(n_layers=2, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ffn=14336, vocab=2048,
+                           max_pos=48, rms_eps=1e-5, rope_base=500000.0),
+     {"default": synth.Q4_K, "down": synth.Q6_K, "head": synth.Q6_K, "embed": synth.Q8_0}),
+    ("small-mixed", dict(n_layers=3, d_model=512, n_heads=8, n_kv_heads=2, head_dim=64, d_ffn=1024, vocab=512,
+                         max_pos=16, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q8_0, "gate": synth.Q4_0, "down": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q4_K}),
+])
+def test_decode_steps_match_cpu_composition(dev, name, cfg, fmts):
+    host, model = build(dev, cfg, fmts, seed=3)
+    ref = llama_ref.LlamaRef(cfg, host)
+    rng = np.random.default_rng(5)
+    tokens = rng.integers(0, cfg["vocab"], 4)
+    for pos, tok in enumerate(tokens):
+        nt, logits = model.decode(int(tok), pos)
+        rt, rlogits, _ = ref.step(ref.embed(int(tok)), pos)
+        # logits within 1e-3 of the CPU result (max-norm); the Q8_0 re-quantization of every
+        # activation amplifies f32 rounding differences a little, layer after layer
+        assert rel(logits, rlogits) <= 1e-3, (name, pos)
+        top2 = np.sort(rlogits)[-2:]
+        if top2[1] - top2[0] > 2e-3 * np.max(np.abs(rlogits)):
+            assert nt == rt, (name, pos)
+        assert nt == int(np.argmax(logits))
+    # the device KV cache holds what the CPU composition wrote
+    kptr, vptr, nbytes = model.kv_cache()
+    kc = np.empty(nbytes // 4, np.float32)
+    hip._check(hip.lib().candy_hip_d2h(dev.handle, kc.ctypes.data, kptr, nbytes))
+    kc = kc.reshape(ref.k_cache.shape)
+    assert rel(kc[:, :, :len(tokens)], ref.k_cache[:, :, :len(tokens)].astype(np.float64)) <= 1e-3
+
+
+def test_decode_errors(dev):
+    cfg = dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, head_dim=128, d_ffn=256, vocab=64, max_pos=4,
+               rms_eps=1e-5, rope_base=10000.0)
+    model = hip.Llama(dev, **cfg)
+    with pytest.raises(hip.CandyHipError, match="embedding table not set"):
+        model.decode(0, 0)
+    with pytest.raises(hip.CandyHipError, match="must be"):
+        model.set_qweight(hip.W_Q, 0, dev.qtensor(synth.Q4_K, 8, 256, synth.random_weight(synth.Q4_K, 8, 256, 1)))
+    host, model = build(dev, cfg, {"default": synth.Q4_K}, seed=1)
+    with pytest.raises(hip.CandyHipError, match="outside the cache"):
+        model.decode(0, 4)
+    with pytest.raises(hip.CandyHipError, match="outside the vocabulary"):
+        model.decode(64, 0)

@@ -1,0 +1,125 @@
+"""GPU parity of QMatMul against the CPU oracle: max_n |gpu - ref| / max_n |ref| <= 1e-3
+(the f32 accumulation order differs; integer block dots are exact on both sides)."""
+import numpy as np
+import pytest
+
+from candy_amd import hip, synth
+from oracle import oracle as o
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3  # the stated bar; observed distances are ~1e-6
+FORMATS = [synth.Q4_0, synth.Q4_0_GGML, synth.Q8_0, synth.Q4_K, synth.Q6_K]
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = hip.Device(0)
+    yield d
+    d.close()
+
+
+def rel_err(got, want):
+    return float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))) / np.max(np.abs(want)))
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("rows,cols", [(64, 256), (37, 512), (256, 4096), (130, 11008), (8, 14336)])
+def test_matvec_matches_oracle(dev, fmt, rows, cols):
+    w = synth.random_weight(fmt, rows, cols, seed=rows * 7 + cols + fmt)
+    x = synth.random_activations(1, cols, seed=cols + fmt)
+    q = dev.qtensor(fmt, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    want = o.qmatmul(fmt, w, rows, cols, x)
+    assert got.shape == (1, rows)
+    assert rel_err(got, want) <= TOL
+    assert rel_err(got, want) <= 2e-5  # much tighter in practice; catches a dropped block or scale
+
+
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q8_0, synth.Q6_K, synth.Q4_0])
+@pytest.mark.parametrize("m", [2, 3, 5, 8, 15])
+def test_small_batch_matches_oracle(dev, fmt, m):
+    rows, cols = 96, 4096
+    w = synth.random_weight(fmt, rows, cols, seed=m + fmt)
+    x = synth.random_activations(m, cols, seed=m * 3 + fmt)
+    q = dev.qtensor(fmt, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    want = o.qmatmul(fmt, w, rows, cols, x)
+    assert got.shape == (m, rows)
+    assert rel_err(got, want) <= 2e-5
+
+
+def test_config_q4_0_4096x4096(dev):
+    # BASELINE config 0: Q4_0 4096x4096, one f32 N(0,1) vector, seeded
+    rows = cols = 4096
+    w = synth.random_weight(synth.Q4_0, rows, cols, seed=20240)
+    x = synth.random_activations(1, cols, seed=20241)
+    q = dev.qtensor(synth.Q4_0, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    sub = np.arange(0, rows, 16)  # the oracle on a row subset keeps the test in seconds
+    wb = w.reshape(rows, -1)[sub].reshape(-1)
+    want = o.qmatmul(synth.Q4_0, wb, len(sub), cols, x)
+    assert rel_err(got[:, sub], want) <= 2e-5
+    # and against candy's literal CPU composition (dequantize + naive f32 loops) on the
+    # Q8_0-dequantized activations: same mathematics, different rounding
+    xdq = o.dequantize(synth.Q8_0, o.quantize_q8_0(x)).reshape(1, cols)
+    lit = o.matmul_dequant_f32(synth.Q4_0, wb, len(sub), cols, xdq)
+    assert rel_err(got[:, sub], lit) <= 1e-4
+
+
+@pytest.mark.parametrize("fmt", [synth.Q8_0, synth.Q4_K])
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)])
+def test_config_sweep_full_shapes(dev, fmt, rows, cols):
+    # BASELINE config 1 at full size: oracle on a strided row subset + linearity over the whole output
+    w = synth.random_weight(fmt, rows, cols, seed=rows + cols + fmt)
+    x = synth.random_activations(1, cols, seed=3 * rows + fmt)
+    q = dev.qtensor(fmt, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    sub = np.arange(0, rows, max(1, rows // 128))
+    rb = synth.weight_nbytes(fmt, 1, cols)
+    wb = w.reshape(rows, rb)[sub].reshape(-1)
+    want = o.qmatmul(fmt, wb, len(sub), cols, x)
+    assert rel_err(got[:, sub], want) <= 2e-5
+    # exact scaling property over every row: x -> 2x doubles Q8_0 scales, leaves quants unchanged
+    got2 = dev.qmatmul(q, 2 * x)
+    assert np.array_equal(got2, 2 * got)
+
+
+def test_q6_k_head_shape(dev):
+    rows, cols = 32000, 4096
+    w = synth.random_weight(synth.Q6_K, rows, cols, seed=606)
+    x = synth.random_activations(1, cols, seed=607)
+    q = dev.qtensor(synth.Q6_K, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    sub = np.arange(0, rows, 250)
+    wb = w.reshape(rows, -1)[sub].reshape(-1)
+    assert rel_err(got[:, sub], o.qmatmul(synth.Q6_K, wb, len(sub), cols, x)) <= 2e-5
+
+
+def test_qmatmul_from_prequantized_blocks(dev):
+    rows, cols, m = 64, 1024, 3
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=1)
+    x = synth.random_activations(m, cols, seed=2)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    xb = o.quantize_q8_0(x)
+    assert np.array_equal(dev.qmatmul_q8(q, xb, m), dev.qmatmul(q, x))
+
+
+def test_zero_and_extreme_activations(dev):
+    rows, cols = 32, 512
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=4)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    assert np.all(dev.qmatmul(q, np.zeros((1, cols), np.float32)) == 0)
+    x = synth.random_activations(1, cols, seed=5) * np.float32(1e4)
+    assert rel_err(dev.qmatmul(q, x), o.qmatmul(synth.Q4_K, w, rows, cols, x)) <= 2e-5
+
+
+def test_qmatmul_errors(dev):
+    with pytest.raises(hip.CandyHipError, match="multiple of the block size"):
+        dev.qtensor(synth.Q4_K, 4, 100, np.zeros(10, np.uint8))
+    with pytest.raises(hip.CandyHipError, match="bytes"):
+        dev.qtensor(synth.Q4_K, 4, 256, np.zeros(10, np.uint8))
+    with pytest.raises(hip.CandyHipError, match="unknown quantized format"):
+        dev.qtensor(99, 4, 256, np.zeros(10, np.uint8))
+    with pytest.raises(hip.CandyHipError, match="invalid matrix dimensions"):
+        dev.qtensor(synth.Q4_K, 0, 256, np.zeros(0, np.uint8))
