@@ -63,11 +63,21 @@ __device__ __forceinline__ int dot4_i8(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
 }
 
+// Cross-lane moves on the DPP path (no LDS traffic, no waits).
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, BANK_MASK, true));
+}
+
 // Sum over the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    v += dpp_move<0xB1>(v);        // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);        // quad_perm [2,3,0,1]
+    v += dpp_move<0x141>(v);       // row_half_mirror
+    v += dpp_move<0x140>(v);       // row_mirror: every lane of a 16-lane row holds the row sum
+    v += dpp_move<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_move<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3: lane 63 holds the total
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

@@ -12,6 +12,10 @@
 // (64 weights of a Q4_K super-block, 32 weights otherwise) per step, so consecutive lanes read
 // consecutive bytes of the row; the R rows' loads are issued together to keep many bytes in
 // flight per wavefront.  Per-row partial sums are reduced across the 64 lanes at the end.
+#include <algorithm>
+#include <cstdlib>
+#include <type_traits>
+
 #include "blocks.h"
 #include "internal.h"
 
@@ -40,19 +44,25 @@ __device__ __forceinline__ void stage_activations(const int8_t *__restrict__ xq,
     __syncthreads();
 }
 
+// Weight loads.  Plain (cached) loads on purpose: a 128-byte line of a row is touched by up to
+// three load instructions of the same wavefront (header, two halves of the nibbles), and a
+// non-temporal hint makes the later ones fetch the line again.
+template <class T>
+__device__ __forceinline__ T ldg_stream(const T *p) { return *p; }
+
 // ------------------------------------------------------------------ per-format units
 
 struct UnitQ4K {
     static constexpr int ELEMS = 64;        // two 32-value sub-blocks sharing 32 bytes of nibbles
     static constexpr int ROW_ALIGN = 16;
-    struct W { uint4 hdr, q0, q1; };
+    struct W { u32x4 hdr, q0, q1; };
     __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 144; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const uint8_t *blk = row + (size_t)(u >> 2) * 144;
-        w.hdr = *(const uint4 *)blk;
-        const uint4 *q = (const uint4 *)(blk + 16 + (u & 3) * 32);
-        w.q0 = q[0];
-        w.q1 = q[1];
+        w.hdr = ldg_stream((const u32x4 *)blk);
+        const u32x4 *q = (const u32x4 *)(blk + 16 + (u & 3) * 32);
+        w.q0 = ldg_stream(q);
+        w.q1 = ldg_stream(q + 1);
     }
     // sum over the unit of w*x, with x = d_x * q_x: quantized.cu:2239-2263
     __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
@@ -87,8 +97,8 @@ struct UnitQ8_0 {
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const BlockQ8_0 *blk = (const BlockQ8_0 *)row + u;
         w.d = blk->d;
-        w.q0 = *(const u32x4_a2 *)(blk->qs);
-        w.q1 = *(const u32x4_a2 *)(blk->qs + 16);
+        w.q0 = ldg_stream((const u32x4_a2 *)(blk->qs));
+        w.q1 = ldg_stream((const u32x4_a2 *)(blk->qs + 16));
     }
     // quantized.cu:2058-2073
     __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
@@ -110,7 +120,7 @@ struct UnitQ4_0 {
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const BlockQ4_0 *blk = (const BlockQ4_0 *)row + u;
         w.d = blk->d;
-        w.q = *(const u32x4_a2 *)(blk->qs);
+        w.q = ldg_stream((const u32x4_a2 *)(blk->qs));
     }
     // Sum (q-8)*x = sum q*x - 8*sum x, all in integers. quantized.cu:1919-1941 gets the
     // second term from the Q8_1 block's float sum; with Q8_0 activations it is the exact integer.
@@ -152,9 +162,9 @@ struct UnitQ6K {
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const BlockQ6K *blk = (const BlockQ6K *)row + (u >> 3);
         const int ip = (u >> 2) & 1, j = u & 3;
-        w.ql0 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 8 * j);
-        w.ql1 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 32 + 8 * j);
-        w.qh = *(const u32x2_a2 *)(blk->qh + 32 * ip + 8 * j);
+        w.ql0 = ldg_stream((const u32x2_a2 *)(blk->ql + 64 * ip + 8 * j));
+        w.ql1 = ldg_stream((const u32x2_a2 *)(blk->ql + 64 * ip + 32 + 8 * j));
+        w.qh = ldg_stream((const u32x2_a2 *)(blk->qh + 32 * ip + 8 * j));
         const int8_t *sc = blk->scales + 8 * ip + (j >> 1);
         w.sc = (uint32_t)(uint8_t)sc[0] | ((uint32_t)(uint8_t)sc[2] << 8) | ((uint32_t)(uint8_t)sc[4] << 16) |
                ((uint32_t)(uint8_t)sc[6] << 24);
@@ -185,8 +195,79 @@ struct UnitQ6K {
     }
 };
 
-// ------------------------------------------------------------------ kernel
+// ------------------------------------------------------------------ kernels
+// Nothing in these kernels branches around a memory operation: out-of-range lanes load a
+// clamped (valid) address and their contribution is dropped afterwards.  That keeps the
+// hardware load counter exact, so waiting for the activations (issued first, returned first)
+// leaves the weight loads in flight.
 
+// Batch-1 kernel.  ITER = ceil(units / 64) is a compile-time bound: every weight load of the
+// wavefront's R rows is in flight before anything waits.  The grid covers all rows at once.
+template <class U, int ITER, int R, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec1(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
+                                                        const Q8Scale *__restrict__ xs, float *__restrict__ y,
+                                                        int N, int K) {
+    constexpr int T = WAVES * 64;
+    constexpr int CAP = ITER * 64 * U::ELEMS;       // activation bytes the LDS image is sized for
+    constexpr int AQ = (CAP / 16 + T - 1) / T;      // 16-byte chunks of quants per thread
+    constexpr int AS = (CAP / 32 + T - 1) / T;      // 8-byte scales per thread
+    extern __shared__ __align__(16) uint8_t smem[];  // sized for AQ*T chunks + AS*T scales: no bounds checks
+    int8_t *sq = (int8_t *)smem;
+    Q8Scale *ss = (Q8Scale *)(smem + skewed(AQ * T * 16));
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int units = K / U::ELEMS;
+    const size_t rb = U::row_bytes(K);
+    const int qchunks = K >> 4, sblocks = K >> 5;
+
+    uint4 aq[AQ];
+    uint2 as[AS];
+#pragma unroll
+    for (int i = 0; i < AQ; ++i) aq[i] = ((const uint4 *)xq)[min(tid + i * T, qchunks - 1)];
+#pragma unroll
+    for (int i = 0; i < AS; ++i) as[i] = ((const uint2 *)xs)[min(tid + i * T, sblocks - 1)];
+
+    const int row0 = (blockIdx.x * WAVES + wave) * R;
+    typename U::W w[R][ITER];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint8_t *row = W + (size_t)min(row0 + r, N - 1) * rb;
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[r][it]);
+    }
+
+    // chunks past the row's end land in the padding of the LDS image
+#pragma unroll
+    for (int i = 0; i < AQ; ++i) {
+        const int c = tid + i * T;
+        ((uint4 *)sq)[c + (c >> 4)] = aq[i];
+    }
+#pragma unroll
+    for (int i = 0; i < AS; ++i) ((uint2 *)ss)[tid + i * T] = as[i];
+    __syncthreads();
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int u = it * 64 + lane;
+        const bool live = u < units;
+        const int uc = live ? u : units - 1;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float v = U::dot(w[r][it], uc, sq, ss);
+            acc[r] += live ? v : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float v = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < N) y[row0 + r] = v;
+    }
+}
+
+// General kernel: NB activation rows (small batch) and any contraction length; each wavefront
+// owns R weight rows and walks the row 64 units at a time.
 template <class U, int NB, int R, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
                                                        const Q8Scale *__restrict__ xs, float *__restrict__ y,
@@ -210,17 +291,20 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.0f;
 
-    for (int u = lane; u < units; u += 64) {
+    for (int u0 = 0; u0 < units; u0 += 64) {
+        const int u = u0 + lane;
+        const bool live = u < units;
+        const int uc = live ? u : units - 1;
         typename U::W w[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int row = min(row0 + r, N - 1);  // tail rows recompute the last row, never stored
-            U::load(W + (size_t)row * rb, u, w[r]);
-        }
+        for (int r = 0; r < R; ++r) U::load(W + (size_t)min(row0 + r, N - 1) * rb, uc, w[r]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-            for (int r = 0; r < R; ++r) acc[r][nb] += U::dot(w[r], u, sq + nb * q_bytes, ss + nb * blocks_per_row);
+            for (int r = 0; r < R; ++r) {
+                const float v = U::dot(w[r], uc, sq + nb * q_bytes, ss + nb * blocks_per_row);
+                acc[r][nb] += live ? v : 0.0f;
+            }
     }
 
 #pragma unroll
@@ -230,6 +314,22 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict
             const float v = wave_sum(acc[r][nb]);
             if (lane == 0 && row0 + r < N) y[(size_t)nb * N + row0 + r] = v;
         }
+}
+
+template <class U, int ITER, int R, int WAVES>
+static int launch1(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                   float *y) {
+    const int N = (int)w->rows, K = (int)w->cols;
+    constexpr int T = WAVES * 64, CAP = ITER * 64 * U::ELEMS;
+    constexpr int AQ = (CAP / 16 + T - 1) / T, AS = (CAP / 32 + T - 1) / T;
+    constexpr size_t smem = (size_t)AQ * T * 16 + (((size_t)AQ * T * 16 >> 8) << 4) + (size_t)AS * T * sizeof(Q8Scale);
+    static_assert(smem <= 64 * 1024, "LDS image too large");
+    const int rows_per_wg = R * WAVES;
+    const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
+    hipLaunchKernelGGL((k_matvec1<U, ITER, R, WAVES>), dim3(grid), dim3(WAVES * 64), smem, dev->stream,
+                       (const uint8_t *)w->data, qs, scales, y, N, K);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
 }
 
 template <class U, int NB, int R, int WAVES>
@@ -252,6 +352,20 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
                       int64_t m, float *y) {
     const int64_t K = w->cols, N = w->rows;
     const int64_t sstride = K >> 5;
+    if (m == 1) {
+        const int iter = (int)((K / U::ELEMS + 63) / 64);
+        switch (iter) {
+        case 1: return launch1<U, 1, 1, 4>(dev, w, qs, scales, y);
+        case 2: return launch1<U, 2, 1, 4>(dev, w, qs, scales, y);
+        case 3: return launch1<U, 3, 1, 4>(dev, w, qs, scales, y);
+        case 4: return launch1<U, 4, 1, 4>(dev, w, qs, scales, y);
+        case 5: return launch1<U, 5, 1, 4>(dev, w, qs, scales, y);
+        case 6: return launch1<U, 6, 1, 4>(dev, w, qs, scales, y);
+        case 7: return launch1<U, 7, 1, 4>(dev, w, qs, scales, y);
+        case 8: return launch1<U, 8, 1, 4>(dev, w, qs, scales, y);
+        default: break;  // longer rows take the looping kernel
+        }
+    }
     int64_t done = 0;
     while (done < m) {
         const int64_t left = m - done;
