@@ -179,6 +179,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the other shapes of the batch-1 sweep")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B decode leg")
     ap.add_argument("--decode-steps", type=int, default=32)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a kernel of known traffic for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE MI355X; --gpus must be 1 (no collectives, no sharding)")
@@ -188,6 +190,13 @@ def main():
     log("device:", dev.name)
     fmt, rows, cols = synth.Q4_K, 4096, 11008
     alg = algorithmic_bytes(fmt, rows, cols)
+    if args.calibrate_copy:
+        a, b = dev.alloc(256 << 20), dev.alloc(256 << 20)
+        a.zero()
+        hip._check(hip.lib().candy_hip_d2d(dev.handle, b.ptr, a.ptr, 256 << 20))
+        dev.synchronize()
+        a.free()
+        b.free()
 
     # headline: whole f32-in -> f32-out path
     ms_step, n_copies = time_matvec(dev, fmt, rows, cols, args.steps, args.warmup, quantize_each=True)
