@@ -33,6 +33,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
 ROTATE_BYTES = 640 << 20  # distinct weight bytes cycled through (last-level cache is 256 MB)
 
 
@@ -178,6 +179,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the other shapes of the batch-1 sweep")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B decode leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the batched-prefill (MFMA) leg")
     ap.add_argument("--decode-steps", type=int, default=32)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for counter runs)")
@@ -238,6 +240,20 @@ def main():
                           "frac": round(gb / HBM_PEAK_GBPS, 4)})
             log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
         out["sweep"] = sweep
+
+    if not args.no_prefill:
+        # batched prefill: Q4_K 14336x4096 x f32 [M, 4096]; MFMA peak = dense fp16 (the operand type used)
+        pre = []
+        r, k = 14336, 4096
+        for m in (16, 128, 512):
+            ms, _ = time_matvec(dev, synth.Q4_K, r, k, 200, 20, quantize_each=True, seed=m, m=m)
+            flops = 2.0 * m * r * k
+            byts = algorithmic_bytes(synth.Q4_K, r, k, m)
+            pre.append({"m": m, "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
+                        "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                        "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+            log(f"  prefill q4_k {r}x{k} M={m}: {ms * 1e3:.1f} us, {pre[-1]['TFLOPs']} TFLOP/s, {pre[-1]['GBps']} GB/s")
+        out["prefill"] = pre
 
     if not args.no_decode:
         out["decode"] = decode_leg(dev, args.decode_steps, 4)

@@ -91,8 +91,16 @@ int launch_q8_blocks_to_planar(candy_hip_device *dev, const void *blocks, int64_
 // matvec.hip: y[m, rows] for m in 1..15 from planar activations.
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                   const Q8Scale *scales, int64_t m, float *y);
-// mmq.hip: MFMA tile kernel for m >= 16.
+// mmq.hip: MFMA tile kernel for m >= 16. half_ws: mmq_m_pad(m) * cols fp16 values of scratch.
+int64_t mmq_m_pad(int64_t m);
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
-               const Q8Scale *scales, int64_t m, float *y);
+               const Q8Scale *scales, int64_t m, float *y, void *half_ws);
+// Workspace carved for one contraction: planar quants, scales and (m >= 16) fp16 activations.
+struct ActWorkspace {
+    int8_t *qs;
+    Q8Scale *scales;
+    void *half_ws;
+};
+int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quants, ActWorkspace *out);
 
 }  // namespace candy

@@ -382,6 +382,18 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
     return CANDY_HIP_OK;
 }
 
+int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quants, ActWorkspace *out) {
+    const size_t q_bytes = need_quants ? (((size_t)(m * cols) + 255) & ~(size_t)255) : 0;
+    const size_t s_bytes = need_quants ? (((size_t)(m * (cols >> 5)) * sizeof(Q8Scale) + 255) & ~(size_t)255) : 0;
+    const size_t h_bytes = m >= 16 ? (size_t)(mmq_m_pad(m) * cols) * 2 : 0;
+    void *ws = nullptr;
+    if (int rc = workspace(dev, q_bytes + s_bytes + h_bytes + 256, &ws)) return rc;
+    out->qs = (int8_t *)ws;
+    out->scales = (Q8Scale *)((uint8_t *)ws + q_bytes);
+    out->half_ws = h_bytes ? (uint8_t *)ws + q_bytes + s_bytes : nullptr;
+    return CANDY_HIP_OK;
+}
+
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                   int64_t m, float *y) {
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && w->cols <= 0x7FFFFFFF, "matrix too large");
@@ -401,48 +413,41 @@ using namespace candy;
 
 extern "C" {
 
-static int qmatmul_common(candy_hip_device *dev, const candy_hip_qtensor *w, int64_t m, float *dev_y,
-                          size_t *q_off, size_t *s_off, size_t *total) {
+static int qmatmul_check(candy_hip_device *dev, const candy_hip_qtensor *w, int64_t m, float *dev_y) {
     CANDY_REQUIRE(w, "rhs qtensor is nil");
     CANDY_REQUIRE(dev && w->dev == dev, "rhs storage must live on the same HIP device");
     CANDY_REQUIRE(m >= 0, "invalid matrix dimensions");
     CANDY_REQUIRE(m == 0 || dev_y, "output is nil");
-    const size_t qb = (size_t)m * (size_t)w->cols;
-    *q_off = 0;
-    *s_off = (qb + 255) & ~(size_t)255;
-    *total = *s_off + (size_t)m * (size_t)(w->cols >> 5) * sizeof(Q8Scale);
     return CANDY_HIP_OK;
 }
 
+static int contract(candy_hip_device *dev, const candy_hip_qtensor *w, const ActWorkspace &a, int64_t m, float *y) {
+    return m < 16 ? launch_matvec(dev, w, a.qs, a.scales, m, y) : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws);
+}
+
 int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m, float *dev_y) {
-    size_t q_off, s_off, total;
-    if (int rc = qmatmul_common(dev, w, m, dev_y, &q_off, &s_off, &total)) return rc;
+    if (int rc = qmatmul_check(dev, w, m, dev_y)) return rc;
     if (m == 0) return CANDY_HIP_OK;
     CANDY_REQUIRE(dev_x, "lhs is nil");
     CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "lhs must be 16-byte aligned");
     if (int rc = use_device(dev)) return rc;
-    void *ws = nullptr;
-    if (int rc = workspace(dev, total, &ws)) return rc;
-    int8_t *qs = (int8_t *)ws + q_off;
-    Q8Scale *sc = (Q8Scale *)((uint8_t *)ws + s_off);
-    if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, qs, sc, nullptr)) return rc;
-    return m < 16 ? launch_matvec(dev, w, qs, sc, m, dev_y) : launch_mmq(dev, w, qs, sc, m, dev_y);
+    ActWorkspace a;
+    if (int rc = act_workspace(dev, m, w->cols, true, &a)) return rc;
+    if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, a.qs, a.scales, nullptr)) return rc;
+    return contract(dev, w, a, m, dev_y);
 }
 
 int candy_hip_qmatmul_q8(candy_hip_device *dev, const candy_hip_qtensor *w, const void *dev_x_q8_0, int64_t m,
                          float *dev_y) {
-    size_t q_off, s_off, total;
-    if (int rc = qmatmul_common(dev, w, m, dev_y, &q_off, &s_off, &total)) return rc;
+    if (int rc = qmatmul_check(dev, w, m, dev_y)) return rc;
     if (m == 0) return CANDY_HIP_OK;
     CANDY_REQUIRE(dev_x_q8_0, "lhs is nil");
     CANDY_REQUIRE(((uintptr_t)dev_x_q8_0 & 1) == 0, "lhs blocks must be 2-byte aligned");
     if (int rc = use_device(dev)) return rc;
-    void *ws = nullptr;
-    if (int rc = workspace(dev, total, &ws)) return rc;
-    int8_t *qs = (int8_t *)ws + q_off;
-    Q8Scale *sc = (Q8Scale *)((uint8_t *)ws + s_off);
-    if (int rc = launch_q8_blocks_to_planar(dev, dev_x_q8_0, m * (w->cols >> 5), qs, sc)) return rc;
-    return m < 16 ? launch_matvec(dev, w, qs, sc, m, dev_y) : launch_mmq(dev, w, qs, sc, m, dev_y);
+    ActWorkspace a;
+    if (int rc = act_workspace(dev, m, w->cols, true, &a)) return rc;
+    if (int rc = launch_q8_blocks_to_planar(dev, dev_x_q8_0, m * (w->cols >> 5), a.qs, a.scales)) return rc;
+    return contract(dev, w, a, m, dev_y);
 }
 
 int candy_hip_qact_create(candy_hip_device *dev, int64_t max_m, int64_t max_cols, candy_hip_qact **out) {
@@ -498,8 +503,13 @@ int candy_hip_qmatmul_qact(candy_hip_device *dev, const candy_hip_qtensor *w, co
                   (long long)a->cols, (long long)w->cols);
     CANDY_REQUIRE(dev_y, "output is nil");
     if (int rc = use_device(dev)) return rc;
-    return a->m < 16 ? launch_matvec(dev, w, a->qs, a->scales, a->m, dev_y)
-                     : launch_mmq(dev, w, a->qs, a->scales, a->m, dev_y);
+    ActWorkspace ws{a->qs, a->scales, nullptr};
+    if (a->m >= 16) {
+        ActWorkspace extra;
+        if (int rc = act_workspace(dev, a->m, a->cols, false, &extra)) return rc;
+        ws.half_ws = extra.half_ws;
+    }
+    return contract(dev, w, ws, a->m, dev_y);
 }
 
 int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws, const float *dev_x,
@@ -513,18 +523,14 @@ int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *cons
     CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "lhs must be 16-byte aligned");
     if (int rc = use_device(dev)) return rc;
     const int64_t K = ws[0]->cols;
-    const size_t s_off = ((size_t)(m * K) + 255) & ~(size_t)255;
-    void *wsp = nullptr;
-    if (int rc = workspace(dev, s_off + (size_t)(m * (K >> 5)) * sizeof(Q8Scale), &wsp)) return rc;
-    int8_t *qs = (int8_t *)wsp;
-    Q8Scale *sc = (Q8Scale *)((uint8_t *)wsp + s_off);
-    if (int rc = launch_quantize_q8(dev, dev_x, m, K, qs, sc, nullptr)) return rc;
+    ActWorkspace a;
+    if (int rc = act_workspace(dev, m, K, true, &a)) return rc;
+    if (int rc = launch_quantize_q8(dev, dev_x, m, K, a.qs, a.scales, nullptr)) return rc;
     CANDY_HIP_TRY(hipEventRecord(dev->ev_start, dev->stream));
     for (int i = 0; i < iters; ++i) {
         if (quantize_each)
-            if (int rc = launch_quantize_q8(dev, dev_x, m, K, qs, sc, nullptr)) return rc;
-        const candy_hip_qtensor *w = ws[i % n_ws];
-        if (int rc = m < 16 ? launch_matvec(dev, w, qs, sc, m, dev_y) : launch_mmq(dev, w, qs, sc, m, dev_y)) return rc;
+            if (int rc = launch_quantize_q8(dev, dev_x, m, K, a.qs, a.scales, nullptr)) return rc;
+        if (int rc = contract(dev, ws[i % n_ws], a, m, dev_y)) return rc;
     }
     CANDY_HIP_TRY(hipEventRecord(dev->ev_stop, dev->stream));
     CANDY_HIP_TRY(hipEventSynchronize(dev->ev_stop));
