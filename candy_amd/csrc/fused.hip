@@ -1,0 +1,282 @@
+// Decode-step matvecs with the neighbouring f32 stages folded in, so a Llama block is five
+// launches instead of ten and no activation makes a round trip through HBM between them:
+//   prologue RMS:   RMSNorm (reduce.go:3071-3092) of the f32 input + Q8_0 quantization
+//                   (quantized.cu:3521-3558), recomputed by every workgroup under the shadow of
+//                   its own weight loads (the weights dominate the time; the input is 16 KB);
+//   epilogue PAIR:  the workgroup owns 32 consecutive rows of BOTH gate and up, so it can apply
+//                   SiLU (unary.go:3353-3366) * Mul and quantize the 32 results to one Q8_0 block
+//                   for the down projection;
+//   epilogue RES:   residual Add (backend.go:21) on the output.
+// The contraction itself is the batch-1 kernel of matvec.hip (same units, same exact load
+// counting: inputs first, then every weight load, nothing branches around a memory operation).
+#include "blocks.h"
+#include "internal.h"
+#include "units.h"
+
+namespace candy {
+
+enum { PRO_Q8 = 0, PRO_RMS = 1 };
+enum { EPI_PLAIN = 0, EPI_PAIR = 1 };
+
+struct FusedArgs {
+    MatvecJobs jobs;        // PLAIN: up to 3 weights; PAIR: j[0] = gate, j[1] = up (same shape)
+    // prologue
+    const int8_t *xq;       // PRO_Q8: planar Q8_0 activations
+    const Q8Scale *xs;
+    const float *x;         // PRO_RMS: f32 input row, RMSNorm weight, epsilon
+    const float *alpha;
+    float eps;
+    // PAIR epilogue output: planar Q8_0 of silu(gate.x) * (up.x)
+    int8_t *oq;
+    Q8Scale *os;
+    int K;
+};
+
+__device__ __forceinline__ float silu_exact(float x) { return x / (1.0f + expf(-x)); }
+
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec_fused(const FusedArgs a) {
+    constexpr int T = WAVES * 64;
+    constexpr int CAP = ITER * 64 * U::ELEMS;       // activation values the LDS image is sized for
+    constexpr int AQ = (CAP / 16 + T - 1) / T;      // PRO_Q8: 16-byte chunks of quants per thread
+    constexpr int AS = (CAP / 32 + T - 1) / T;      // PRO_Q8: 8-byte scales per thread
+    constexpr int XF = (CAP / 4 + T - 1) / T;       // PRO_RMS: float4 of input per thread
+    constexpr int NW = EPI == EPI_PAIR ? 2 : 1;     // weights contracted per wavefront
+    extern __shared__ __align__(16) uint8_t smem[];
+    int8_t *sq = (int8_t *)smem;
+    constexpr int QBYTES = (PRO == PRO_Q8 ? AQ * T * 16 : XF * T * 4);
+    Q8Scale *ss = (Q8Scale *)(smem + QBYTES + ((QBYTES >> 8) << 4));
+    __shared__ float s_red[WAVES];
+    __shared__ float s_act[32];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = a.K;
+    const int units = K / U::ELEMS;
+    const size_t rb = U::row_bytes(K);
+
+    int ji = 0, wg = blockIdx.x;
+    if (EPI == EPI_PLAIN) {
+        ji = (int)(blockIdx.x >= (unsigned)a.jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)a.jobs.j[1].wg_end);
+        wg = blockIdx.x - (ji > 0 ? a.jobs.j[ji - 1].wg_end : 0);
+    }
+    const int N = a.jobs.j[ji].N;
+
+    // ---- inputs first (oldest entries of the in-order return queue)
+    uint4 aq[AQ];
+    uint2 as[AS];
+    float4 xv[XF], av[XF];
+    if (PRO == PRO_Q8) {
+        const int qchunks = K >> 4, sblocks = K >> 5;
+#pragma unroll
+        for (int i = 0; i < AQ; ++i) aq[i] = ((const uint4 *)a.xq)[min(tid + i * T, qchunks - 1)];
+#pragma unroll
+        for (int i = 0; i < AS; ++i) as[i] = ((const uint2 *)a.xs)[min(tid + i * T, sblocks - 1)];
+    } else {
+        const int n4 = K >> 2;
+#pragma unroll
+        for (int i = 0; i < XF; ++i) {
+            const int c = min(tid + i * T, n4 - 1);
+            xv[i] = ((const float4 *)a.x)[c];
+            av[i] = ((const float4 *)a.alpha)[c];
+        }
+    }
+
+    // ---- every weight load of the wavefront
+    const int row0 = (wg * WAVES + wave) * R;
+    typename U::W w[NW][R][ITER];
+#pragma unroll
+    for (int m = 0; m < NW; ++m) {
+        const uint8_t *Wm = EPI == EPI_PAIR ? a.jobs.j[m].W : a.jobs.j[ji].W;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint8_t *row = Wm + (size_t)min(row0 + r, N - 1) * rb;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
+        }
+    }
+
+    // ---- park the quantized activations in LDS
+    if (PRO == PRO_Q8) {
+#pragma unroll
+        for (int i = 0; i < AQ; ++i) {
+            const int c = tid + i * T;
+            ((uint4 *)sq)[c + (c >> 4)] = aq[i];
+        }
+#pragma unroll
+        for (int i = 0; i < AS; ++i) ((uint2 *)ss)[tid + i * T] = as[i];
+    } else {
+        const int n4 = K >> 2;
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < XF; ++i) {
+            const float4 v = xv[i];
+            const float t = v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            s += (tid + i * T < n4) ? t : 0.0f;
+        }
+        s = wave_sum(s);
+        if (lane == 0) s_red[wave] = s;
+        __syncthreads();
+        float tot = 0.0f;
+#pragma unroll
+        for (int i = 0; i < WAVES; ++i) tot += s_red[i];
+        const float mean = tot / (float)K;
+        const float scale = 1.0f / (float)sqrt((double)(mean + a.eps));
+#pragma unroll
+        for (int i = 0; i < XF; ++i) {
+            const int c = tid + i * T;
+            const float4 v = xv[i], al = av[i];
+            const float4 xn = make_float4(scale * v.x * al.x, scale * v.y * al.y, scale * v.z * al.z, scale * v.w * al.w);
+            __half h;
+            int bsum;
+            const uint32_t packed = quantize_q8_lane4(xn, h, bsum);
+            *(uint32_t *)(sq + skewed(4 * c)) = packed;  // c past the row lands in the padding
+            if ((c & 7) == 0) {
+                Q8Scale sc;
+                sc.d = __half2float(h);
+                sc.bsum = bsum;
+                ss[c >> 3] = sc;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- contraction
+    float acc[NW][R];
+#pragma unroll
+    for (int m = 0; m < NW; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int u = it * 64 + lane;
+        const bool live = u < units;
+        const int uc = live ? u : units - 1;
+#pragma unroll
+        for (int m = 0; m < NW; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float v = U::dot(w[m][r][it], uc, sq, ss);
+                acc[m][r] += live ? v : 0.0f;
+            }
+    }
+
+    if (EPI == EPI_PLAIN) {
+        float *y = a.jobs.j[ji].y;  // may alias res (h += W.x)
+        const float *res = a.jobs.j[ji].res;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float v = wave_sum(acc[0][r]);
+            if (lane == 0 && row0 + r < N) y[row0 + r] = res ? res[row0 + r] + v : v;
+        }
+    } else {
+        static_assert(EPI != EPI_PAIR || R * WAVES == 32, "a PAIR workgroup owns one 32-value block");
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float g = wave_sum(acc[0][r]), u = wave_sum(acc[1][r]);
+            if (lane == 0) s_act[wave * R + r] = silu_exact(g) * u;
+        }
+        __syncthreads();
+        if (wave == 0) {
+            __half h;
+            int bsum;
+            const int q = quantize_q8_lane1(s_act[lane & 31], h, bsum);
+            const int blk = wg;  // N % 32 == 0: every workgroup holds a whole block
+            if (lane < 32) a.oq[(size_t)blk * 32 + lane] = (int8_t)q;
+            if (lane == 0) {
+                Q8Scale sc;
+                sc.d = __half2float(h);
+                sc.bsum = bsum;
+                a.os[blk] = sc;
+            }
+        }
+    }
+}
+
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
+static int launch_fused_cfg(candy_hip_device *dev, FusedArgs a) {
+    constexpr int T = WAVES * 64, CAP = ITER * 64 * U::ELEMS;
+    constexpr int AQ = (CAP / 16 + T - 1) / T, AS = (CAP / 32 + T - 1) / T, XF = (CAP / 4 + T - 1) / T;
+    constexpr size_t QBYTES = PRO == PRO_Q8 ? (size_t)AQ * T * 16 : (size_t)XF * T * 4;
+    constexpr size_t SBYTES = PRO == PRO_Q8 ? (size_t)AS * T * 8 : ((size_t)XF * T / 8 + 1) * 8;
+    constexpr size_t smem = QBYTES + ((QBYTES >> 8) << 4) + SBYTES;
+    static_assert(smem <= 60 * 1024, "LDS image too large");
+    const int rows_per_wg = R * WAVES;
+    int total = 0;
+    if (EPI == EPI_PAIR) {
+        total = a.jobs.j[0].N / 32;
+    } else {
+        for (int i = 0; i < 3; ++i) {
+            if (i < a.jobs.n) total += (a.jobs.j[i].N + rows_per_wg - 1) / rows_per_wg;
+            a.jobs.j[i].wg_end = total;
+        }
+    }
+    hipLaunchKernelGGL((k_matvec_fused<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)total), dim3(T), smem, dev->stream, a);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+// Tile shapes: PLAIN keeps the batch-1 kernel's one row per wavefront when the input is already
+// quantized; with the RMSNorm prologue a workgroup takes 16 rows so that the (redundant) prologue
+// is amortised; PAIR is 8 wavefronts x 4 rows of each of the two weights.
+template <class U, int ITER>
+static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro, int epi) {
+    if (epi == EPI_PAIR) {
+        if constexpr (ITER <= 2) {  // two weights x 4 rows x ITER units must stay in registers
+            return pro == PRO_RMS ? launch_fused_cfg<U, ITER, 4, 8, PRO_RMS, EPI_PAIR>(dev, a)
+                                  : launch_fused_cfg<U, ITER, 4, 8, PRO_Q8, EPI_PAIR>(dev, a);
+        } else {
+            return CANDY_HIP_ERR_UNSUPPORTED;
+        }
+    }
+    if (pro == PRO_RMS) {
+        if constexpr (ITER <= 2) return launch_fused_cfg<U, ITER, 4, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+        else return launch_fused_cfg<U, ITER, 2, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+    }
+    return launch_fused_cfg<U, ITER, 1, 4, PRO_Q8, EPI_PLAIN>(dev, a);
+}
+
+template <class U>
+static int launch_fused_fmt(candy_hip_device *dev, const FusedArgs &a, int pro, int epi) {
+    const int iter = (a.K / U::ELEMS + 63) / 64;
+    switch (iter) {
+    case 1: return launch_fused_iter<U, 1>(dev, a, pro, epi);
+    case 2: return launch_fused_iter<U, 2>(dev, a, pro, epi);
+    case 3: return launch_fused_iter<U, 3>(dev, a, pro, epi);
+    case 4: return launch_fused_iter<U, 4>(dev, a, pro, epi);
+    default: return CANDY_HIP_ERR_UNSUPPORTED;
+    }
+}
+
+// Returns CANDY_HIP_ERR_UNSUPPORTED (without setting the error text) when no instantiation covers
+// the request; the caller then runs the unfused sequence.
+int launch_matvec_fused(candy_hip_device *dev, const FusedLaunch &L) {
+    const int n = L.n;
+    if (n < 1 || n > 3) return CANDY_HIP_ERR_UNSUPPORTED;
+    const candy_hip_qtensor *w0 = L.w[0];
+    for (int i = 1; i < n; ++i)
+        if (L.w[i]->fmt != w0->fmt || L.w[i]->cols != w0->cols) return CANDY_HIP_ERR_UNSUPPORTED;
+    const int pro = L.x ? PRO_RMS : PRO_Q8, epi = L.pair ? EPI_PAIR : EPI_PLAIN;
+    if (L.pair && (n != 2 || L.w[0]->rows != L.w[1]->rows || w0->rows % 32 != 0)) return CANDY_HIP_ERR_UNSUPPORTED;
+    if (w0->cols > 0x7FFFFFFF) return CANDY_HIP_ERR_UNSUPPORTED;
+    FusedArgs a{};
+    a.jobs.n = n;
+    for (int i = 0; i < n; ++i) {
+        if (L.w[i]->rows > 0x7FFFFFFF) return CANDY_HIP_ERR_UNSUPPORTED;
+        a.jobs.j[i].W = (const uint8_t *)L.w[i]->data;
+        a.jobs.j[i].y = L.y[i];
+        a.jobs.j[i].res = L.res[i];
+        a.jobs.j[i].N = (int)L.w[i]->rows;
+    }
+    a.xq = L.xq; a.xs = L.xs; a.x = L.x; a.alpha = L.alpha; a.eps = L.eps; a.oq = L.oq; a.os = L.os;
+    a.K = (int)w0->cols;
+    switch (w0->fmt) {
+    case CANDY_HIP_Q4_K: return launch_fused_fmt<UnitQ4K>(dev, a, pro, epi);
+    case CANDY_HIP_Q8_0: return launch_fused_fmt<UnitQ8_0>(dev, a, pro, epi);
+    case CANDY_HIP_Q4_0: return launch_fused_fmt<UnitQ4_0<false>>(dev, a, pro, epi);
+    case CANDY_HIP_Q4_0_GGML: return launch_fused_fmt<UnitQ4_0<true>>(dev, a, pro, epi);
+    case CANDY_HIP_Q6_K: return launch_fused_fmt<UnitQ6K>(dev, a, pro, epi);
+    default: return CANDY_HIP_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace candy

@@ -67,6 +67,21 @@ struct candy_hip_qtensor {
     bool owned = false;
 };
 
+namespace candy {
+// Kernel argument of the batch-1 matvec: up to three weights that share one activation row.
+struct MatvecJob {
+    const uint8_t *W;
+    float *y;
+    const float *res;  // optional residual added to the output (may alias y)
+    int N;
+    int wg_end;        // cumulative workgroup count, filled by the launcher
+};
+struct MatvecJobs {
+    MatvecJob j[3];
+    int n;
+};
+}  // namespace candy
+
 struct candy_hip_qact {
     candy_hip_device *dev = nullptr;
     int64_t max_m = 0, max_cols = 0;  // capacity
@@ -91,10 +106,60 @@ int launch_q8_blocks_to_planar(candy_hip_device *dev, const void *blocks, int64_
 // matvec.hip: y[m, rows] for m in 1..15 from planar activations.
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                   const Q8Scale *scales, int64_t m, float *y);
+// matvec.hip: one activation row against up to three weights in one launch, optional residuals.
+int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *ws, float *const *ys,
+                        const float *const *res, int n, const int8_t *qs, const Q8Scale *scales);
 // mmq.hip: MFMA tile kernel for m >= 16. half_ws: mmq_m_pad(m) * cols fp16 values of scratch.
 int64_t mmq_m_pad(int64_t m);
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                const Q8Scale *scales, int64_t m, float *y, void *half_ws);
+// ops.hip: fused decode-step stages (all enqueue on dev->stream, no allocation, no sync).
+int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
+                          int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales);
+int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *act_out,
+                          int8_t *qs, Q8Scale *scales);
+// fused.hip: batch-1 contraction of one activation row with up to three weights, with optional
+// RMSNorm+quantize prologue (x != nullptr, else planar Q8_0 in xq/xs), residuals, or the
+// gate/up SiLU*Mul+quantize epilogue (pair). Returns CANDY_HIP_ERR_UNSUPPORTED when the shape
+// has no fused instantiation (caller falls back to the unfused sequence).
+struct FusedLaunch {
+    int n = 0;
+    const candy_hip_qtensor *w[3] = {nullptr, nullptr, nullptr};
+    float *y[3] = {nullptr, nullptr, nullptr};
+    const float *res[3] = {nullptr, nullptr, nullptr};
+    const int8_t *xq = nullptr;
+    const Q8Scale *xs = nullptr;
+    const float *x = nullptr, *alpha = nullptr;
+    float eps = 0.0f;
+    bool pair = false;
+    int8_t *oq = nullptr;
+    Q8Scale *os = nullptr;
+};
+int launch_matvec_fused(candy_hip_device *dev, const FusedLaunch &launch);
+// attention.hip
+struct AttnLaunch {
+    const float *q = nullptr;      // [n_heads, head_dim]; pre-Rope when k_new is set
+    const float *k_new = nullptr;  // optional pre-Rope key / value rows of the new token, [n_kv_heads, head_dim]
+    const float *v_new = nullptr;
+    const float *cos_t = nullptr;  // Rope tables [max_pos, head_dim/2] (with k_new)
+    const float *sin_t = nullptr;
+    float *k_cache = nullptr;      // this layer's cache, cache_stride elements between kv heads
+    float *v_cache = nullptr;
+    const int *pos_ptr = nullptr;  // position of the new token in device memory, or
+    int n_pos = 0;                 // number of cached positions to attend when pos_ptr is null
+    int64_t cache_stride = 0;
+    float scale = 1.0f;
+    int n_heads = 0, n_kv_heads = 0, head_dim = 0, n_splits = 1;
+    void *scratch = nullptr;       // attention_scratch_bytes() of device memory
+    float *out = nullptr;          // optional f32 output [n_heads, head_dim]
+    int8_t *oq = nullptr;          // optional planar Q8_0 output
+    Q8Scale *os = nullptr;
+};
+int attention_splits(const candy_hip_device *dev, int64_t n_kv_heads, int64_t max_pos);
+size_t attention_scratch_bytes(int n_heads, int n_kv_heads, int head_dim, int n_splits);
+int launch_attention(candy_hip_device *dev, const AttnLaunch &launch);
+// runtime.hip: zero-fill with a kernel (safe to capture into a HIP graph, unlike a memset node)
+int launch_zero(candy_hip_device *dev, void *dptr, size_t bytes);
 // Workspace carved for one contraction: planar quants, scales and (m >= 16) fp16 activations.
 struct ActWorkspace {
     int8_t *qs;

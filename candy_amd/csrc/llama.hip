@@ -4,6 +4,7 @@
 // BackendStorage calls (backend.go) a candy model would issue, with the quantized Linear in
 // place of MatMul.
 #include <cmath>
+#include <cstdlib>
 #include <vector>
 
 #include "blocks.h"
@@ -23,46 +24,28 @@ struct candy_hip_llama {
     // device buffers
     float *k_cache = nullptr, *v_cache = nullptr;  // [n_layers][n_kv_heads][max_pos][head_dim]
     float *cos_t = nullptr, *sin_t = nullptr;      // [max_pos][head_dim/2]
-    float *h = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *att = nullptr;
-    float *gate_o = nullptr, *up_o = nullptr, *act = nullptr, *tmp = nullptr, *logits = nullptr;
+    float *h = nullptr, *q = nullptr, *k = nullptr, *v = nullptr;
+    float *gate_o = nullptr, *up_o = nullptr, *logits = nullptr;
     int8_t *xq = nullptr;           // planar Q8_0 quants of the current activation
     candy::Q8Scale *xs = nullptr;
     uint32_t *next_tok = nullptr;
     int64_t *tok_id = nullptr;
+    int *d_pos = nullptr;                         // position of the token being decoded (device copy)
+    void *attn_scratch = nullptr;                 // attention split partials
+    int n_splits = 1;
+    hipGraph_t graph = nullptr;                   // the captured step (layers + head + argmax)
+    hipGraphExec_t graph_exec = nullptr;
+    bool graph_dirty = true;
+    bool use_graph = true;
     std::vector<void *> owned;
 };
 
 namespace candy {
 
-// RoPE on the new q and k rows (reduce.go:3987-4006 with t = 1: pairs (i, i + d/2), cos/sin row
-// of this position), then k and v go to row `pos` of their kv head's cache.
-__global__ __launch_bounds__(256) void k_rope_store(float *__restrict__ q, const float *__restrict__ k,
-                                                    const float *__restrict__ v, const float *__restrict__ cos_row,
-                                                    const float *__restrict__ sin_row, int n_heads, int n_kv_heads,
-                                                    int head_dim, int pos, int max_pos, float *__restrict__ k_cache,
-                                                    float *__restrict__ v_cache) {
-    const int half = head_dim >> 1;
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    const int nq = n_heads * half, nk = n_kv_heads * half;
-    if (idx < nq) {
-        const int hh = idx / half, i = idx - hh * half;
-        float *p = q + hh * head_dim;
-        const float a = p[i], b = p[i + half], c = cos_row[i], s = sin_row[i];
-        p[i] = a * c - b * s;
-        p[i + half] = a * s + b * c;
-    } else if (idx < nq + nk) {
-        const int j = idx - nq;
-        const int hh = j / half, i = j - hh * half;
-        const float *p = k + hh * head_dim;
-        const float a = p[i], b = p[i + half], c = cos_row[i], s = sin_row[i];
-        float *kd = k_cache + ((size_t)hh * max_pos + pos) * head_dim;
-        kd[i] = a * c - b * s;
-        kd[i + half] = a * s + b * c;
-        const float *pv = v + hh * head_dim;
-        float *vd = v_cache + ((size_t)hh * max_pos + pos) * head_dim;
-        vd[i] = pv[i];
-        vd[i + half] = pv[i + half];
-    }
+// Parks the step's position and token id in device memory (read by the captured kernels).
+__global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok) {
+    *pos_dst = pos;
+    if (tok >= 0) *tok_dst = tok;
 }
 
 }  // namespace candy
@@ -78,14 +61,6 @@ static int dev_alloc(candy_hip_llama *m, T **p, size_t count) {
     return CANDY_HIP_OK;
 }
 
-static int linear(candy_hip_llama *m, const candy_hip_qtensor *w, float *y) {
-    return launch_matvec(m->dev, w, m->xq, m->xs, 1, y);
-}
-
-static int quantize(candy_hip_llama *m, const float *x, int64_t n) {
-    return launch_quantize_q8(m->dev, x, 1, n, m->xq, m->xs, nullptr);
-}
-
 extern "C" {
 
 int candy_hip_qindex_select(candy_hip_device *dev, const candy_hip_qtensor *q, const int64_t *dev_ids, int64_t n_ids,
@@ -99,7 +74,7 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
                       cfg->head_dim > 0 && cfg->d_ffn > 0 && cfg->vocab > 0 && cfg->max_pos > 0,
                   "every size in the config must be positive");
     CANDY_REQUIRE(cfg->n_heads % cfg->n_kv_heads == 0, "n_heads must be a multiple of n_kv_heads");
-    CANDY_REQUIRE(cfg->head_dim % 2 == 0 && cfg->head_dim <= 256, "head_dim must be even and <= 256");
+    CANDY_REQUIRE(cfg->head_dim == 64 || cfg->head_dim == 128, "head_dim must be 64 or 128");
     CANDY_REQUIRE(cfg->d_model % 256 == 0 && cfg->d_ffn % 256 == 0 && (cfg->n_heads * cfg->head_dim) % 256 == 0,
                   "d_model, d_ffn and n_heads*head_dim must be multiples of 256");
     if (int rc = use_device(dev)) return rc;
@@ -116,20 +91,24 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
     if (!rc) rc = dev_alloc(m, &m->cos_t, (size_t)cfg->max_pos * half);
     if (!rc) rc = dev_alloc(m, &m->sin_t, (size_t)cfg->max_pos * half);
     if (!rc) rc = dev_alloc(m, &m->h, (size_t)cfg->d_model);
-    if (!rc) rc = dev_alloc(m, &m->xn, widest);
     if (!rc) rc = dev_alloc(m, &m->q, (size_t)cfg->n_heads * cfg->head_dim);
     if (!rc) rc = dev_alloc(m, &m->k, (size_t)cfg->n_kv_heads * cfg->head_dim);
     if (!rc) rc = dev_alloc(m, &m->v, (size_t)cfg->n_kv_heads * cfg->head_dim);
-    if (!rc) rc = dev_alloc(m, &m->att, (size_t)cfg->n_heads * cfg->head_dim);
     if (!rc) rc = dev_alloc(m, &m->gate_o, (size_t)cfg->d_ffn);
     if (!rc) rc = dev_alloc(m, &m->up_o, (size_t)cfg->d_ffn);
-    if (!rc) rc = dev_alloc(m, &m->act, (size_t)cfg->d_ffn);
-    if (!rc) rc = dev_alloc(m, &m->tmp, (size_t)cfg->d_model);
     if (!rc) rc = dev_alloc(m, &m->logits, (size_t)cfg->vocab);
     if (!rc) rc = dev_alloc(m, &m->xq, widest);
     if (!rc) rc = dev_alloc(m, &m->xs, widest / 32);
     if (!rc) rc = dev_alloc(m, &m->next_tok, 1);
     if (!rc) rc = dev_alloc(m, &m->tok_id, 1);
+    if (!rc) rc = dev_alloc(m, &m->d_pos, 1);
+    m->n_splits = attention_splits(dev, cfg->n_kv_heads, cfg->max_pos);
+    if (!rc) {
+        uint8_t *p = nullptr;
+        rc = dev_alloc(m, &p, attention_scratch_bytes(cfg->n_heads, cfg->n_kv_heads, cfg->head_dim, m->n_splits));
+        m->attn_scratch = p;
+    }
+    m->use_graph = getenv("CANDY_HIP_NO_GRAPH") == nullptr;
     if (!rc) rc = candy_hip_zero(dev, m->k_cache, kv * sizeof(float));
     if (!rc) rc = candy_hip_zero(dev, m->v_cache, kv * sizeof(float));
     if (!rc) {
@@ -154,6 +133,10 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
 
 int candy_hip_llama_free(candy_hip_llama *m) {
     if (!m) return CANDY_HIP_OK;
+    (void)hipSetDevice(m->dev->ordinal);
+    (void)hipStreamSynchronize(m->dev->stream);
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
     for (void *p : m->owned) (void)candy_hip_free(m->dev, p);
     delete m;
     return CANDY_HIP_OK;
@@ -177,6 +160,7 @@ int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const 
     case CANDY_HIP_W_EMBED: rows = c.vocab; cols = c.d_model; break;
     default: return fail(CANDY_HIP_ERR_INVALID, "weight kind %d is not a quantized matrix", which);
     }
+    m->graph_dirty = true;
     CANDY_REQUIRE(w->rows == rows && w->cols == cols, "weight kind %d must be %lld x %lld, got %lld x %lld", which,
                   (long long)rows, (long long)cols, (long long)w->rows, (long long)w->cols);
     if (which == CANDY_HIP_W_HEAD) { m->head = w; return CANDY_HIP_OK; }
@@ -197,11 +181,18 @@ int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const 
 
 int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const float *dev_alpha) {
     CANDY_REQUIRE(m && dev_alpha, "nil argument");
+    m->graph_dirty = true;
     if (which == CANDY_HIP_W_OUT_NORM) { m->out_norm = dev_alpha; return CANDY_HIP_OK; }
     CANDY_REQUIRE(which == CANDY_HIP_W_ATTN_NORM || which == CANDY_HIP_W_FFN_NORM, "weight kind %d is not a norm", which);
     CANDY_REQUIRE(layer >= 0 && layer < m->cfg.n_layers, "layer %d out of range", layer);
     if (which == CANDY_HIP_W_ATTN_NORM) m->layers[layer].attn_norm = dev_alpha;
     else m->layers[layer].ffn_norm = dev_alpha;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_llama_set_graph(candy_hip_llama *m, int enable) {
+    CANDY_REQUIRE(m, "model is nil");
+    m->use_graph = enable != 0;
     return CANDY_HIP_OK;
 }
 
@@ -224,48 +215,118 @@ static int llama_check_complete(const candy_hip_llama *m) {
     return CANDY_HIP_OK;
 }
 
-static int llama_step(candy_hip_llama *m, int32_t pos, const float **dev_logits, int32_t *next_token) {
+// Enqueues one decode step (hidden state in m->h, position in *m->d_pos) on the stream:
+// 10 launches per layer. Everything it touches is owned by the model, nothing allocates or
+// synchronises, so the sequence can be captured once and replayed for every token.
+// y_i = W_i . q8(rmsnorm(h) * alpha) for up to three weights: one fused launch, or
+// RMSNorm+quantize then the batch-1 kernel when no fused instantiation covers the shape.
+static int norm_linear(candy_hip_llama *m, const float *alpha, const candy_hip_qtensor *const *ws, float *const *ys,
+                       int n) {
+    const candy_hip_llama_config &c = m->cfg;
+    FusedLaunch F;
+    F.n = n;
+    for (int i = 0; i < n; ++i) { F.w[i] = ws[i]; F.y[i] = ys[i]; }
+    F.x = m->h; F.alpha = alpha; F.eps = c.rms_eps;
+    int rc = launch_matvec_fused(m->dev, F);
+    if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+    if ((rc = launch_rms_norm_quant(m->dev, m->h, alpha, c.rms_eps, 1, c.d_model, nullptr, m->xq, m->xs))) return rc;
+    return launch_matvec_multi(m->dev, ws, ys, nullptr, n, m->xq, m->xs);
+}
+
+// h += W . (quantized activations in xq/xs)
+static int linear_residual(candy_hip_llama *m, const candy_hip_qtensor *w) {
+    FusedLaunch F;
+    F.n = 1; F.w[0] = w; F.y[0] = m->h; F.res[0] = m->h; F.xq = m->xq; F.xs = m->xs;
+    int rc = launch_matvec_fused(m->dev, F);
+    if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+    const candy_hip_qtensor *ws[1] = {w};
+    float *ys[1] = {m->h};
+    const float *res[1] = {m->h};
+    return launch_matvec_multi(m->dev, ws, ys, res, 1, m->xq, m->xs);
+}
+
+// Enqueues one decode step (hidden state in m->h, position in *m->d_pos) on the stream: six
+// launches per layer. Everything it touches is owned by the model, nothing allocates or
+// synchronises, so the sequence can be captured once and replayed for every token.
+static int llama_enqueue_step(candy_hip_llama *m) {
     const candy_hip_llama_config &c = m->cfg;
     candy_hip_device *dev = m->dev;
-    const int64_t qd = (int64_t)c.n_heads * c.head_dim;
     const size_t layer_kv = (size_t)c.n_kv_heads * c.max_pos * c.head_dim;
-    const int half = c.head_dim / 2;
     const float scale = 1.0f / std::sqrt((float)c.head_dim);
     int rc;
     for (int l = 0; l < c.n_layers; ++l) {
         const candy_hip_llama::Layer &L = m->layers[l];
         float *kc = m->k_cache + (size_t)l * layer_kv, *vc = m->v_cache + (size_t)l * layer_kv;
-        if ((rc = candy_hip_rms_norm(dev, m->h, L.attn_norm, c.rms_eps, 1, c.d_model, m->xn))) return rc;
-        if ((rc = quantize(m, m->xn, c.d_model))) return rc;
-        if ((rc = linear(m, L.wq, m->q))) return rc;
-        if ((rc = linear(m, L.wk, m->k))) return rc;
-        if ((rc = linear(m, L.wv, m->v))) return rc;
-        const int threads = (c.n_heads + c.n_kv_heads) * half;
-        hipLaunchKernelGGL(k_rope_store, dim3((threads + 255) / 256), dim3(256), 0, dev->stream, m->q, m->k, m->v,
-                           m->cos_t + (size_t)pos * half, m->sin_t + (size_t)pos * half, c.n_heads, c.n_kv_heads,
-                           c.head_dim, pos, c.max_pos, kc, vc);
-        CANDY_LAUNCH_CHECK();
-        if ((rc = candy_hip_attention_decode(dev, m->q, kc, vc, c.n_heads, c.n_kv_heads, c.head_dim, pos + 1,
-                                             (int64_t)c.max_pos * c.head_dim, scale, m->att)))
-            return rc;
-        if ((rc = quantize(m, m->att, qd))) return rc;
-        if ((rc = linear(m, L.wo, m->tmp))) return rc;
-        if ((rc = candy_hip_add(dev, m->h, m->tmp, c.d_model, m->h))) return rc;
-        if ((rc = candy_hip_rms_norm(dev, m->h, L.ffn_norm, c.rms_eps, 1, c.d_model, m->xn))) return rc;
-        if ((rc = quantize(m, m->xn, c.d_model))) return rc;
-        if ((rc = linear(m, L.gate, m->gate_o))) return rc;
-        if ((rc = linear(m, L.up, m->up_o))) return rc;
-        if ((rc = candy_hip_silu_mul(dev, m->gate_o, m->up_o, c.d_ffn, m->act))) return rc;
-        if ((rc = quantize(m, m->act, c.d_ffn))) return rc;
-        if ((rc = linear(m, L.down, m->tmp))) return rc;
-        if ((rc = candy_hip_add(dev, m->h, m->tmp, c.d_model, m->h))) return rc;
+        {   // RMSNorm + quantize + q/k/v
+            const candy_hip_qtensor *ws[3] = {L.wq, L.wk, L.wv};
+            float *ys[3] = {m->q, m->k, m->v};
+            if ((rc = norm_linear(m, L.attn_norm, ws, ys, 3))) return rc;
+        }
+        {   // Rope on q and the new k, append k/v to the cache, attention; the merge quantizes for Wo
+            AttnLaunch A;
+            A.q = m->q; A.k_new = m->k; A.v_new = m->v; A.cos_t = m->cos_t; A.sin_t = m->sin_t;
+            A.k_cache = kc; A.v_cache = vc; A.pos_ptr = m->d_pos;
+            A.cache_stride = (int64_t)c.max_pos * c.head_dim; A.scale = scale;
+            A.n_heads = c.n_heads; A.n_kv_heads = c.n_kv_heads; A.head_dim = c.head_dim; A.n_splits = m->n_splits;
+            A.scratch = m->attn_scratch;
+            A.oq = m->xq; A.os = m->xs;
+            if ((rc = launch_attention(dev, A))) return rc;
+        }
+        if ((rc = linear_residual(m, L.wo))) return rc;  // h += Wo . att
+        {   // RMSNorm + quantize + gate/up + SiLU*Mul + quantize
+            FusedLaunch F;
+            F.n = 2; F.w[0] = L.gate; F.w[1] = L.up; F.pair = true;
+            F.x = m->h; F.alpha = L.ffn_norm; F.eps = c.rms_eps; F.oq = m->xq; F.os = m->xs;
+            rc = launch_matvec_fused(dev, F);
+            if (rc == CANDY_HIP_ERR_UNSUPPORTED) {
+                const candy_hip_qtensor *ws[2] = {L.gate, L.up};
+                float *ys[2] = {m->gate_o, m->up_o};
+                if ((rc = norm_linear(m, L.ffn_norm, ws, ys, 2))) return rc;
+                rc = launch_silu_mul_quant(dev, m->gate_o, m->up_o, c.d_ffn, nullptr, m->xq, m->xs);
+            }
+            if (rc) return rc;
+        }
+        if ((rc = linear_residual(m, L.down))) return rc;  // h += Wdown . act
     }
-    if ((rc = candy_hip_rms_norm(dev, m->h, m->out_norm, c.rms_eps, 1, c.d_model, m->xn))) return rc;
-    if ((rc = quantize(m, m->xn, c.d_model))) return rc;
-    if ((rc = linear(m, m->head, m->logits))) return rc;
+    {
+        const candy_hip_qtensor *ws[1] = {m->head};
+        float *ys[1] = {m->logits};
+        if ((rc = norm_linear(m, m->out_norm, ws, ys, 1))) return rc;
+    }
+    return candy_hip_argmax(dev, m->logits, 1, c.vocab, m->next_tok);
+}
+
+static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const float *dev_hidden,
+                      const float **dev_logits, int32_t *next_token) {
+    candy_hip_device *dev = m->dev;
+    int rc;
+    hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token);
+    CANDY_LAUNCH_CHECK();
+    if (dev_hidden) {
+        if ((rc = candy_hip_d2d(dev, m->h, dev_hidden, (size_t)m->cfg.d_model * sizeof(float)))) return rc;
+    } else {
+        if ((rc = candy_hip_qindex_select(dev, m->embed, m->tok_id, 1, m->h))) return rc;
+    }
+    if (m->use_graph) {
+        if (m->graph_dirty) {
+            if (m->graph_exec) CANDY_HIP_TRY(hipGraphExecDestroy(m->graph_exec));
+            if (m->graph) CANDY_HIP_TRY(hipGraphDestroy(m->graph));
+            m->graph_exec = nullptr;
+            m->graph = nullptr;
+            CANDY_HIP_TRY(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
+            rc = llama_enqueue_step(m);
+            hipError_t e = hipStreamEndCapture(dev->stream, &m->graph);
+            if (rc) return rc;
+            CANDY_HIP_TRY(e);
+            CANDY_HIP_TRY(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
+            m->graph_dirty = false;
+        }
+        CANDY_HIP_TRY(hipGraphLaunch(m->graph_exec, dev->stream));
+    } else {
+        if ((rc = llama_enqueue_step(m))) return rc;
+    }
     if (dev_logits) *dev_logits = m->logits;
     if (next_token) {
-        if ((rc = candy_hip_argmax(dev, m->logits, 1, c.vocab, m->next_tok))) return rc;
         uint32_t t = 0;
         if ((rc = candy_hip_d2h(dev, &t, m->next_tok, sizeof(t)))) return rc;
         *next_token = (int32_t)t;
@@ -279,8 +340,7 @@ int candy_hip_llama_decode_hidden(candy_hip_llama *m, const float *dev_hidden, i
     CANDY_REQUIRE(pos >= 0 && pos < m->cfg.max_pos, "position %d outside the cache (max_pos %d)", pos, m->cfg.max_pos);
     if (int rc = llama_check_complete(m)) return rc;
     if (int rc = use_device(m->dev)) return rc;
-    if (int rc = candy_hip_d2d(m->dev, m->h, dev_hidden, (size_t)m->cfg.d_model * sizeof(float))) return rc;
-    return llama_step(m, pos, dev_logits, next_token);
+    return llama_step(m, pos, -1, dev_hidden, dev_logits, next_token);
 }
 
 int candy_hip_llama_decode(candy_hip_llama *m, int32_t token, int32_t pos, const float **dev_logits,
@@ -291,10 +351,7 @@ int candy_hip_llama_decode(candy_hip_llama *m, int32_t token, int32_t pos, const
     CANDY_REQUIRE(pos >= 0 && pos < m->cfg.max_pos, "position %d outside the cache (max_pos %d)", pos, m->cfg.max_pos);
     if (int rc = llama_check_complete(m)) return rc;
     if (int rc = use_device(m->dev)) return rc;
-    const int64_t id = token;
-    if (int rc = candy_hip_h2d(m->dev, m->tok_id, &id, sizeof(id))) return rc;
-    if (int rc = candy_hip_qindex_select(m->dev, m->embed, m->tok_id, 1, m->h)) return rc;
-    return llama_step(m, pos, dev_logits, next_token);
+    return llama_step(m, pos, token, nullptr, dev_logits, next_token);
 }
 
 }  // extern "C"

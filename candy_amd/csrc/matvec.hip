@@ -18,12 +18,9 @@
 
 #include "blocks.h"
 #include "internal.h"
+#include "units.h"
 
 namespace candy {
-
-// LDS image of the activations: quants with 16 bytes of skew per 256 bytes (keeps 16-byte
-// reads of lanes that are 32 or 64 bytes apart on distinct banks), then the scales.
-__device__ __forceinline__ int skewed(int byte_off) { return byte_off + ((byte_off >> 8) << 4); }
 
 template <int NB, int THREADS>
 __device__ __forceinline__ void stage_activations(const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs,
@@ -44,157 +41,6 @@ __device__ __forceinline__ void stage_activations(const int8_t *__restrict__ xq,
     __syncthreads();
 }
 
-// Weight loads.  Plain (cached) loads on purpose: a 128-byte line of a row is touched by up to
-// three load instructions of the same wavefront (header, two halves of the nibbles), and a
-// non-temporal hint makes the later ones fetch the line again.
-template <class T>
-__device__ __forceinline__ T ldg_stream(const T *p) { return *p; }
-
-// ------------------------------------------------------------------ per-format units
-
-struct UnitQ4K {
-    static constexpr int ELEMS = 64;        // two 32-value sub-blocks sharing 32 bytes of nibbles
-    static constexpr int ROW_ALIGN = 16;
-    struct W { u32x4 hdr, q0, q1; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 144; }
-    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
-        const uint8_t *blk = row + (size_t)(u >> 2) * 144;
-        w.hdr = ldg_stream((const u32x4 *)blk);
-        const u32x4 *q = (const u32x4 *)(blk + 16 + (u & 3) * 32);
-        w.q0 = ldg_stream(q);
-        w.q1 = ldg_stream(q + 1);
-    }
-    // sum over the unit of w*x, with x = d_x * q_x: quantized.cu:2239-2263
-    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
-        const uint4 *xa = (const uint4 *)(sq + skewed(u * 64));
-        const uint4 x0 = xa[0], x1 = xa[1], x2 = xa[2], x3 = xa[3];
-        const Q8Scale s0 = ss[2 * u], s1 = ss[2 * u + 1];
-        uint32_t sc2, m2;
-        q4k_scale_min_pair(w.hdr.y, w.hdr.z, w.hdr.w, u & 3, sc2, m2);
-        const uint32_t M = 0x0F0F0F0Fu;
-        int lo = 0, hi = 0;
-        lo = dot4_i8(w.q0.x & M, x0.x, lo); hi = dot4_i8((w.q0.x >> 4) & M, x2.x, hi);
-        lo = dot4_i8(w.q0.y & M, x0.y, lo); hi = dot4_i8((w.q0.y >> 4) & M, x2.y, hi);
-        lo = dot4_i8(w.q0.z & M, x0.z, lo); hi = dot4_i8((w.q0.z >> 4) & M, x2.z, hi);
-        lo = dot4_i8(w.q0.w & M, x0.w, lo); hi = dot4_i8((w.q0.w >> 4) & M, x2.w, hi);
-        lo = dot4_i8(w.q1.x & M, x1.x, lo); hi = dot4_i8((w.q1.x >> 4) & M, x3.x, hi);
-        lo = dot4_i8(w.q1.y & M, x1.y, lo); hi = dot4_i8((w.q1.y >> 4) & M, x3.y, hi);
-        lo = dot4_i8(w.q1.z & M, x1.z, lo); hi = dot4_i8((w.q1.z >> 4) & M, x3.z, hi);
-        lo = dot4_i8(w.q1.w & M, x1.w, lo); hi = dot4_i8((w.q1.w >> 4) & M, x3.w, hi);
-        const float d = half_bits_to_float((uint16_t)(w.hdr.x & 0xFFFF));
-        const float dmin = half_bits_to_float((uint16_t)(w.hdr.x >> 16));
-        const float sd = s0.d * (float)(lo * (int)(sc2 & 0xFF)) + s1.d * (float)(hi * (int)(sc2 >> 8));
-        const float sm = s0.d * (float)(s0.bsum * (int)(m2 & 0xFF)) + s1.d * (float)(s1.bsum * (int)(m2 >> 8));
-        return d * sd - dmin * sm;
-    }
-};
-
-struct UnitQ8_0 {
-    static constexpr int ELEMS = 32;
-    static constexpr int ROW_ALIGN = 2;
-    struct W { u32x4 q0, q1; uint16_t d; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 34; }
-    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
-        const BlockQ8_0 *blk = (const BlockQ8_0 *)row + u;
-        w.d = blk->d;
-        w.q0 = ldg_stream((const u32x4_a2 *)(blk->qs));
-        w.q1 = ldg_stream((const u32x4_a2 *)(blk->qs + 16));
-    }
-    // quantized.cu:2058-2073
-    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
-        const uint4 *xa = (const uint4 *)(sq + skewed(u * 32));
-        const uint4 x0 = xa[0], x1 = xa[1];
-        int s = 0;
-        s = dot4_i8(w.q0.x, x0.x, s); s = dot4_i8(w.q0.y, x0.y, s); s = dot4_i8(w.q0.z, x0.z, s); s = dot4_i8(w.q0.w, x0.w, s);
-        s = dot4_i8(w.q1.x, x1.x, s); s = dot4_i8(w.q1.y, x1.y, s); s = dot4_i8(w.q1.z, x1.z, s); s = dot4_i8(w.q1.w, x1.w, s);
-        return (half_bits_to_float(w.d) * ss[u].d) * (float)s;
-    }
-};
-
-template <bool GGML_ORDER>
-struct UnitQ4_0 {
-    static constexpr int ELEMS = 32;
-    static constexpr int ROW_ALIGN = 2;
-    struct W { u32x4 q; uint16_t d; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 18; }
-    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
-        const BlockQ4_0 *blk = (const BlockQ4_0 *)row + u;
-        w.d = blk->d;
-        w.q = ldg_stream((const u32x4_a2 *)(blk->qs));
-    }
-    // Sum (q-8)*x = sum q*x - 8*sum x, all in integers. quantized.cu:1919-1941 gets the
-    // second term from the Q8_1 block's float sum; with Q8_0 activations it is the exact integer.
-    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
-        const uint4 *xa = (const uint4 *)(sq + skewed(u * 32));
-        const uint4 x0 = xa[0], x1 = xa[1];
-        const Q8Scale sx = ss[u];
-        const uint32_t M = 0x0F0F0F0Fu;
-        int s = 0;
-        if (GGML_ORDER) {
-            // low nibble of byte j pairs with x[j], high nibble with x[j+16] (quantized.cu:2426-2433)
-            s = dot4_i8(w.q.x & M, x0.x, s); s = dot4_i8((w.q.x >> 4) & M, x1.x, s);
-            s = dot4_i8(w.q.y & M, x0.y, s); s = dot4_i8((w.q.y >> 4) & M, x1.y, s);
-            s = dot4_i8(w.q.z & M, x0.z, s); s = dot4_i8((w.q.z >> 4) & M, x1.z, s);
-            s = dot4_i8(w.q.w & M, x0.w, s); s = dot4_i8((w.q.w >> 4) & M, x1.w, s);
-        } else {
-            // candy CPU order (quantized.go:87-92): byte j holds elements 2j (low) and 2j+1 (high);
-            // gather the even and odd activation bytes of each 8-element run
-            const uint32_t xs8[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-            const uint32_t qw[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t even = __builtin_amdgcn_perm(xs8[2 * j + 1], xs8[2 * j], 0x06040200u);
-                const uint32_t odd = __builtin_amdgcn_perm(xs8[2 * j + 1], xs8[2 * j], 0x07050301u);
-                s = dot4_i8(qw[j] & M, even, s);
-                s = dot4_i8((qw[j] >> 4) & M, odd, s);
-            }
-        }
-        s -= 8 * sx.bsum;
-        return (half_bits_to_float(w.d) * sx.d) * (float)s;
-    }
-};
-
-struct UnitQ6K {
-    static constexpr int ELEMS = 32;   // 8 values from each 32-value quarter of one 128-value half
-    static constexpr int ROW_ALIGN = 2;
-    struct W { u32x2 ql0, ql1, qh; uint32_t sc; uint16_t d; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 210; }
-    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
-        const BlockQ6K *blk = (const BlockQ6K *)row + (u >> 3);
-        const int ip = (u >> 2) & 1, j = u & 3;
-        w.ql0 = ldg_stream((const u32x2_a2 *)(blk->ql + 64 * ip + 8 * j));
-        w.ql1 = ldg_stream((const u32x2_a2 *)(blk->ql + 64 * ip + 32 + 8 * j));
-        w.qh = ldg_stream((const u32x2_a2 *)(blk->qh + 32 * ip + 8 * j));
-        const int8_t *sc = blk->scales + 8 * ip + (j >> 1);
-        w.sc = (uint32_t)(uint8_t)sc[0] | ((uint32_t)(uint8_t)sc[2] << 8) | ((uint32_t)(uint8_t)sc[4] << 16) |
-               ((uint32_t)(uint8_t)sc[6] << 24);
-        w.d = blk->d;
-    }
-    // quantized.cu:2367-2389: d * sum over 16-value groups of d8 * (dot * scale); the -32 offset is
-    // applied as dot(q,x) - 32*sum(x) in integers.
-    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
-        const int sb = u >> 3, ip = (u >> 2) & 1, j = u & 3;
-        const int blk0 = sb * 8 + ip * 4;  // first of the four 32-value activation blocks
-        float sumf = 0.0f;
-        const uint32_t M = 0x0F0F0F0Fu, H = 0x30303030u, ones = 0x01010101u;
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-            const uint2 x = *(const uint2 *)(sq + skewed((blk0 + qd) * 32 + 8 * j));
-            const u32x2 ql = (qd & 1) ? w.ql1 : w.ql0;
-            const uint32_t lx = (qd < 2) ? (ql.x & M) : ((ql.x >> 4) & M);
-            const uint32_t ly = (qd < 2) ? (ql.y & M) : ((ql.y >> 4) & M);
-            const uint32_t vx = lx | (((w.qh.x >> (2 * qd)) << 4) & H);
-            const uint32_t vy = ly | (((w.qh.y >> (2 * qd)) << 4) & H);
-            int dq = dot4_i8(vy, x.y, dot4_i8(vx, x.x, 0));
-            const int sx = dot4_i8(ones, x.y, dot4_i8(ones, x.x, 0));
-            dq -= 32 * sx;
-            const int scale = (int)(int8_t)((w.sc >> (8 * qd)) & 0xFF);
-            sumf += ss[blk0 + qd].d * (float)(dq * scale);
-        }
-        return half_bits_to_float(w.d) * sumf;
-    }
-};
-
 // ------------------------------------------------------------------ kernels
 // Nothing in these kernels branches around a memory operation: out-of-range lanes load a
 // clamped (valid) address and their contribution is dropped afterwards.  That keeps the
@@ -204,9 +50,15 @@ struct UnitQ6K {
 // Batch-1 kernel.  ITER = ceil(units / 64) is a compile-time bound: every weight load of the
 // wavefront's R rows is in flight before anything waits.  The grid covers all rows at once.
 template <class U, int ITER, int R, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_matvec1(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
-                                                        const Q8Scale *__restrict__ xs, float *__restrict__ y,
-                                                        int N, int K) {
+__global__ __launch_bounds__(WAVES * 64) void k_matvec1(const MatvecJobs jobs, const int8_t *__restrict__ xq,
+                                                        const Q8Scale *__restrict__ xs, int K) {
+    // which of the (up to three) weights sharing this activation does the workgroup belong to
+    const int ji = (int)(blockIdx.x >= (unsigned)jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)jobs.j[1].wg_end);
+    const int wg = blockIdx.x - (ji > 0 ? jobs.j[ji - 1].wg_end : 0);
+    const uint8_t *__restrict__ W = jobs.j[ji].W;
+    float *y = jobs.j[ji].y;  // may alias res (h += W.x)
+    const float *res = jobs.j[ji].res;
+    const int N = jobs.j[ji].N;
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;       // activation bytes the LDS image is sized for
     constexpr int AQ = (CAP / 16 + T - 1) / T;      // 16-byte chunks of quants per thread
@@ -226,7 +78,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1(const uint8_t *__restric
 #pragma unroll
     for (int i = 0; i < AS; ++i) as[i] = ((const uint2 *)xs)[min(tid + i * T, sblocks - 1)];
 
-    const int row0 = (blockIdx.x * WAVES + wave) * R;
+    const int row0 = (wg * WAVES + wave) * R;
     typename U::W w[R][ITER];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -262,7 +114,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1(const uint8_t *__restric
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const float v = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) y[row0 + r] = v;
+        if (lane == 0 && row0 + r < N) y[row0 + r] = res ? res[row0 + r] + v : v;  // Add (backend.go:21) folded in
     }
 }
 
@@ -317,19 +169,50 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict
 }
 
 template <class U, int ITER, int R, int WAVES>
-static int launch1(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                   float *y) {
-    const int N = (int)w->rows, K = (int)w->cols;
+static int launch1(candy_hip_device *dev, MatvecJobs jobs, int K, const int8_t *qs, const Q8Scale *scales) {
     constexpr int T = WAVES * 64, CAP = ITER * 64 * U::ELEMS;
     constexpr int AQ = (CAP / 16 + T - 1) / T, AS = (CAP / 32 + T - 1) / T;
     constexpr size_t smem = (size_t)AQ * T * 16 + (((size_t)AQ * T * 16 >> 8) << 4) + (size_t)AS * T * sizeof(Q8Scale);
     static_assert(smem <= 64 * 1024, "LDS image too large");
     const int rows_per_wg = R * WAVES;
-    const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
-    hipLaunchKernelGGL((k_matvec1<U, ITER, R, WAVES>), dim3(grid), dim3(WAVES * 64), smem, dev->stream,
-                       (const uint8_t *)w->data, qs, scales, y, N, K);
+    int total = 0;
+    for (int i = 0; i < 3; ++i) {
+        if (i < jobs.n) total += (jobs.j[i].N + rows_per_wg - 1) / rows_per_wg;
+        jobs.j[i].wg_end = total;  // unused slots end where the last real one does
+    }
+    hipLaunchKernelGGL((k_matvec1<U, ITER, R, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), smem, dev->stream, jobs,
+                       qs, scales, K);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
+}
+
+template <class U>
+static int launch_jobs_fmt(candy_hip_device *dev, const MatvecJobs &jobs, int64_t K, const int8_t *qs,
+                           const Q8Scale *scales) {
+    const int iter = (int)((K / U::ELEMS + 63) / 64);
+    switch (iter) {
+    case 1: return launch1<U, 1, 1, 4>(dev, jobs, (int)K, qs, scales);
+    case 2: return launch1<U, 2, 1, 4>(dev, jobs, (int)K, qs, scales);
+    case 3: return launch1<U, 3, 1, 4>(dev, jobs, (int)K, qs, scales);
+    case 4: return launch1<U, 4, 1, 4>(dev, jobs, (int)K, qs, scales);
+    case 5: return launch1<U, 5, 1, 4>(dev, jobs, (int)K, qs, scales);
+    case 6: return launch1<U, 6, 1, 4>(dev, jobs, (int)K, qs, scales);
+    case 7: return launch1<U, 7, 1, 4>(dev, jobs, (int)K, qs, scales);
+    case 8: return launch1<U, 8, 1, 4>(dev, jobs, (int)K, qs, scales);
+    default: return CANDY_HIP_ERR_UNSUPPORTED;  // longer rows take the looping kernel
+    }
+}
+
+static int launch_jobs(candy_hip_device *dev, int fmt, const MatvecJobs &jobs, int64_t K, const int8_t *qs,
+                       const Q8Scale *scales) {
+    switch (fmt) {
+    case CANDY_HIP_Q4_K: return launch_jobs_fmt<UnitQ4K>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q8_0: return launch_jobs_fmt<UnitQ8_0>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q4_0: return launch_jobs_fmt<UnitQ4_0<false>>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q4_0_GGML: return launch_jobs_fmt<UnitQ4_0<true>>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q6_K: return launch_jobs_fmt<UnitQ6K>(dev, jobs, K, qs, scales);
+    default: return fail(CANDY_HIP_ERR_INVALID, "unknown quantized format %d", fmt);
+    }
 }
 
 template <class U, int NB, int R, int WAVES>
@@ -353,18 +236,13 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
     const int64_t K = w->cols, N = w->rows;
     const int64_t sstride = K >> 5;
     if (m == 1) {
-        const int iter = (int)((K / U::ELEMS + 63) / 64);
-        switch (iter) {
-        case 1: return launch1<U, 1, 1, 4>(dev, w, qs, scales, y);
-        case 2: return launch1<U, 2, 1, 4>(dev, w, qs, scales, y);
-        case 3: return launch1<U, 3, 1, 4>(dev, w, qs, scales, y);
-        case 4: return launch1<U, 4, 1, 4>(dev, w, qs, scales, y);
-        case 5: return launch1<U, 5, 1, 4>(dev, w, qs, scales, y);
-        case 6: return launch1<U, 6, 1, 4>(dev, w, qs, scales, y);
-        case 7: return launch1<U, 7, 1, 4>(dev, w, qs, scales, y);
-        case 8: return launch1<U, 8, 1, 4>(dev, w, qs, scales, y);
-        default: break;  // longer rows take the looping kernel
-        }
+        MatvecJobs jobs{};
+        jobs.n = 1;
+        jobs.j[0].W = (const uint8_t *)w->data;
+        jobs.j[0].y = y;
+        jobs.j[0].N = (int)N;
+        const int rc = launch_jobs_fmt<U>(dev, jobs, K, qs, scales);
+        if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     }
     int64_t done = 0;
     while (done < m) {
@@ -378,6 +256,34 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
         else if (left >= 2 && K <= 16384) { rc = launch_one<U, 2, 2, 4>(dev, w, q, s, yo); done += 2; }
         else { rc = launch_one<U, 1, 2, 4>(dev, w, q, s, yo); done += 1; }
         if (rc) return rc;
+    }
+    return CANDY_HIP_OK;
+}
+
+// Batch-1 contraction of one quantized activation row against up to three weights in ONE launch
+// (q/k/v, gate/up), each with an optional residual added to its output.  Weights must share
+// format and contraction length; otherwise, or for very long rows, one launch per weight.
+int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *ws, float *const *ys,
+                        const float *const *res, int n, const int8_t *qs, const Q8Scale *scales) {
+    CANDY_REQUIRE(n >= 1 && n <= 3, "internal: 1..3 weights per launch");
+    bool same = true;
+    for (int i = 1; i < n; ++i) same = same && ws[i]->fmt == ws[0]->fmt && ws[i]->cols == ws[0]->cols;
+    if (same) {
+        MatvecJobs jobs{};
+        jobs.n = n;
+        for (int i = 0; i < n; ++i) {
+            CANDY_REQUIRE(ws[i]->rows <= 0x7FFFFFFF && ws[i]->cols <= 0x7FFFFFFF, "matrix too large");
+            jobs.j[i].W = (const uint8_t *)ws[i]->data;
+            jobs.j[i].y = ys[i];
+            jobs.j[i].res = res ? res[i] : nullptr;
+            jobs.j[i].N = (int)ws[i]->rows;
+        }
+        const int rc = launch_jobs(dev, ws[0]->fmt, jobs, ws[0]->cols, qs, scales);
+        if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+    }
+    for (int i = 0; i < n; ++i) {
+        if (res && res[i]) return fail(CANDY_HIP_ERR_UNSUPPORTED, "residual epilogue needs the batch-1 kernel");
+        if (int rc = launch_matvec(dev, ws[i], qs, scales, 1, ys[i])) return rc;
     }
     return CANDY_HIP_OK;
 }

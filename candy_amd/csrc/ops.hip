@@ -150,118 +150,100 @@ __global__ __launch_bounds__(256) void k_matmul_f32(const float *__restrict__ a,
     c[(bb * m + i) * n + j] = sum;
 }
 
-// ------------------------------------------------------------------ attention over the f32 KV cache
-// Split over positions (grid = kv heads x splits): each workgroup streams its slice of K and V
-// once for all query heads that share the kv head, keeps a running (max, sum, weighted V) per
-// query head, and a second kernel merges the splits.  head_dim is 128 here: a wavefront holds
-// one cache row as 64 lanes x float2.
 
-template <int GROUP>
-__global__ __launch_bounds__(256) void k_attn_partial(const float *__restrict__ q, const float *__restrict__ kc,
-                                                      const float *__restrict__ vc, int head_dim, int n_pos,
-                                                      int64_t cache_stride, float scale, int n_splits,
-                                                      float *__restrict__ part_o, float *__restrict__ part_ml) {
-    // part_o: [n_heads][n_splits][head_dim]; part_ml: [n_heads][n_splits][2] (max, sum)
-    const int kvh = blockIdx.x, split = blockIdx.y;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int per = (n_pos + n_splits - 1) / n_splits;
-    const int p0 = split * per, p1 = min(n_pos, p0 + per);
-    const float *kh = kc + (size_t)kvh * cache_stride;
-    const float *vh = vc + (size_t)kvh * cache_stride;
-    const int hd2 = head_dim >> 1;  // float2 per row
-    const int loops = (hd2 + 63) >> 6;  // 1 for head_dim 128
+// ------------------------------------------------------------------ fused decode-step kernels
+// Each produces the planar Q8_0 activations the next quantized Linear consumes, so the f32
+// intermediate never makes a round trip through a separate quantize launch.  The arithmetic of
+// each stage is the unfused one (RMSNorm: reduce.go:3071-3092; SiLU: unary.go:3353-3366; Mul;
+// activation quantization: quantized.cu:3521-3558).
 
-    // each wave: positions p0+wave, p0+wave+4, ...
-    float m_run[GROUP], l_run[GROUP];
-    float2 o_run[GROUP][2];
-    float2 qv[GROUP][2];
-#pragma unroll
-    for (int g = 0; g < GROUP; ++g) {
-        m_run[g] = -3.402823466e+38f;
-        l_run[g] = 0.0f;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            o_run[g][t] = make_float2(0.f, 0.f);
-            const int c = lane + 64 * t;
-            qv[g][t] = (t < loops && c < hd2) ? ((const float2 *)(q + (size_t)(kvh * GROUP + g) * head_dim))[c]
-                                              : make_float2(0.f, 0.f);
-        }
+// RMSNorm of one row followed by Q8_0 quantization. cols % 32 == 0. One workgroup per row.
+__global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict__ x, const float *__restrict__ alpha,
+                                                        float eps, int cols, float *__restrict__ xn_out,
+                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales) {
+    __shared__ float red[16];
+    const float4 *xr = (const float4 *)(x + (size_t)blockIdx.x * cols);
+    const int n4 = cols >> 2;
+    float s = 0.0f;
+    for (int c = threadIdx.x; c < n4; c += 256) {
+        const float4 v = xr[c];
+        s += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
-    for (int p = p0 + wave; p < p1; p += 4) {
-        float2 kv[2], vv[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int c = lane + 64 * t;
-            const bool ok = t < loops && c < hd2;
-            kv[t] = ok ? ((const float2 *)(kh + (size_t)p * head_dim))[c] : make_float2(0.f, 0.f);
-            vv[t] = ok ? ((const float2 *)(vh + (size_t)p * head_dim))[c] : make_float2(0.f, 0.f);
-        }
-#pragma unroll
-        for (int g = 0; g < GROUP; ++g) {
-            float s = qv[g][0].x * kv[0].x + qv[g][0].y * kv[0].y + qv[g][1].x * kv[1].x + qv[g][1].y * kv[1].y;
-            s = wave_sum(s) * scale;
-            const float m_new = fmaxf(m_run[g], s);
-            const float corr = expf(m_run[g] - m_new), pw = expf(s - m_new);
-            l_run[g] = l_run[g] * corr + pw;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                o_run[g][t].x = o_run[g][t].x * corr + pw * vv[t].x;
-                o_run[g][t].y = o_run[g][t].y * corr + pw * vv[t].y;
+    s = block_reduce<false>(s, red);
+    const float mean = s / (float)cols;
+    const float scale = 1.0f / (float)sqrt((double)(mean + eps));
+    const int n4_pad = (n4 + 255) & ~255;  // whole wavefronts take part in the cross-lane steps
+    for (int c = threadIdx.x; c < n4_pad; c += 256) {
+        const bool live = c < n4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) {
+            v = xr[c];
+            if (alpha) {
+                const float4 a = ((const float4 *)alpha)[c];
+                v = make_float4(scale * v.x * a.x, scale * v.y * a.y, scale * v.z * a.z, scale * v.w * a.w);
+            } else {
+                v = make_float4(scale * v.x, scale * v.y, scale * v.z, scale * v.w);
             }
-            m_run[g] = m_new;
         }
-    }
-    // merge the 4 waves through LDS
-    __shared__ float sm[4][GROUP], sl[4][GROUP];
-    __shared__ float2 so[4][GROUP][128];
-#pragma unroll
-    for (int g = 0; g < GROUP; ++g) {
-        if (lane == 0) { sm[wave][g] = m_run[g]; sl[wave][g] = l_run[g]; }
-#pragma unroll
-        for (int t = 0; t < 2; ++t) so[wave][g][lane + 64 * t] = o_run[g][t];
-    }
-    __syncthreads();
-    // thread -> (g, column c of float2)
-    for (int idx = threadIdx.x; idx < GROUP * hd2; idx += 256) {
-        const int g = idx / hd2, c = idx - g * hd2;
-        float m = sm[0][g];
-        for (int w = 1; w < 4; ++w) m = fmaxf(m, sm[w][g]);
-        float l = 0.0f;
-        float2 o = make_float2(0.f, 0.f);
-        for (int w = 0; w < 4; ++w) {
-            const float f = expf(sm[w][g] - m);
-            l += sl[w][g] * f;
-            o.x += so[w][g][c].x * f;
-            o.y += so[w][g][c].y * f;
-        }
-        const int h = kvh * GROUP + g;
-        ((float2 *)(part_o + ((size_t)h * n_splits + split) * head_dim))[c] = o;
-        if (c == 0) {
-            part_ml[((size_t)h * n_splits + split) * 2 + 0] = m;
-            part_ml[((size_t)h * n_splits + split) * 2 + 1] = l;
+        __half h;
+        int bsum;
+        const uint32_t packed = quantize_q8_lane4(v, h, bsum);
+        if (!live) continue;
+        const size_t i = (size_t)blockIdx.x * n4 + c;
+        if (xn_out) ((float4 *)xn_out)[i] = v;
+        qs[i] = packed;
+        if ((c & 7) == 0) {
+            Q8Scale sc;
+            sc.d = __half2float(h);
+            sc.bsum = bsum;
+            scales[i >> 3] = sc;
         }
     }
 }
 
-__global__ __launch_bounds__(128) void k_attn_merge(const float *__restrict__ part_o, const float *__restrict__ part_ml,
-                                                    int head_dim, int n_splits, float *__restrict__ out) {
-    const int h = blockIdx.x;
-    float m = -3.402823466e+38f;
-    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part_ml[((size_t)h * n_splits + s) * 2]);
-    float l = 0.0f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float ls = part_ml[((size_t)h * n_splits + s) * 2 + 1];
-        l += ls * expf(part_ml[((size_t)h * n_splits + s) * 2] - m);
+// silu(gate) * up, then Q8_0 quantization. n % 32 == 0.
+__global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict__ gate, const float4 *__restrict__ up,
+                                                        int64_t n4, float4 *__restrict__ act_out,
+                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool live = i < n4;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (live) {
+        const float4 g = gate[i], u = up[i];
+        v = make_float4(silu_f(g.x) * u.x, silu_f(g.y) * u.y, silu_f(g.z) * u.z, silu_f(g.w) * u.w);
     }
-    const float inv = 1.0f / l;
-    for (int c = threadIdx.x; c < head_dim; c += blockDim.x) {
-        float o = 0.0f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float f = expf(part_ml[((size_t)h * n_splits + s) * 2] - m);
-            o += part_o[((size_t)h * n_splits + s) * head_dim + c] * f;
-        }
-        out[(size_t)h * head_dim + c] = o * inv;
+    __half h;
+    int bsum;
+    const uint32_t packed = quantize_q8_lane4(v, h, bsum);
+    if (!live) return;
+    if (act_out) act_out[i] = v;
+    qs[i] = packed;
+    if ((i & 7) == 0) {
+        Q8Scale sc;
+        sc.d = __half2float(h);
+        sc.bsum = bsum;
+        scales[i >> 3] = sc;
     }
+}
+
+// ------------------------------------------------------------------ launchers shared with llama.hip
+int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
+                          int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales) {
+    CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0 && cols <= 0x7FFFFFFF, "rms_norm_quant needs cols %% 32 == 0");
+    hipLaunchKernelGGL(k_rms_norm_quant, dim3((unsigned)rows), dim3(256), 0, dev->stream, x, alpha, eps, (int)cols,
+                       xn_out, (uint32_t *)qs, scales);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *act_out,
+                          int8_t *qs, Q8Scale *scales) {
+    CANDY_REQUIRE(n % 32 == 0 && n > 0, "silu_mul_quant needs n %% 32 == 0");
+    const int64_t n4 = n >> 2;
+    hipLaunchKernelGGL(k_silu_mul_quant, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, dev->stream,
+                       (const float4 *)gate, (const float4 *)up, n4, (float4 *)act_out, (uint32_t *)qs, scales);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
 }
 
 }  // namespace candy
@@ -361,46 +343,6 @@ int candy_hip_index_select(candy_hip_device *dev, const float *table, int64_t n_
     CANDY_REQUIRE(table && dev_ids && out, "nil pointer");
     if (int rc = use_device(dev)) return rc;
     hipLaunchKernelGGL(k_index_select, dim3((unsigned)n_ids), dim3(256), 0, dev->stream, table, width, dev_ids, out);
-    CANDY_LAUNCH_CHECK();
-    return CANDY_HIP_OK;
-}
-
-int candy_hip_attention_decode(candy_hip_device *dev, const float *q, const float *k_cache, const float *v_cache,
-                               int64_t n_heads, int64_t n_kv_heads, int64_t head_dim, int64_t n_pos,
-                               int64_t cache_stride, float scale, float *out) {
-    CANDY_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "invalid head counts %lld / %lld",
-                  (long long)n_heads, (long long)n_kv_heads);
-    CANDY_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256, "head_dim %lld unsupported (even, <= 256)",
-                  (long long)head_dim);
-    CANDY_REQUIRE(n_pos > 0 && cache_stride >= n_pos * head_dim, "invalid cache shape");
-    CANDY_REQUIRE(q && k_cache && v_cache && out, "nil pointer");
-    const int group = (int)(n_heads / n_kv_heads);
-    CANDY_REQUIRE(group == 1 || group == 2 || group == 4 || group == 8, "query heads per kv head must be 1, 2, 4 or 8");
-    if (int rc = use_device(dev)) return rc;
-    // enough workgroups to fill the chip, at least 64 positions per split
-    int n_splits = (int)((2 * (int64_t)dev->num_cus + n_kv_heads - 1) / n_kv_heads);
-    const int max_splits = (int)((n_pos + 63) / 64);
-    if (n_splits > max_splits) n_splits = max_splits;
-    if (n_splits < 1) n_splits = 1;
-    const size_t po_bytes = (size_t)n_heads * n_splits * head_dim * sizeof(float);
-    const size_t ml_bytes = (size_t)n_heads * n_splits * 2 * sizeof(float);
-    void *ws = nullptr;
-    if (int rc = workspace(dev, po_bytes + ml_bytes, &ws)) return rc;
-    float *part_o = (float *)ws, *part_ml = (float *)((uint8_t *)ws + po_bytes);
-    dim3 grid((unsigned)n_kv_heads, (unsigned)n_splits);
-#define CANDY_ATTN(G)                                                                                          \
-    hipLaunchKernelGGL((k_attn_partial<G>), grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, (int)head_dim, \
-                       (int)n_pos, cache_stride, scale, n_splits, part_o, part_ml)
-    switch (group) {
-    case 1: CANDY_ATTN(1); break;
-    case 2: CANDY_ATTN(2); break;
-    case 4: CANDY_ATTN(4); break;
-    default: CANDY_ATTN(8); break;
-    }
-#undef CANDY_ATTN
-    CANDY_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_attn_merge, dim3((unsigned)n_heads), dim3(128), 0, dev->stream, part_o, part_ml, (int)head_dim,
-                       n_splits, out);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }

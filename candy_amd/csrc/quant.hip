@@ -18,28 +18,12 @@ __global__ __launch_bounds__(256) void k_quantize_q8_0(const float4 *__restrict_
     const bool active = i < n4;  // n4 is a multiple of 8, so a block's 8 lanes agree
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (active) v = x[i];
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
-    const float d = amax / 127.0f;
-    int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
-    if (amax != 0.0f) {
-        q0 = (int)roundf(v.x / d);
-        q1 = (int)roundf(v.y / d);
-        q2 = (int)roundf(v.z / d);
-        q3 = (int)roundf(v.w / d);
-    }
-    int s = q0 + q1 + q2 + q3;
-    s += __shfl_xor(s, 1, 64);
-    s += __shfl_xor(s, 2, 64);
-    s += __shfl_xor(s, 4, 64);
+    __half h;
+    int s;
+    const uint32_t packed = quantize_q8_lane4(v, h, s);
     if (!active) return;
-    const uint32_t packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
-                            ((uint32_t)(q3 & 0xFF) << 24);
     const int64_t b = i >> 3;
     const int part = (int)(i & 7);
-    const __half h = __float2half_rn(d);
     if (qs) qs[i] = packed;
     if (scales && part == 0) {
         Q8Scale sc;

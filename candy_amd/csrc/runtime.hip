@@ -60,6 +60,27 @@ int workspace(candy_hip_device *dev, size_t bytes, void **out) {
     return CANDY_HIP_OK;
 }
 
+__global__ __launch_bounds__(256) void k_zero_bytes(uint8_t *p, size_t bytes) {
+    // 16 bytes per thread where aligned, byte stores for the ragged head and tail
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 16;
+    if (i >= bytes) return;
+    if ((((uintptr_t)p + i) & 15) == 0 && i + 16 <= bytes) {
+        *(uint4 *)(p + i) = make_uint4(0, 0, 0, 0);
+    } else {
+        for (size_t j = i; j < i + 16 && j < bytes; ++j) p[j] = 0;
+    }
+}
+
+int launch_zero(candy_hip_device *dev, void *dptr, size_t bytes) {
+    if (bytes == 0) return CANDY_HIP_OK;
+    const size_t threads = (bytes + 15) / 16;
+    const size_t grid = (threads + 255) / 256;
+    CANDY_REQUIRE(grid <= 0x7FFFFFFF, "buffer too large to zero in one launch");
+    hipLaunchKernelGGL(k_zero_bytes, dim3((unsigned)grid), dim3(256), 0, dev->stream, (uint8_t *)dptr, bytes);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
 }  // namespace candy
 
 using namespace candy;
@@ -160,7 +181,13 @@ int candy_hip_zero(candy_hip_device *dev, void *dptr, size_t bytes) {
     if (bytes == 0) return CANDY_HIP_OK;
     CANDY_REQUIRE(dptr, "dptr is nil");
     if (int rc = use_device(dev)) return rc;
-    CANDY_HIP_TRY(hipMemsetAsync(dptr, 0, bytes, dev->stream));
+    // a fill kernel rather than a memset node: callers may capture this into a HIP graph
+    size_t done = 0;
+    while (done < bytes) {
+        const size_t chunk = bytes - done < (size_t(1) << 36) ? bytes - done : (size_t(1) << 36);
+        if (int rc = launch_zero(dev, (uint8_t *)dptr + done, chunk)) return rc;
+        done += chunk;
+    }
     return CANDY_HIP_OK;
 }
 

@@ -83,6 +83,7 @@ SIGNATURES = {
     "candy_hip_llama_free": (c_int, [c_void_p]),
     "candy_hip_llama_set_qweight": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "candy_hip_llama_set_norm": (c_int, [c_void_p, c_int, c_int, c_void_p]),
+    "candy_hip_llama_set_graph": (c_int, [c_void_p, c_int]),
     "candy_hip_llama_kv_cache": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_size_t)]),
     "candy_hip_llama_decode": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_llama_decode_hidden": (c_int, [c_void_p, c_void_p, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
@@ -388,6 +389,9 @@ class Llama:
         buf = self.dev.from_numpy(np.ascontiguousarray(alpha, np.float32))
         self._keep.append(buf)
         _check(lib().candy_hip_llama_set_norm(self.handle, which, layer, buf.ptr))
+
+    def set_graph(self, enable: bool):
+        _check(lib().candy_hip_llama_set_graph(self.handle, int(enable)))
 
     def kv_cache(self):
         k, v, n = c_void_p(), c_void_p(), c_size_t()

@@ -187,6 +187,10 @@ int candy_hip_llama_free(candy_hip_llama *m);
 /* The model borrows the tensors; they must outlive it. */
 int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const candy_hip_qtensor *w);
 int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const float *dev_alpha);
+/* The decode step is captured into a HIP graph on first use and replayed afterwards (the
+ * position and token travel through device memory); enable = 0 launches the kernels one by
+ * one instead.  Results are identical either way. */
+int candy_hip_llama_set_graph(candy_hip_llama *m, int enable);
 /* f32 KV cache, [n_layers][n_kv_heads][max_pos][head_dim] for K and the same for V. */
 int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, size_t *bytes_each);
 /* One decode step: token id at position pos -> logits [vocab] (device pointer owned by the

@@ -88,6 +88,26 @@ def test_decode_steps_match_cpu_composition(dev, name, cfg, fmts):
     assert rel(kc[:, :, :len(tokens)], ref.k_cache[:, :, :len(tokens)].astype(np.float64)) <= 1e-3
 
 
+def test_graph_replay_equals_eager_launches(dev):
+    # the captured step is replayed for every token; every replay must give what one-by-one
+    # launches give, with other work and synchronisations in between
+    cfg = dict(n_layers=2, d_model=1024, n_heads=8, n_kv_heads=4, head_dim=128, d_ffn=2816, vocab=1024, max_pos=12,
+               rms_eps=1e-5, rope_base=10000.0)
+    fm = {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}
+    _, eager = build(dev, cfg, fm, seed=9)
+    _, graph = build(dev, cfg, fm, seed=9)
+    eager.set_graph(False)
+    tokens = [5, 900, 17, 17, 3, 64, 1000, 2]
+    for pos, tok in enumerate(tokens):
+        et, el = eager.decode(tok, pos)
+        gt, gl = graph.decode(tok, pos)
+        assert np.array_equal(el, gl), pos
+        assert et == gt
+        # unrelated work on the same device between replays
+        dev.softmax(np.arange(64, dtype=np.float32), 64)
+        dev.synchronize()
+
+
 def test_decode_errors(dev):
     cfg = dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, head_dim=128, d_ffn=256, vocab=64, max_pos=4,
                rms_eps=1e-5, rope_base=10000.0)
