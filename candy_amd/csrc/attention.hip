@@ -130,19 +130,39 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
         }
     };
 
-    // cached positions: wavefront w, half hw, slot u takes position base + 2u + hw
-    for (int base = p0 + wave * 2 * UNR; base < p1; base += 4 * 2 * UNR) {
-        vecf kv[UNR], vv[UNR];
-        bool valid[UNR];
+    // cached positions: wavefront w, half hw, slot u takes position base + 2u + hw.  The next
+    // batch of rows is requested before the current one is absorbed, so two batches (up to
+    // 16 KB) are in flight per wavefront.
+    auto fetch = [&](int base, vecf (&kv)[UNR], vecf (&vv)[UNR], bool (&valid)[UNR]) {
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
             const int p = base + 2 * u + hw;
             valid[u] = p < p1;
-            const size_t off = (size_t)min(p, p1 - 1) * HD + hl * VEC;
-            kv[u] = *(const vecf *)(kh + off);
-            vv[u] = *(const vecf *)(vh + off);
+            const size_t off = (size_t)max(min(p, p1 - 1), 0) * HD + hl * VEC;
+            // every cache byte is read once, by one instruction: stream it past the caches
+            kv[u] = __builtin_nontemporal_load((const vecf *)(kh + off));
+            vv[u] = __builtin_nontemporal_load((const vecf *)(vh + off));
         }
-        absorb(kv, vv, valid);
+    };
+    {
+        constexpr int STEP = 4 * 2 * UNR;
+        int base = p0 + wave * 2 * UNR;
+        vecf kv[UNR], vv[UNR], kn[UNR], vn[UNR];
+        bool valid[UNR], vnext[UNR];
+        if (base < p1) fetch(base, kv, vv, valid);
+        while (base < p1) {
+            const int nb = base + STEP;
+            if (nb < p1) fetch(nb, kn, vn, vnext);
+            absorb(kv, vv, valid);
+            if (nb >= p1) break;
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) {
+                kv[u] = kn[u];
+                vv[u] = vn[u];
+                valid[u] = vnext[u];
+            }
+            base = nb;
+        }
     }
 
     // the new token: Rope its key, append both rows to the cache, attend to them from registers

@@ -69,6 +69,11 @@ __device__ __forceinline__ float dpp_move(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, BANK_MASK, true));
 }
 
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ int dpp_move_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, BANK_MASK, true);
+}
+
 // Sum over the 64 lanes of a wavefront; every lane gets the total.
 __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_move<0xB1>(v);        // quad_perm [1,0,3,2]
@@ -86,22 +91,17 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 
-// Planar Q8_0 activation scale (the matvec / MFMA kernels read quants and scales separately).
-struct Q8ScaleDev {
-    float d;
-    int32_t bsum;
-};
-
 // Q8_0 quantization of 4 consecutive values held by one lane; the 8 lanes that share a 32-value
 // block must be consecutive lanes of one wavefront (lane % 8 == position in the block) and all
 // active.  quantize_q8_1 (quantized.cu:3521-3558) without its `sum`: amax over the block,
 // d = amax / 127 (IEEE division), q = amax == 0 ? 0 : roundf(x / d).
 // Returns the 4 quants packed little-endian; d_half / bsum are valid in every lane of the block.
 __device__ __forceinline__ uint32_t quantize_q8_lane4(float4 v, __half &d_half, int &bsum) {
+    // 8-lane reductions on the DPP path: two quad permutes, then the mirror within each 8 lanes
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    amax = fmaxf(amax, dpp_move<0xB1>(amax));
+    amax = fmaxf(amax, dpp_move<0x4E>(amax));
+    amax = fmaxf(amax, dpp_move<0x141>(amax));
     const float d = amax / 127.0f;
     int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
     if (amax != 0.0f) {
@@ -111,27 +111,33 @@ __device__ __forceinline__ uint32_t quantize_q8_lane4(float4 v, __half &d_half, 
         q3 = (int)roundf(v.w / d);
     }
     int s = q0 + q1 + q2 + q3;
-    s += __shfl_xor(s, 1, 64);
-    s += __shfl_xor(s, 2, 64);
-    s += __shfl_xor(s, 4, 64);
+    s += dpp_move_i<0xB1>(s);
+    s += dpp_move_i<0x4E>(s);
+    s += dpp_move_i<0x141>(s);
     bsum = s;
     d_half = __float2half_rn(d);
     return (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
            ((uint32_t)(q3 & 0xFF) << 24);
 }
 
-
 // Same quantization with one value per lane: the 32 lanes of a block are consecutive lanes
 // (lane % 32 == position in the block), all active.
 __device__ __forceinline__ int quantize_q8_lane1(float v, __half &d_half, int &bsum) {
+    // 32-lane reductions: quad permutes, half mirror, mirror (16-lane row), then the neighbouring row
     float amax = fabsf(v);
-#pragma unroll
-    for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    amax = fmaxf(amax, dpp_move<0xB1>(amax));
+    amax = fmaxf(amax, dpp_move<0x4E>(amax));
+    amax = fmaxf(amax, dpp_move<0x141>(amax));
+    amax = fmaxf(amax, dpp_move<0x140>(amax));
+    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
     const float d = amax / 127.0f;
     const int q = amax != 0.0f ? (int)roundf(v / d) : 0;
     int s = q;
-#pragma unroll
-    for (int off = 1; off < 32; off <<= 1) s += __shfl_xor(s, off, 64);
+    s += dpp_move_i<0xB1>(s);
+    s += dpp_move_i<0x4E>(s);
+    s += dpp_move_i<0x141>(s);
+    s += dpp_move_i<0x140>(s);
+    s += __shfl_xor(s, 16, 64);
     bsum = s;
     d_half = __float2half_rn(d);
     return q;

@@ -35,7 +35,7 @@ struct FusedArgs {
 __device__ __forceinline__ float silu_exact(float x) { return x / (1.0f + expf(-x)); }
 
 template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void k_matvec_fused(const FusedArgs a) {
+__global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1) void k_matvec_fused(const FusedArgs a) {
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;       // activation values the LDS image is sized for
     constexpr int AQ = (CAP / 16 + T - 1) / T;      // PRO_Q8: 16-byte chunks of quants per thread
