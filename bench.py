@@ -34,6 +34,9 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
+# HBM bytes one launch of the Q4_K 4096x11008 matvec moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by a copy kernel of known size (profiles/matvec_q4k_4096x11008.md): 24985 KiB read + 32 KiB written
+MATVEC_TRAFFIC_BYTES = (24985 + 32) * 1024
 ROTATE_BYTES = 640 << 20  # distinct weight bytes cycled through (last-level cache is 256 MB)
 
 
@@ -219,7 +222,7 @@ def main():
                    "algorithmic_bytes_per_step": alg, "distinct_weight_copies": n_copies,
                    "device": dev.name},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MATVEC_TRAFFIC_BYTES,
                      "kernel": "k_matvec<UnitQ4K>", "us_per_launch": round(ms_kernel * 1e3, 3)},
     }
 
@@ -240,6 +243,35 @@ def main():
                           "frac": round(gb / HBM_PEAK_GBPS, 4)})
             log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
         out["sweep"] = sweep
+
+    if not args.no_sweep:
+        # the two conversions, both HBM-bound: dequantize writes 4 B per weight, quantize reads 4 B per value
+        conv = []
+        for f, name in ((synth.Q4_K, "q4_k"), (synth.Q6_K, "q6_k"), (synth.Q8_0, "q8_0"), (synth.Q4_0, "q4_0")):
+            r, k = 4096, 11008
+            nb = synth.weight_nbytes(f, r, k)
+            base = synth.random_weight(f, r, k, seed=500 + f)
+            ws = [dev.qtensor(f, r, k, base) for _ in range(3)]
+            outb = dev.alloc(4 * r * k)
+            dev.dequantize_sweep(ws, outb, 5)
+            ms = dev.dequantize_sweep(ws, outb, 30) / 30
+            byts = nb + 4 * r * k
+            conv.append({"op": "dequantize", "fmt": name, "rows": r, "cols": k, "us": round(ms * 1e3, 2),
+                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+            log(f"  dequantize {name} {r}x{k}: {ms * 1e3:.1f} us, {conv[-1]['GBps']} GB/s")
+            for w in ws:
+                w.free()
+            outb.free()
+        for r, k, copies in ((1, 4096, 1), (512, 4096, 32)):
+            x = dev.from_numpy(synth.random_activations(r * copies, k, seed=9))
+            outb = dev.alloc(r * k // 32 * 34 + 64)
+            dev.quantize_sweep(x, r * k, copies, r, k, outb, 20)
+            ms = dev.quantize_sweep(x, r * k, copies, r, k, outb, 200) / 200
+            byts = 4 * r * k + r * k // 32 * 34
+            conv.append({"op": "quantize_q8_0", "rows": r, "cols": k, "us": round(ms * 1e3, 2),
+                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+            log(f"  quantize_q8_0 {r}x{k}: {ms * 1e3:.2f} us, {conv[-1]['GBps']} GB/s")
+        out["conversions"] = conv
 
     if not args.no_prefill:
         # batched prefill: Q4_K 14336x4096 x f32 [M, 4096]; MFMA peak = dense fp16 (the operand type used)

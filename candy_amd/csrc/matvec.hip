@@ -252,7 +252,8 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
         float *yo = y + done * N;
         int rc;
         // LDS holds NB activation rows; keep the workgroup's share under 64 KB
-        if (left >= 4 && K <= 8192) { rc = launch_one<U, 4, 2, 4>(dev, w, q, s, yo); done += 4; }
+        if (left >= 8 && K <= 5632) { rc = launch_one<U, 8, 2, 4>(dev, w, q, s, yo); done += 8; }
+        else if (left >= 4 && K <= 11264) { rc = launch_one<U, 4, 2, 4>(dev, w, q, s, yo); done += 4; }
         else if (left >= 2 && K <= 16384) { rc = launch_one<U, 2, 2, 4>(dev, w, q, s, yo); done += 2; }
         else { rc = launch_one<U, 1, 2, 4>(dev, w, q, s, yo); done += 1; }
         if (rc) return rc;
@@ -327,8 +328,13 @@ static int qmatmul_check(candy_hip_device *dev, const candy_hip_qtensor *w, int6
     return CANDY_HIP_OK;
 }
 
+static int mmq_min_m() {
+    static const int v = getenv("CANDY_HIP_MMQ_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_MIN_M")) : 16;
+    return v < 16 ? 16 : v;
+}
+
 static int contract(candy_hip_device *dev, const candy_hip_qtensor *w, const ActWorkspace &a, int64_t m, float *y) {
-    return m < 16 ? launch_matvec(dev, w, a.qs, a.scales, m, y) : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws);
+    return m < mmq_min_m() ? launch_matvec(dev, w, a.qs, a.scales, m, y) : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws);
 }
 
 int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m, float *dev_y) {

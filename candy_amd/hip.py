@@ -89,6 +89,9 @@ SIGNATURES = {
     "candy_hip_llama_decode_hidden": (c_int, [c_void_p, c_void_p, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_qmatmul_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int64, c_void_p, c_int, c_int,
                                         POINTER(c_float)]),
+    "candy_hip_dequantize_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int, POINTER(c_float)]),
+    "candy_hip_quantize_sweep": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p, c_int,
+                                         POINTER(c_float)]),
     "candy_hip_timer_start": (c_int, [c_void_p]),
     "candy_hip_timer_stop": (c_int, [c_void_p, POINTER(c_float)]),
 }
@@ -348,6 +351,19 @@ class Device:
         ms = c_float(0)
         _check(lib().candy_hip_qmatmul_sweep(self.handle, arr, len(weights), x_buf.ptr, m, y_buf.ptr, iters,
                                              int(quantize_each), byref(ms)))
+        return ms.value
+
+    def dequantize_sweep(self, weights: list, out_buf: "Buffer", iters: int) -> float:
+        arr = (c_void_p * len(weights))(*[w.handle for w in weights])
+        ms = c_float(0)
+        _check(lib().candy_hip_dequantize_sweep(self.handle, arr, len(weights), out_buf.ptr, iters, byref(ms)))
+        return ms.value
+
+    def quantize_sweep(self, x_buf: "Buffer", x_stride: int, n_x: int, rows: int, cols: int, out_buf: "Buffer",
+                       iters: int) -> float:
+        ms = c_float(0)
+        _check(lib().candy_hip_quantize_sweep(self.handle, x_buf.ptr, x_stride, n_x, rows, cols, out_buf.ptr, iters,
+                                              byref(ms)))
         return ms.value
 
     def timer_start(self):

@@ -211,6 +211,13 @@ int candy_hip_llama_decode_hidden(candy_hip_llama *m, const float *dev_hidden, i
 int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws,
                             const float *dev_x, int64_t m, float *dev_y, int iters, int quantize_each,
                             float *elapsed_ms);
+/* Same for the two bandwidth-bound conversions: `iters` dequantizations rotating over ws[]
+ * (dev_out holds rows*cols f32), and `iters` Q8_0 quantizations of x[rows, cols] rotating over
+ * n_x inputs spaced x_stride elements apart (dev_out_blocks holds rows*cols/32 blocks). */
+int candy_hip_dequantize_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws,
+                               float *dev_out, int iters, float *elapsed_ms);
+int candy_hip_quantize_sweep(candy_hip_device *dev, const float *dev_x, int64_t x_stride, int n_x, int64_t rows,
+                             int64_t cols, void *dev_out_blocks, int iters, float *elapsed_ms);
 int candy_hip_timer_start(candy_hip_device *dev);
 int candy_hip_timer_stop(candy_hip_device *dev, float *elapsed_ms);   /* synchronises */
 
