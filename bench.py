@@ -125,6 +125,75 @@ def build_7b(dev, n_layers=32, max_pos=2176, seed=4000):
     return cfg, model
 
 
+def build_8b(dev, max_pos, seed=8000):
+    """Random-init Llama-3-8B-shaped decoder: GQA 32/8, FFN 14336, vocab 128256; Q4_K attention and
+    gate/up, Q6_K down and head, Q8_0 embedding rows."""
+    from candy_amd import hip, synth
+    cfg = dict(n_layers=32, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ffn=14336, vocab=128256,
+               max_pos=max_pos, rms_eps=1e-5, rope_base=500000.0)
+    model = hip.Llama(dev, **cfg)
+    shapes = [(hip.W_Q, 4096, 4096, synth.Q4_K), (hip.W_K, 1024, 4096, synth.Q4_K), (hip.W_V, 1024, 4096, synth.Q4_K),
+              (hip.W_O, 4096, 4096, synth.Q4_K), (hip.W_GATE, 14336, 4096, synth.Q4_K),
+              (hip.W_UP, 14336, 4096, synth.Q4_K), (hip.W_DOWN, 4096, 14336, synth.Q6_K)]
+    ones = np.ones(4096, np.float32)
+    t0 = time.perf_counter()
+    nbytes = 0
+    for l in range(cfg["n_layers"]):
+        for kind, r, k, f in shapes:
+            seed += 1
+            model.set_qweight(kind, l, dev.qtensor(f, r, k, synth.random_weight(f, r, k, seed, synth.unit_scale(f))))
+            nbytes += synth.weight_nbytes(f, r, k)
+        model.set_norm(hip.W_ATTN_NORM, l, ones)
+        model.set_norm(hip.W_FFN_NORM, l, ones)
+        if l % 8 == 7:
+            log(f"  built layer {l + 1}/32 ({time.perf_counter() - t0:.0f} s)")
+    model.set_norm(hip.W_OUT_NORM, -1, ones)
+    model.set_qweight(hip.W_HEAD, -1, dev.qtensor(synth.Q6_K, 128256, 4096, synth.random_weight(
+        synth.Q6_K, 128256, 4096, seed + 1, synth.unit_scale(synth.Q6_K))))
+    model.set_qweight(hip.W_EMBED, -1, dev.qtensor(synth.Q8_0, 128256, 4096, synth.random_weight(
+        synth.Q8_0, 128256, 4096, seed + 2, synth.unit_scale(synth.Q8_0))))
+    return cfg, model, nbytes + synth.weight_nbytes(synth.Q6_K, 128256, 4096)
+
+
+def llama3_leg(dev, n_prompt=512, n_decode=128):
+    """Prefill a seeded random prompt in one batched pass, then decode greedily at batch 1."""
+    log("building random-init Llama-3-8B shape (Q4_K / Q6_K down+head / Q8_0 embedding) ...")
+    cfg, model, weight_bytes = build_8b(dev, max_pos=n_prompt + n_decode + 8)
+    prompt = [int(t) for t in np.random.default_rng(4321).integers(0, cfg["vocab"], n_prompt)]
+    model.prefill(prompt[:64], 0, want_logits=False)  # warm-up: allocates the prompt buffers' first size
+    model.prefill(prompt, 0, want_logits=False)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        tok, _ = model.prefill(prompt, 0, want_logits=False)
+    dev.synchronize()
+    pre_s = (time.perf_counter() - t0) / reps
+    pos = n_prompt
+    for _ in range(4):
+        tok, _ = model.decode(tok, pos, want_logits=False)
+        pos += 1
+    dev.synchronize()
+    t0 = time.perf_counter()
+    toks = []
+    for _ in range(n_decode - 4):
+        tok, _ = model.decode(tok, pos, want_logits=False)
+        toks.append(tok)
+        pos += 1
+    dev.synchronize()
+    dec_s = (time.perf_counter() - t0) / (n_decode - 4)
+    kv_mid = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * (n_prompt + n_decode // 2) * cfg["head_dim"] * 4
+    bpt = weight_bytes + kv_mid
+    per_layer_macs = (2 * 4096 * 4096 + 2 * 1024 * 4096 + 3 * 14336 * 4096)
+    lin_flops = 2.0 * n_prompt * per_layer_macs * cfg["n_layers"]
+    model.free()
+    return {"prefill_tokens": n_prompt, "prefill_ms": round(pre_s * 1e3, 2), "prefill_tok_s": round(n_prompt / pre_s, 1),
+            "prefill_linear_TFLOPs": round(lin_flops / pre_s / 1e12, 1),
+            "decode_tokens": n_decode - 4, "decode_ms_per_token": round(dec_s * 1e3, 4), "decode_tok_s": round(1 / dec_s, 2),
+            "decode_bytes_per_token": bpt, "decode_hbm_frac": round(bpt / dec_s / 1e9 / HBM_PEAK_GBPS, 4),
+            "tokens": toks[:8]}
+
+
 def prefill_kv(dev, model, cfg, n_pos, seed=9):
     """KV cache positions [0, n_pos) <- N(0,1) f32."""
     from candy_amd import hip
@@ -183,6 +252,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the other shapes of the batch-1 sweep")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the batched-prefill (MFMA) leg")
+    ap.add_argument("--no-llama3", action="store_true", help="skip the Llama-3-8B-shaped prefill + decode leg")
     ap.add_argument("--decode-steps", type=int, default=32)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for counter runs)")
@@ -274,7 +344,8 @@ def main():
         out["conversions"] = conv
 
     if not args.no_prefill:
-        # batched prefill: Q4_K 14336x4096 x f32 [M, 4096]; MFMA peak = dense fp16 (the operand type used)
+        # batched prefill: Q4_K 14336x4096 x f32 [M, 4096] on the int8 matrix cores; mfma_frac is quoted against
+        # the dense fp16 peak (2.5 PFLOP/s), the int8 peak is twice that
         pre = []
         r, k = 14336, 4096
         for m in (16, 128, 512):
@@ -290,6 +361,10 @@ def main():
     if not args.no_decode:
         out["decode"] = decode_leg(dev, args.decode_steps, 4)
         log("decode:", out["decode"])
+
+    if not args.no_llama3:
+        out["llama3_8b"] = llama3_leg(dev)
+        log("llama3-8b shape:", out["llama3_8b"])
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(rows, cols)

@@ -170,5 +170,16 @@ struct ActWorkspace {
     void *half_ws;
 };
 int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quants, ActWorkspace *out);
+// matvec.hip: y[m, rows] = x . W^T for any m from planar activations that live OUTSIDE the device
+// workspace (the tile kernel may carve its fp16 scratch from it).
+int mmq_min_m();
+int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                    int64_t m, float *y);
+// prefill.hip: prompt stages of the decoder (n tokens at positions pos0 ..).
+int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, const float *v, const float *cos_t,
+                           const float *sin_t, float *k_cache, float *v_cache, int n, int pos0, int n_heads,
+                           int n_kv_heads, int head_dim, int64_t cache_stride);
+int launch_attn_prefill(candy_hip_device *dev, const float *q, const float *k_cache, const float *v_cache, float *out,
+                        int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride, float scale);
 
 }  // namespace candy

@@ -38,6 +38,16 @@ struct candy_hip_llama {
     bool graph_dirty = true;
     bool use_graph = true;
     std::vector<void *> owned;
+    // prompt buffers, grown on demand to the longest prompt seen: [n][width] activations
+    struct Prompt {
+        int cap = 0;
+        int64_t *ids = nullptr;
+        float *h = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *att = nullptr, *tmp = nullptr;
+        float *gate = nullptr, *up = nullptr;
+        int8_t *xq = nullptr;
+        candy::Q8Scale *xs = nullptr;
+        std::vector<void *> owned;
+    } pf;
 };
 
 namespace candy {
@@ -57,6 +67,15 @@ static int dev_alloc(candy_hip_llama *m, T **p, size_t count) {
     void *d = nullptr;
     if (int rc = candy_hip_alloc(m->dev, count * sizeof(T), &d)) return rc;
     m->owned.push_back(d);
+    *p = (T *)d;
+    return CANDY_HIP_OK;
+}
+
+template <class T>
+static int prompt_alloc(candy_hip_llama *m, T **p, size_t count) {
+    void *d = nullptr;
+    if (int rc = candy_hip_alloc(m->dev, count * sizeof(T), &d)) return rc;
+    m->pf.owned.push_back(d);
     *p = (T *)d;
     return CANDY_HIP_OK;
 }
@@ -138,6 +157,7 @@ int candy_hip_llama_free(candy_hip_llama *m) {
     if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
     if (m->graph) (void)hipGraphDestroy(m->graph);
     for (void *p : m->owned) (void)candy_hip_free(m->dev, p);
+    for (void *p : m->pf.owned) (void)candy_hip_free(m->dev, p);
     delete m;
     return CANDY_HIP_OK;
 }
@@ -329,6 +349,103 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
     if (next_token) {
         uint32_t t = 0;
         if ((rc = candy_hip_d2h(dev, &t, m->next_tok, sizeof(t)))) return rc;
+        *next_token = (int32_t)t;
+    }
+    return CANDY_HIP_OK;
+}
+
+static int prompt_reserve(candy_hip_llama *m, int n) {
+    candy_hip_llama::Prompt &P = m->pf;
+    if (n <= P.cap) return CANDY_HIP_OK;
+    const candy_hip_llama_config &c = m->cfg;
+    CANDY_HIP_TRY(hipStreamSynchronize(m->dev->stream));
+    for (void *p : P.owned) (void)candy_hip_free(m->dev, p);
+    P.owned.clear();
+    P.cap = 0;
+    const size_t N = (size_t)n, qd = (size_t)c.n_heads * c.head_dim, kvd = (size_t)c.n_kv_heads * c.head_dim;
+    const size_t widest = std::max(std::max((size_t)c.d_model, (size_t)c.d_ffn), qd);
+    int rc = CANDY_HIP_OK;
+    if (!rc) rc = prompt_alloc(m, &P.ids, N);
+    if (!rc) rc = prompt_alloc(m, &P.h, N * c.d_model);
+    if (!rc) rc = prompt_alloc(m, &P.q, N * qd);
+    if (!rc) rc = prompt_alloc(m, &P.k, N * kvd);
+    if (!rc) rc = prompt_alloc(m, &P.v, N * kvd);
+    if (!rc) rc = prompt_alloc(m, &P.att, N * qd);
+    if (!rc) rc = prompt_alloc(m, &P.tmp, N * c.d_model);
+    if (!rc) rc = prompt_alloc(m, &P.gate, N * c.d_ffn);
+    if (!rc) rc = prompt_alloc(m, &P.up, N * c.d_ffn);
+    if (!rc) rc = prompt_alloc(m, &P.xq, N * widest);
+    if (!rc) rc = prompt_alloc(m, &P.xs, N * (widest / 32));
+    if (rc) return rc;
+    P.cap = n;
+    return CANDY_HIP_OK;
+}
+
+// The prompt pass: the decode step's sequence with n rows per activation. Linears go through the
+// batched contraction (MFMA tiles from 16 rows up), attention is causal over the cache, and only
+// the last row goes through the final norm and the head.
+static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
+    const candy_hip_llama_config &c = m->cfg;
+    candy_hip_device *dev = m->dev;
+    candy_hip_llama::Prompt &P = m->pf;
+    const size_t layer_kv = (size_t)c.n_kv_heads * c.max_pos * c.head_dim;
+    const int64_t cache_stride = (int64_t)c.max_pos * c.head_dim;
+    const int64_t qd = (int64_t)c.n_heads * c.head_dim;
+    const float scale = 1.0f / std::sqrt((float)c.head_dim);
+    int rc;
+    if ((rc = candy_hip_qindex_select(dev, m->embed, P.ids, n, P.h))) return rc;
+    for (int l = 0; l < c.n_layers; ++l) {
+        const candy_hip_llama::Layer &L = m->layers[l];
+        float *kc = m->k_cache + (size_t)l * layer_kv, *vc = m->v_cache + (size_t)l * layer_kv;
+        if ((rc = launch_rms_norm_quant(dev, P.h, L.attn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs))) return rc;
+        if ((rc = launch_contract(dev, L.wq, P.xq, P.xs, n, P.q))) return rc;
+        if ((rc = launch_contract(dev, L.wk, P.xq, P.xs, n, P.k))) return rc;
+        if ((rc = launch_contract(dev, L.wv, P.xq, P.xs, n, P.v))) return rc;
+        if ((rc = launch_prefill_rope_kv(dev, P.q, P.k, P.v, m->cos_t, m->sin_t, kc, vc, n, pos0, c.n_heads,
+                                         c.n_kv_heads, c.head_dim, cache_stride)))
+            return rc;
+        if ((rc = launch_attn_prefill(dev, P.q, kc, vc, P.att, n, pos0, c.n_heads, c.n_kv_heads, c.head_dim,
+                                      cache_stride, scale)))
+            return rc;
+        if ((rc = launch_quantize_q8(dev, P.att, n, qd, P.xq, P.xs, nullptr))) return rc;
+        if ((rc = launch_contract(dev, L.wo, P.xq, P.xs, n, P.tmp))) return rc;
+        if ((rc = candy_hip_add(dev, P.h, P.tmp, (int64_t)n * c.d_model, P.h))) return rc;
+        if ((rc = launch_rms_norm_quant(dev, P.h, L.ffn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs))) return rc;
+        if ((rc = launch_contract(dev, L.gate, P.xq, P.xs, n, P.gate))) return rc;
+        if ((rc = launch_contract(dev, L.up, P.xq, P.xs, n, P.up))) return rc;
+        if ((rc = launch_silu_mul_quant(dev, P.gate, P.up, (int64_t)n * c.d_ffn, nullptr, P.xq, P.xs))) return rc;
+        if ((rc = launch_contract(dev, L.down, P.xq, P.xs, n, P.tmp))) return rc;
+        if ((rc = candy_hip_add(dev, P.h, P.tmp, (int64_t)n * c.d_model, P.h))) return rc;
+    }
+    if ((rc = candy_hip_d2d(dev, m->h, P.h + (size_t)(n - 1) * c.d_model, (size_t)c.d_model * sizeof(float)))) return rc;
+    const candy_hip_qtensor *ws[1] = {m->head};
+    float *ys[1] = {m->logits};
+    if ((rc = norm_linear(m, m->out_norm, ws, ys, 1))) return rc;
+    return candy_hip_argmax(dev, m->logits, 1, c.vocab, m->next_tok);
+}
+
+int candy_hip_llama_prefill(candy_hip_llama *m, const int32_t *tokens, int32_t n_tokens, int32_t pos0,
+                            const float **dev_logits, int32_t *next_token) {
+    CANDY_REQUIRE(m, "model is nil");
+    CANDY_REQUIRE(m->embed, "embedding table not set");
+    CANDY_REQUIRE(tokens && n_tokens > 0, "prompt is empty");
+    CANDY_REQUIRE(pos0 >= 0 && (int64_t)pos0 + n_tokens <= m->cfg.max_pos,
+                  "positions %d..%lld outside the cache (max_pos %d)", pos0, (long long)pos0 + n_tokens - 1,
+                  m->cfg.max_pos);
+    std::vector<int64_t> ids((size_t)n_tokens);
+    for (int32_t i = 0; i < n_tokens; ++i) {
+        CANDY_REQUIRE(tokens[i] >= 0 && tokens[i] < m->cfg.vocab, "token %d outside the vocabulary", tokens[i]);
+        ids[(size_t)i] = tokens[i];
+    }
+    if (int rc = llama_check_complete(m)) return rc;
+    if (int rc = use_device(m->dev)) return rc;
+    if (int rc = prompt_reserve(m, n_tokens)) return rc;
+    if (int rc = candy_hip_h2d(m->dev, m->pf.ids, ids.data(), ids.size() * sizeof(int64_t))) return rc;
+    if (int rc = llama_enqueue_prompt(m, n_tokens, pos0)) return rc;
+    if (dev_logits) *dev_logits = m->logits;
+    if (next_token) {
+        uint32_t t = 0;
+        if (int rc = candy_hip_d2h(m->dev, &t, m->next_tok, sizeof(t))) return rc;
         *next_token = (int32_t)t;
     }
     return CANDY_HIP_OK;

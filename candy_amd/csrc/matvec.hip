@@ -314,6 +314,19 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
     }
 }
 
+int mmq_min_m() {
+    static const int v = getenv("CANDY_HIP_MMQ_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_MIN_M")) : 16;
+    return v < 16 ? 16 : v;
+}
+
+int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                    int64_t m, float *y) {
+    if (m < mmq_min_m()) return launch_matvec(dev, w, qs, scales, m, y);
+    ActWorkspace extra;
+    if (int rc = act_workspace(dev, m, w->cols, false, &extra)) return rc;
+    return launch_mmq(dev, w, qs, scales, m, y, extra.half_ws);
+}
+
 }  // namespace candy
 
 using namespace candy;
@@ -326,11 +339,6 @@ static int qmatmul_check(candy_hip_device *dev, const candy_hip_qtensor *w, int6
     CANDY_REQUIRE(m >= 0, "invalid matrix dimensions");
     CANDY_REQUIRE(m == 0 || dev_y, "output is nil");
     return CANDY_HIP_OK;
-}
-
-static int mmq_min_m() {
-    static const int v = getenv("CANDY_HIP_MMQ_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_MIN_M")) : 16;
-    return v < 16 ? 16 : v;
 }
 
 static int contract(candy_hip_device *dev, const candy_hip_qtensor *w, const ActWorkspace &a, int64_t m, float *y) {
@@ -415,13 +423,7 @@ int candy_hip_qmatmul_qact(candy_hip_device *dev, const candy_hip_qtensor *w, co
                   (long long)a->cols, (long long)w->cols);
     CANDY_REQUIRE(dev_y, "output is nil");
     if (int rc = use_device(dev)) return rc;
-    ActWorkspace ws{a->qs, a->scales, nullptr};
-    if (a->m >= 16) {
-        ActWorkspace extra;
-        if (int rc = act_workspace(dev, a->m, a->cols, false, &extra)) return rc;
-        ws.half_ws = extra.half_ws;
-    }
-    return contract(dev, w, ws, a->m, dev_y);
+    return launch_contract(dev, w, a->qs, a->scales, a->m, dev_y);
 }
 
 int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws, const float *dev_x,

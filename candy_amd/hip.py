@@ -87,6 +87,8 @@ SIGNATURES = {
     "candy_hip_llama_kv_cache": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_size_t)]),
     "candy_hip_llama_decode": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_llama_decode_hidden": (c_int, [c_void_p, c_void_p, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
+    "candy_hip_llama_prefill": (c_int, [c_void_p, POINTER(c_int32), c_int32, c_int32, POINTER(c_void_p),
+                                        POINTER(c_int32)]),
     "candy_hip_qmatmul_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int64, c_void_p, c_int, c_int,
                                         POINTER(c_float)]),
     "candy_hip_dequantize_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int, POINTER(c_float)]),
@@ -423,6 +425,13 @@ class Llama:
         buf = self.dev.from_numpy(np.ascontiguousarray(hidden, np.float32))
         lg, nt = c_void_p(), c_int32(-1)
         _check(lib().candy_hip_llama_decode_hidden(self.handle, buf.ptr, pos, byref(lg), byref(nt)))
+        return self._result(lg, nt, want_logits)
+
+    def prefill(self, tokens, pos0: int = 0, want_logits: bool = True):
+        """Batched prompt pass; returns (greedy next token, logits) of the last prompt token."""
+        ids = (c_int32 * len(tokens))(*[int(t) for t in tokens])
+        lg, nt = c_void_p(), c_int32(-1)
+        _check(lib().candy_hip_llama_prefill(self.handle, ids, len(tokens), pos0, byref(lg), byref(nt)))
         return self._result(lg, nt, want_logits)
 
     def _result(self, lg, nt, want_logits):

@@ -200,6 +200,13 @@ int candy_hip_llama_decode(candy_hip_llama *m, int32_t token, int32_t pos, const
 /* Same step with the hidden state of the token given directly instead of an embedding row. */
 int candy_hip_llama_decode_hidden(candy_hip_llama *m, const float *dev_hidden, int32_t pos,
                                   const float **dev_logits, int32_t *next_token);
+/* Prompt pass: n_tokens token ids (host memory) enter the cache at positions pos0 .. pos0+n_tokens-1
+ * in one batched pass -- every Linear is one [n_tokens, K] x W^T contraction (the MatMul call shape
+ * of nn/linear.go:58-112 with m = n_tokens; MFMA tiles from 16 rows up), attention is causal over
+ * the cache -- and the logits / greedy next token of the LAST prompt token come back.  Equivalent
+ * to n_tokens successive candy_hip_llama_decode calls up to f32 summation order. */
+int candy_hip_llama_prefill(candy_hip_llama *m, const int32_t *tokens, int32_t n_tokens, int32_t pos0,
+                            const float **dev_logits, int32_t *next_token);
 
 /* ------------------------------------------------------------------ timing (HIP events on the handle's stream) */
 /* Runs `iters` contractions back to back, iteration i using weight ws[i % n_ws] (all the same

@@ -88,6 +88,67 @@ def test_decode_steps_match_cpu_composition(dev, name, cfg, fmts):
     assert rel(kc[:, :, :len(tokens)], ref.k_cache[:, :, :len(tokens)].astype(np.float64)) <= 1e-3
 
 
+PROMPT_CASES = [
+    # (name, cfg, formats, prompt length, bar): lengths on both sides of the 16-row switch to MFMA tiles
+    # and off the 32-query attention tile. Q4_K tiles are integer-exact, so the prompt pass holds the
+    # decode step's 1e-3; a Q6_K down-projection goes through the fp16 tile kernel (3e-4 per matmul,
+    # inside the 1e-3 matmul bar), and what it leaves in the residual stream and the cache
+    # compounds over layers, so that chain is held to 2e-3.
+    ("gqa-q4k-q6k-down", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=2, head_dim=64, d_ffn=1024, vocab=512,
+                              max_pos=64, rms_eps=1e-5, rope_base=500000.0),
+     {"default": synth.Q4_K, "down": synth.Q6_K, "head": synth.Q6_K, "embed": synth.Q8_0}, 37, 2e-3),
+    ("mha-hd128", dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=4, head_dim=128, d_ffn=768, vocab=256,
+                       max_pos=80, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}, 70, 1e-3),
+    ("short-prompt", dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=64, d_ffn=512, vocab=128,
+                          max_pos=16, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q8_0, "gate": synth.Q4_0, "head": synth.Q6_K, "embed": synth.Q4_K}, 5, 1e-3),
+]
+
+
+@pytest.mark.parametrize("name,cfg,fmts,n,bar", PROMPT_CASES)
+def test_prompt_pass_matches_token_by_token_cpu(dev, name, cfg, fmts, n, bar):
+    host, model = build(dev, cfg, fmts, seed=11)
+    ref = llama_ref.LlamaRef(cfg, host)
+    rng = np.random.default_rng(12)
+    tokens = [int(t) for t in rng.integers(0, cfg["vocab"], n)]
+    for pos, tok in enumerate(tokens):  # the CPU composition has no batched form: token by token
+        rt, rlogits, _ = ref.step(ref.embed(tok), pos)
+    nt, logits = model.prefill(tokens, 0)
+    assert rel(logits, rlogits) <= bar, name
+    assert nt == int(np.argmax(logits))
+    kptr, vptr, nbytes = model.kv_cache()
+    for ptr, want in ((kptr, ref.k_cache), (vptr, ref.v_cache)):
+        got = np.empty(nbytes // 4, np.float32)
+        hip._check(hip.lib().candy_hip_d2h(dev.handle, got.ctypes.data, ptr, nbytes))
+        got = got.reshape(want.shape)
+        assert rel(got[:, :, :n], want[:, :, :n].astype(np.float64)) <= bar
+        assert not got[:, :, n:].any()  # nothing written past the prompt
+    # decoding continues from the cache the prompt pass left
+    tok = nt
+    for pos in range(n, n + 3):
+        rt, rlogits, _ = ref.step(ref.embed(tok), pos)
+        gt, glogits = model.decode(tok, pos)
+        assert rel(glogits, rlogits) <= bar, (name, pos)
+        tok = rt
+
+
+def test_prompt_in_two_chunks_equals_one_pass(dev):
+    # a prompt continued at pos0 > 0 attends the positions already in the cache
+    name, cfg, fmts, n, _ = PROMPT_CASES[0]
+    _, a = build(dev, cfg, fmts, seed=13)
+    _, b = build(dev, cfg, fmts, seed=13)
+    tokens = [int(t) for t in np.random.default_rng(14).integers(0, cfg["vocab"], 50)]
+    ta, la = a.prefill(tokens, 0)
+    b.prefill(tokens[:19], 0)
+    tb, lb = b.prefill(tokens[19:], 19)
+    assert rel(lb, la.astype(np.float64)) <= 1e-4
+    with pytest.raises(hip.CandyHipError, match="outside the cache"):
+        a.prefill(tokens, cfg["max_pos"] - 10)
+    with pytest.raises(hip.CandyHipError, match="empty"):
+        a.prefill([], 0)
+
+
 def test_graph_replay_equals_eager_launches(dev):
     # the captured step is replayed for every token; every replay must give what one-by-one
     # launches give, with other work and synchronisations in between
