@@ -113,9 +113,10 @@ int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *w
 int64_t mmq_m_pad(int64_t m);
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                const Q8Scale *scales, int64_t m, float *y, void *half_ws);
-// mmq_i8.hip: Q4_K on v_mfma_i32_16x16x32_i8, bit-for-bit the batch-1 arithmetic. Needs 16-byte aligned w->data and qs.
-int launch_mmq_q4k_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
-                      const Q8Scale *scales, int64_t m, float *y);
+// mmq_i8.hip: Q4_K / Q6_K on v_mfma_i32_16x16x32_i8 with the batch-1 kernels' integer arithmetic.
+bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs);
+int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
+                  const Q8Scale *scales, int64_t m, float *y);
 // ops.hip: fused decode-step stages (all enqueue on dev->stream, no allocation, no sync).
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
                           int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales);

@@ -296,10 +296,9 @@ int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *
     const int64_t K = w->cols;
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && K <= 0x7FFFFFFF && m <= 0x7FFFFFFF, "matrix too large");
     if (K % 64 != 0) return launch_matvec(dev, w, qs, scales, m, y);  // odd block counts: small-batch kernel in slices
-    // Q4_K runs on the int8 matrix cores (exact); the fp16 tile kernel below serves the other formats
+    // Q4_K and Q6_K run on the int8 matrix cores (exact); the fp16 tile kernel below serves the other formats
     static const bool force_fp16 = getenv("CANDY_HIP_MMQ_FP16") != nullptr;
-    if (w->fmt == CANDY_HIP_Q4_K && !force_fp16 && ((uintptr_t)w->data & 15) == 0 && ((uintptr_t)qs & 15) == 0)
-        return launch_mmq_q4k_i8(dev, w, qs, scales, m, y);
+    if (!force_fp16 && mmq_i8_covers(w, qs)) return launch_mmq_i8(dev, w, qs, scales, m, y);
     CANDY_REQUIRE(half_ws, "internal: no workspace for the fp16 activations");
     const int64_t m_pad = mmq_m_pad(m);
     const int64_t runs = m_pad * (K >> 3);

@@ -1,24 +1,31 @@
-// Batched (m >= 16) Q4_K matmul on the integer matrix cores, exact like the matvec:
+// Batched (m >= 16) Q4_K and Q6_K matmul on the integer matrix cores, exact like the matvec:
 // y[m, N] = x[m, K] . W^T with x quantized to Q8_0.
 //
-// mul_mat_q + vec_dot_q4_K_q8_1_impl_mmq (tensor/internal/cuda/kernels/quantized.cu:455-578,
-// :2266-2294) tile the contraction for dp4a; here every 32-value sub-block is one
-// v_mfma_i32_16x16x32_i8 (16 weight rows x 16 activation rows), and the per-sub-block scales are
-// applied to the int32 tile exactly as the batch-1 vec-dot does (quantized.cu:2239-2263):
-//   sumf_d += d8 * float(dot * sc);  sumf_m += d8 * float(bsum * m);  y += d * sumf_d - dmin * sumf_m
-// with d and dmin folded into the per-sub-block factors, so the result matches the CPU contraction
-// to f32 rounding (no fp16 operand rounding). (Running the min term as a small f32 MFMA product
-// instead was measured slower: the kernel is bound by the sum of matrix and vector issue.)
+// mul_mat_q + vec_dot_q4_K_q8_1_impl_mmq / vec_dot_q6_K_q8_1_impl_mmq
+// (tensor/internal/cuda/kernels/quantized.cu:455-578, :2266-2294, :2392-2417) tile the contraction
+// for dp4a; here a 32-value sub-block is one v_mfma_i32_16x16x32_i8 (16 weight rows x 16
+// activation rows) and the scales are applied to the int32 tile as the batch-1 vec-dots do
+// (quantized.cu:2239-2263, :2367-2389):
+//   Q4_K  sumf_d += d8 * float(dot * sc);  sumf_m += d8 * float(bsum * m);  y += d * sumf_d - dmin * sumf_m
+//         (d and dmin folded into the per-sub-block factors)
+//   Q6_K  y += d * sum over 16-value groups of d8 * float(sc * dot): the two groups of a sub-block are two
+//         MFMAs whose A operand is zeroed in the other half (lanes 0-31 hold k 0-15, lanes 32-63 k 16-31),
+//         combined as integers (sc_lo * dot_lo + sc_hi * dot_hi < 2^24, exact in f32).
+// The result differs from the CPU contraction only by f32 summation order (no fp16 operand
+// rounding). Running the Q4_K min term as a small f32 MFMA product instead was measured slower:
+// the kernel is bound by the sum of matrix and vector issue.
 //
 // Work split: a wavefront owns 16 weight rows and all BM = 16*TM activation rows of the
 // workgroup; the four wavefronts of a workgroup share the activation tile in LDS.
 //   * weights are fetched a stage (up to four super-blocks, 1024 values) ahead as 16-byte chunks
-//     that run along the rows, so every wavefront load covers whole cache lines; the stage is then
-//     parked in the wavefront's own LDS slice, from where each lane picks 8 bytes of nibbles per
-//     64-value group in the A-operand layout (row = lane%16, 8 consecutive k per lane);
-//   * the 6-bit scales are unpacked once per (row, pair) by the lane that owns that row in the
+//     that run along the rows, so every wavefront load covers whole cache lines (fetching them
+//     directly in the A-operand layout, 8 bytes per lane from 16 rows, was 1.3x slower); the stage
+//     is parked in the wavefront's own LDS slice, every super-block at a 16-byte aligned slot
+//     (Q6_K blocks are 210 bytes and only 2-byte aligned in memory), from where each lane picks
+//     its A-operand bytes (row = lane%16, 8 consecutive k per lane);
+//   * Q4_K's 6-bit scales are unpacked once per (row, pair) by the lane that owns that row in the
 //     A layout and handed through LDS to the lanes that own the row in the C layout
-//     (4 consecutive weight rows per lane);
+//     (4 consecutive weight rows per lane); Q6_K's int8 scales are read from the slice directly;
 //   * activations: 256 int8 per row per super-block plus {d, d*bsum} per block, loaded one
 //     super-block ahead into registers and parked in LDS between two barriers.
 // The rescale costs 16 VALU instructions per 16x16x32 tile (convert, multiply and two fused
@@ -30,40 +37,189 @@ namespace candy {
 
 typedef int int4v __attribute__((ext_vector_type(4)));
 
-template <int TM>
-__global__ __launch_bounds__(256) void k_mmq_q4k_i8(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
-                                                    const Q8Scale *__restrict__ xs, float *__restrict__ y, int N,
-                                                    int M, int K) {
+constexpr int XROW = 272;  // LDS pitch of an activation row: 256 quants + 16 (bank spread)
+
+__device__ __forceinline__ void wave_lds_fence() {
+    // orders LDS traffic of one wavefront (its LDS operations complete in order): no barrier needed
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Per-format part: what one super-block of the wavefront's 16 rows does to the accumulators.
+//   slice   the wavefront's LDS slice, row r's super-block b at slice + r * pitch + b * SLOT
+//   s_xq    activation tile [16*TM][XROW] int8, s_xs {d, d*bsum} [16*TM][8]
+//   acc     lane (j = lane%16, c = lane/16) holds activation row 16a+j, weight rows 4c+i
+struct TileQ4K {
+    static constexpr int BLOCK = 144, SLOT = 144;
+    typedef u32x4 GlobalChunk;  // rows are 16-byte aligned
+    struct Exchange {
+        uint8_t sc[16 * 8];  // scale / min bytes [row][sub-block]
+        uint8_t mn[16 * 8];
+        float2 dd[16];       // {d, dmin} per row
+    };
+    template <int TM>
+    static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &ex,
+                                                      const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        const uint8_t *wl = slice + j * pitch + SLOT * b;  // the row this lane feeds into the A operand
+        {   // lane (row j, pair c) unpacks one pair of 6-bit scales and parks it for the C-layout owners
+            const u32x4 h = *(const u32x4 *)wl;
+            uint32_t sc2, m2;
+            q4k_scale_min_pair(h.y, h.z, h.w, c, sc2, m2);
+            *(uint16_t *)&ex.sc[j * 8 + 2 * c] = (uint16_t)sc2;
+            *(uint16_t *)&ex.mn[j * 8 + 2 * c] = (uint16_t)m2;
+            if (c == 0)
+                ex.dd[j] = make_float2(half_bits_to_float((uint16_t)(h.x & 0xFFFF)), half_bits_to_float((uint16_t)(h.x >> 16)));
+        }
+        wave_lds_fence();
+        // my four C rows are 4c .. 4c+3: 8 scale bytes, 8 min bytes, {d, dmin} each
+        const u32x4 scA = *(const u32x4 *)&ex.sc[32 * c], scB = *(const u32x4 *)&ex.sc[32 * c + 16];
+        const u32x4 mnA = *(const u32x4 *)&ex.mn[32 * c], mnB = *(const u32x4 *)&ex.mn[32 * c + 16];
+        const float4 dd0 = *(const float4 *)&ex.dd[4 * c], dd1 = *(const float4 *)&ex.dd[4 * c + 2];
+        wave_lds_fence();  // the slots are rewritten by the next super-block
+        const uint32_t scw[8] = {scA.x, scA.y, scA.z, scA.w, scB.x, scB.y, scB.z, scB.w};
+        const uint32_t mnw[8] = {mnA.x, mnA.y, mnA.z, mnA.w, mnB.x, mnB.y, mnB.z, mnB.w};
+        const float dw[4] = {dd0.x, dd0.z, dd1.x, dd1.z}, dmn[4] = {dd0.y, dd0.w, dd1.y, dd1.w};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const u32x2 qa = *(const u32x2 *)(wl + 16 + 32 * (t >> 1) + 8 * c);
+            const int sh = (t & 1) * 4;
+            const uint32_t lo = (qa.x >> sh) & 0x0F0F0F0Fu, hi = (qa.y >> sh) & 0x0F0F0F0Fu;
+            const long afrag = (long)(((uint64_t)hi << 32) | lo);
+            float dsc[4], dmf[4];  // d * sc and dmin * m of my four weight rows for this sub-block
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                dsc[i] = dw[i] * (float)((scw[2 * i + (t >> 2)] >> (8 * (t & 3))) & 0xFF);
+                dmf[i] = dmn[i] * (float)((mnw[2 * i + (t >> 2)] >> (8 * (t & 3))) & 0xFF);
+            }
+            int4v d[TM];  // all tiles of the sub-block first, so the matrix pipe runs under the rescale
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
+                d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const float2 sx = s_xs[(16 * a + j) * 8 + t];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[a][i] += sx.x * ((float)d[a][i] * dsc[i]);  // d8 * d * sc * dot
+                    acc[a][i] -= dmf[i] * sx.y;                     // d8 * bsum * dmin * m
+                }
+            }
+        }
+    }
+};
+
+struct TileQ6K {
+    static constexpr int BLOCK = 210, SLOT = 224;  // 14 chunks: the last one runs 14 bytes into the next block
+    typedef u32x4_a2 GlobalChunk;                  // blocks sit on 2-byte boundaries
+    struct Exchange {};
+    template <int TM>
+    static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &,
+                                                      const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        const uint8_t *wl = slice + j * pitch + SLOT * b;
+        // scales[16] (int8) and d of my four C rows, straight from the slice
+        u32x4 scq[4];
+        float dw[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint8_t *row = slice + (4 * c + i) * pitch + SLOT * b;
+            scq[i] = *(const u32x4 *)(row + 192);
+            dw[i] = half_bits_to_float(*(const uint16_t *)(row + 208));
+        }
+        float part[TM][4];  // sum over the super-block of d8 * (sc . dot), before the row's d
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[a][i] = 0.0f;
+        const bool low_half = c < 2;  // my 8 values belong to the sub-block's first 16-value group
+#pragma unroll
+        for (int ip = 0; ip < 2; ++ip) {
+            // element 128*ip + 32*quarter + il: ql[64*ip + 32*(quarter&1) + il] low/high nibble, qh[32*ip + il] bit pair
+            const u32x2 qla = *(const u32x2 *)(wl + 64 * ip + 8 * c), qlb = *(const u32x2 *)(wl + 64 * ip + 32 + 8 * c);
+            const u32x2 qh = *(const u32x2 *)(wl + 128 + 32 * ip + 8 * c);
+#pragma unroll
+            for (int quarter = 0; quarter < 4; ++quarter) {
+                const int t = 4 * ip + quarter;
+                const u32x2 ql = (quarter & 1) ? qlb : qla;
+                uint32_t w2[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const uint32_t nib = (quarter & 2) ? (ql[e] >> 4) & 0x0F0F0F0Fu : ql[e] & 0x0F0F0F0Fu;
+                    const uint32_t top = quarter == 0 ? (qh[e] << 4) : quarter == 1 ? (qh[e] << 2)
+                                       : quarter == 2 ? qh[e] : (qh[e] >> 2);
+                    const uint32_t q6 = nib | (top & 0x30303030u);
+                    // bytewise q6 - 32 (0..63 -> -32..31): bias by 128 so no byte borrows, then flip the bias off
+                    w2[e] = ((q6 | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
+                }
+                const long full = (long)(((uint64_t)w2[1] << 32) | w2[0]);
+                const long a_lo = low_half ? full : 0, a_hi = low_half ? 0 : full;
+                int sc_lo[4], sc_hi[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {  // scales[2t], scales[2t+1], sign-extended
+                    const uint32_t word = scq[i][t >> 1];
+                    sc_lo[i] = (int)(word << (24 - 16 * (t & 1))) >> 24;
+                    sc_hi[i] = (int)(word << (16 - 16 * (t & 1))) >> 24;
+                }
+                int4v dl[TM], dh[TM];
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
+                    dl[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+                    dh[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+                }
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    const float dx = s_xs[(16 * a + j) * 8 + t].x;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        part[a][i] += dx * (float)(__mul24(dh[a][i], sc_hi[i]) + __mul24(dl[a][i], sc_lo[i]));  // |dot| < 2^17
+                }
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[a][i] += dw[i] * part[a][i];
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+template <class F, int TM, int STG>
+__global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
+                                                const Q8Scale *__restrict__ xs, float *__restrict__ y, int N, int M,
+                                                int K) {
     constexpr int BM = 16 * TM;
-    constexpr int XROW = 272;                              // LDS pitch of an activation row: 256 quants + 16 (bank spread)
-    constexpr int STG = TM <= 2 ? 4 : (TM == 4 ? 2 : 1);   // super-blocks per stage: deep prefetch where m is small
-    constexpr int XSC = (BM * 8 + 255) / 256;              // activation scales per thread per super-block
+    constexpr int XSC = (BM * 8 + 255) / 256;  // activation scales per thread per super-block
+    // slice pitch: an odd multiple of 16 bytes, so the 16 rows of an 8-byte pick fall in distinct banks
+    constexpr int WPITCH = STG * F::SLOT + (((STG * F::SLOT / 16) & 1) ? 32 : 16);
+    static_assert((WPITCH / 16) % 2 == 1, "pitch must be an odd number of 16-byte units");
     __shared__ __align__(16) int8_t s_xq[BM * XROW];
-    __shared__ __align__(16) float2 s_xs[BM * 8];     // {d, d * bsum} per (row, block)
-    constexpr int WPITCH = STG * 144 + (STG == 1 ? 32 : 16);  // odd multiple of 16 bytes: conflict-free 8-byte picks
-    __shared__ __align__(16) uint8_t s_w[4][16 * WPITCH];   // per wavefront: the current stage's weight rows
-    __shared__ __align__(16) uint8_t s_sc[4][16 * 8];      // per wavefront: scale / min bytes [row][sub-block]
-    __shared__ __align__(16) uint8_t s_mn[4][16 * 8];
-    __shared__ __align__(16) float2 s_dd[4][16];           // {d, dmin} per row
+    __shared__ __align__(16) float2 s_xs[BM * 8];          // {d, d * bsum} per (row, block)
+    __shared__ __align__(16) uint8_t s_w[4][16 * WPITCH];  // per wavefront: the current stage's weight rows
+    __shared__ __align__(16) typename F::Exchange s_ex[4];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 15, c = lane >> 4;
     const int n0 = blockIdx.x * 64 + wave * 16, m0 = blockIdx.y * BM;
     const int nsb = K >> 8;
-    const size_t rb = (size_t)nsb * 144;
+    const size_t rb = (size_t)nsb * F::BLOCK;
 
-    // weights of one stage: 16 rows x STG blocks, fetched as whole 16-byte chunks that run along the
-    // rows (full cache lines per wavefront load), kept in registers while in flight, then parked in
-    // the wavefront's own LDS slice from where the lanes pick their A-operand bytes
-    constexpr int CPR = 9 * STG;                       // 16-byte chunks per row per stage
-    constexpr int WCH = (16 * CPR + 63) / 64;          // chunks per lane
+    // weights of one stage: 16 rows x STG blocks as 16-byte chunks along the rows, in registers
+    // while in flight, then parked in the wavefront's LDS slice
+    constexpr int CPB = F::SLOT / 16;           // chunks per block
+    constexpr int CPR = CPB * STG;              // chunks per row per stage
+    constexpr int WCH = (16 * CPR + 63) / 64;   // chunks per lane
     u32x4 wr[WCH];
     auto load_stage = [&](int s0) {
 #pragma unroll
         for (int i = 0; i < WCH; ++i) {
             const int q = min(lane + 64 * i, 16 * CPR - 1), row = q / CPR, col = q % CPR;
-            const int sb = min(s0 + col / 9, nsb - 1);
-            wr[i] = *(const u32x4 *)(W + (size_t)min(n0 + row, N - 1) * rb + (size_t)sb * 144 + (col % 9) * 16);
+            const int sb = min(s0 + col / CPB, nsb - 1);
+            wr[i] = *(const typename F::GlobalChunk *)(W + (size_t)min(n0 + row, N - 1) * rb + (size_t)sb * F::BLOCK +
+                                                       (col % CPB) * 16);
         }
     };
     auto park_stage = [&]() {
@@ -103,15 +259,10 @@ __global__ __launch_bounds__(256) void k_mmq_q4k_i8(const uint8_t *__restrict__ 
         for (int i = 0; i < 4; ++i) acc[a][i] = 0.0f;
 
     for (int s0 = 0; s0 < nsb; s0 += STG) {
-        // the slice is private to the wavefront, whose LDS operations complete in order: no barrier
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        wave_lds_fence();  // this wavefront is done reading the previous stage
         park_stage();
         load_stage(s0 + STG);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const uint8_t *wl = &s_w[wave][j * WPITCH];  // the row this lane feeds into the A operand
+        wave_lds_fence();
 #pragma unroll
         for (int b = 0; b < STG; ++b) {
             const int s = s0 + b;
@@ -126,55 +277,10 @@ __global__ __launch_bounds__(256) void k_mmq_q4k_i8(const uint8_t *__restrict__ 
                     const int e = tid + i * 256;
                     if (BM * 8 % 256 == 0 || e < BM * 8) s_xs[e] = make_float2(xsd[i], xsd[i] * (float)xsb[i]);
                 }
-                // scales: lane (row j, pair c) unpacks one pair and parks it for the C-layout owners
-                {
-                    const u32x4 h = *(const u32x4 *)(wl + 144 * b);
-                    uint32_t sc2, m2;
-                    q4k_scale_min_pair(h.y, h.z, h.w, c, sc2, m2);
-                    *(uint16_t *)&s_sc[wave][j * 8 + 2 * c] = (uint16_t)sc2;
-                    *(uint16_t *)&s_mn[wave][j * 8 + 2 * c] = (uint16_t)m2;
-                    if (c == 0)
-                        s_dd[wave][j] = make_float2(half_bits_to_float((uint16_t)(h.x & 0xFFFF)),
-                                                    half_bits_to_float((uint16_t)(h.x >> 16)));
-                }
                 __syncthreads();
                 load_x(s + 1);  // the next super-block's activations fly under this one's MFMAs
-                // my four C rows are 4c .. 4c+3: 8 scale bytes, 8 min bytes, {d, dmin} each
-                const u32x4 scA = *(const u32x4 *)&s_sc[wave][32 * c], scB = *(const u32x4 *)&s_sc[wave][32 * c + 16];
-                const u32x4 mnA = *(const u32x4 *)&s_mn[wave][32 * c], mnB = *(const u32x4 *)&s_mn[wave][32 * c + 16];
-                const float4 dd0 = *(const float4 *)&s_dd[wave][4 * c], dd1 = *(const float4 *)&s_dd[wave][4 * c + 2];
-                const uint32_t scw[8] = {scA.x, scA.y, scA.z, scA.w, scB.x, scB.y, scB.z, scB.w};
-                const uint32_t mnw[8] = {mnA.x, mnA.y, mnA.z, mnA.w, mnB.x, mnB.y, mnB.z, mnB.w};
-                const float dw[4] = {dd0.x, dd0.z, dd1.x, dd1.z}, dmn[4] = {dd0.y, dd0.w, dd1.y, dd1.w};
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const u32x2 qa = *(const u32x2 *)(wl + 144 * b + 16 + 32 * (t >> 1) + 8 * c);
-                    const int sh = (t & 1) * 4;
-                    const uint32_t lo = (qa.x >> sh) & 0x0F0F0F0Fu, hi = (qa.y >> sh) & 0x0F0F0F0Fu;
-                    const long afrag = (long)(((uint64_t)hi << 32) | lo);
-                    float dsc[4], dmf[4];  // d * sc and dmin * m of my four weight rows for this sub-block
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        dsc[i] = dw[i] * (float)((scw[2 * i + (t >> 2)] >> (8 * (t & 3))) & 0xFF);
-                        dmf[i] = dmn[i] * (float)((mnw[2 * i + (t >> 2)] >> (8 * (t & 3))) & 0xFF);
-                    }
-                    int4v d[TM];  // all tiles of the sub-block first, so the matrix pipe runs under the rescale
-#pragma unroll
-                    for (int a = 0; a < TM; ++a) {
-                        const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
-                        d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
-                    }
-#pragma unroll
-                    for (int a = 0; a < TM; ++a) {
-                        const float2 sx = s_xs[(16 * a + j) * 8 + t];
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            acc[a][i] += sx.x * ((float)d[a][i] * dsc[i]);  // d8 * d * sc * dot
-                            acc[a][i] -= dmf[i] * sx.y;                     // d8 * bsum * dmin * m
-                        }
-                    }
-                }
-                __syncthreads();  // the tile and the scale slots are rewritten next
+                F::template superblock<TM>(s_w[wave], WPITCH, b, j, c, s_ex[wave], s_xq, s_xs, acc);
+                __syncthreads();  // the activation tile is rewritten next
             }
         }
     }
@@ -195,22 +301,39 @@ __global__ __launch_bounds__(256) void k_mmq_q4k_i8(const uint8_t *__restrict__ 
     }
 }
 
-int launch_mmq_q4k_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                      int64_t m, float *y) {
+template <class F>
+static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                     int64_t m, float *y) {
     const int N = (int)w->rows, K = (int)w->cols, M = (int)m;
     const unsigned gx = (unsigned)((N + 63) / 64);
-#define CANDY_MMQ_I8(TMV)                                                                                         \
-    hipLaunchKernelGGL((k_mmq_q4k_i8<TMV>), dim3(gx, (unsigned)((M + 16 * TMV - 1) / (16 * TMV))), dim3(256), 0, \
+    constexpr int DEEP = F::SLOT == 144 ? 4 : 2;  // super-blocks per stage where m is small (LDS budget)
+#define CANDY_MMQ_I8(TMV, STGV)                                                                                       \
+    hipLaunchKernelGGL((k_mmq_i8<F, TMV, STGV>), dim3(gx, (unsigned)((M + 16 * TMV - 1) / (16 * TMV))), dim3(256), 0, \
                        dev->stream, (const uint8_t *)w->data, qs, scales, y, N, M, K)
     // the largest tile height that still leaves about 1.5 wavefronts per SIMD: a wavefront walks the
     // whole contraction on its own, so a grid below that leaves load latency exposed
     const int64_t strips = (N + 15) / 16, want = 1536;
-    if (M > 32 && strips * ((M + 63) / 64) >= want) CANDY_MMQ_I8(4);
-    else if (M > 16 && strips * ((M + 31) / 32) >= want) CANDY_MMQ_I8(2);
-    else CANDY_MMQ_I8(1);
+    if (M > 32 && strips * ((M + 63) / 64) >= want) CANDY_MMQ_I8(4, 2);
+    else if (M > 16 && strips * ((M + 31) / 32) >= want) CANDY_MMQ_I8(2, DEEP);
+    else CANDY_MMQ_I8(1, DEEP);
 #undef CANDY_MMQ_I8
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
+}
+
+bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs) {
+    if (((uintptr_t)qs & 15) != 0 || w->cols % 256 != 0) return false;
+    if (w->fmt == CANDY_HIP_Q4_K) return ((uintptr_t)w->data & 15) == 0;
+    // the last chunk of a Q6_K row runs 14 bytes past the block: only buffers allocated by the library
+    // (which pads them) are known to have that room after the last row
+    if (w->fmt == CANDY_HIP_Q6_K) return w->owned && ((uintptr_t)w->data & 1) == 0;
+    return false;
+}
+
+int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                  int64_t m, float *y) {
+    return w->fmt == CANDY_HIP_Q4_K ? launch_i8<TileQ4K>(dev, w, qs, scales, m, y)
+                                    : launch_i8<TileQ6K>(dev, w, qs, scales, m, y);
 }
 
 }  // namespace candy

@@ -1,7 +1,7 @@
 """GPU parity of the batched (m >= 16) QMatMul, the MFMA tile kernels, against the CPU oracle.
-Bar: max|gpu - ref| / max|ref| <= 1e-3. The fp16 tile kernel (Q4_0, Q8_0, Q6_K) rounds its operands
-to fp16 and lands near 2e-4; the Q4_K kernel multiplies int8 on the matrix cores and differs from
-the oracle's integer dots only by f32 summation order, so it is held to 2e-5."""
+Bar: max|gpu - ref| / max|ref| <= 1e-3. The fp16 tile kernel (Q4_0, Q8_0) rounds its operands to
+fp16 and lands near 2e-4; the Q4_K / Q6_K kernel multiplies int8 on the matrix cores and differs
+from the oracle's integer dots only by f32 summation order, so it is held to 2e-5."""
 import numpy as np
 import pytest
 
@@ -39,14 +39,15 @@ def test_tile_kernel_matches_oracle(dev, fmt, m):
     assert np.max(per_row) <= 2 * TOL
 
 
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K])
 @pytest.mark.parametrize("m", [16, 31, 32, 48, 65, 129, 300])
 @pytest.mark.parametrize("rows,cols", [(1, 256), (15, 768), (67, 1280), (130, 2304), (1030, 512)])
-def test_q4k_int8_tiles_are_integer_exact(dev, m, rows, cols):
+def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
     # rows off every 4/16/64 boundary, block counts off every stage length, m off every tile height
-    w = synth.random_weight(synth.Q4_K, rows, cols, seed=rows + m)
+    w = synth.random_weight(fmt, rows, cols, seed=rows + m)
     x = synth.random_activations(m, cols, seed=cols + m)
-    got = dev.qmatmul(dev.qtensor(synth.Q4_K, rows, cols, w), x)
-    want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
+    got = dev.qmatmul(dev.qtensor(fmt, rows, cols, w), x)
+    want = o.qmatmul(fmt, w, rows, cols, x)
     assert got.shape == (m, rows)
     assert rel_err(got, want) <= 2e-5
 
