@@ -100,9 +100,30 @@ __global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ src, 
     const float *xr = src + (size_t)blockIdx.x * cols;
     float best = -3.402823466e+38f;
     uint32_t bi = 0xFFFFFFFFu;
-    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
-        const float v = xr[c];
-        if (v > best) { best = v; bi = (uint32_t)c; }
+    if ((cols & 3) == 0 && ((uintptr_t)xr & 15) == 0) {
+        // four independent 16-byte loads in flight per thread: one block has to cover a whole vocabulary row
+        const float4 *x4 = (const float4 *)xr;
+        const int n4 = cols >> 2, step = (int)blockDim.x;
+        for (int c0 = threadIdx.x; c0 < n4; c0 += 4 * step) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = x4[min(c0 + u * step, n4 - 1)];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int c = c0 + u * step;
+                if (c >= n4) break;
+                // ascending index within the thread, strict >: the first maximum wins
+                if (v[u].x > best) { best = v[u].x; bi = (uint32_t)(4 * c); }
+                if (v[u].y > best) { best = v[u].y; bi = (uint32_t)(4 * c + 1); }
+                if (v[u].z > best) { best = v[u].z; bi = (uint32_t)(4 * c + 2); }
+                if (v[u].w > best) { best = v[u].w; bi = (uint32_t)(4 * c + 3); }
+            }
+        }
+    } else {
+        for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+            const float v = xr[c];
+            if (v > best) { best = v; bi = (uint32_t)c; }
+        }
     }
     // lexicographic (value desc, index asc) reduction
 #pragma unroll

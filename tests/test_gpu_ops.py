@@ -111,6 +111,20 @@ def test_argmax_first_maximum_wins(dev):
     assert list(dev.argmax(x, 32000))[:3] == [5, 0, 31999]
 
 
+@pytest.mark.parametrize("cols", [128256, 32001, 4099, 7, 1])
+def test_argmax_wide_and_ragged_rows(dev, cols):
+    # rows wider than one pass of the block, widths that are not a multiple of 4 (rows then start
+    # off a 16-byte boundary), ties on both sides of a vector boundary
+    rng = np.random.default_rng(cols)
+    x = rng.standard_normal((3, cols)).astype(np.float32)
+    x[1, cols - 1] = 99.0
+    x[1, cols // 2] = 99.0
+    x[2, :] = np.float32(-np.inf)      # reduce.go:846-862: nothing beats -MaxFloat32 -> 0
+    got = list(dev.argmax(x, cols))
+    assert got == list(o.fast_argmax(x, cols))
+    assert got[1] == cols // 2 and got[2] == 0
+
+
 def test_index_select(dev):
     rng = np.random.default_rng(4)
     table = rng.standard_normal((50, 96)).astype(np.float32)
