@@ -20,11 +20,14 @@ __device__ __forceinline__ int skewed(int byte_off) { return byte_off + ((byte_o
 
 // ------------------------------------------------------------------ per-format units
 
+// SPAN: bytes that 64 consecutive units occupy in a row when that is a whole number of 16-byte
+// chunks although single blocks are not 16-byte aligned (0: the unit's own loads are aligned).
 struct UnitQ4K {
     static constexpr int ELEMS = 64;        // two 32-value sub-blocks sharing 32 bytes of nibbles
     static constexpr int ROW_ALIGN = 16;
+    static constexpr int SPAN = 0;
     struct W { u32x4 hdr, q0, q1; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 144; }
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 144; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const uint8_t *blk = row + (size_t)(u >> 2) * 144;
         w.hdr = *(const u32x4 *)blk;
@@ -51,8 +54,9 @@ struct UnitQ4K {
         lo = dot4_i8(w.q1.w & M, x1.w, lo); hi = dot4_i8((w.q1.w >> 4) & M, x3.w, hi);
         const float d = half_bits_to_float((uint16_t)(w.hdr.x & 0xFFFF));
         const float dmin = half_bits_to_float((uint16_t)(w.hdr.x >> 16));
-        const float sd = s0.d * (float)(lo * (int)(sc2 & 0xFF)) + s1.d * (float)(hi * (int)(sc2 >> 8));
-        const float sm = s0.d * (float)(s0.bsum * (int)(m2 & 0xFF)) + s1.d * (float)(s1.bsum * (int)(m2 >> 8));
+        // every factor fits 24 bits (|dot| <= 32*15*127, |bsum| <= 32*127, scales < 64): full-rate v_mul_i32_i24
+        const float sd = s0.d * (float)__mul24(lo, (int)(sc2 & 0xFF)) + s1.d * (float)__mul24(hi, (int)(sc2 >> 8));
+        const float sm = s0.d * (float)__mul24(s0.bsum, (int)(m2 & 0xFF)) + s1.d * (float)__mul24(s1.bsum, (int)(m2 >> 8));
         return d * sd - dmin * sm;
     }
 };
@@ -60,8 +64,9 @@ struct UnitQ4K {
 struct UnitQ8_0 {
     static constexpr int ELEMS = 32;
     static constexpr int ROW_ALIGN = 2;
+    static constexpr int SPAN = 64 * 34;
     struct W { u32x4 q0, q1; uint16_t d; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 34; }
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 34; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const BlockQ8_0 *blk = (const BlockQ8_0 *)row + u;
         w.d = blk->d;
@@ -83,8 +88,9 @@ template <bool GGML_ORDER>
 struct UnitQ4_0 {
     static constexpr int ELEMS = 32;
     static constexpr int ROW_ALIGN = 2;
+    static constexpr int SPAN = 64 * 18;
     struct W { u32x4 q; uint16_t d; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 18; }
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 18; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const BlockQ4_0 *blk = (const BlockQ4_0 *)row + u;
         w.d = blk->d;
@@ -125,8 +131,9 @@ struct UnitQ4_0 {
 struct UnitQ6K {
     static constexpr int ELEMS = 32;   // 8 values from each 32-value quarter of one 128-value half
     static constexpr int ROW_ALIGN = 2;
+    static constexpr int SPAN = 0;     // picking the unit's scattered bytes out of an LDS slice was measured slower
     struct W { u32x2 ql0, ql1, qh; uint32_t sc; uint16_t d; };
-    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 210; }
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 210; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
         const BlockQ6K *blk = (const BlockQ6K *)row + (u >> 3);
         const int ip = (u >> 2) & 1, j = u & 3;
