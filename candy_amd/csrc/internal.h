@@ -117,6 +117,9 @@ int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *
 bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs);
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                   const Q8Scale *scales, int64_t m, float *y);
+// mmq_f16.hip: Q4_K with prompt-sized batches on big fp16 tiles. xh: fp16 activations [mmq_m_pad(m)][K].
+bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m);
+int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y);
 // ops.hip: fused decode-step stages (all enqueue on dev->stream, no allocation, no sync).
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
                           int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales);

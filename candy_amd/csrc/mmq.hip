@@ -289,16 +289,18 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const _
     return launch_tile<F, 128, 128, 64>(dev, w, xh, m, y);
 }
 
-int64_t mmq_m_pad(int64_t m) { return (m + 127) / 128 * 128; }  // a multiple of every tile height
+int64_t mmq_m_pad(int64_t m) { return (m + 255) / 256 * 256; }  // a multiple of every tile height
 
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int64_t m,
                float *y, void *half_ws) {
     const int64_t K = w->cols;
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && K <= 0x7FFFFFFF && m <= 0x7FFFFFFF, "matrix too large");
     if (K % 64 != 0) return launch_matvec(dev, w, qs, scales, m, y);  // odd block counts: small-batch kernel in slices
-    // Q4_K and Q6_K run on the int8 matrix cores (exact); the fp16 tile kernel below serves the other formats
+    // prompt-sized batches of Q4_K: big fp16 tiles (the integer kernel is bound by its per-sub-block rescale there);
+    // smaller batches of Q4_K and Q6_K: int8 matrix cores (exact); the fp16 tile kernel below serves the rest
     static const bool force_fp16 = getenv("CANDY_HIP_MMQ_FP16") != nullptr;
-    if (!force_fp16 && mmq_i8_covers(w, qs)) return launch_mmq_i8(dev, w, qs, scales, m, y);
+    const bool big = !force_fp16 && mmq_f16_big_covers(w, m);
+    if (!force_fp16 && !big && mmq_i8_covers(w, qs)) return launch_mmq_i8(dev, w, qs, scales, m, y);
     CANDY_REQUIRE(half_ws, "internal: no workspace for the fp16 activations");
     const int64_t m_pad = mmq_m_pad(m);
     const int64_t runs = m_pad * (K >> 3);
@@ -306,6 +308,7 @@ int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *
                        m_pad, K, (half8 *)half_ws);
     CANDY_LAUNCH_CHECK();
     const _Float16 *xh = (const _Float16 *)half_ws;
+    if (big) return launch_mmq_f16_big(dev, w, xh, m, y);
     switch (w->fmt) {
     case CANDY_HIP_Q4_K: return launch_fmt<MmqQ4K>(dev, w, xh, m, y);
     case CANDY_HIP_Q8_0: return launch_fmt<MmqQ8_0>(dev, w, xh, m, y);

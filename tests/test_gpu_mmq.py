@@ -1,7 +1,8 @@
 """GPU parity of the batched (m >= 16) QMatMul, the MFMA tile kernels, against the CPU oracle.
-Bar: max|gpu - ref| / max|ref| <= 1e-3. The fp16 tile kernel (Q4_0, Q8_0) rounds its operands to
-fp16 and lands near 2e-4; the Q4_K / Q6_K kernel multiplies int8 on the matrix cores and differs
-from the oracle's integer dots only by f32 summation order, so it is held to 2e-5."""
+Bar: max|gpu - ref| / max|ref| <= 1e-3. The fp16 tile kernels (Q4_0, Q8_0, and Q4_K from 256
+activation rows up) round their operands to fp16 and land near 3e-4; the Q4_K / Q6_K int8 kernel
+multiplies integers on the matrix cores and differs from the oracle's integer dots only by f32
+summation order, so it is held to 2e-5."""
 import numpy as np
 import pytest
 
@@ -49,7 +50,23 @@ def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
     got = dev.qmatmul(dev.qtensor(fmt, rows, cols, w), x)
     want = o.qmatmul(fmt, w, rows, cols, x)
     assert got.shape == (m, rows)
-    assert rel_err(got, want) <= 2e-5
+    # Q4_K with 256 rows or more runs on the fp16 tiles (operands rounded to fp16)
+    assert rel_err(got, want) <= (5e-4 if (fmt == synth.Q4_K and m >= 256) else 2e-5)
+
+
+@pytest.mark.parametrize("m", [256, 257, 300, 512, 700])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (127, 512), (129, 1024), (300, 2304), (1030, 768)])
+def test_q4k_big_fp16_tiles(dev, m, rows, cols):
+    # rows off the 128-row tile, m off the 256-row tile, odd and even super-block counts
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=3 * rows + m)
+    x = synth.random_activations(m, cols, seed=cols + 7 * m)
+    got = dev.qmatmul(dev.qtensor(synth.Q4_K, rows, cols, w), x)
+    want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
+    assert got.shape == (m, rows)
+    assert rel_err(got, want) <= 5e-4  # observed 3e-4; a dropped block or a wrong scale costs far more
+    if rows >= 100:  # per activation row (a max over few outputs is no scale to measure against)
+        per_row = np.max(np.abs(got - want), axis=1) / np.max(np.abs(want), axis=1)
+        assert np.max(per_row) <= 2 * TOL
 
 
 @pytest.mark.parametrize("fmt,rows,cols", [(synth.Q8_0, 70, 96), (synth.Q4_0, 33, 160), (synth.Q8_0, 64, 32)])
