@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void k_mmq(const uint8_t *__restrict__ W, cons
     const int steps = K / BK;
 
     typename F::Raw raw[TPT];
-    uint4 xr[XPT];
+    u32x4 xr[XPT];
     auto gload = [&](int ks) {
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void k_mmq(const uint8_t *__restrict__ W, cons
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             const int c = min(tid + i * 256, XCH - 1), r = c / (BK / 8), kc = c % (BK / 8);
-            xr[i] = *(const uint4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BK + kc * 8);
+            xr[i] = *(const u32x4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BK + kc * 8);
         }
     };
     gload(0);
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void k_mmq(const uint8_t *__restrict__ W, cons
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             const int c = tid + i * 256;
-            if (XCH % 256 == 0 || c < XCH) *(uint4 *)&sB[(c / (BK / 8)) * LD + (c % (BK / 8)) * 8] = xr[i];
+            if (XCH % 256 == 0 || c < XCH) *(u32x4 *)&sB[(c / (BK / 8)) * LD + (c % (BK / 8)) * 8] = xr[i];
         }
         __syncthreads();
         if (ks + 1 < steps) gload(ks + 1);

@@ -158,15 +158,15 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_q4k_f16(const uint8_t *__r
             if (sb >= n_sb) break;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
+                // One straight-line block per step (loads past the end are clamped to valid addresses and
+                // the last step stages a buffer nobody reads).
                 const int ks = sb * 4 + g;
                 compute(g & 1);
-                if (ks + 1 < steps) {
-                    // (g + 1) & 1 is both the activation slot and the LDS buffer of step ks + 1
-                    if (g < 3) stage(g + 1, half, (g + 1) & 1, (g + 1) & 1);
-                    else stage(0, half ^ 1, 0, 0);
-                    if (ks + 3 < steps) gload_b(ks + 3, (g + 1) & 1);
-                }
-                if (g == 3 && sb + 2 < n_sb) gload_a(sb + 2, half);
+                // (g + 1) & 1 is both the activation slot and the LDS buffer of step ks + 1
+                if (g < 3) stage(g + 1, half, (g + 1) & 1, (g + 1) & 1);
+                else stage(0, half ^ 1, 0, 0);
+                gload_b(min(ks + 3, steps - 1), (g + 1) & 1);
+                if (g == 3) gload_a(min(sb + 2, n_sb - 1), half);
                 __syncthreads();
             }
         }
@@ -211,14 +211,7 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
 
 // xh: fp16 activations [mmq_m_pad(m)][K], rows past m zero.
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y) {
-    static const int variant = getenv("CANDY_HIP_MMQ_BIG_VARIANT") ? atoi(getenv("CANDY_HIP_MMQ_BIG_VARIANT")) : 0;
-    switch (variant) {
-    case 1: return launch_big<128, 256, 2, 2>(dev, w, xh, m, y);
-    case 2: return launch_big<128, 128, 2, 2>(dev, w, xh, m, y);
-    case 3: return launch_big<128, 128, 2, 4>(dev, w, xh, m, y);
-    case 4: return launch_big<256, 256, 2, 4>(dev, w, xh, m, y);
-    default: return launch_big<128, 256, 2, 4>(dev, w, xh, m, y);
-    }
+    return launch_big<128, 256, 2, 4>(dev, w, xh, m, y);
 }
 
 }  // namespace candy
