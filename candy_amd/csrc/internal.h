@@ -56,6 +56,9 @@ struct candy_hip_device {
     // Workspace for quantized activations (grown on demand, never shrunk).
     void *ws = nullptr;
     size_t ws_bytes = 0;
+    // Partial sums of the split-K tile kernel (same policy).
+    void *ws_split = nullptr;
+    size_t ws_split_bytes = 0;
 };
 
 struct candy_hip_qtensor {
@@ -96,6 +99,8 @@ namespace candy {
 int use_device(const candy_hip_device *dev);
 // Returns a workspace of at least `bytes` bytes (256-byte aligned).
 int workspace(candy_hip_device *dev, size_t bytes, void **out);
+// Second buffer, for the split-K partial sums (lives beside the activation workspace).
+int splitk_workspace(candy_hip_device *dev, size_t bytes, void **out);
 
 // quant.hip: x[rows, cols] -> planar int8 quants + scales; optionally also 34-byte blocks.
 int launch_quantize_q8(candy_hip_device *dev, const float *x, int64_t rows, int64_t cols,

@@ -1,24 +1,27 @@
-// Large-batch (m >= 256) Q4_K matmul on the fp16 matrix cores: y[m, N] = x[m, K] . W^T.
+// Prompt-sized batches (m >= 256) of Q4_K and Q6_K on the fp16 matrix cores: y[m, N] = x[m, K] . W^T.
 //
-// Replaces mul_mat_q / load_tiles_q4_K (tensor/internal/cuda/kernels/quantized.cu:455-578,
-// :4116-4205) for prompt-sized batches.  With hundreds of activation rows the contraction is a dense
-// GEMM, and the per-sub-block rescale that keeps the integer kernel exact costs several times the
-// matrix-core time; here the scales are folded into the operands instead:
-//   * weights are dequantized exactly as dequantize_block_q4_K does (quantized.cu:1008-1041:
-//     (d*sc)*q - dmin*m, evaluated in f32) and rounded once to fp16;
+// Replaces mul_mat_q / load_tiles_q4_K / load_tiles_q6_K (tensor/internal/cuda/kernels/quantized.cu
+// :455-578, :4116-4205) for prompt-sized batches.  With hundreds of activation rows the contraction
+// is a dense GEMM, and the per-sub-block rescale that keeps the integer kernel exact costs several
+// times the matrix-core time; here the scales are folded into the operands instead:
+//   * weights are dequantized exactly as dequantize_block_q4_K / dequantize_block_q6_K do
+//     (quantized.cu:1008-1041: (d*sc)*q - dmin*m; :1103-1128: d*sc*(q-32); evaluated in f32) and
+//     rounded once to fp16;
 //   * activations are the Q8_0 values d_x * q_x (exact in f32) rounded once to fp16;
 //   * products accumulate in f32 (v_mfma_f32_16x16x32_f16).
 // Both roundings are 2^-12 relative per element; the result stays a few 1e-4 (max-norm) from the
 // CPU contraction, inside the 1e-3 bar.
 //
-// Tiling: a workgroup owns BN weight rows x BM activation rows and walks K in steps of 64 (one
-// 32-byte nibble group of a super-block = two sub-blocks).  Every thread dequantizes 16 weights per
-// step (8 bytes of nibbles: 8 low + 8 high) into an LDS tile, the fp16 activations go into a second
-// LDS tile, both double-buffered so one barrier per step suffices, and the next step's global
-// loads are issued before the current step's MFMAs.  Each wavefront owns a (BN/WN) x (BM/WM)
-// sub-tile; LDS rows are padded to 144 bytes so that the 16-byte operand reads of a wavefront
-// spread over all banks.  Workgroups are numbered so that those sharing an XCD (and its L2) work
-// on neighbouring weight tiles of the same activation tile.
+// Tiling: a workgroup owns 128 weight rows x 256 activation rows and walks K in steps of 64.  Every
+// thread dequantizes 16 weights per step into an LDS tile, the fp16 activations go into a second
+// LDS tile, both double-buffered so one barrier per step suffices.  Global requests run ahead in
+// registers: a thread's share of a whole super-block of weights four steps ahead (HBM), the
+// activations two steps ahead (L2).  Each of the 8 wavefronts owns a 64 x 64 sub-tile; LDS rows are
+// padded to 144 bytes so that the 16-byte operand reads of a wavefront spread over all banks.
+// Workgroups are numbered so that those sharing an XCD (and its L2) work on neighbouring weight
+// tiles of the same activation tile.  When the output has too few tiles to fill the chip
+// (N = 4096 or 1024 projections), K is split over several workgroups per tile; their partial sums
+// go to a scratch buffer and a second kernel adds them in a fixed order (bitwise reproducible).
 #include <cstdlib>
 
 #include "blocks.h"
@@ -32,14 +35,91 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int BIG_BK = 64;
 constexpr int BIG_PITCH = BIG_BK + 8;  // halves per LDS row (144 bytes)
 
-template <int BN, int BM, int WN, int WM>
-__global__ __launch_bounds__(WN * WM * 64) void k_mmq_q4k_f16(const uint8_t *__restrict__ W,
-                                                              const _Float16 *__restrict__ xh,
-                                                              float *__restrict__ y, int N, int M, int K, int n_tiles,
-                                                              int m_tiles) {
+// ------------------------------------------------------------------ per-format policies
+// A task is (row, quarter c in 0..3) of one 64-wide step g in 0..3 of a super-block: 16 weights.
+//   load():    the task's bytes of a whole super-block -> registers (requested four steps ahead)
+//   dequant(): step g's 16 weights as two 8-value chunks and their positions (in halves) in the
+//              64-wide LDS row
+
+struct BigQ4K {
+    static constexpr int BLOCK = 144;
+    struct Raw { u32x4 hdr; u32x2 q[4]; };  // header + bytes 8c..8c+7 of each 32-byte nibble group
+    __device__ static __forceinline__ void load(const uint8_t *blk, int c, Raw &r) {
+        r.hdr = *(const u32x4 *)blk;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) r.q[g] = *(const u32x2 *)(blk + 16 + g * 32 + c * 8);
+    }
+    // group g holds sub-blocks 2g (low nibbles, k = 0..31 of the step) and 2g+1 (high nibbles, k = 32..63)
+    __device__ static __forceinline__ void dequant(const Raw &r, int g, int c, half8 &o0, half8 &o1, int &k0, int &k1) {
+        uint32_t sc2, m2;
+        q4k_scale_min_pair(r.hdr.y, r.hdr.z, r.hdr.w, g, sc2, m2);
+        const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
+        const float d_lo = d * (float)(sc2 & 0xFF), d_hi = d * (float)((sc2 >> 8) & 0xFF);
+        const float m_lo = dmin * (float)(m2 & 0xFF), m_hi = dmin * (float)((m2 >> 8) & 0xFF);
+        const u32x2 q = r.q[g];
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+            const uint32_t byte = ((l < 4 ? q.x : q.y) >> (8 * (l & 3))) & 0xFF;
+            o0[l] = (_Float16)(d_lo * (float)(byte & 0xF) - m_lo);
+            o1[l] = (_Float16)(d_hi * (float)(byte >> 4) - m_hi);
+        }
+        k0 = c * 8;
+        k1 = 32 + c * 8;
+    }
+};
+
+struct BigQ6K {
+    static constexpr int BLOCK = 210;
+    // per half ip: ql bytes 64ip+16c..+15 (low nibbles: quarters 0/1, high nibbles: quarters 2/3) and qh bytes
+    // 32ip+16(c&1)..+15; the four scales of this quarter-column (8ip + 4p + c) packed in one word; d
+    struct Raw { u32x4 ql[2], qh[2]; uint32_t sc4; uint32_t d; };
+    __device__ static __forceinline__ void load(const uint8_t *blk, int c, Raw &r) {
+#pragma unroll
+        for (int ip = 0; ip < 2; ++ip) {
+            r.ql[ip] = *(const u32x4_a2 *)(blk + 64 * ip + 16 * c);
+            r.qh[ip] = *(const u32x4_a2 *)(blk + 128 + 32 * ip + 16 * (c & 1));
+        }
+        const uint8_t *sc = blk + 192 + c;
+        r.sc4 = (uint32_t)sc[0] | ((uint32_t)sc[4] << 8) | ((uint32_t)sc[8] << 16) | ((uint32_t)sc[12] << 24);
+        r.d = *(const uint16_t *)(blk + 208);
+    }
+    // step g = 2*ip + p covers k = 128ip + 64p .. +63: quarters 2p and 2p+1 of half ip; this task owns
+    // values 16c..16c+15 of the step, i.e. quarter 2p + (c>>1), il = 16(c&1)..+15, one scale
+    __device__ static __forceinline__ void dequant(const Raw &r, int g, int c, half8 &o0, half8 &o1, int &k0, int &k1) {
+        const int ip = g >> 1, p = g & 1;
+        const int shift = 2 * (2 * p + (c >> 1));
+        const float dsc = half_bits_to_float((uint16_t)r.d) * (float)(int)(int8_t)((r.sc4 >> (8 * g)) & 0xFF);
+        const float off = -32.0f * dsc;
+        const uint32_t qlw[4] = {r.ql[ip].x, r.ql[ip].y, r.ql[ip].z, r.ql[ip].w};
+        const uint32_t qhw[4] = {r.qh[ip].x, r.qh[ip].y, r.qh[ip].z, r.qh[ip].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo4 = (qlw[j] >> (4 * p)) & 0x0F0F0F0Fu;
+            const uint32_t hi2 = ((qhw[j] >> shift) & 0x03030303u) << 4;
+            const uint32_t q = lo4 | hi2;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const _Float16 v = (_Float16)(dsc * (float)((q >> (8 * b)) & 0xFF) + off);  // = d*sc*(q-32), exact in f32
+                if (j < 2) o0[4 * j + b] = v;
+                else o1[4 * (j - 2) + b] = v;
+            }
+        }
+        k0 = 16 * c;
+        k1 = 16 * c + 8;
+    }
+};
+
+// ------------------------------------------------------------------ tile kernel
+// grid = tiles * n_split; workgroup (tile, split) contracts super-blocks [split*sb_per, ...) and writes
+// its tile to out + split * M * N (out = y when n_split == 1).
+template <class F, int BN, int BM, int WN, int WM>
+__global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xh,
+                                                          float *__restrict__ out, int N, int M, int K, int n_tiles,
+                                                          int m_tiles, int sb_per) {
     constexpr int T = WN * WM * 64;
     constexpr int TN = BN / WN / 16, TM = BM / WM / 16;
-    constexpr int ATK = BN * 4 / T;   // quarter-row dequantization tasks per thread per step
+    constexpr int ATK = BN * 4 / T;   // dequantization tasks per thread per step
     constexpr int BCH = BM * 8 / T;   // 16-byte activation chunks per thread per step
     static_assert(BN * 4 % T == 0 && BM * 8 % T == 0 && TN >= 1 && TM >= 1, "tile shape");
     extern __shared__ __align__(16) uint8_t smem_raw[];
@@ -51,30 +131,28 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_q4k_f16(const uint8_t *__r
 
     // tile numbering: the hardware deals workgroups round-robin to the 8 XCDs; give each XCD a
     // contiguous run of weight tiles inside one activation tile
-    int v = blockIdx.x;
     const int total = n_tiles * m_tiles;
-    if ((total & 7) == 0) v = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+    const int split = blockIdx.x / total;
+    int v = blockIdx.x - split * total;
+    if ((total & 7) == 0) v = (v & 7) * (total >> 3) + (v >> 3);
     const int mt = v / n_tiles, nt = v - mt * n_tiles;
     const int n0 = nt * BN, m0 = mt * BM;
 
-    const size_t rb = (size_t)(K >> 8) * 144;
-    const int steps = K / BIG_BK;
+    const size_t rb = (size_t)(K >> 8) * F::BLOCK;
+    const int sb0 = split * sb_per;
+    const int n_sb = min(K >> 8, sb0 + sb_per) - sb0;  // >= 1 by construction of the grid
+    const int steps = n_sb * 4;
+    W += (size_t)sb0 * F::BLOCK;
+    xh += (size_t)sb0 * 256;
+    out += (size_t)split * M * N;
 
-    // Register pipeline.  Weights: the 16-byte header and this thread's four 8-byte nibble runs (one per
-    // 64-value group) of a whole super-block are requested one super-block (four steps) ahead, far
-    // enough for HBM.  Activations (L2-resident): requested two steps ahead.
-    // Task (row, quarter c) of step g dequantizes bytes 8c..8c+7 of group g: 8 low + 8 high nibbles.
-    u32x4 hdr[2][ATK];
-    u32x2 qs[2][ATK][4];
+    typename F::Raw raw[2][ATK];
     u32x4 xr[2][BCH];
     auto gload_a = [&](int sb, int slot) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < ATK; ++i) {
             const int task = tid + i * T, row = task >> 2, c = task & 3;
-            const uint8_t *blk = W + (size_t)min(n0 + row, N - 1) * rb + (size_t)sb * 144;
-            hdr[slot][i] = *(const u32x4 *)blk;
-#pragma unroll
-            for (int g = 0; g < 4; ++g) qs[slot][i][g] = *(const u32x2 *)(blk + 16 + g * 32 + c * 8);
+            F::load(W + (size_t)min(n0 + row, N - 1) * rb + (size_t)sb * F::BLOCK, c, raw[slot][i]);
         }
     };
     auto gload_b = [&](int ks, int slot) __attribute__((always_inline)) {
@@ -90,23 +168,11 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_q4k_f16(const uint8_t *__r
 #pragma unroll
         for (int i = 0; i < ATK; ++i) {
             const int task = tid + i * T, row = task >> 2, c = task & 3;
-            const u32x4 h = hdr[aslot][i];
-            const u32x2 q = qs[aslot][i][g];
-            uint32_t sc2, m2;
-            q4k_scale_min_pair(h.y, h.z, h.w, g, sc2, m2);
-            const float d = half_bits_to_float((uint16_t)(h.x & 0xFFFF));
-            const float dmin = half_bits_to_float((uint16_t)(h.x >> 16));
-            const float d_lo = d * (float)(sc2 & 0xFF), d_hi = d * (float)((sc2 >> 8) & 0xFF);
-            const float m_lo = dmin * (float)(m2 & 0xFF), m_hi = dmin * (float)((m2 >> 8) & 0xFF);
-            half8 lo, hi;
-#pragma unroll
-            for (int l = 0; l < 8; ++l) {
-                const uint32_t byte = ((l < 4 ? q.x : q.y) >> (8 * (l & 3))) & 0xFF;
-                lo[l] = (_Float16)(d_lo * (float)(byte & 0xF) - m_lo);
-                hi[l] = (_Float16)(d_hi * (float)(byte >> 4) - m_hi);
-            }
-            *(half8 *)&a[row * BIG_PITCH + c * 8] = lo;
-            *(half8 *)&a[row * BIG_PITCH + 32 + c * 8] = hi;
+            half8 o0, o1;
+            int k0, k1;
+            F::dequant(raw[aslot][i], g, c, o0, o1, k0, k1);
+            *(half8 *)&a[row * BIG_PITCH + k0] = o0;
+            *(half8 *)&a[row * BIG_PITCH + k1] = o1;
         }
 #pragma unroll
         for (int i = 0; i < BCH; ++i) {
@@ -143,11 +209,10 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_q4k_f16(const uint8_t *__r
     // other buffer.  Staging step 4*sb+4 (g == 3) is the first use of super-block sb+1, which was
     // requested when super-block sb was first used.  Super-blocks alternate between the two register
     // slots, so the loop body covers two of them.
-    const int n_sb = K >> 8;
     gload_a(0, 0);
     gload_b(0, 0);
     gload_b(1, 1);
-    if (n_sb > 1) gload_a(1, 1);
+    gload_a(min(1, n_sb - 1), 1);
     stage(0, 0, 0, 0);
     gload_b(2, 0);
     __syncthreads();
@@ -180,7 +245,7 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_q4k_f16(const uint8_t *__r
             const int m = m0 + wm * (BM / WM) + tm * 16 + (lane & 15);
             const int n = n0 + wn * (BN / WN) + tn * 16 + 4 * (lane >> 4);
             if (m >= M) continue;
-            float *dst = y + (size_t)m * N + n;
+            float *dst = out + (size_t)m * N + n;
             if (n + 3 < N && (N & 3) == 0) {
                 *(float4 *)dst = make_float4(acc[tn][tm][0], acc[tn][tm][1], acc[tn][tm][2], acc[tn][tm][3]);
             } else {
@@ -191,27 +256,75 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_q4k_f16(const uint8_t *__r
         }
 }
 
-template <int BN, int BM, int WN, int WM>
+// y[i] = part[0][i] + part[1][i] + ... in that order
+__global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ part, float *__restrict__ y, size_t count,
+                                                    int n_split) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= count) return;
+    if (i + 4 <= count && ((uintptr_t)y & 15) == 0 && (count & 3) == 0) {
+        float4 s = *(const float4 *)(part + i);
+        for (int k = 1; k < n_split; ++k) {
+            const float4 v = *(const float4 *)(part + (size_t)k * count + i);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        *(float4 *)(y + i) = s;
+    } else {
+        for (size_t j = i; j < i + 4 && j < count; ++j) {
+            float s = part[j];
+            for (int k = 1; k < n_split; ++k) s += part[(size_t)k * count + j];
+            y[j] = s;
+        }
+    }
+}
+
+template <class F, int BN, int BM, int WN, int WM>
 static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y) {
     const int N = (int)w->rows, K = (int)w->cols;
     const int n_tiles = (N + BN - 1) / BN, m_tiles = (int)((m + BM - 1) / BM);
+    const int tiles = n_tiles * m_tiles, n_sb = K >> 8;
+    // split K until the grid covers the chip, keeping at least two super-blocks (8 steps) per workgroup
+    int n_split = 1;
+    if (tiles < (3 * dev->num_cus) / 4) {
+        n_split = (dev->num_cus + tiles - 1) / tiles;
+        if (n_split > n_sb / 2) n_split = n_sb / 2;
+        if (n_split > 16) n_split = 16;
+        if (n_split < 1) n_split = 1;
+    }
+    const int sb_per = (n_sb + n_split - 1) / n_split;
+    n_split = (n_sb + sb_per - 1) / sb_per;  // no empty splits
+    float *out = y;
+    if (n_split > 1) {
+        void *p = nullptr;
+        if (int rc = splitk_workspace(dev, (size_t)n_split * (size_t)m * N * sizeof(float), &p)) return rc;
+        out = (float *)p;
+    }
     constexpr size_t smem = (size_t)2 * (BN + BM) * BIG_PITCH * sizeof(_Float16);
-    CANDY_HIP_TRY(hipFuncSetAttribute((const void *)k_mmq_q4k_f16<BN, BM, WN, WM>,
+    CANDY_HIP_TRY(hipFuncSetAttribute((const void *)k_mmq_f16<F, BN, BM, WN, WM>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL((k_mmq_q4k_f16<BN, BM, WN, WM>), dim3((unsigned)(n_tiles * m_tiles)), dim3(WN * WM * 64), smem,
-                       dev->stream, (const uint8_t *)w->data, xh, y, N, (int)m, K, n_tiles, m_tiles);
+    hipLaunchKernelGGL((k_mmq_f16<F, BN, BM, WN, WM>), dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem,
+                       dev->stream, (const uint8_t *)w->data, xh, out, N, (int)m, K, n_tiles, m_tiles, sb_per);
     CANDY_LAUNCH_CHECK();
+    if (n_split > 1) {
+        const size_t count = (size_t)m * N;
+        hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((count / 4 + 256) / 256)), dim3(256), 0, dev->stream, out, y, count,
+                           n_split);
+        CANDY_LAUNCH_CHECK();
+    }
     return CANDY_HIP_OK;
 }
 
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
     static const int min_m = getenv("CANDY_HIP_MMQ_BIG_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_BIG_MIN_M")) : 256;
-    return w->fmt == CANDY_HIP_Q4_K && m >= min_m && w->cols % 256 == 0 && ((uintptr_t)w->data & 15) == 0;
+    if (m < min_m || w->cols % 256 != 0) return false;
+    if (w->fmt == CANDY_HIP_Q4_K) return ((uintptr_t)w->data & 15) == 0;
+    if (w->fmt == CANDY_HIP_Q6_K) return ((uintptr_t)w->data & 1) == 0;
+    return false;
 }
 
 // xh: fp16 activations [mmq_m_pad(m)][K], rows past m zero.
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y) {
-    return launch_big<128, 256, 2, 4>(dev, w, xh, m, y);
+    if (w->fmt == CANDY_HIP_Q6_K) return launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y);
+    return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y);
 }
 
 }  // namespace candy

@@ -60,6 +60,20 @@ int workspace(candy_hip_device *dev, size_t bytes, void **out) {
     return CANDY_HIP_OK;
 }
 
+int splitk_workspace(candy_hip_device *dev, size_t bytes, void **out) {
+    if (bytes > dev->ws_split_bytes) {
+        CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
+        if (dev->ws_split) CANDY_HIP_TRY(hipFree(dev->ws_split));
+        dev->ws_split = nullptr;
+        dev->ws_split_bytes = 0;
+        size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        CANDY_HIP_TRY(hipMalloc(&dev->ws_split, want));
+        dev->ws_split_bytes = want;
+    }
+    *out = dev->ws_split;
+    return CANDY_HIP_OK;
+}
+
 __global__ __launch_bounds__(256) void k_zero_bytes(uint8_t *p, size_t bytes) {
     // 16 bytes per thread where aligned, byte stores for the ragged head and tail
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 16;
@@ -135,6 +149,7 @@ int candy_hip_close(candy_hip_device *dev) {
     (void)hipSetDevice(dev->ordinal);
     if (dev->stream) (void)hipStreamSynchronize(dev->stream);
     if (dev->ws) (void)hipFree(dev->ws);
+    if (dev->ws_split) (void)hipFree(dev->ws_split);
     if (dev->ev_start) (void)hipEventDestroy(dev->ev_start);
     if (dev->ev_stop) (void)hipEventDestroy(dev->ev_stop);
     if (dev->stream) (void)hipStreamDestroy(dev->stream);

@@ -50,18 +50,20 @@ def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
     got = dev.qmatmul(dev.qtensor(fmt, rows, cols, w), x)
     want = o.qmatmul(fmt, w, rows, cols, x)
     assert got.shape == (m, rows)
-    # Q4_K with 256 rows or more runs on the fp16 tiles (operands rounded to fp16)
-    assert rel_err(got, want) <= (5e-4 if (fmt == synth.Q4_K and m >= 256) else 2e-5)
+    # 256 activation rows or more run on the fp16 tiles (operands rounded to fp16)
+    assert rel_err(got, want) <= (5e-4 if m >= 256 else 2e-5)
 
 
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K])
 @pytest.mark.parametrize("m", [256, 257, 300, 512, 700])
-@pytest.mark.parametrize("rows,cols", [(1, 256), (127, 512), (129, 1024), (300, 2304), (1030, 768)])
-def test_q4k_big_fp16_tiles(dev, m, rows, cols):
-    # rows off the 128-row tile, m off the 256-row tile, odd and even super-block counts
-    w = synth.random_weight(synth.Q4_K, rows, cols, seed=3 * rows + m)
+@pytest.mark.parametrize("rows,cols", [(1, 256), (127, 512), (129, 1024), (300, 2304), (1030, 768), (130, 4352)])
+def test_big_fp16_tiles(dev, fmt, m, rows, cols):
+    # rows off the 128-row tile, m off the 256-row tile, odd and even super-block counts; the few-tile
+    # shapes split K over several workgroups (17 super-blocks: uneven splits)
+    w = synth.random_weight(fmt, rows, cols, seed=3 * rows + m)
     x = synth.random_activations(m, cols, seed=cols + 7 * m)
-    got = dev.qmatmul(dev.qtensor(synth.Q4_K, rows, cols, w), x)
-    want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
+    got = dev.qmatmul(dev.qtensor(fmt, rows, cols, w), x)
+    want = o.qmatmul(fmt, w, rows, cols, x)
     assert got.shape == (m, rows)
     assert rel_err(got, want) <= 5e-4  # observed 3e-4; a dropped block or a wrong scale costs far more
     if rows >= 100:  # per activation row (a max over few outputs is no scale to measure against)
@@ -99,12 +101,16 @@ def test_config_prefill_q4k_14336x4096(dev, m):
         assert rel_err(got[r:r + 1], dev.qmatmul(q, x[r:r + 1])) <= TOL
 
 
-def test_mixed_format_prefill_q6k_down_proj(dev):
-    rows, cols, m = 4096, 14336, 64
+@pytest.mark.parametrize("m", [64, 512])
+def test_mixed_format_prefill_q6k_down_proj(dev, m):
+    rows, cols = 4096, 14336
     w = synth.random_weight(synth.Q6_K, rows, cols, seed=5)
     x = synth.random_activations(m, cols, seed=6)
-    got = dev.qmatmul(dev.qtensor(synth.Q6_K, rows, cols, w), x)
+    q = dev.qtensor(synth.Q6_K, rows, cols, w)
+    got = dev.qmatmul(q, x)
     sub = np.arange(0, rows, 128)
     rb = synth.weight_nbytes(synth.Q6_K, 1, cols)
     want = o.qmatmul(synth.Q6_K, w.reshape(rows, rb)[sub].reshape(-1), len(sub), cols, x)
     assert rel_err(got[:, sub], want) <= TOL
+    # split-K partial sums are added in a fixed order: the same call gives the same bits
+    assert np.array_equal(got, dev.qmatmul(q, x))
