@@ -344,15 +344,17 @@ def main():
         out["conversions"] = conv
 
     if not args.no_prefill:
-        # batched prefill: Q4_K 14336x4096 x f32 [M, 4096] on the int8 matrix cores; mfma_frac is quoted against
-        # the dense fp16 peak (2.5 PFLOP/s), the int8 peak is twice that
+        # batched prefill: Q4_K 14336x4096 x f32 [M, 4096], f32 in -> f32 out (activation quantization included).
+        # m < 256 runs on the int8 matrix cores (exact integer dots), m >= 256 on fp16 tiles; mfma_frac is quoted
+        # against the dense fp16 peak (2.5 PFLOP/s) for both (the int8 peak is twice that)
         pre = []
         r, k = 14336, 4096
         for m in (16, 128, 512):
             ms, _ = time_matvec(dev, synth.Q4_K, r, k, 200, 20, quantize_each=True, seed=m, m=m)
             flops = 2.0 * m * r * k
             byts = algorithmic_bytes(synth.Q4_K, r, k, m)
-            pre.append({"m": m, "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
+            pre.append({"m": m, "kernel": "k_mmq_q4k_i8 (int8 MFMA)" if m < 256 else "k_mmq_f16<BigQ4K> (fp16 MFMA)",
+                        "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
                         "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
             log(f"  prefill q4_k {r}x{k} M={m}: {ms * 1e3:.1f} us, {pre[-1]['TFLOPs']} TFLOP/s, {pre[-1]['GBps']} GB/s")
