@@ -120,6 +120,17 @@ __device__ __forceinline__ uint32_t quantize_q8_lane4(float4 v, __half &d_half, 
            ((uint32_t)(q3 & 0xFF) << 24);
 }
 
+// The 4 quantized values of a lane as fp16(d * q): what the fp16 tile kernels contract with
+// (d = the fp16-rounded block scale widened to f32; the product is exact in f32, one rounding).
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half4v q8_lane4_to_half(uint32_t packed, __half d_half) {
+    const float d = __half2float(d_half);
+    half4v r;
+#pragma unroll
+    for (int l = 0; l < 4; ++l) r[l] = (_Float16)(d * (float)(int8_t)((packed >> (8 * l)) & 0xFF));
+    return r;
+}
+
 // Same quantization with one value per lane: the 32 lanes of a block are consecutive lanes
 // (lane % 32 == position in the block), all active.
 __device__ __forceinline__ int quantize_q8_lane1(float v, __half &d_half, int &bsum) {

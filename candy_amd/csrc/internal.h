@@ -103,8 +103,9 @@ int workspace(candy_hip_device *dev, size_t bytes, void **out);
 int splitk_workspace(candy_hip_device *dev, size_t bytes, void **out);
 
 // quant.hip: x[rows, cols] -> planar int8 quants + scales; optionally also 34-byte blocks.
+// xh (optional): also the fp16 values d * q, row-major like x (what the fp16 tile kernels contract with).
 int launch_quantize_q8(candy_hip_device *dev, const float *x, int64_t rows, int64_t cols,
-                       int8_t *qs, Q8Scale *scales, void *blocks);
+                       int8_t *qs, Q8Scale *scales, void *blocks, _Float16 *xh = nullptr);
 // quant.hip: Q8_0 blocks -> planar form.
 int launch_q8_blocks_to_planar(candy_hip_device *dev, const void *blocks, int64_t n_blocks,
                                int8_t *qs, Q8Scale *scales);
@@ -116,20 +117,26 @@ int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *w
                         const float *const *res, int n, const int8_t *qs, const Q8Scale *scales);
 // mmq.hip: MFMA tile kernel for m >= 16. half_ws: mmq_m_pad(m) * cols fp16 values of scratch.
 int64_t mmq_m_pad(int64_t m);
+// Whether launch_mmq / launch_contract add `res` in the contraction's own epilogue (then res may alias y).
+bool mmq_fuses_residual(const candy_hip_qtensor *w, int64_t m);
+// xh_ready (optional): the activations already expanded to fp16 [>= mmq_m_pad(m) rows][cols] (rows past m
+// may hold anything); res (optional, may alias y): y = res + x . W^T.
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
-               const Q8Scale *scales, int64_t m, float *y, void *half_ws);
+               const Q8Scale *scales, int64_t m, float *y, void *half_ws, const _Float16 *xh_ready = nullptr,
+               const float *res = nullptr);
 // mmq_i8.hip: Q4_K / Q6_K on v_mfma_i32_16x16x32_i8 with the batch-1 kernels' integer arithmetic.
 bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs);
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                   const Q8Scale *scales, int64_t m, float *y);
 // mmq_f16.hip: Q4_K with prompt-sized batches on big fp16 tiles. xh: fp16 activations [mmq_m_pad(m)][K].
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m);
-int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y);
+int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
+                       const float *res = nullptr);
 // ops.hip: fused decode-step stages (all enqueue on dev->stream, no allocation, no sync).
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
-                          int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales);
+                          int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales, _Float16 *xh = nullptr);
 int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *act_out,
-                          int8_t *qs, Q8Scale *scales);
+                          int8_t *qs, Q8Scale *scales, _Float16 *xh = nullptr);
 // fused.hip: batch-1 contraction of one activation row with up to three weights, with optional
 // RMSNorm+quantize prologue (x != nullptr, else planar Q8_0 in xq/xs), residuals, or the
 // gate/up SiLU*Mul+quantize epilogue (pair). Returns CANDY_HIP_ERR_UNSUPPORTED when the shape
@@ -183,7 +190,7 @@ int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quan
 // workspace (the tile kernel may carve its fp16 scratch from it).
 int mmq_min_m();
 int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                    int64_t m, float *y);
+                    int64_t m, float *y, const _Float16 *xh_ready = nullptr, const float *res = nullptr);
 // prefill.hip: prompt stages of the decoder (n tokens at positions pos0 ..).
 int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, const float *v, const float *cos_t,
                            const float *sin_t, float *k_cache, float *v_cache, int n, int pos0, int n_heads,

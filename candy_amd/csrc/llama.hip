@@ -46,6 +46,7 @@ struct candy_hip_llama {
         float *gate = nullptr, *up = nullptr;
         int8_t *xq = nullptr;
         candy::Q8Scale *xs = nullptr;
+        _Float16 *xh = nullptr;  // the quantized activations as fp16 (d * q), for the fp16 tile kernels
         std::vector<void *> owned;
     } pf;
 };
@@ -376,6 +377,7 @@ static int prompt_reserve(candy_hip_llama *m, int n) {
     if (!rc) rc = prompt_alloc(m, &P.up, N * c.d_ffn);
     if (!rc) rc = prompt_alloc(m, &P.xq, N * widest);
     if (!rc) rc = prompt_alloc(m, &P.xs, N * (widest / 32));
+    if (!rc) rc = prompt_alloc(m, &P.xh, (size_t)mmq_m_pad(n) * widest);  // the tile kernel reads whole tiles of rows
     if (rc) return rc;
     P.cap = n;
     return CANDY_HIP_OK;
@@ -397,25 +399,35 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
     for (int l = 0; l < c.n_layers; ++l) {
         const candy_hip_llama::Layer &L = m->layers[l];
         float *kc = m->k_cache + (size_t)l * layer_kv, *vc = m->v_cache + (size_t)l * layer_kv;
-        if ((rc = launch_rms_norm_quant(dev, P.h, L.attn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs))) return rc;
-        if ((rc = launch_contract(dev, L.wq, P.xq, P.xs, n, P.q))) return rc;
-        if ((rc = launch_contract(dev, L.wk, P.xq, P.xs, n, P.k))) return rc;
-        if ((rc = launch_contract(dev, L.wv, P.xq, P.xs, n, P.v))) return rc;
+        // Where a projection runs on the fp16 tiles, the kernel that quantizes its input also writes the
+        // fp16 expansion (one conversion for q/k/v, one for gate/up), and the residual add rides in the
+        // projection's epilogue.
+        auto xh_for = [&](const candy_hip_qtensor *w) { return mmq_f16_big_covers(w, n) ? P.xh : nullptr; };
+        auto add_linear = [&](const candy_hip_qtensor *w) -> int {  // P.h += (quantized activations) . w^T
+            if (mmq_fuses_residual(w, n)) return launch_contract(dev, w, P.xq, P.xs, n, P.h, xh_for(w), P.h);
+            if (int e = launch_contract(dev, w, P.xq, P.xs, n, P.tmp)) return e;
+            return candy_hip_add(dev, P.h, P.tmp, (int64_t)n * c.d_model, P.h);
+        };
+        _Float16 *xh = (xh_for(L.wq) || xh_for(L.wk) || xh_for(L.wv)) ? P.xh : nullptr;
+        if ((rc = launch_rms_norm_quant(dev, P.h, L.attn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs, xh))) return rc;
+        if ((rc = launch_contract(dev, L.wq, P.xq, P.xs, n, P.q, xh_for(L.wq)))) return rc;
+        if ((rc = launch_contract(dev, L.wk, P.xq, P.xs, n, P.k, xh_for(L.wk)))) return rc;
+        if ((rc = launch_contract(dev, L.wv, P.xq, P.xs, n, P.v, xh_for(L.wv)))) return rc;
         if ((rc = launch_prefill_rope_kv(dev, P.q, P.k, P.v, m->cos_t, m->sin_t, kc, vc, n, pos0, c.n_heads,
                                          c.n_kv_heads, c.head_dim, cache_stride)))
             return rc;
         if ((rc = launch_attn_prefill(dev, P.q, kc, vc, P.att, n, pos0, c.n_heads, c.n_kv_heads, c.head_dim,
                                       cache_stride, scale)))
             return rc;
-        if ((rc = launch_quantize_q8(dev, P.att, n, qd, P.xq, P.xs, nullptr))) return rc;
-        if ((rc = launch_contract(dev, L.wo, P.xq, P.xs, n, P.tmp))) return rc;
-        if ((rc = candy_hip_add(dev, P.h, P.tmp, (int64_t)n * c.d_model, P.h))) return rc;
-        if ((rc = launch_rms_norm_quant(dev, P.h, L.ffn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs))) return rc;
-        if ((rc = launch_contract(dev, L.gate, P.xq, P.xs, n, P.gate))) return rc;
-        if ((rc = launch_contract(dev, L.up, P.xq, P.xs, n, P.up))) return rc;
-        if ((rc = launch_silu_mul_quant(dev, P.gate, P.up, (int64_t)n * c.d_ffn, nullptr, P.xq, P.xs))) return rc;
-        if ((rc = launch_contract(dev, L.down, P.xq, P.xs, n, P.tmp))) return rc;
-        if ((rc = candy_hip_add(dev, P.h, P.tmp, (int64_t)n * c.d_model, P.h))) return rc;
+        if ((rc = launch_quantize_q8(dev, P.att, n, qd, P.xq, P.xs, nullptr, xh_for(L.wo)))) return rc;
+        if ((rc = add_linear(L.wo))) return rc;  // h += Wo . att
+        xh = (xh_for(L.gate) || xh_for(L.up)) ? P.xh : nullptr;
+        if ((rc = launch_rms_norm_quant(dev, P.h, L.ffn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs, xh))) return rc;
+        if ((rc = launch_contract(dev, L.gate, P.xq, P.xs, n, P.gate, xh_for(L.gate)))) return rc;
+        if ((rc = launch_contract(dev, L.up, P.xq, P.xs, n, P.up, xh_for(L.up)))) return rc;
+        if ((rc = launch_silu_mul_quant(dev, P.gate, P.up, (int64_t)n * c.d_ffn, nullptr, P.xq, P.xs, xh_for(L.down))))
+            return rc;
+        if ((rc = add_linear(L.down))) return rc;  // h += Wdown . act
     }
     if ((rc = candy_hip_d2d(dev, m->h, P.h + (size_t)(n - 1) * c.d_model, (size_t)c.d_model * sizeof(float)))) return rc;
     const candy_hip_qtensor *ws[1] = {m->head};

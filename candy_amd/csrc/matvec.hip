@@ -432,11 +432,15 @@ int mmq_min_m() {
 }
 
 int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                    int64_t m, float *y) {
-    if (m < mmq_min_m()) return launch_matvec(dev, w, qs, scales, m, y);
+                    int64_t m, float *y, const _Float16 *xh_ready, const float *res) {
+    if (m < mmq_min_m()) {
+        CANDY_REQUIRE(res != y, "internal: in-place residual needs the fused epilogue");
+        if (int rc = launch_matvec(dev, w, qs, scales, m, y)) return rc;
+        return res ? candy_hip_add(dev, res, y, m * w->rows, y) : CANDY_HIP_OK;
+    }
     ActWorkspace extra;
     if (int rc = act_workspace(dev, m, w->cols, false, &extra)) return rc;
-    return launch_mmq(dev, w, qs, scales, m, y, extra.half_ws);
+    return launch_mmq(dev, w, qs, scales, m, y, extra.half_ws, xh_ready, res);
 }
 
 }  // namespace candy

@@ -291,16 +291,41 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const _
 
 int64_t mmq_m_pad(int64_t m) { return (m + 255) / 256 * 256; }  // a multiple of every tile height
 
+static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                        int64_t m, float *y, void *half_ws, const _Float16 *xh_ready, const float *res, bool *res_done);
+
+static bool force_old_fp16() {
+    static const bool v = getenv("CANDY_HIP_MMQ_FP16") != nullptr;
+    return v;
+}
+
+bool mmq_fuses_residual(const candy_hip_qtensor *w, int64_t m) {
+    return m >= mmq_min_m() && w->cols % 64 == 0 && !force_old_fp16() && mmq_f16_big_covers(w, m);
+}
+
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int64_t m,
-               float *y, void *half_ws) {
+               float *y, void *half_ws, const _Float16 *xh_ready, const float *res) {
+    CANDY_REQUIRE(res != y || mmq_fuses_residual(w, m), "internal: in-place residual needs the fused epilogue");
+    bool res_done = false;
+    if (int rc = mmq_dispatch(dev, w, qs, scales, m, y, half_ws, xh_ready, res, &res_done)) return rc;
+    if (res && !res_done) return candy_hip_add(dev, res, y, m * w->rows, y);  // kernels without a residual epilogue
+    return CANDY_HIP_OK;
+}
+
+static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
+                        int64_t m, float *y, void *half_ws, const _Float16 *xh_ready, const float *res, bool *res_done) {
     const int64_t K = w->cols;
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && K <= 0x7FFFFFFF && m <= 0x7FFFFFFF, "matrix too large");
     if (K % 64 != 0) return launch_matvec(dev, w, qs, scales, m, y);  // odd block counts: small-batch kernel in slices
     // prompt-sized batches of Q4_K: big fp16 tiles (the integer kernel is bound by its per-sub-block rescale there);
     // smaller batches of Q4_K and Q6_K: int8 matrix cores (exact); the fp16 tile kernel below serves the rest
-    static const bool force_fp16 = getenv("CANDY_HIP_MMQ_FP16") != nullptr;
+    const bool force_fp16 = force_old_fp16();
     const bool big = !force_fp16 && mmq_f16_big_covers(w, m);
     if (!force_fp16 && !big && mmq_i8_covers(w, qs)) return launch_mmq_i8(dev, w, qs, scales, m, y);
+    if (big && xh_ready) {
+        *res_done = res != nullptr;
+        return launch_mmq_f16_big(dev, w, xh_ready, m, y, res);
+    }
     CANDY_REQUIRE(half_ws, "internal: no workspace for the fp16 activations");
     const int64_t m_pad = mmq_m_pad(m);
     const int64_t runs = m_pad * (K >> 3);
@@ -308,7 +333,10 @@ int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *
                        m_pad, K, (half8 *)half_ws);
     CANDY_LAUNCH_CHECK();
     const _Float16 *xh = (const _Float16 *)half_ws;
-    if (big) return launch_mmq_f16_big(dev, w, xh, m, y);
+    if (big) {
+        *res_done = res != nullptr;
+        return launch_mmq_f16_big(dev, w, xh, m, y, res);
+    }
     switch (w->fmt) {
     case CANDY_HIP_Q4_K: return launch_fmt<MmqQ4K>(dev, w, xh, m, y);
     case CANDY_HIP_Q8_0: return launch_fmt<MmqQ8_0>(dev, w, xh, m, y);

@@ -113,10 +113,10 @@ struct BigQ6K {
 // ------------------------------------------------------------------ tile kernel
 // grid = tiles * n_split; workgroup (tile, split) contracts super-blocks [split*sb_per, ...) and writes
 // its tile to out + split * M * N (out = y when n_split == 1).
-template <class F, int BN, int BM, int WN, int WM>
+template <class F, int BN, int BM, int WN, int WM, bool RES>
 __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xh,
-                                                          float *__restrict__ out, int N, int M, int K, int n_tiles,
-                                                          int m_tiles, int sb_per) {
+                                                          float *out, const float *res, int N, int M, int K,
+                                                          int n_tiles, int m_tiles, int sb_per) {
     constexpr int T = WN * WM * 64;
     constexpr int TN = BN / WN / 16, TM = BM / WM / 16;
     constexpr int ATK = BN * 4 / T;   // dequantization tasks per thread per step
@@ -246,18 +246,24 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
             const int n = n0 + wn * (BN / WN) + tn * 16 + 4 * (lane >> 4);
             if (m >= M) continue;
             float *dst = out + (size_t)m * N + n;
+            const float *r = RES ? res + (size_t)m * N + n : nullptr;  // may alias dst: read before the store
             if (n + 3 < N && (N & 3) == 0) {
-                *(float4 *)dst = make_float4(acc[tn][tm][0], acc[tn][tm][1], acc[tn][tm][2], acc[tn][tm][3]);
+                float4 o = make_float4(acc[tn][tm][0], acc[tn][tm][1], acc[tn][tm][2], acc[tn][tm][3]);
+                if (r) {
+                    const float4 rv = *(const float4 *)r;
+                    o = make_float4(rv.x + o.x, rv.y + o.y, rv.z + o.z, rv.w + o.w);
+                }
+                *(float4 *)dst = o;
             } else {
 #pragma unroll
                 for (int l = 0; l < 4; ++l)
-                    if (n + l < N) dst[l] = acc[tn][tm][l];
+                    if (n + l < N) dst[l] = r ? r[l] + acc[tn][tm][l] : acc[tn][tm][l];
             }
         }
 }
 
-// y[i] = part[0][i] + part[1][i] + ... in that order
-__global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ part, float *__restrict__ y, size_t count,
+// y[i] = (res[i] +) part[0][i] + part[1][i] + ... in that order; res may alias y
+__global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ part, float *y, const float *res, size_t count,
                                                     int n_split) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= count) return;
@@ -267,18 +273,23 @@ __global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ pa
             const float4 v = *(const float4 *)(part + (size_t)k * count + i);
             s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
         }
+        if (res) {
+            const float4 r = *(const float4 *)(res + i);
+            s = make_float4(r.x + s.x, r.y + s.y, r.z + s.z, r.w + s.w);
+        }
         *(float4 *)(y + i) = s;
     } else {
         for (size_t j = i; j < i + 4 && j < count; ++j) {
             float s = part[j];
             for (int k = 1; k < n_split; ++k) s += part[(size_t)k * count + j];
-            y[j] = s;
+            y[j] = res ? res[j] + s : s;
         }
     }
 }
 
 template <class F, int BN, int BM, int WN, int WM>
-static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y) {
+static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
+                      const float *res) {
     const int N = (int)w->rows, K = (int)w->cols;
     const int n_tiles = (N + BN - 1) / BN, m_tiles = (int)((m + BM - 1) / BM);
     const int tiles = n_tiles * m_tiles, n_sb = K >> 8;
@@ -299,15 +310,16 @@ static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _
         out = (float *)p;
     }
     constexpr size_t smem = (size_t)2 * (BN + BM) * BIG_PITCH * sizeof(_Float16);
-    CANDY_HIP_TRY(hipFuncSetAttribute((const void *)k_mmq_f16<F, BN, BM, WN, WM>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL((k_mmq_f16<F, BN, BM, WN, WM>), dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem,
-                       dev->stream, (const uint8_t *)w->data, xh, out, N, (int)m, K, n_tiles, m_tiles, sb_per);
+    const bool epi_res = res && n_split == 1;  // otherwise the split sum adds it
+    auto kern = epi_res ? k_mmq_f16<F, BN, BM, WN, WM, true> : k_mmq_f16<F, BN, BM, WN, WM, false>;
+    CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream,
+                       (const uint8_t *)w->data, xh, out, epi_res ? res : nullptr, N, (int)m, K, n_tiles, m_tiles, sb_per);
     CANDY_LAUNCH_CHECK();
     if (n_split > 1) {
         const size_t count = (size_t)m * N;
-        hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((count / 4 + 256) / 256)), dim3(256), 0, dev->stream, out, y, count,
-                           n_split);
+        hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((count / 4 + 256) / 256)), dim3(256), 0, dev->stream, out, y, res,
+                           count, n_split);
         CANDY_LAUNCH_CHECK();
     }
     return CANDY_HIP_OK;
@@ -322,9 +334,10 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
 }
 
 // xh: fp16 activations [mmq_m_pad(m)][K], rows past m zero.
-int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y) {
-    if (w->fmt == CANDY_HIP_Q6_K) return launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y);
-    return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y);
+int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
+                       const float *res) {
+    if (w->fmt == CANDY_HIP_Q6_K) return launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
+    return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
 }
 
 }  // namespace candy

@@ -181,7 +181,8 @@ __global__ __launch_bounds__(256) void k_matmul_f32(const float *__restrict__ a,
 // RMSNorm of one row followed by Q8_0 quantization. cols % 32 == 0. One workgroup per row.
 __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict__ x, const float *__restrict__ alpha,
                                                         float eps, int cols, float *__restrict__ xn_out,
-                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales) {
+                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
+                                                        half4v *__restrict__ xh) {
     __shared__ float red[16];
     const float4 *xr = (const float4 *)(x + (size_t)blockIdx.x * cols);
     const int n4 = cols >> 2;
@@ -213,6 +214,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict_
         const size_t i = (size_t)blockIdx.x * n4 + c;
         if (xn_out) ((float4 *)xn_out)[i] = v;
         qs[i] = packed;
+        if (xh) xh[i] = q8_lane4_to_half(packed, h);
         if ((c & 7) == 0) {
             Q8Scale sc;
             sc.d = __half2float(h);
@@ -225,7 +227,8 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict_
 // silu(gate) * up, then Q8_0 quantization. n % 32 == 0.
 __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict__ gate, const float4 *__restrict__ up,
                                                         int64_t n4, float4 *__restrict__ act_out,
-                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales) {
+                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
+                                                        half4v *__restrict__ xh) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const bool live = i < n4;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -239,6 +242,7 @@ __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict
     if (!live) return;
     if (act_out) act_out[i] = v;
     qs[i] = packed;
+    if (xh) xh[i] = q8_lane4_to_half(packed, h);
     if ((i & 7) == 0) {
         Q8Scale sc;
         sc.d = __half2float(h);
@@ -249,20 +253,21 @@ __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict
 
 // ------------------------------------------------------------------ launchers shared with llama.hip
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
-                          int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales) {
+                          int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales, _Float16 *xh) {
     CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0 && cols <= 0x7FFFFFFF, "rms_norm_quant needs cols %% 32 == 0");
     hipLaunchKernelGGL(k_rms_norm_quant, dim3((unsigned)rows), dim3(256), 0, dev->stream, x, alpha, eps, (int)cols,
-                       xn_out, (uint32_t *)qs, scales);
+                       xn_out, (uint32_t *)qs, scales, (half4v *)xh);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
 
 int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *act_out,
-                          int8_t *qs, Q8Scale *scales) {
+                          int8_t *qs, Q8Scale *scales, _Float16 *xh) {
     CANDY_REQUIRE(n % 32 == 0 && n > 0, "silu_mul_quant needs n %% 32 == 0");
     const int64_t n4 = n >> 2;
     hipLaunchKernelGGL(k_silu_mul_quant, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, dev->stream,
-                       (const float4 *)gate, (const float4 *)up, n4, (float4 *)act_out, (uint32_t *)qs, scales);
+                       (const float4 *)gate, (const float4 *)up, n4, (float4 *)act_out, (uint32_t *)qs, scales,
+                       (half4v *)xh);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }

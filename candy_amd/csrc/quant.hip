@@ -13,7 +13,7 @@ namespace candy {
 // One lane owns 4 consecutive values; the 8 lanes of a block reduce with cross-lane xor.
 __global__ __launch_bounds__(256) void k_quantize_q8_0(const float4 *__restrict__ x, int64_t n4,
                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
-                                                       uint8_t *__restrict__ blocks) {
+                                                       uint8_t *__restrict__ blocks, half4v *__restrict__ xh) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const bool active = i < n4;  // n4 is a multiple of 8, so a block's 8 lanes agree
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -25,6 +25,7 @@ __global__ __launch_bounds__(256) void k_quantize_q8_0(const float4 *__restrict_
     const int64_t b = i >> 3;
     const int part = (int)(i & 7);
     if (qs) qs[i] = packed;
+    if (xh) xh[i] = q8_lane4_to_half(packed, h);
     if (scales && part == 0) {
         Q8Scale sc;
         sc.d = __half2float(h);
@@ -62,13 +63,13 @@ __global__ __launch_bounds__(256) void k_q8_blocks_to_planar(const BlockQ8_0 *__
 }
 
 int launch_quantize_q8(candy_hip_device *dev, const float *x, int64_t rows, int64_t cols, int8_t *qs, Q8Scale *scales,
-                       void *blocks) {
+                       void *blocks, _Float16 *xh) {
     const int64_t n4 = rows * cols / 4;
     if (n4 == 0) return CANDY_HIP_OK;
     const int64_t grid = (n4 + 255) / 256;
     CANDY_REQUIRE(grid <= 0x7FFFFFFF, "activation too large");
     hipLaunchKernelGGL(k_quantize_q8_0, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const float4 *)x, n4,
-                       (uint32_t *)qs, scales, (uint8_t *)blocks);
+                       (uint32_t *)qs, scales, (uint8_t *)blocks, (half4v *)xh);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
