@@ -7,7 +7,10 @@
 //   k_prefill_rope_kv   Rope (reduce.go:3987-4006: pairs (j, j + d/2)) on q in place and on k, and the
 //                       new k / v rows written into the f32 cache [kv_head][position][head_dim]
 //   k_attn_prefill      causal attention of 32 queries of one head against the cache, f32 on the
-//                       vector ALU with K / V / probabilities tiled through LDS, online softmax
+//                       vector ALU with K / V / probabilities tiled through LDS, online softmax (head_dim 64)
+//   k_attn_prefill_mfma the same for head_dim 128 on the matrix cores, 64 queries per workgroup
+#include <cstdlib>
+
 #include "blocks.h"
 #include "internal.h"
 
@@ -150,6 +153,219 @@ __global__ __launch_bounds__(256) void k_attn_prefill(const float *__restrict__ 
     }
 }
 
+// ------------------------------------------------------------------ causal attention on the matrix cores
+// head_dim 128.  grid (n_heads, ceil(n / 64)), 4 wavefronts, wavefront w owns query rows 16w .. 16w+15 of
+// the tile.  Keys and values are walked in tiles of 32 positions through LDS.  Scores S = Q.K^T and
+// outputs O += P.V run on v_mfma_f32_16x16x32_f16 with every f32 operand split into an fp16 head and an
+// fp16 tail (x = hi + lo, |lo| <= 2^-11 |x|): hi.hi + hi.lo + lo.hi carries 22 bits of each operand into
+// the f32 accumulators, so the result stays at f32-like distance from the CPU composition while the
+// vector ALU only does the softmax.  (The arithmetic being replaced is MatMul / FastSoftmax / MatMul,
+// backend.go:78,147; online softmax as in the vector-ALU kernel above.)
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4h __attribute__((ext_vector_type(4)));
+typedef _Float16 half2h __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+struct HiLo { _Float16 hi, lo; };
+__device__ __forceinline__ HiLo split_half(float x) {
+    HiLo r;
+    r.hi = (_Float16)x;
+    r.lo = (_Float16)(x - (float)r.hi);
+    return r;
+}
+
+// 16-lane row reductions on the DPP path (C-layout columns live in the 16 lanes of a row)
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    v = fmaxf(v, dpp_move<0x140>(v));
+    return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);
+    return v;
+}
+
+__global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restrict__ q, const float *__restrict__ k_cache,
+                                                           const float *__restrict__ v_cache, float *__restrict__ out,
+                                                           int n, int pos0, int n_heads, int n_kv_heads,
+                                                           int64_t cache_stride, float scale) {
+    constexpr int HD = 128, QT = 64, KT = 32;
+    constexpr int KP = HD + 8;   // K tile pitch in halves (272 bytes: the 16 rows of an operand read hit distinct banks)
+    constexpr int VP = KT + 8;   // V^T tile pitch in halves (80 bytes, same property)
+    constexpr int PP = KT + 8;   // P tile pitch
+    __shared__ __align__(16) _Float16 s_k[2][KT * KP];        // [hi/lo][key][d]
+    __shared__ __align__(16) _Float16 s_vt[2][HD * VP];       // [hi/lo][d][key]
+    __shared__ __align__(16) _Float16 s_p[4][2][16 * PP];     // per wavefront [hi/lo][row][key]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, c4 = lane >> 4;
+    const int head = blockIdx.x, i0 = blockIdx.y * QT;
+    const int kvh = head / (n_heads / n_kv_heads);
+    const float *kh = k_cache + (size_t)kvh * cache_stride, *vh = v_cache + (size_t)kvh * cache_stride;
+    const int n_keys = pos0 + min(i0 + QT, n);   // positions the tile's last query may see
+    const int wave_last = pos0 + i0 + 16 * wave + 15;  // last position any row of this wavefront may see
+
+    // Q as the A operand (row = query r16, 8 consecutive d per k-step), pre-scaled, split hi / lo
+    half8 qh[4], ql[4];
+    {
+        const int i = min(i0 + 16 * wave + r16, n - 1);
+        const float *qr = q + ((size_t)i * n_heads + head) * HD;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const float4 a = *(const float4 *)(qr + ks * 32 + c4 * 8), b = *(const float4 *)(qr + ks * 32 + c4 * 8 + 4);
+            const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const HiLo t = split_half(v[e] * scale);
+                qh[ks][e] = t.hi;
+                ql[ks][e] = t.lo;
+            }
+        }
+    }
+    // C layout: lane holds rows 4*c4 + j (j = 0..3) of the wavefront's 16 queries, column r16
+    float m_run[4], l_run[4];
+    float4v o[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { m_run[j] = -INFINITY; l_run[j] = 0.0f; }
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) o[dt] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    // global -> register requests of a tile: K: thread -> (key, 4 consecutive d), 4 passes; V: thread -> (key pair,
+    // 4 consecutive d), 2 passes.  The next tile is requested before the current one is consumed.
+    float4 kreg[4], vreg[2][2];
+    auto request = [&](int p0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int e = tid + it * 256, key = e >> 5, d4 = e & 31;
+            kreg[it] = *(const float4 *)(kh + (size_t)min(p0 + key, n_keys - 1) * HD + 4 * d4);
+        }
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int e = tid + it * 256, kp = e >> 5, d4 = e & 31;
+            vreg[it][0] = *(const float4 *)(vh + (size_t)min(p0 + 2 * kp, n_keys - 1) * HD + 4 * d4);
+            vreg[it][1] = *(const float4 *)(vh + (size_t)min(p0 + 2 * kp + 1, n_keys - 1) * HD + 4 * d4);
+        }
+    };
+    request(0);
+    for (int p0 = 0; p0 < n_keys; p0 += KT) {
+        __syncthreads();  // previous tile fully consumed
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int e = tid + it * 256, key = e >> 5, d4 = e & 31;
+            const float4 kv = kreg[it];
+            half4h hi, lo;
+            const float kvv[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const HiLo t = split_half(kvv[c]);
+                hi[c] = t.hi;
+                lo[c] = t.lo;
+            }
+            *(half4h *)&s_k[0][key * KP + 4 * d4] = hi;
+            *(half4h *)&s_k[1][key * KP + 4 * d4] = lo;
+        }
+        // V transposed: two keys of one d share a 32-bit store
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int e = tid + it * 256, kp = e >> 5, d4 = e & 31;
+            const float4 v0 = vreg[it][0], v1 = vreg[it][1];
+            const float a[4] = {v0.x, v0.y, v0.z, v0.w}, b[4] = {v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                half2h hi, lo;
+                const HiLo ta = split_half(a[c]), tb = split_half(b[c]);
+                hi[0] = ta.hi; lo[0] = ta.lo;
+                hi[1] = tb.hi; lo[1] = tb.lo;
+                *(half2h *)&s_vt[0][(4 * d4 + c) * VP + 2 * kp] = hi;
+                *(half2h *)&s_vt[1][(4 * d4 + c) * VP + 2 * kp] = lo;
+            }
+        }
+        if (p0 + KT < n_keys) request(p0 + KT);
+        __syncthreads();
+        if (p0 > wave_last) continue;  // every key of the tile is in the future of all 16 rows (the barriers above stay uniform)
+
+        // ---- S = Q.K^T for 32 keys: two 16-key column tiles
+        float4v s_acc[2];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const int off = (nt * 16 + r16) * KP + ks * 32 + c4 * 8;
+                const half8 kh8 = *(const half8 *)&s_k[0][off], kl8 = *(const half8 *)&s_k[1][off];
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql[ks], kh8, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[ks], kl8, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[ks], kh8, acc, 0, 0, 0);
+            }
+            s_acc[nt] = acc;
+        }
+        // ---- online softmax per row
+        float corr[4];
+        _Float16 *ph = &s_p[wave][0][0], *pl = &s_p[wave][1][0];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int qpos = pos0 + i0 + 16 * wave + 4 * c4 + j;
+            float sv[2];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                const bool ok = p0 + nt * 16 + r16 <= qpos;
+                sv[nt] = ok ? s_acc[nt][j] : -INFINITY;
+                mx = fmaxf(mx, sv[nt]);
+            }
+            mx = row16_max(mx);
+            const float m_new = fmaxf(m_run[j], mx);  // position 0 is visible to every row: finite from the first tile on
+            corr[j] = expf(m_run[j] - m_new);
+            float ps = 0.0f;
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                const float pw = expf(sv[nt] - m_new);  // exp(-inf) = 0 for masked keys
+                ps += pw;
+                const HiLo t = split_half(pw);
+                ph[(4 * c4 + j) * PP + nt * 16 + r16] = t.hi;
+                pl[(4 * c4 + j) * PP + nt * 16 + r16] = t.lo;
+            }
+            ps = row16_sum(ps);
+            l_run[j] = l_run[j] * corr[j] + ps;
+            m_run[j] = m_new;
+        }
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[dt][j] *= corr[j];
+        // the wavefront's own P tile: its LDS operations complete in order, no workgroup barrier needed
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // ---- O += P.V: P as the A operand (row r16, keys 8*c4 .. +7), V^T rows as the B operand
+        const half8 pa_h = *(const half8 *)&ph[r16 * PP + c4 * 8], pa_l = *(const half8 *)&pl[r16 * PP + c4 * 8];
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+            const int off = (dt * 16 + r16) * VP + c4 * 8;
+            const half8 vh8 = *(const half8 *)&s_vt[0][off], vl8 = *(const half8 *)&s_vt[1][off];
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_l, vh8, o[dt], 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_h, vl8, o[dt], 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_h, vh8, o[dt], 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int i = i0 + 16 * wave + 4 * c4 + j;
+        if (i >= n) continue;
+        const float inv = 1.0f / l_run[j];
+        float *dst = out + ((size_t)i * n_heads + head) * HD + r16;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) dst[dt * 16] = o[dt][j] * inv;
+    }
+}
+
 int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, const float *v, const float *cos_t,
                            const float *sin_t, float *k_cache, float *v_cache, int n, int pos0, int n_heads,
                            int n_kv_heads, int head_dim, int64_t cache_stride) {
@@ -165,7 +381,11 @@ int launch_attn_prefill(candy_hip_device *dev, const float *q, const float *k_ca
     CANDY_REQUIRE(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
     CANDY_REQUIRE(n > 0 && pos0 >= 0 && n_heads % n_kv_heads == 0, "invalid attention shape");
     const dim3 grid((unsigned)n_heads, (unsigned)((n + 31) / 32));
-    if (head_dim == 128)
+    static const bool valu_only = getenv("CANDY_HIP_ATTN_PREFILL_VALU") != nullptr;  // comparison runs
+    if (head_dim == 128 && !valu_only)
+        hipLaunchKernelGGL(k_attn_prefill_mfma, dim3((unsigned)n_heads, (unsigned)((n + 63) / 64)), dim3(256), 0, dev->stream,
+                           q, k_cache, v_cache, out, n, pos0, n_heads, n_kv_heads, cache_stride, scale);
+    else if (head_dim == 128)
         hipLaunchKernelGGL(k_attn_prefill<128>, grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n, pos0,
                            n_heads, n_kv_heads, cache_stride, scale);
     else

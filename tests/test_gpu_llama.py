@@ -98,6 +98,9 @@ PROMPT_CASES = [
     ("mha-hd128", dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=4, head_dim=128, d_ffn=768, vocab=256,
                        max_pos=80, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}, 70, 1e-3),
+    ("gqa-hd128-long", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=2, head_dim=128, d_ffn=512, vocab=256,
+                            max_pos=224, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}, 203, 1e-3),
     ("short-prompt", dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=64, d_ffn=512, vocab=128,
                           max_pos=16, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q8_0, "gate": synth.Q4_0, "head": synth.Q6_K, "embed": synth.Q4_K}, 5, 1e-3),
