@@ -134,15 +134,17 @@ def test_prompt_pass_matches_token_by_token_cpu(dev, name, cfg, fmts, n, bar):
         tok = rt
 
 
-def test_prompt_in_two_chunks_equals_one_pass(dev):
-    # a prompt continued at pos0 > 0 attends the positions already in the cache
-    name, cfg, fmts, n, _ = PROMPT_CASES[0]
+@pytest.mark.parametrize("case,n,cut", [(0, 50, 19), (2, 150, 77)])
+def test_prompt_in_two_chunks_equals_one_pass(dev, case, n, cut):
+    # a prompt continued at pos0 > 0 attends the positions already in the cache (head_dim 64: vector-ALU
+    # attention; head_dim 128: the matrix-core kernel, second chunk starting off every tile boundary)
+    name, cfg, fmts, _, _ = PROMPT_CASES[case]
     _, a = build(dev, cfg, fmts, seed=13)
     _, b = build(dev, cfg, fmts, seed=13)
-    tokens = [int(t) for t in np.random.default_rng(14).integers(0, cfg["vocab"], 50)]
+    tokens = [int(t) for t in np.random.default_rng(14).integers(0, cfg["vocab"], n)]
     ta, la = a.prefill(tokens, 0)
-    b.prefill(tokens[:19], 0)
-    tb, lb = b.prefill(tokens[19:], 19)
+    b.prefill(tokens[:cut], 0)
+    tb, lb = b.prefill(tokens[cut:], cut)
     assert rel(lb, la.astype(np.float64)) <= 1e-4
     with pytest.raises(hip.CandyHipError, match="outside the cache"):
         a.prefill(tokens, cfg["max_pos"] - 10)
