@@ -9,6 +9,9 @@
 
 #include "blocks.h"
 #include "internal.h"
+#include <cstdio>
+
+#include "persist.h"
 
 struct candy_hip_llama {
     candy_hip_device *dev = nullptr;
@@ -28,11 +31,19 @@ struct candy_hip_llama {
     float *gate_o = nullptr, *up_o = nullptr, *logits = nullptr;
     int8_t *xq = nullptr;           // planar Q8_0 quants of the current activation
     candy::Q8Scale *xs = nullptr;
-    uint32_t *next_tok = nullptr;
+    uint32_t *next_tok = nullptr;   // [2]: greedy token, then the persistent kernel's time-out flag
     int64_t *tok_id = nullptr;
     int *d_pos = nullptr;                         // position of the token being decoded (device copy)
     void *attn_scratch = nullptr;                 // attention split partials
     int n_splits = 1;
+    // the step as one persistent kernel (persist.hip), when the configuration is one it covers
+    bool persist_wanted = false, persist_broken = false, persist_ready = false;
+    int last_path = 0;
+    candy::u64 *p_prof = nullptr;  // phase stamps of the last persistent step (CANDY_HIP_PERSIST_PROF)
+    std::vector<candy::PersistLayer> p_host;
+    candy::PersistLayer *p_layers = nullptr;
+    unsigned *p_epoch = nullptr;
+    candy::u64 *p_xchg = nullptr;
     hipGraph_t graph = nullptr;                   // the captured step (layers + head + argmax)
     hipGraphExec_t graph_exec = nullptr;
     bool graph_dirty = true;
@@ -54,9 +65,11 @@ struct candy_hip_llama {
 namespace candy {
 
 // Parks the step's position and token id in device memory (read by the captured kernels).
-__global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok) {
+__global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok, unsigned *epoch) {
     *pos_dst = pos;
     if (tok >= 0) *tok_dst = tok;
+    const unsigned e = *epoch + 1;  // tags of the persistent kernel's exchange words: never 0, new every step
+    *epoch = e == 0 ? 1 : e;
 }
 
 }  // namespace candy
@@ -119,7 +132,10 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
     if (!rc) rc = dev_alloc(m, &m->logits, (size_t)cfg->vocab);
     if (!rc) rc = dev_alloc(m, &m->xq, widest);
     if (!rc) rc = dev_alloc(m, &m->xs, widest / 32);
-    if (!rc) rc = dev_alloc(m, &m->next_tok, 1);
+    if (!rc) rc = dev_alloc(m, &m->next_tok, 2);
+    if (!rc) rc = candy_hip_zero(dev, m->next_tok, 2 * sizeof(uint32_t));
+    if (!rc) rc = dev_alloc(m, &m->p_epoch, 1);
+    if (!rc) rc = candy_hip_zero(dev, m->p_epoch, sizeof(unsigned));
     if (!rc) rc = dev_alloc(m, &m->tok_id, 1);
     if (!rc) rc = dev_alloc(m, &m->d_pos, 1);
     m->n_splits = attention_splits(dev, cfg->n_kv_heads, cfg->max_pos);
@@ -129,6 +145,7 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
         m->attn_scratch = p;
     }
     m->use_graph = getenv("CANDY_HIP_NO_GRAPH") == nullptr;
+    m->persist_wanted = getenv("CANDY_HIP_PERSIST") != nullptr;  // opt-in: measured slower than the launches so far
     if (!rc) rc = candy_hip_zero(dev, m->k_cache, kv * sizeof(float));
     if (!rc) rc = candy_hip_zero(dev, m->v_cache, kv * sizeof(float));
     if (!rc) {
@@ -155,6 +172,20 @@ int candy_hip_llama_free(candy_hip_llama *m) {
     if (!m) return CANDY_HIP_OK;
     (void)hipSetDevice(m->dev->ordinal);
     (void)hipStreamSynchronize(m->dev->stream);
+    if (m->p_prof) {  // the last step's phase stamps (100 MHz clock), one line per workgroup and layer
+        const size_t n = (size_t)m->dev->num_cus * (size_t)(m->cfg.n_layers + 1) * candy::PROF_SLOTS;
+        std::vector<candy::u64> h(n);
+        const char *path = getenv("CANDY_HIP_PERSIST_PROF");
+        FILE *f = path ? fopen(path, "w") : nullptr;
+        if (f && hipMemcpy(h.data(), m->p_prof, n * sizeof(candy::u64), hipMemcpyDeviceToHost) == hipSuccess)
+            for (size_t i = 0; i < n; i += candy::PROF_SLOTS) {
+                const size_t row = i / candy::PROF_SLOTS;
+                fprintf(f, "%zu %zu", row / (size_t)(m->cfg.n_layers + 1), row % (size_t)(m->cfg.n_layers + 1));
+                for (int j = 0; j < candy::PROF_SLOTS; ++j) fprintf(f, " %llu", h[i + j]);
+                fprintf(f, "\n");
+            }
+        if (f) fclose(f);
+    }
     if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
     if (m->graph) (void)hipGraphDestroy(m->graph);
     for (void *p : m->owned) (void)candy_hip_free(m->dev, p);
@@ -217,6 +248,19 @@ int candy_hip_llama_set_graph(candy_hip_llama *m, int enable) {
     return CANDY_HIP_OK;
 }
 
+int candy_hip_llama_set_persistent(candy_hip_llama *m, int enable) {
+    CANDY_REQUIRE(m, "model is nil");
+    m->persist_wanted = enable != 0;
+    m->graph_dirty = true;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_llama_decode_path(candy_hip_llama *m, int *path) {
+    CANDY_REQUIRE(m && path, "model or output is nil");
+    *path = m->last_path;
+    return CANDY_HIP_OK;
+}
+
 int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, size_t *bytes_each) {
     CANDY_REQUIRE(m, "model is nil");
     if (dev_k) *dev_k = m->k_cache;
@@ -269,7 +313,83 @@ static int linear_residual(candy_hip_llama *m, const candy_hip_qtensor *w) {
 // Enqueues one decode step (hidden state in m->h, position in *m->d_pos) on the stream: six
 // launches per layer. Everything it touches is owned by the model, nothing allocates or
 // synchronises, so the sequence can be captured once and replayed for every token.
+// Whether the persistent kernel covers this model on this device (persist.hip states what it covers).
+static bool persist_covers(const candy_hip_llama *m) {
+    const candy_hip_llama_config &c = m->cfg;
+    const int G = m->dev->num_cus;
+    if (c.head_dim != 128 || c.n_heads != c.n_kv_heads || c.n_heads * c.head_dim != c.d_model) return false;
+    if (c.d_model > 4096 || c.d_model % 256 || c.d_ffn > 16384 || c.d_ffn % 256 || 6 * c.n_layers + 2 >= 4096) return false;
+    if (G % c.n_heads) return false;
+    const int S = G / c.n_heads;
+    if (S < 1 || S > 128 || 128 % S) return false;  // a split's merge uses S * (128 / S + 2) <= 384 threads
+    auto q4k = [](const candy_hip_qtensor *w) { return w->fmt == CANDY_HIP_Q4_K && ((uintptr_t)w->data & 15) == 0; };
+    for (const candy_hip_llama::Layer &L : m->layers)
+        if (!q4k(L.wq) || !q4k(L.wk) || !q4k(L.wv) || !q4k(L.wo) || !q4k(L.gate) || !q4k(L.up) || !q4k(L.down)) return false;
+    return q4k(m->head) || (m->head->fmt == CANDY_HIP_Q6_K && ((uintptr_t)m->head->data & 1) == 0);
+}
+
+// Exchange buffers (allocated and cleared once) and the layer table (uploaded again whenever a weight
+// changed).  Runs outside stream capture; the upload is ordered on the stream before the next step.
+static size_t persist_part_words(const candy_hip_llama *m) {
+    return (size_t)m->cfg.n_heads * (size_t)(m->dev->num_cus / m->cfg.n_heads) * (128 + 2);
+}
+
+static int persist_prepare(candy_hip_llama *m) {
+    const candy_hip_llama_config &c = m->cfg;
+    candy_hip_device *dev = m->dev;
+    const size_t D = (size_t)c.d_model, F = (size_t)c.d_ffn;
+    const size_t words = 2 * (D + D + 3 * D + persist_part_words(m) + D + F) + 2 * (size_t)dev->num_cus;
+    if (!m->p_xchg) {
+        if (int rc = dev_alloc(m, &m->p_xchg, words)) return rc;
+        if (int rc = candy_hip_zero(dev, m->p_xchg, words * sizeof(u64))) return rc;
+        if (int rc = dev_alloc(m, &m->p_layers, (size_t)c.n_layers)) return rc;
+    }
+    if (!m->p_prof && getenv("CANDY_HIP_PERSIST_PROF"))
+        if (int rc = dev_alloc(m, &m->p_prof, (size_t)dev->num_cus * (size_t)(c.n_layers + 1) * candy::PROF_SLOTS)) return rc;
+    CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));  // a step still in flight reads the table being replaced
+    m->p_host.resize((size_t)c.n_layers);
+    for (int l = 0; l < c.n_layers; ++l) {
+        const candy_hip_llama::Layer &L = m->layers[l];
+        PersistLayer &P = m->p_host[(size_t)l];
+        auto addr = [](const void *p) { return (candy::u64)(uintptr_t)p; };
+        P.wq = addr(L.wq->data); P.wk = addr(L.wk->data); P.wv = addr(L.wv->data); P.wo = addr(L.wo->data);
+        P.gate = addr(L.gate->data); P.up = addr(L.up->data); P.down = addr(L.down->data);
+        P.attn_norm = addr(L.attn_norm); P.ffn_norm = addr(L.ffn_norm);
+    }
+    if (int rc = candy_hip_h2d(dev, m->p_layers, m->p_host.data(), m->p_host.size() * sizeof(PersistLayer))) return rc;
+    m->persist_ready = true;
+    return CANDY_HIP_OK;
+}
+
+// The step as one launch (nothing here allocates or synchronises: it may be captured).
+static int persist_enqueue(candy_hip_llama *m) {
+    const candy_hip_llama_config &c = m->cfg;
+    candy_hip_device *dev = m->dev;
+    const size_t D = (size_t)c.d_model, F = (size_t)c.d_ffn;
+    const size_t part = persist_part_words(m);
+    PersistArgs a{};
+    a.layers = m->p_layers;
+    a.n_layers = c.n_layers; a.d_model = c.d_model; a.n_heads = c.n_heads; a.d_ffn = c.d_ffn; a.vocab = c.vocab;
+    a.max_pos = c.max_pos; a.eps = c.rms_eps; a.scale = 1.0f / std::sqrt((float)c.head_dim);
+    a.out_norm = m->out_norm; a.head = (const uint8_t *)m->head->data; a.head_is_q6k = m->head->fmt == CANDY_HIP_Q6_K;
+    a.cos_t = m->cos_t; a.sin_t = m->sin_t; a.k_cache = m->k_cache; a.v_cache = m->v_cache;
+    a.h_in = m->h; a.pos_ptr = m->d_pos; a.epoch_ptr = m->p_epoch;
+    u64 *p = m->p_xchg;
+    a.x_ha = p; p += 2 * D;
+    a.x_hb = p; p += 2 * D;
+    a.x_qkv = p; p += 6 * D;
+    a.x_part = p; p += 2 * part;
+    a.x_att = p; p += 2 * D;
+    a.x_act = p; p += 2 * F;
+    a.x_best = p;
+    a.logits = m->logits; a.next_tok = m->next_tok; a.fail = m->next_tok + 1;
+    a.spin_limit = 1 << 15;
+    a.prof = m->p_prof;
+    return launch_decode_step(dev, a);
+}
+
 static int llama_enqueue_step(candy_hip_llama *m) {
+    if (m->persist_ready) return persist_enqueue(m);
     const candy_hip_llama_config &c = m->cfg;
     candy_hip_device *dev = m->dev;
     const size_t layer_kv = (size_t)c.n_kv_heads * c.max_pos * c.head_dim;
@@ -318,15 +438,23 @@ static int llama_enqueue_step(candy_hip_llama *m) {
 }
 
 static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const float *dev_hidden,
+                      const float **dev_logits, int32_t *next_token);
+
+static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const float *dev_hidden,
                       const float **dev_logits, int32_t *next_token) {
     candy_hip_device *dev = m->dev;
     int rc;
-    hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token);
+    hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token, m->p_epoch);
     CANDY_LAUNCH_CHECK();
     if (dev_hidden) {
         if ((rc = candy_hip_d2d(dev, m->h, dev_hidden, (size_t)m->cfg.d_model * sizeof(float)))) return rc;
     } else {
         if ((rc = candy_hip_qindex_select(dev, m->embed, m->tok_id, 1, m->h))) return rc;
+    }
+    if (m->graph_dirty || !m->use_graph) {
+        m->persist_ready = false;
+        if (m->persist_wanted && !m->persist_broken && persist_covers(m))
+            if ((rc = persist_prepare(m))) return rc;
     }
     if (m->use_graph) {
         if (m->graph_dirty) {
@@ -347,11 +475,21 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
         if ((rc = llama_enqueue_step(m))) return rc;
     }
     if (dev_logits) *dev_logits = m->logits;
-    if (next_token) {
-        uint32_t t = 0;
-        if ((rc = candy_hip_d2h(dev, &t, m->next_tok, sizeof(t)))) return rc;
-        *next_token = (int32_t)t;
+    if (next_token || m->persist_ready) {
+        uint32_t t[2] = {0, 0};  // token, time-out flag of the persistent kernel
+        if ((rc = candy_hip_d2h(dev, t, m->next_tok, sizeof(t)))) return rc;
+        if (t[1] != 0) {
+            // a workgroup gave up waiting for another (the grid was not resident as a whole): nothing of the
+            // step is trusted; clear the flag and redo it kernel by kernel, from now on
+            m->persist_broken = true;
+            m->persist_ready = false;
+            m->graph_dirty = true;
+            if ((rc = candy_hip_zero(dev, m->next_tok + 1, sizeof(uint32_t)))) return rc;
+            return llama_step(m, pos, token, dev_hidden, dev_logits, next_token);
+        }
+        if (next_token) *next_token = (int32_t)t[0];
     }
+    m->last_path = m->persist_ready ? 1 : 0;
     return CANDY_HIP_OK;
 }
 

@@ -84,6 +84,8 @@ SIGNATURES = {
     "candy_hip_llama_set_qweight": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "candy_hip_llama_set_norm": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "candy_hip_llama_set_graph": (c_int, [c_void_p, c_int]),
+    "candy_hip_llama_set_persistent": (c_int, [c_void_p, c_int]),
+    "candy_hip_llama_decode_path": (c_int, [c_void_p, POINTER(c_int)]),
     "candy_hip_llama_kv_cache": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_size_t)]),
     "candy_hip_llama_decode": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_llama_decode_hidden": (c_int, [c_void_p, c_void_p, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
@@ -410,6 +412,15 @@ class Llama:
 
     def set_graph(self, enable: bool):
         _check(lib().candy_hip_llama_set_graph(self.handle, int(enable)))
+
+    def set_persistent(self, enable: bool):
+        _check(lib().candy_hip_llama_set_persistent(self.handle, int(enable)))
+
+    def decode_path(self) -> int:
+        """0: the last decode step ran kernel by kernel; 1: as the persistent kernel."""
+        p = c_int(-1)
+        _check(lib().candy_hip_llama_decode_path(self.handle, byref(p)))
+        return p.value
 
     def kv_cache(self):
         k, v, n = c_void_p(), c_void_p(), c_size_t()

@@ -191,6 +191,17 @@ int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const flo
  * position and token travel through device memory); enable = 0 launches the kernels one by
  * one instead.  Results are identical either way. */
 int candy_hip_llama_set_graph(candy_hip_llama *m, int enable);
+/* Experimental, off by default: where the model's shape allows (head_dim 128, one kv head per query
+ * head, Q4_K layer weights, d_model <= 4096, d_ffn <= 16384) the decode step can run as ONE persistent
+ * kernel, one workgroup per compute unit, whose phases hand their results on through tagged words in
+ * device memory, instead of six launches per layer.  enable = 1 selects it (so does the environment
+ * variable CANDY_HIP_PERSIST); a model it does not cover, or a device on which its workgroups cannot
+ * all be resident, keeps the launches.  Results agree to f32 summation order.  As measured on the 7B
+ * shape it is the slower of the two.  No counterpart in the reference, which has no model code and runs
+ * one op per call. */
+int candy_hip_llama_set_persistent(candy_hip_llama *m, int enable);
+/* How the last decode step ran: 0 = kernel by kernel, 1 = the persistent kernel. */
+int candy_hip_llama_decode_path(candy_hip_llama *m, int *path);
 /* f32 KV cache, [n_layers][n_kv_heads][max_pos][head_dim] for K and the same for V. */
 int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, size_t *bytes_each);
 /* One decode step: token id at position pos -> logits [vocab] (device pointer owned by the
