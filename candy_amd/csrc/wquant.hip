@@ -1,0 +1,314 @@
+// Weight quantizers from f32: Q4_0 (both element orders), Q4_K, Q6_K.
+//
+// candy names these kernels (tensor/internal/metal/kernels/kernels.go:563-592: quantize_q4_0,
+// quantize_q4_k, quantize_q6_k ...) but holds no implementation; the arithmetic is that of ggml's
+// published reference quantizers (quantize_row_q4_0_ref; quantize_row_q4_K_ref with make_qkx2_quants;
+// quantize_row_q6_K_ref with make_qx_quants), every f32 operation rounding once, in their order, so the
+// blocks come out bit for bit as a CPU evaluation of the same steps gives them.  This file is compiled
+// with -ffp-contract=off for that reason (a fused multiply-add rounds once where the steps round twice).
+//
+// A load-time operation: one thread per block (32 values) or super-block (256 values), the candidate
+// search of the K formats running serially in that thread.  Inputs must be finite.
+#include "blocks.h"
+#include "internal.h"
+
+namespace candy {
+
+// Round to nearest, ties to even (|f| <= 4194303): adding 1.5 * 2^23 leaves the integer in the mantissa.
+__device__ __forceinline__ int rne_int(float f) {
+    const float v = f + 12582912.0f;
+    return (int)(__float_as_uint(v) & 0x007FFFFFu) - 0x00400000;
+}
+__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+// The f32 value is rounded to fp16 as it stands: left to the compiler, a product feeding the conversion
+// is folded into one mixed-precision multiply-add with a +0 addend, which turns a -0 product into +0.
+__device__ __forceinline__ uint16_t f32_to_half_bits(float f) {
+    asm volatile("" : "+v"(f));
+    return __half_as_ushort(__float2half_rn(f));
+}
+
+// ------------------------------------------------------------------ Q4_0
+// The value of largest magnitude maps to level -8 (d = max / -8 keeps its sign), the others to
+// (int)(x / d + 8.5) capped at 15.  ggml_order: byte j = elements j (low nibble) and j + 16 (high);
+// otherwise candy's CPU order, byte j = elements 2j and 2j + 1 (quantized.go:85-93).
+__global__ __launch_bounds__(256) void k_wquant_q4_0(const float *__restrict__ x, int64_t nb, BlockQ4_0 *__restrict__ out,
+                                                     int ggml_order) {
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= nb) return;
+    const float4 *src = (const float4 *)(x + 32 * b);
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float4 t = src[i];
+        v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+    }
+    float amax = 0.0f, vmax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const float a = fabsf(v[i]);
+        if (amax < a) { amax = a; vmax = v[i]; }
+    }
+    const float d = vmax / -8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint32_t q[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const int l = (int)(v[i] * id + 8.5f);
+        q[i] = (uint32_t)(l < 15 ? l : 15);
+    }
+    BlockQ4_0 *y = out + b;
+    y->d = f32_to_half_bits(d);
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+        y->qs[j] = ggml_order ? (uint8_t)(q[j] | (q[j + 16] << 4)) : (uint8_t)(q[2 * j] | (q[2 * j + 1] << 4));
+}
+
+// ------------------------------------------------------------------ Q4_K
+// Levels 0..15 with scale and non-positive minimum for 32 values (make_qkx2_quants with rmin -1,
+// rdelta 0.1, 20 steps, squared error): min/max rounding first, then 21 nearby scales, each followed by
+// the weighted least-squares fit of (scale, min) to the levels it yields; the best weighted error wins.
+// Returns the scale; neg_min receives -min.
+__device__ float search_affine32(const float *x, const float *w, uint8_t *L, float &neg_min) {
+    float lo = x[0], hi = x[0];
+    float sum_w = w[0], sum_x = sum_w * x[0];
+    for (int i = 1; i < 32; ++i) {
+        if (x[i] < lo) lo = x[i];
+        if (x[i] > hi) hi = x[i];
+        sum_w += w[i];
+        sum_x += w[i] * x[i];
+    }
+    if (lo > 0.0f) lo = 0.0f;
+    if (hi == lo) {
+        for (int i = 0; i < 32; ++i) L[i] = 0;
+        neg_min = -lo;
+        return 0.0f;
+    }
+    float iscale = 15.0f / (hi - lo);
+    float scale = 1.0f / iscale;
+    float best = 0.0f;
+    for (int i = 0; i < 32; ++i) {
+        const int l = clampi(rne_int(iscale * (x[i] - lo)), 0, 15);
+        L[i] = (uint8_t)l;
+        float diff = scale * (float)l + lo - x[i];
+        diff = diff * diff;
+        best += w[i] * diff;
+    }
+    uint8_t cand[32];
+    for (int is = 0; is <= 20; ++is) {
+        iscale = (-1.0f + 0.1f * (float)is + 15.0f) / (hi - lo);
+        float sum_l = 0.0f, sum_l2 = 0.0f, sum_xl = 0.0f;
+        for (int i = 0; i < 32; ++i) {
+            const int l = clampi(rne_int(iscale * (x[i] - lo)), 0, 15);
+            cand[i] = (uint8_t)l;
+            sum_l += w[i] * (float)l;
+            sum_l2 += w[i] * (float)l * (float)l;
+            sum_xl += w[i] * (float)l * x[i];
+        }
+        const float det = sum_w * sum_l2 - sum_l * sum_l;
+        if (det > 0.0f) {
+            float s = (sum_w * sum_xl - sum_x * sum_l) / det;
+            float m = (sum_l2 * sum_x - sum_l * sum_xl) / det;
+            if (m > 0.0f) {
+                m = 0.0f;
+                s = sum_xl / sum_l2;
+            }
+            float err = 0.0f;
+            for (int i = 0; i < 32; ++i) {
+                float diff = s * (float)cand[i] + m - x[i];
+                diff = diff * diff;
+                err += w[i] * diff;
+            }
+            if (err < best) {
+                for (int i = 0; i < 32; ++i) L[i] = cand[i];
+                best = err;
+                scale = s;
+                lo = m;
+            }
+        }
+    }
+    neg_min = -lo;
+    return scale;
+}
+
+// One super-block: per-sub-block (scale, min) with weights rms + |x|, both stored in 6 bits relative to
+// their maxima (d, dmin in fp16, packed as get_scale_min_k4 of quantized.cu:993-1005 unpacks them), then
+// the levels assigned again with the STORED scales (a sub-block whose stored scale is 0 keeps the search's).
+__global__ __launch_bounds__(64) void k_wquant_q4_k(const float *__restrict__ x, int64_t nb, BlockQ4K *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (b >= nb) return;
+    const float *xb = x + 256 * b;
+    uint8_t L[256];
+    float scales[8], mins[8];
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int j = 0; j < 8; ++j) {
+        float xs[32], w[32];
+        float sum_x2 = 0.0f;
+        for (int l = 0; l < 32; ++l) {
+            xs[l] = xb[32 * j + l];
+            sum_x2 += xs[l] * xs[l];
+        }
+        const float av = sqrtf(sum_x2 / 32.0f);
+        for (int l = 0; l < 32; ++l) w[l] = av + fabsf(xs[l]);
+        scales[j] = search_affine32(xs, w, L + 32 * j, mins[j]);
+        if (scales[j] > max_scale) max_scale = scales[j];
+        if (mins[j] > max_min) max_min = mins[j];
+    }
+    const float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    uint8_t sc6[8], mn6[8], packed[12];
+    for (int j = 0; j < 8; ++j) {
+        const int ls = rne_int(inv_scale * scales[j]), lm = rne_int(inv_min * mins[j]);
+        sc6[j] = (uint8_t)(ls < 63 ? ls : 63);
+        mn6[j] = (uint8_t)(lm < 63 ? lm : 63);
+    }
+    for (int j = 0; j < 4; ++j) {
+        packed[j] = (uint8_t)(sc6[j] | ((sc6[j + 4] >> 4) << 6));
+        packed[j + 4] = (uint8_t)(mn6[j] | ((mn6[j + 4] >> 4) << 6));
+        packed[j + 8] = (uint8_t)((sc6[j + 4] & 0xF) | ((mn6[j + 4] & 0xF) << 4));
+    }
+    BlockQ4K *y = out + b;
+    const uint16_t dh = f32_to_half_bits(max_scale / 63.0f), mh = f32_to_half_bits(max_min / 63.0f);
+    y->d = dh;
+    y->dmin = mh;
+    for (int j = 0; j < 12; ++j) y->scales[j] = packed[j];
+    const float df = half_bits_to_float(dh), mf = half_bits_to_float(mh);
+    for (int j = 0; j < 8; ++j) {
+        const float d = df * (float)sc6[j];
+        if (d == 0.0f) continue;
+        const float dm = mf * (float)mn6[j];
+        for (int i = 0; i < 32; ++i) L[32 * j + i] = (uint8_t)clampi(rne_int((xb[32 * j + i] + dm) / d), 0, 15);
+    }
+    for (int g = 0; g < 4; ++g)
+        for (int l = 0; l < 32; ++l) y->qs[32 * g + l] = (uint8_t)(L[64 * g + l] | (L[64 * g + 32 + l] << 4));
+}
+
+// ------------------------------------------------------------------ Q6_K
+// Symmetric levels -32..31 for 16 values (make_qx_quants, weights x^2): the value of largest magnitude
+// maps to -32, then 18 nearby scales are tried and the largest (sum w x l)^2 / (sum w l^2) wins.
+// L receives level + 32.
+__device__ float search_symmetric16(const float *x, int8_t *L) {
+    float vmax = 0.0f, amax = 0.0f;
+    for (int i = 0; i < 16; ++i) {
+        const float a = fabsf(x[i]);
+        if (a > amax) { amax = a; vmax = x[i]; }
+    }
+    if (amax < 1e-15f) {
+        for (int i = 0; i < 16; ++i) L[i] = 0;
+        return 0.0f;
+    }
+    float iscale = -32.0f / vmax;
+    float sumlx = 0.0f, suml2 = 0.0f;
+    for (int i = 0; i < 16; ++i) {
+        const int l = clampi(rne_int(iscale * x[i]), -32, 31);
+        L[i] = (int8_t)(l + 32);
+        const float w = x[i] * x[i];
+        sumlx += w * x[i] * (float)l;
+        suml2 += w * (float)l * (float)l;
+    }
+    float scale = suml2 != 0.0f ? sumlx / suml2 : 0.0f;
+    float best = scale * sumlx;
+    for (int is = -9; is <= 9; ++is) {
+        if (is == 0) continue;
+        iscale = -(32.0f + 0.1f * (float)is) / vmax;
+        sumlx = 0.0f;
+        suml2 = 0.0f;
+        for (int i = 0; i < 16; ++i) {
+            const int l = clampi(rne_int(iscale * x[i]), -32, 31);
+            const float w = x[i] * x[i];
+            sumlx += w * x[i] * (float)l;
+            suml2 += w * (float)l * (float)l;
+        }
+        if (suml2 > 0.0f && sumlx * sumlx > best * suml2) {
+            for (int i = 0; i < 16; ++i) L[i] = (int8_t)(32 + clampi(rne_int(iscale * x[i]), -32, 31));
+            scale = sumlx / suml2;
+            best = scale * sumlx;
+        }
+    }
+    return scale;
+}
+
+// One super-block: sixteen group scales, the one of largest magnitude mapping to -128 in int8 (d in
+// fp16 keeps its sign), levels assigned again with the STORED scales, packed as quantized.cu:1103-1128
+// reads them (ql: low nibbles of two quarters per byte, qh: the two high bits of four quarters).
+__global__ __launch_bounds__(64) void k_wquant_q6_k(const float *__restrict__ x, int64_t nb, BlockQ6K *__restrict__ out) {
+    const int64_t b = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (b >= nb) return;
+    const float *xb = x + 256 * b;
+    int8_t L[256];
+    float scales[16];
+    float max_scale = 0.0f, max_abs = 0.0f;
+    for (int g = 0; g < 16; ++g) {
+        float xs[16];
+        for (int i = 0; i < 16; ++i) xs[i] = xb[16 * g + i];
+        const float s = search_symmetric16(xs, L + 16 * g);
+        scales[g] = s;
+        if (fabsf(s) > max_abs) { max_abs = fabsf(s); max_scale = s; }
+    }
+    BlockQ6K *y = out + b;
+    if (max_abs < 1e-15f) {
+        uint16_t *z = (uint16_t *)y;  // 210 bytes, 2-byte aligned
+        for (int i = 0; i < 105; ++i) z[i] = 0;
+        return;
+    }
+    const float iscale = -128.0f / max_scale;
+    const uint16_t dh = f32_to_half_bits(1.0f / iscale);
+    int8_t sc8[16];
+    for (int g = 0; g < 16; ++g) {
+        const int v = rne_int(iscale * scales[g]);
+        sc8[g] = (int8_t)(v < 127 ? v : 127);
+    }
+    const float df = half_bits_to_float(dh);
+    for (int g = 0; g < 16; ++g) {
+        const float d = df * (float)sc8[g];
+        if (d == 0.0f) continue;
+        for (int i = 0; i < 16; ++i) L[16 * g + i] = (int8_t)(clampi(rne_int(xb[16 * g + i] / d), -32, 31) + 32);
+    }
+    y->d = dh;
+    for (int g = 0; g < 16; ++g) y->scales[g] = sc8[g];
+    for (int h = 0; h < 2; ++h)
+        for (int l = 0; l < 32; ++l) {
+            const uint32_t a0 = (uint8_t)L[128 * h + l], a1 = (uint8_t)L[128 * h + 32 + l];
+            const uint32_t a2 = (uint8_t)L[128 * h + 64 + l], a3 = (uint8_t)L[128 * h + 96 + l];
+            y->ql[64 * h + l] = (uint8_t)((a0 & 0xF) | ((a2 & 0xF) << 4));
+            y->ql[64 * h + 32 + l] = (uint8_t)((a1 & 0xF) | ((a3 & 0xF) << 4));
+            y->qh[32 * h + l] = (uint8_t)((a0 >> 4) | ((a1 >> 4) << 2) | ((a2 >> 4) << 4) | ((a3 >> 4) << 6));
+        }
+}
+
+}  // namespace candy
+
+using namespace candy;
+
+int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64_t rows, int64_t cols, void *dev_out_blocks) {
+    CANDY_REQUIRE(dev, "device is nil");
+    const int qk = candy_hip_block_elems(fmt);
+    CANDY_REQUIRE(qk != 0, "unknown block format %d", fmt);
+    CANDY_REQUIRE(rows >= 0 && cols >= 0, "invalid matrix dimensions");
+    CANDY_REQUIRE(cols % qk == 0, "cols %lld is not a multiple of the block size %d", (long long)cols, qk);
+    if (fmt == CANDY_HIP_Q8_0) return candy_hip_quantize_q8_0(dev, dev_x, rows, cols, dev_out_blocks);
+    if (rows * cols == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dev_x && dev_out_blocks, "nil pointer");
+    CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "input must be 16-byte aligned");
+    CANDY_REQUIRE(((uintptr_t)dev_out_blocks & 1) == 0, "output blocks must be 2-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    const int64_t nb = rows * cols / qk;
+    const int per = qk == 32 ? 256 : 64;
+    const int64_t grid = (nb + per - 1) / per;
+    CANDY_REQUIRE(grid <= 0x7FFFFFFF, "matrix too large");
+    switch (fmt) {
+    case CANDY_HIP_Q4_0:
+    case CANDY_HIP_Q4_0_GGML:
+        hipLaunchKernelGGL(k_wquant_q4_0, dim3((unsigned)grid), dim3(256), 0, dev->stream, dev_x, nb,
+                           (BlockQ4_0 *)dev_out_blocks, fmt == CANDY_HIP_Q4_0_GGML ? 1 : 0);
+        break;
+    case CANDY_HIP_Q4_K:
+        hipLaunchKernelGGL(k_wquant_q4_k, dim3((unsigned)grid), dim3(64), 0, dev->stream, dev_x, nb, (BlockQ4K *)dev_out_blocks);
+        break;
+    case CANDY_HIP_Q6_K:
+        hipLaunchKernelGGL(k_wquant_q6_k, dim3((unsigned)grid), dim3(64), 0, dev->stream, dev_x, nb, (BlockQ6K *)dev_out_blocks);
+        break;
+    default: CANDY_REQUIRE(false, "no quantizer for format %d", fmt);
+    }
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}

@@ -60,6 +60,7 @@ SIGNATURES = {
     "candy_hip_dequantize_blocks": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "candy_hip_dequantize": (c_int, [c_void_p, c_void_p, c_void_p]),
     "candy_hip_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "candy_hip_quantize": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p]),
     "candy_hip_qmatmul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "candy_hip_qmatmul_q8": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "candy_hip_qact_create": (c_int, [c_void_p, c_int64, c_int64, POINTER(c_void_p)]),
@@ -178,6 +179,22 @@ class QTensor:
         _check(lib().candy_hip_qtensor_upload(dev.handle, fmt, rows, cols, b.ctypes.data, b.nbytes, byref(h)))
         self.dev, self.fmt, self.rows, self.cols, self.nbytes, self.handle = dev, fmt, rows, cols, b.nbytes, h.value
 
+    @classmethod
+    def quantize(cls, dev: "Device", fmt: int, x: np.ndarray) -> "QTensor":
+        """f32 [rows, cols] -> a weight of format fmt, quantized on the device and kept there."""
+        x = np.ascontiguousarray(x, np.float32)
+        rows, cols = x.reshape(-1, x.shape[-1]).shape
+        nbytes = lib().candy_hip_qweight_bytes(fmt, rows, cols)
+        src = dev.from_numpy(x)
+        dst = dev.alloc(max(nbytes, 2))
+        _check(lib().candy_hip_quantize(dev.handle, fmt, src.ptr, rows, cols, dst.ptr))
+        q = cls.__new__(cls)
+        h = c_void_p()
+        _check(lib().candy_hip_qtensor_wrap(dev.handle, fmt, rows, cols, dst.ptr, nbytes, byref(h)))
+        q.dev, q.fmt, q.rows, q.cols, q.nbytes, q.handle = dev, fmt, rows, cols, nbytes, h.value
+        q._blocks = dst  # the wrapped device memory stays owned here
+        return q
+
     def free(self):
         if self.handle is not None and self.dev.handle is not None:
             _check(lib().candy_hip_qtensor_free(self.handle))
@@ -245,6 +262,17 @@ class Device:
         dst = self.alloc(max(rows * cols // 32 * 34, 2))
         _check(lib().candy_hip_quantize_q8_0(self.handle, src.ptr, rows, cols, dst.ptr))
         return dst.download(np.uint8, rows * cols // 32 * 34)
+
+    def quantize(self, fmt: int, x: np.ndarray) -> np.ndarray:
+        """f32 [rows, cols] -> the blocks of format fmt (host bytes), quantized on the device."""
+        x = np.ascontiguousarray(x, np.float32)
+        x2 = x.reshape(-1, x.shape[-1]) if x.ndim > 1 else x.reshape(1, -1)
+        rows, cols = x2.shape
+        nbytes = lib().candy_hip_qweight_bytes(fmt, rows, cols)
+        src = self.from_numpy(x2)
+        dst = self.alloc(max(nbytes, 2))
+        _check(lib().candy_hip_quantize(self.handle, fmt, src.ptr, rows, cols, dst.ptr))
+        return dst.download(np.uint8, nbytes)
 
     def qmatmul(self, w: QTensor, x: np.ndarray) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32).reshape(-1, w.cols)

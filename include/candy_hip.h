@@ -99,6 +99,14 @@ int candy_hip_dequantize(candy_hip_device *dev, const candy_hip_qtensor *q, floa
 int candy_hip_quantize_q8_0(candy_hip_device *dev, const float *dev_x, int64_t rows, int64_t cols,
                             void *dev_out_blocks);
 
+/* Weight quantizer: f32 [rows, cols] (device) -> blocks of fmt (device, rows*cols/qk of them), cols a
+ * multiple of the block.  candy only names these kernels (tensor/internal/metal/kernels/kernels.go:563-592,
+ * quantize_q4_0 ... quantize_q6_k) and has no implementation; the arithmetic is ggml's reference
+ * quantizers (quantize_row_q4_0_ref, quantize_row_q4_K_ref, quantize_row_q6_K_ref), step for step in f32;
+ * Q8_0 is candy_hip_quantize_q8_0.  Wrap the result with candy_hip_qtensor_wrap.  Inputs must be finite. */
+int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64_t rows, int64_t cols,
+                       void *dev_out_blocks);
+
 /* y[m, rows] = x[m, cols] . W^T, activations quantized to Q8_0 on the device first.
  * m < 16 runs the bandwidth-bound matvec family (QCU:2787-2871 mul_mat_vec_q and its entry
  * points :2874, :2906, :2930, :2946); m >= 16 the MFMA tile kernel (QCU:455-578 mul_mat_q).

@@ -33,6 +33,20 @@
  *   co_dequantize Q6_K    QCU:1103-1128. Pinned: exact value in Fractions.
  *   co_quantize_q8_0      QCU:3521-3558 without the `sum` half. Pinned: float64 evaluation
  *                         of round-half-away(x/d) with numpy float32 division; invariants.
+ *   co_quantize (Q4_0 / Q4_0_GGML / Q4_K / Q6_K)
+ *                         PARITY UNPINNED against the original.  candy has no quantizer from f32
+ *                         (only kernel names, tensor/internal/metal/kernels/kernels.go:563-592);
+ *                         the algorithm is ggml's published reference quantizer, which is not in
+ *                         the checkout: quantize_row_q4_0_ref, quantize_row_q4_K_ref with
+ *                         make_qkx2_quants, quantize_row_q6_K_ref with make_qx_quants
+ *                         (ggml/src/ggml-quants.c of llama.cpp, 2024 releases; candle's
+ *                         k_quants.rs `from_float` is a port of the same).  Restated here from
+ *                         the published algorithm.  What the tests do pin: Q4_0 against an
+ *                         independent numpy evaluation of its closed form; for the K formats the
+ *                         level-assignment pass against the stored scales (recomputed from the
+ *                         block in Fractions), the error bound of the result, that the searched
+ *                         scale is never worse in the weighted objective than plain rounding,
+ *                         special blocks (zeros, constants, a single spike), and determinism.
  *   co_vec_dot_q8_0       QCU:2058-2073, 2239-2263, 2367-2389 (shape of the float
  *                         combination); integer parts pinned with Python ints, the float
  *                         result against exact-arithmetic sum of dequantized products.
@@ -247,6 +261,279 @@ int co_quantize_q8_0(const float *x, int64_t rows, int64_t cols, void *out_block
         out[b].d = co_f32_to_fp16(d);
     }
     return 0;
+}
+
+/* ---- weight quantizers from f32 (ggml's reference quantizers, see the header: parity unpinned) ---- */
+
+/* Round to nearest, ties to even, by the 1.5 * 2^23 trick; |f| <= 4194303. */
+static int nearest_int(float f) {
+    const float v = f + 12582912.0f;
+    return (int)(f32_to_bits(v) & 0x007FFFFFu) - 0x00400000;
+}
+
+/* quantize_row_q4_0_ref: the element of largest magnitude maps to level -8 (so d carries its sign);
+ * levels are (int8)(x / d + 8.5) capped at 15.  ggml_order: low nibbles hold elements 0..15 and high
+ * nibbles 16..31 (QCU:862-866); otherwise candy's CPU order, byte i = elements 2i, 2i+1 (QGO:85-93). */
+static void quantize_block_q4_0(const float *x, co_block_q4_0 *y, int ggml_order) {
+    float amax = 0.0f, max = 0.0f;
+    for (int j = 0; j < 32; ++j) {
+        const float v = x[j];
+        if (amax < fabsf(v)) { amax = fabsf(v); max = v; }
+    }
+    const float d = max / -8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    y->d = co_f32_to_fp16(d);
+    uint8_t q[32];
+    for (int j = 0; j < 32; ++j) {
+        const int v = (int)(int8_t)(x[j] * id + 8.5f);
+        q[j] = (uint8_t)(v < 15 ? v : 15);
+    }
+    for (int j = 0; j < 16; ++j)
+        y->qs[j] = ggml_order ? (uint8_t)(q[j] | (q[j + 16] << 4)) : (uint8_t)(q[2 * j] | (q[2 * j + 1] << 4));
+}
+
+/* make_qkx2_quants: levels 0..nmax with scale and (non-positive) minimum for n values; starts from
+ * min/max rounding and tries nstep+1 nearby scales, each followed by the weighted least-squares fit
+ * of (scale, min) to the levels it yields; keeps the best weighted squared error.  Returns the scale,
+ * *the_min receives -min (>= 0). */
+static float make_qkx2_quants(int n, int nmax, const float *x, const float *weights, uint8_t *L, float *the_min,
+                              uint8_t *Laux, float rmin, float rdelta, int nstep) {
+    float min = x[0], max = x[0];
+    float sum_w = weights[0], sum_x = sum_w * x[0];
+    for (int i = 1; i < n; ++i) {
+        if (x[i] < min) min = x[i];
+        if (x[i] > max) max = x[i];
+        const float w = weights[i];
+        sum_w += w;
+        sum_x += w * x[i];
+    }
+    if (min > 0.0f) min = 0.0f;
+    if (max == min) {
+        for (int i = 0; i < n; ++i) L[i] = 0;
+        *the_min = -min;
+        return 0.0f;
+    }
+    float iscale = (float)nmax / (max - min);
+    float scale = 1.0f / iscale;
+    float best = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        int l = nearest_int(iscale * (x[i] - min));
+        l = l < 0 ? 0 : (l > nmax ? nmax : l);
+        L[i] = (uint8_t)l;
+        float diff = scale * (float)L[i] + min - x[i];
+        diff = diff * diff;
+        best += weights[i] * diff;
+    }
+    if (nstep < 1) {
+        *the_min = -min;
+        return scale;
+    }
+    for (int is = 0; is <= nstep; ++is) {
+        iscale = (rmin + rdelta * (float)is + (float)nmax) / (max - min);
+        float sum_l = 0.0f, sum_l2 = 0.0f, sum_xl = 0.0f;
+        for (int i = 0; i < n; ++i) {
+            int l = nearest_int(iscale * (x[i] - min));
+            l = l < 0 ? 0 : (l > nmax ? nmax : l);
+            Laux[i] = (uint8_t)l;
+            const float w = weights[i];
+            sum_l += w * (float)l;
+            sum_l2 += w * (float)l * (float)l;
+            sum_xl += w * (float)l * x[i];
+        }
+        const float D = sum_w * sum_l2 - sum_l * sum_l;
+        if (D > 0.0f) {
+            float this_scale = (sum_w * sum_xl - sum_x * sum_l) / D;
+            float this_min = (sum_l2 * sum_x - sum_l * sum_xl) / D;
+            if (this_min > 0.0f) {
+                this_min = 0.0f;
+                this_scale = sum_xl / sum_l2;
+            }
+            float mad = 0.0f;
+            for (int i = 0; i < n; ++i) {
+                float diff = this_scale * (float)Laux[i] + this_min - x[i];
+                diff = diff * diff;
+                mad += weights[i] * diff;
+            }
+            if (mad < best) {
+                for (int i = 0; i < n; ++i) L[i] = Laux[i];
+                best = mad;
+                scale = this_scale;
+                min = this_min;
+            }
+        }
+    }
+    *the_min = -min;
+    return scale;
+}
+
+/* quantize_row_q4_K_ref for one super-block: eight 32-value sub-blocks get (scale, min) from
+ * make_qkx2_quants with weights rms + |x|; scales and mins are stored in 6 bits relative to their
+ * maxima (d, dmin in fp16), then the levels are assigned again with the STORED scales. */
+static void quantize_block_q4_k(const float *x, co_block_q4_k *y) {
+    uint8_t L[256], Laux[32];
+    float weights[32], mins[8], scales[8];
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int j = 0; j < 8; ++j) {
+        float sum_x2 = 0.0f;
+        for (int l = 0; l < 32; ++l) sum_x2 += x[32 * j + l] * x[32 * j + l];
+        const float av_x = sqrtf(sum_x2 / 32.0f);
+        for (int l = 0; l < 32; ++l) weights[l] = av_x + fabsf(x[32 * j + l]);
+        scales[j] = make_qkx2_quants(32, 15, x + 32 * j, weights, L + 32 * j, &mins[j], Laux, -1.0f, 0.1f, 20);
+        if (scales[j] > max_scale) max_scale = scales[j];
+        if (mins[j] > max_min) max_min = mins[j];
+    }
+    const float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    memset(y->scales, 0, sizeof(y->scales));
+    for (int j = 0; j < 8; ++j) {
+        int ls = nearest_int(inv_scale * scales[j]);
+        int lm = nearest_int(inv_min * mins[j]);
+        ls = ls < 63 ? ls : 63;
+        lm = lm < 63 ? lm : 63;
+        if (j < 4) {
+            y->scales[j] = (uint8_t)ls;
+            y->scales[j + 4] = (uint8_t)lm;
+        } else {
+            y->scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+            y->scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+            y->scales[j] |= (uint8_t)((lm >> 4) << 6);
+        }
+    }
+    y->dm[0] = co_f32_to_fp16(max_scale / 63.0f);
+    y->dm[1] = co_f32_to_fp16(max_min / 63.0f);
+    for (int j = 0; j < 8; ++j) {
+        uint8_t sc, m;
+        co_get_scale_min_k4(j, y->scales, &sc, &m);
+        const float d = co_fp16_to_f32(y->dm[0]) * (float)sc;
+        if (d == 0.0f) continue;  /* keeps the levels of the search */
+        const float dm = co_fp16_to_f32(y->dm[1]) * (float)m;
+        for (int ii = 0; ii < 32; ++ii) {
+            int l = nearest_int((x[32 * j + ii] + dm) / d);
+            l = l < 0 ? 0 : (l > 15 ? 15 : l);
+            L[32 * j + ii] = (uint8_t)l;
+        }
+    }
+    uint8_t *q = y->qs;
+    for (int j = 0; j < 256; j += 64) {
+        for (int l = 0; l < 32; ++l) q[l] = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
+        q += 32;
+    }
+}
+
+/* make_qx_quants with rmse_type 1 (weights x^2) and no external weights: symmetric levels
+ * -nmax..nmax-1 stored as L = level + nmax; the value of largest magnitude maps to -nmax; 18 nearby
+ * scales are tried and the one with the largest (sum w x l)^2 / (sum w l^2) kept. */
+static float make_qx_quants(int n, int nmax, const float *x, int8_t *L) {
+    float max = 0.0f, amax = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        const float ax = fabsf(x[i]);
+        if (ax > amax) { amax = ax; max = x[i]; }
+    }
+    if (amax < 1e-15f) {
+        for (int i = 0; i < n; ++i) L[i] = 0;
+        return 0.0f;
+    }
+    float iscale = -(float)nmax / max;
+    float sumlx = 0.0f, suml2 = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        int l = nearest_int(iscale * x[i]);
+        l = l < -nmax ? -nmax : (l > nmax - 1 ? nmax - 1 : l);
+        L[i] = (int8_t)(l + nmax);
+        const float w = x[i] * x[i];
+        sumlx += w * x[i] * (float)l;
+        suml2 += w * (float)l * (float)l;
+    }
+    float scale = suml2 != 0.0f ? sumlx / suml2 : 0.0f;
+    float best = scale * sumlx;
+    for (int is = -9; is <= 9; ++is) {
+        if (is == 0) continue;
+        iscale = -((float)nmax + 0.1f * (float)is) / max;
+        sumlx = suml2 = 0.0f;
+        for (int i = 0; i < n; ++i) {
+            int l = nearest_int(iscale * x[i]);
+            l = l < -nmax ? -nmax : (l > nmax - 1 ? nmax - 1 : l);
+            const float w = x[i] * x[i];
+            sumlx += w * x[i] * (float)l;
+            suml2 += w * (float)l * (float)l;
+        }
+        if (suml2 > 0.0f && sumlx * sumlx > best * suml2) {
+            for (int i = 0; i < n; ++i) {
+                int l = nearest_int(iscale * x[i]);
+                l = l < -nmax ? -nmax : (l > nmax - 1 ? nmax - 1 : l);
+                L[i] = (int8_t)(nmax + l);
+            }
+            scale = sumlx / suml2;
+            best = scale * sumlx;
+        }
+    }
+    return scale;
+}
+
+/* quantize_row_q6_K_ref for one super-block: sixteen 16-value groups, each with a make_qx_quants
+ * scale; the scale of largest magnitude maps to -128 in int8 (d in fp16 carries its sign), then
+ * the levels -32..31 are assigned again with the STORED scales and packed as QCU:1103-1128 reads them. */
+static void quantize_block_q6_k(const float *x, co_block_q6_k *y) {
+    int8_t L[256];
+    float scales[16];
+    float max_scale = 0.0f, max_abs_scale = 0.0f;
+    for (int ib = 0; ib < 16; ++ib) {
+        const float scale = make_qx_quants(16, 32, x + 16 * ib, L + 16 * ib);
+        scales[ib] = scale;
+        const float abs_scale = fabsf(scale);
+        if (abs_scale > max_abs_scale) { max_abs_scale = abs_scale; max_scale = scale; }
+    }
+    if (max_abs_scale < 1e-15f) {
+        memset(y, 0, sizeof(*y));
+        return;
+    }
+    const float iscale = -128.0f / max_scale;
+    y->d = co_f32_to_fp16(1.0f / iscale);
+    for (int ib = 0; ib < 16; ++ib) {
+        const int v = nearest_int(iscale * scales[ib]);
+        y->scales[ib] = (int8_t)(v < 127 ? v : 127);
+    }
+    for (int j = 0; j < 16; ++j) {
+        const float d = co_fp16_to_f32(y->d) * (float)y->scales[j];
+        if (d == 0.0f) continue;
+        for (int ii = 0; ii < 16; ++ii) {
+            int l = nearest_int(x[16 * j + ii] / d);
+            l = l < -32 ? -32 : (l > 31 ? 31 : l);
+            L[16 * j + ii] = (int8_t)(l + 32);
+        }
+    }
+    uint8_t *ql = y->ql, *qh = y->qh;
+    for (int j = 0; j < 256; j += 128) {
+        for (int l = 0; l < 32; ++l) {
+            const uint8_t q1 = (uint8_t)L[j + l] & 0xF, q2 = (uint8_t)L[j + l + 32] & 0xF;
+            const uint8_t q3 = (uint8_t)L[j + l + 64] & 0xF, q4 = (uint8_t)L[j + l + 96] & 0xF;
+            ql[l] = (uint8_t)(q1 | (q3 << 4));
+            ql[l + 32] = (uint8_t)(q2 | (q4 << 4));
+            qh[l] = (uint8_t)(((uint8_t)L[j + l] >> 4) | (((uint8_t)L[j + l + 32] >> 4) << 2) |
+                              (((uint8_t)L[j + l + 64] >> 4) << 4) | (((uint8_t)L[j + l + 96] >> 4) << 6));
+        }
+        ql += 64;
+        qh += 32;
+    }
+}
+
+int co_quantize(int fmt, const float *x, int64_t rows, int64_t cols, void *out_blocks) {
+    const int qk = co_block_elems(fmt);
+    if (qk == 0 || rows < 0 || cols < 0 || cols % qk != 0) return -1;
+    const int64_t nb = rows * cols / qk;
+    switch (fmt) {
+    case CO_Q8_0: return co_quantize_q8_0(x, rows, cols, out_blocks);
+    case CO_Q4_0:
+    case CO_Q4_0_GGML:
+        for (int64_t b = 0; b < nb; ++b) quantize_block_q4_0(x + 32 * b, (co_block_q4_0 *)out_blocks + b, fmt == CO_Q4_0_GGML);
+        return 0;
+    case CO_Q4_K:
+        for (int64_t b = 0; b < nb; ++b) quantize_block_q4_k(x + 256 * b, (co_block_q4_k *)out_blocks + b);
+        return 0;
+    case CO_Q6_K:
+        for (int64_t b = 0; b < nb; ++b) quantize_block_q6_k(x + 256 * b, (co_block_q6_k *)out_blocks + b);
+        return 0;
+    default: return -1;
+    }
 }
 
 /* ---- integer vec-dots against Q8_0 activation blocks ---- */

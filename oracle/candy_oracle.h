@@ -46,6 +46,10 @@ int co_dequantize(int fmt, const void *blocks, int64_t n_blocks, float *y);
 /* x: rows*cols f32, cols % 32 == 0. out: rows*cols/32 Q8_0 blocks (34 B each). */
 int co_quantize_q8_0(const float *x, int64_t rows, int64_t cols, void *out_blocks);
 
+/* Weight quantizer from f32 for any of the formats (ggml's reference quantizers; Q8_0 is the one
+ * above): x is rows*cols f32, cols a multiple of the block; out receives rows*cols/qk blocks. */
+int co_quantize(int fmt, const float *x, int64_t rows, int64_t cols, void *out_blocks);
+
 /* One weight row (k/qk blocks) against one activation row (k/32 Q8_0 blocks). */
 float co_vec_dot_q8_0(int fmt, const void *w_row, const void *x_q8_0, int64_t k);
 

@@ -45,6 +45,8 @@ def lib() -> ctypes.CDLL:
         L.co_get_scale_min_k4.restype = None
         L.co_dequantize.argtypes = [ctypes.c_int, vp, i64, vp]
         L.co_quantize_q8_0.argtypes = [vp, i64, i64, vp]
+        L.co_quantize.argtypes = [ctypes.c_int, vp, i64, i64, vp]
+        L.co_quantize.restype = ctypes.c_int
         L.co_vec_dot_q8_0.argtypes = [ctypes.c_int, vp, vp, i64]
         L.co_vec_dot_q8_0.restype = f32
         L.co_qmatmul.argtypes = [ctypes.c_int, vp, i64, i64, vp, i64, vp]
@@ -131,6 +133,20 @@ def quantize_q8_0(x, rows: int | None = None, cols: int | None = None) -> np.nda
     out = np.empty(rows * cols // 32 * 34, np.uint8)
     rc = lib().co_quantize_q8_0(_p(x), rows, cols, _p(out))
     assert rc == 0, "cols must be a multiple of 32"
+    return out
+
+
+def quantize(fmt: int, x, rows: int | None = None, cols: int | None = None) -> np.ndarray:
+    """f32 [rows, cols] -> blocks of fmt (ggml's reference quantizers; parity unpinned, see candy_oracle.c)."""
+    x = _f32(x)
+    if rows is None:
+        x2 = x.reshape(-1, x.shape[-1]) if x.ndim > 1 else x.reshape(1, -1)
+        rows, cols = x2.shape
+    qk = block_elems(fmt)
+    assert qk and cols % qk == 0, "cols must be a multiple of the block"
+    out = np.empty(rows * cols // qk * block_bytes(fmt), np.uint8)
+    rc = lib().co_quantize(fmt, _p(x), rows, cols, _p(out))
+    assert rc == 0
     return out
 
 
