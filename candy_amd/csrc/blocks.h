@@ -27,6 +27,45 @@ struct __attribute__((packed)) BlockQ6K {
     int8_t scales[16];
     uint16_t d;
 };
+// quantized.go:13-31, 39-52, 62-67, 78-82
+struct __attribute__((packed)) BlockQ4_1 {
+    uint16_t d, m;
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ5_0 {
+    uint16_t d;
+    uint8_t qh[4];
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ5_1 {
+    uint16_t d, m;
+    uint8_t qh[4];
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ2K {
+    uint8_t scales[16];
+    uint8_t qs[64];
+    uint16_t d, dmin;
+};
+struct __attribute__((packed)) BlockQ3K {
+    uint8_t hmask[32];
+    uint8_t qs[64];
+    uint8_t scales[12];
+    uint16_t d;
+};
+struct __attribute__((packed)) BlockQ5K {
+    uint16_t d, dmin;
+    uint8_t scales[12];
+    uint8_t qh[32];
+    uint8_t qs[128];
+};
+struct __attribute__((packed)) BlockQ8K {
+    float d;
+    int8_t qs[256];
+    int16_t bsums[16];
+};
+static_assert(sizeof(BlockQ4_1) == 20 && sizeof(BlockQ5_0) == 22 && sizeof(BlockQ5_1) == 24, "block size");
+static_assert(sizeof(BlockQ2K) == 84 && sizeof(BlockQ3K) == 110 && sizeof(BlockQ5K) == 176 && sizeof(BlockQ8K) == 292, "block size");
 static_assert(sizeof(BlockQ4_0) == 18 && sizeof(BlockQ8_0) == 34, "block size");
 static_assert(sizeof(BlockQ4K) == 144 && sizeof(BlockQ6K) == 210, "block size");
 

@@ -101,6 +101,12 @@ int use_device(const candy_hip_device *dev);
 int workspace(candy_hip_device *dev, size_t bytes, void **out);
 // Second buffer, for the split-K partial sums (lives beside the activation workspace).
 int splitk_workspace(candy_hip_device *dev, size_t bytes, void **out);
+// Formats with the per-length batch-1 kernels (residual epilogue, several weights per launch) and the fused
+// decode kernels; the others contract through the general small-batch kernel.
+inline bool format_has_batch1_kernel(int fmt) {
+    return fmt == CANDY_HIP_Q4_K || fmt == CANDY_HIP_Q6_K || fmt == CANDY_HIP_Q8_0 || fmt == CANDY_HIP_Q4_0 ||
+           fmt == CANDY_HIP_Q4_0_GGML;
+}
 
 // quant.hip: x[rows, cols] -> planar int8 quants + scales; optionally also 34-byte blocks.
 // xh (optional): also the fp16 values d * q, row-major like x (what the fp16 tile kernels contract with).

@@ -29,6 +29,7 @@ struct candy_hip_llama {
     float *cos_t = nullptr, *sin_t = nullptr;      // [max_pos][head_dim/2]
     float *h = nullptr, *q = nullptr, *k = nullptr, *v = nullptr;
     float *gate_o = nullptr, *up_o = nullptr, *logits = nullptr;
+    float *proj = nullptr;  // [d_model]: a projection's output before the residual add, for formats without that epilogue
     int8_t *xq = nullptr;           // planar Q8_0 quants of the current activation
     candy::Q8Scale *xs = nullptr;
     uint32_t *next_tok = nullptr;   // [2]: greedy token, then the persistent kernel's time-out flag
@@ -128,6 +129,7 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
     if (!rc) rc = dev_alloc(m, &m->k, (size_t)cfg->n_kv_heads * cfg->head_dim);
     if (!rc) rc = dev_alloc(m, &m->v, (size_t)cfg->n_kv_heads * cfg->head_dim);
     if (!rc) rc = dev_alloc(m, &m->gate_o, (size_t)cfg->d_ffn);
+    if (!rc) rc = dev_alloc(m, &m->proj, (size_t)cfg->d_model);
     if (!rc) rc = dev_alloc(m, &m->up_o, (size_t)cfg->d_ffn);
     if (!rc) rc = dev_alloc(m, &m->logits, (size_t)cfg->vocab);
     if (!rc) rc = dev_alloc(m, &m->xq, widest);
@@ -307,7 +309,10 @@ static int linear_residual(candy_hip_llama *m, const candy_hip_qtensor *w) {
     const candy_hip_qtensor *ws[1] = {w};
     float *ys[1] = {m->h};
     const float *res[1] = {m->h};
-    return launch_matvec_multi(m->dev, ws, ys, res, 1, m->xq, m->xs);
+    if (format_has_batch1_kernel(w->fmt)) return launch_matvec_multi(m->dev, ws, ys, res, 1, m->xq, m->xs);
+    // the other formats: general kernel into a buffer of its own, then the add
+    if ((rc = launch_matvec(m->dev, w, m->xq, m->xs, 1, m->proj))) return rc;
+    return candy_hip_add(m->dev, m->h, m->proj, w->rows, m->h);
 }
 
 // Enqueues one decode step (hidden state in m->h, position in *m->d_pos) on the stream: six

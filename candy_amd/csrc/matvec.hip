@@ -19,6 +19,7 @@
 #include "blocks.h"
 #include "internal.h"
 #include "units.h"
+#include "formats_more.h"
 
 namespace candy {
 
@@ -323,7 +324,9 @@ static int launch_jobs(candy_hip_device *dev, int fmt, const MatvecJobs &jobs, i
     case CANDY_HIP_Q4_0: return launch_jobs_fmt<UnitQ4_0<false>>(dev, jobs, K, qs, scales);
     case CANDY_HIP_Q4_0_GGML: return launch_jobs_fmt<UnitQ4_0<true>>(dev, jobs, K, qs, scales);
     case CANDY_HIP_Q6_K: return launch_jobs_fmt<UnitQ6K>(dev, jobs, K, qs, scales);
-    default: return fail(CANDY_HIP_ERR_INVALID, "unknown quantized format %d", fmt);
+    default:
+        if (format_info(fmt).elems != 0) return CANDY_HIP_ERR_UNSUPPORTED;  // the other formats: one launch per weight
+        return fail(CANDY_HIP_ERR_INVALID, "unknown quantized format %d", fmt);
     }
 }
 
@@ -342,19 +345,29 @@ static int launch_one(candy_hip_device *dev, const candy_hip_qtensor *w, const i
     return CANDY_HIP_OK;
 }
 
+// Units of the secondary formats go through the general kernel only (no per-length batch-1 variants).
+template <class U, class = void>
+struct GeneralOnly { static constexpr bool value = false; };
+template <class U>
+struct GeneralOnly<U, std::enable_if_t<U::GENERAL_ONLY>> { static constexpr bool value = true; };
+template <class U>
+static constexpr bool general_only() { return GeneralOnly<U>::value; }
+
 template <class U>
 static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                       int64_t m, float *y) {
     const int64_t K = w->cols, N = w->rows;
     const int64_t sstride = K >> 5;
-    if (m == 1) {
-        MatvecJobs jobs{};
-        jobs.n = 1;
-        jobs.j[0].W = (const uint8_t *)w->data;
-        jobs.j[0].y = y;
-        jobs.j[0].N = (int)N;
-        const int rc = launch_jobs_fmt<U>(dev, jobs, K, qs, scales);
-        if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+    if constexpr (!general_only<U>()) {
+        if (m == 1) {
+            MatvecJobs jobs{};
+            jobs.n = 1;
+            jobs.j[0].W = (const uint8_t *)w->data;
+            jobs.j[0].y = y;
+            jobs.j[0].N = (int)N;
+            const int rc = launch_jobs_fmt<U>(dev, jobs, K, qs, scales);
+            if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+        }
     }
     int64_t done = 0;
     while (done < m) {
@@ -422,6 +435,14 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
     case CANDY_HIP_Q4_0: return launch_fmt<UnitQ4_0<false>>(dev, w, qs, scales, m, y);
     case CANDY_HIP_Q4_0_GGML: return launch_fmt<UnitQ4_0<true>>(dev, w, qs, scales, m, y);
     case CANDY_HIP_Q6_K: return launch_fmt<UnitQ6K>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q4_1: return launch_fmt<UnitQ4_1<false>>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q4_1_GGML: return launch_fmt<UnitQ4_1<true>>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q5_0: return launch_fmt<UnitQ5<false>>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q5_1: return launch_fmt<UnitQ5<true>>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q2_K: return launch_fmt<UnitQ2K>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q3_K: return launch_fmt<UnitQ3K>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q5_K: return launch_fmt<UnitQ5K>(dev, w, qs, scales, m, y);
+    case CANDY_HIP_Q8_K: return fail(CANDY_HIP_ERR_UNSUPPORTED, "Q8_K weights only dequantize (the reference has no vec-dot for them)");
     default: return fail(CANDY_HIP_ERR_INVALID, "unknown quantized format %d", w->fmt);
     }
 }

@@ -317,6 +317,10 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     const int64_t K = w->cols;
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && K <= 0x7FFFFFFF && m <= 0x7FFFFFFF, "matrix too large");
     if (K % 64 != 0) return launch_matvec(dev, w, qs, scales, m, y);  // odd block counts: small-batch kernel in slices
+    switch (w->fmt) {  // the formats with tile kernels; the others contract in slices of the small-batch kernel
+    case CANDY_HIP_Q4_K: case CANDY_HIP_Q6_K: case CANDY_HIP_Q8_0: case CANDY_HIP_Q4_0: case CANDY_HIP_Q4_0_GGML: break;
+    default: return launch_matvec(dev, w, qs, scales, m, y);
+    }
     // prompt-sized batches of Q4_K: big fp16 tiles (the integer kernel is bound by its per-sub-block rescale there);
     // smaller batches of Q4_K and Q6_K: int8 matrix cores (exact); the fp16 tile kernel below serves the rest
     const bool force_fp16 = force_old_fp16();

@@ -2,6 +2,7 @@
 // definitions: every product in the dequantizers is exact in f32 (fp16 scale times small
 // integers), so instruction selection cannot change a result.
 #include "blocks.h"
+#include "formats_more.h"
 #include "internal.h"
 
 namespace candy {
@@ -198,6 +199,41 @@ __global__ __launch_bounds__(256) void k_dequant_q6_k(const BlockQ6K *__restrict
     for (int qd = 0; qd < 4; ++qd) out[8 * qd] = make_float4(o[qd][0], o[qd][1], o[qd][2], o[qd][3]);
 }
 
+// The other formats: one lane per float4 of output, F::quad gives values 4j .. 4j+3 of a block.
+template <class F>
+__global__ __launch_bounds__(256) void k_dequant_more(const uint8_t *__restrict__ blocks, int64_t nb,
+                                                      const int64_t *__restrict__ ids, int64_t bpr, float4 *__restrict__ y) {
+    constexpr int LPB = F::ELEMS / 4;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = t / LPB;
+    if (b >= nb) return;
+    y[t] = F::quad(blocks + src_block(b, ids, bpr) * F::BYTES, (int)(t - b * LPB));
+}
+
+template <class F>
+static int launch_dequant_more(candy_hip_device *dev, const void *blocks, int64_t nb, const int64_t *ids, int64_t bpr, float *out) {
+    const int64_t grid = (nb * (F::ELEMS / 4) + 255) / 256;
+    CANDY_REQUIRE(grid <= 0x7FFFFFFF, "too many blocks");
+    hipLaunchKernelGGL(k_dequant_more<F>, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const uint8_t *)blocks, nb, ids,
+                       bpr, (float4 *)out);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+// Alignment the block array of a format needs (its widest aligned load).
+static int block_alignment(int fmt) {
+    switch (fmt) {
+    case CANDY_HIP_Q4_K:
+    case CANDY_HIP_Q5_K: return 16;
+    case CANDY_HIP_Q4_1:
+    case CANDY_HIP_Q4_1_GGML:
+    case CANDY_HIP_Q5_1:
+    case CANDY_HIP_Q2_K:
+    case CANDY_HIP_Q8_K: return 4;
+    default: return 2;
+    }
+}
+
 }  // namespace candy
 
 using namespace candy;
@@ -212,8 +248,19 @@ static int dequantize_impl(candy_hip_device *dev, int fmt, const void *dev_block
     if (n_blocks == 0) return CANDY_HIP_OK;
     CANDY_REQUIRE(dev_blocks && dev_out, "nil pointer");
     CANDY_REQUIRE(((uintptr_t)dev_out & 15) == 0, "output must be 16-byte aligned");
-    CANDY_REQUIRE(((uintptr_t)dev_blocks & (fmt == CANDY_HIP_Q4_K ? 15 : 1)) == 0, "blocks are misaligned");
+    CANDY_REQUIRE(((uintptr_t)dev_blocks & (uintptr_t)(block_alignment(fmt) - 1)) == 0, "blocks are misaligned");
     if (int rc = use_device(dev)) return rc;
+    switch (fmt) {
+    case CANDY_HIP_Q4_1: return launch_dequant_more<FmtQ4_1<false>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q4_1_GGML: return launch_dequant_more<FmtQ4_1<true>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q5_0: return launch_dequant_more<FmtQ5<false>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q5_1: return launch_dequant_more<FmtQ5<true>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q2_K: return launch_dequant_more<FmtQ2K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q3_K: return launch_dequant_more<FmtQ3K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q5_K: return launch_dequant_more<FmtQ5K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q8_K: return launch_dequant_more<FmtQ8K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    default: break;
+    }
     const int lanes_per_block = fmt == CANDY_HIP_Q4_K ? 32 : fmt == CANDY_HIP_Q6_K ? 16 : fmt == CANDY_HIP_Q8_0 ? 8 : 4;
     const int64_t grid = (n_blocks * lanes_per_block + 255) / 256;
     CANDY_REQUIRE(grid <= 0x7FFFFFFF, "too many blocks");

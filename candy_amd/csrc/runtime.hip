@@ -35,6 +35,14 @@ FormatInfo format_info(int fmt) {
     case CANDY_HIP_Q8_0: return {32, 34};
     case CANDY_HIP_Q4_K: return {256, 144};
     case CANDY_HIP_Q6_K: return {256, 210};
+    case CANDY_HIP_Q4_1:
+    case CANDY_HIP_Q4_1_GGML: return {32, 20};
+    case CANDY_HIP_Q5_0: return {32, 22};
+    case CANDY_HIP_Q5_1: return {32, 24};
+    case CANDY_HIP_Q2_K: return {256, 84};
+    case CANDY_HIP_Q3_K: return {256, 110};
+    case CANDY_HIP_Q5_K: return {256, 176};
+    case CANDY_HIP_Q8_K: return {256, 292};
     default: return {0, 0};
     }
 }

@@ -39,7 +39,10 @@ GGML_TYPES = {
     12: ("Q4_K", 256, 144), 13: ("Q5_K", 256, 176), 14: ("Q6_K", 256, 210), 15: ("Q8_K", 256, 292),
 }
 # file type -> format id of the device path
-DEVICE_FORMATS = {GGML_Q4_0: synth.Q4_0_GGML, GGML_Q8_0: synth.Q8_0, GGML_Q4_K: synth.Q4_K, GGML_Q6_K: synth.Q6_K}
+DEVICE_FORMATS = {GGML_Q4_0: synth.Q4_0_GGML, GGML_Q8_0: synth.Q8_0, GGML_Q4_K: synth.Q4_K, GGML_Q6_K: synth.Q6_K,
+                  # files hold Q4_1 in ggml's element order too; the other ids are the device's own
+                  3: synth.Q4_1_GGML, 6: synth.Q5_0, 7: synth.Q5_1, 10: synth.Q2_K, 11: synth.Q3_K, 13: synth.Q5_K,
+                  15: synth.Q8_K}
 
 # metadata value types
 _U8, _I8, _U16, _I16, _U32, _I32, _F32, _BOOL, _STR, _ARR, _U64, _I64, _F64 = range(13)
@@ -171,7 +174,7 @@ class GGUFFile:
         t = self._info(name)
         if t.ggml_type not in DEVICE_FORMATS:
             raise GGUFError(f"tensor {name}: type {GGML_TYPES[t.ggml_type][0]} has no device kernels "
-                            "(Q4_0, Q8_0, Q4_K, Q6_K do)")
+                            "(Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K ... Q6_K, Q8_K do)")
         return DEVICE_FORMATS[t.ggml_type], t.rows, t.cols, self.raw(name)
 
     def _info(self, name: str) -> TensorInfo:

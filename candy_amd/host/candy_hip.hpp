@@ -276,7 +276,11 @@ private:
 };
 
 // ---------------------------------------------------------------- quantized weight + op
-enum class QFormat { Q4_0 = CANDY_HIP_Q4_0, Q8_0 = CANDY_HIP_Q8_0, Q4_K = CANDY_HIP_Q4_K, Q6_K = CANDY_HIP_Q6_K, Q4_0_GGML = CANDY_HIP_Q4_0_GGML };
+enum class QFormat {
+    Q4_0 = CANDY_HIP_Q4_0, Q8_0 = CANDY_HIP_Q8_0, Q4_K = CANDY_HIP_Q4_K, Q6_K = CANDY_HIP_Q6_K, Q4_0_GGML = CANDY_HIP_Q4_0_GGML,
+    Q4_1 = CANDY_HIP_Q4_1, Q4_1_GGML = CANDY_HIP_Q4_1_GGML, Q5_0 = CANDY_HIP_Q5_0, Q5_1 = CANDY_HIP_Q5_1,
+    Q2_K = CANDY_HIP_Q2_K, Q3_K = CANDY_HIP_Q3_K, Q5_K = CANDY_HIP_Q5_K, Q8_K = CANDY_HIP_Q8_K
+};
 
 class QTensor {
 public:

@@ -46,7 +46,19 @@ enum candy_hip_qformat {
     CANDY_HIP_Q8_0 = 8,
     CANDY_HIP_Q4_K = 12,
     CANDY_HIP_Q6_K = 14,
-    CANDY_HIP_Q4_0_GGML = 102  /* element order of QCU:862-866 / GGUF files (low half, high half)   */
+    CANDY_HIP_Q4_0_GGML = 102, /* element order of QCU:862-866 / GGUF files (low half, high half)   */
+    /* The reference's other block formats: dequantize, row gather and QMatMul at any batch through the
+     * general matvec kernel (no matrix-core tiles, no fused decode kernels).  Layouts QGO:13-31, 39-52,
+     * 62-67, 78-82; dequantize QGO:107-116 and QCU:728-795, 870-990, 1054-1102, 1178-1206; vec-dots
+     * QCU:1947-2053, 2108-2135, 2177-2209, 2300-2331. */
+    CANDY_HIP_Q4_1 = 3,        /* 20 B / 32; element order of candy's CPU dequantize, QGO:107-116 */
+    CANDY_HIP_Q4_1_GGML = 103, /* element order of QCU:870-899 / GGUF files */
+    CANDY_HIP_Q5_0 = 6,        /* 22 B / 32 */
+    CANDY_HIP_Q5_1 = 7,        /* 24 B / 32 */
+    CANDY_HIP_Q2_K = 10,       /* 84 B / 256 */
+    CANDY_HIP_Q3_K = 11,       /* 110 B / 256 */
+    CANDY_HIP_Q5_K = 13,       /* 176 B / 256 */
+    CANDY_HIP_Q8_K = 15        /* 292 B / 256; dequantize and row gather only (the reference has no weight vec-dot) */
 };
 
 /* ------------------------------------------------------------------ library / device
@@ -72,7 +84,7 @@ int candy_hip_d2d(candy_hip_device *dev, void *dst_dev, const void *src_dev, siz
 
 /* ------------------------------------------------------------------ block formats */
 int candy_hip_block_elems(int fmt);   /* 32 / 256, 0 if unknown                                   */
-int candy_hip_block_bytes(int fmt);   /* 18 / 34 / 144 / 210, 0 if unknown                        */
+int candy_hip_block_bytes(int fmt);   /* 18 / 34 / 144 / 210 / 20 / 22 / 24 / 84 / 110 / 176 / 292, 0 if unknown */
 /* bytes of a [rows, cols] weight, 0 if fmt is unknown or cols is not a multiple of the block */
 size_t candy_hip_qweight_bytes(int fmt, int64_t rows, int64_t cols);
 

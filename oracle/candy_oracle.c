@@ -31,6 +31,17 @@
  *                         byte-pair patterns.
  *   co_dequantize Q4_K    QCU:1008-1041. Pinned: exact value (one rounding) in Fractions.
  *   co_dequantize Q6_K    QCU:1103-1128. Pinned: exact value in Fractions.
+ *   co_dequantize Q4_1    QGO:107-116 (candy CPU order) and QCU:728-746 (ggml order). Pinned: exact
+ *                         rational values; the two orders are a permutation of each other.
+ *   co_dequantize Q5_0/Q5_1  QCU:749-795 through dequantize_block (QCU:1208-1216). Pinned: exact values.
+ *   co_dequantize Q2_K    QCU:902-935.   Pinned: exact value rounded once (Fractions).
+ *   co_dequantize Q3_K    QCU:936-990.   Pinned: exact value (no rounding happens: 17-bit scale x 3-bit level).
+ *   co_dequantize Q5_K    QCU:1054-1102. Pinned: exact value rounded once.
+ *   co_dequantize Q8_K    QCU:1178-1206. Pinned: exact value rounded once.
+ *   vec-dots of these     QCU:1947-2053 (Q4_1, Q5_0, Q5_1), 2108-2135 (Q2_K), 2177-2209 (Q3_K),
+ *                         2300-2331 (Q5_K): integer dot products per scale group, combined in f32 as the
+ *                         kernels do, the Q8_1 `sum` half replaced by the exact integer block sum.
+ *                         Pinned: against the exact-arithmetic sum of dequantized products.
  *   co_quantize_q8_0      QCU:3521-3558 without the `sum` half. Pinned: float64 evaluation
  *                         of round-half-away(x/d) with numpy float32 division; invariants.
  *   co_quantize (Q4_0 / Q4_0_GGML / Q4_K / Q6_K)
@@ -75,7 +86,18 @@ typedef struct { uint16_t d; uint8_t qs[16]; } co_block_q4_0;
 typedef struct { uint16_t d; int8_t qs[32]; } co_block_q8_0;
 typedef struct { uint16_t dm[2]; uint8_t scales[12]; uint8_t qs[128]; } co_block_q4_k;
 typedef struct { uint8_t ql[128]; uint8_t qh[64]; int8_t scales[16]; uint16_t d; } co_block_q6_k;
+/* QGO:13-31, 39-52, 62-67, 78-82; QCU:310-336, 370-390, 416-431, 447-452 */
+typedef struct { uint16_t dm[2]; uint8_t qs[16]; } co_block_q4_1;
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } co_block_q5_0;
+typedef struct { uint16_t dm[2]; uint8_t qh[4]; uint8_t qs[16]; } co_block_q5_1;
+typedef struct { uint8_t scales[16]; uint8_t qs[64]; uint16_t dm[2]; } co_block_q2_k;
+typedef struct { uint8_t hmask[32]; uint8_t qs[64]; uint8_t scales[12]; uint16_t d; } co_block_q3_k;
+typedef struct { uint16_t dm[2]; uint8_t scales[12]; uint8_t qh[32]; uint8_t qs[128]; } co_block_q5_k;
+typedef struct { float d; int8_t qs[256]; int16_t bsums[16]; } co_block_q8_k;
 #pragma pack(pop)
+_Static_assert(sizeof(co_block_q4_1) == 20 && sizeof(co_block_q5_0) == 22 && sizeof(co_block_q5_1) == 24, "32-value blocks");
+_Static_assert(sizeof(co_block_q2_k) == 84 && sizeof(co_block_q3_k) == 110, "q2_K / q3_K");
+_Static_assert(sizeof(co_block_q5_k) == 176 && sizeof(co_block_q8_k) == 292, "q5_K / q8_K");
 
 _Static_assert(sizeof(co_block_q4_0) == 18, "q4_0");
 _Static_assert(sizeof(co_block_q8_0) == 34, "q8_0");
@@ -85,7 +107,9 @@ _Static_assert(sizeof(co_block_q6_k) == 210, "q6_K");
 int co_block_elems(int fmt) {
     switch (fmt) {
     case CO_Q4_0: case CO_Q4_0_GGML: case CO_Q8_0: return 32;
+    case CO_Q4_1: case CO_Q4_1_GGML: case CO_Q5_0: case CO_Q5_1: return 32;
     case CO_Q4_K: case CO_Q6_K: return 256;
+    case CO_Q2_K: case CO_Q3_K: case CO_Q5_K: case CO_Q8_K: return 256;
     default: return 0;
     }
 }
@@ -96,6 +120,13 @@ int co_block_bytes(int fmt) {
     case CO_Q8_0: return 34;
     case CO_Q4_K: return 144;
     case CO_Q6_K: return 210;
+    case CO_Q4_1: case CO_Q4_1_GGML: return 20;
+    case CO_Q5_0: return 22;
+    case CO_Q5_1: return 24;
+    case CO_Q2_K: return 84;
+    case CO_Q3_K: return 110;
+    case CO_Q5_K: return 176;
+    case CO_Q8_K: return 292;
     default: return 0;
     }
 }
@@ -222,8 +253,130 @@ static void dequant_q6_k(const co_block_q6_k *b, float *y) {
     }
 }
 
+/* QGO:107-116: y[2j] = d*lo(qs[j]) + m, y[2j+1] = d*hi(qs[j]) + m */
+static void dequant_q4_1(const co_block_q4_1 *b, float *y) {
+    const float d = co_fp16_to_f32(b->dm[0]), m = co_fp16_to_f32(b->dm[1]);
+    for (int i = 0; i < 32; i += 2) {
+        y[i] = d * (float)(b->qs[i / 2] & 0xF) + m;
+        y[i + 1] = d * (float)(b->qs[i / 2] >> 4) + m;
+    }
+}
+
+/* QCU:728-746 placed by dequantize_block (QCU:870-899): y[j] = d*lo(qs[j]) + m, y[j+16] = d*hi(qs[j]) + m */
+static void dequant_q4_1_ggml(const co_block_q4_1 *b, float *y) {
+    const float d = co_fp16_to_f32(b->dm[0]), m = co_fp16_to_f32(b->dm[1]);
+    for (int j = 0; j < 16; ++j) {
+        y[j] = d * (float)(b->qs[j] & 0xF) + m;
+        y[j + 16] = d * (float)(b->qs[j] >> 4) + m;
+    }
+}
+
+/* the 5-bit level of element e (0..31): nibble of qs[e % 16] (low for e < 16), bit e of qh on top: QCU:756-763 */
+static int q5_level(const uint8_t *qs, const uint8_t *qh4, int e) {
+    uint32_t qh;
+    memcpy(&qh, qh4, 4);
+    const int nib = e < 16 ? (qs[e] & 0xF) : (qs[e - 16] >> 4);
+    return nib | (int)(((qh >> e) & 1u) << 4);
+}
+
+/* QCU:749-770: (level - 16) * d */
+static void dequant_q5_0(const co_block_q5_0 *b, float *y) {
+    const float d = co_fp16_to_f32(b->d);
+    for (int e = 0; e < 32; ++e) y[e] = ((float)q5_level(b->qs, b->qh, e) - 16.0f) * d;
+}
+
+/* QCU:773-795: level * d + m */
+static void dequant_q5_1(const co_block_q5_1 *b, float *y) {
+    const float d = co_fp16_to_f32(b->dm[0]), m = co_fp16_to_f32(b->dm[1]);
+    for (int e = 0; e < 32; ++e) y[e] = (float)q5_level(b->qs, b->qh, e) * d + m;
+}
+
+/* QCU:902-920: element 128n + 32k + l is bits 2k.. of qs[32n + l]; its 16-value group e/16 has a 4-bit
+ * scale (low nibble) and a 4-bit min (high nibble): y = dall*scale*q - dmin*min */
+static void dequant_q2_k(const co_block_q2_k *b, float *y) {
+    const float dall = co_fp16_to_f32(b->dm[0]), dmin = co_fp16_to_f32(b->dm[1]);
+    for (int e = 0; e < 256; ++e) {
+        const int n = e / 128, k = (e % 128) / 32, l = e % 32;
+        const uint8_t sc = b->scales[e / 16];
+        const int q = (b->qs[32 * n + l] >> (2 * k)) & 3;
+        y[e] = dall * (float)(sc & 0xF) * (float)q - dmin * (float)(sc >> 4);
+    }
+}
+
+/* the 6-bit scale of 16-value group is (0..15) of a Q3_K block: QCU:953-956 */
+static int q3k_scale(const uint8_t *sc, int is) {
+    if (is < 4) return (sc[is] & 0xF) | (((sc[is + 8] >> 0) & 3) << 4);
+    if (is < 8) return (sc[is] & 0xF) | (((sc[is + 4] >> 2) & 3) << 4);
+    if (is < 12) return (sc[is - 8] >> 4) | (((sc[is] >> 4) & 3) << 4);
+    return (sc[is - 8] >> 4) | (((sc[is - 4] >> 6) & 3) << 4);
+}
+
+/* the level -4..3 of element e = 128n + 32j + l: two bits of qs[32n + l], minus 4 unless bit 4n + j of hmask[l] is set */
+static int q3k_level(const co_block_q3_k *b, int e) {
+    const int n = e / 128, j = (e % 128) / 32, l = e % 32;
+    const int q = (b->qs[32 * n + l] >> (2 * j)) & 3;
+    return q - ((b->hmask[l] >> (4 * n + j)) & 1 ? 0 : 4);
+}
+
+/* QCU:936-966: y = d*(scale - 32) * level */
+static void dequant_q3_k(const co_block_q3_k *b, float *y) {
+    const float d_all = co_fp16_to_f32(b->d);
+    for (int e = 0; e < 256; ++e) {
+        const float dl = d_all * (float)(q3k_scale(b->scales, e / 16) - 32);
+        y[e] = dl * (float)q3k_level(b, e);
+    }
+}
+
+/* the 5-bit level of element e of a Q5_K block: sub-block t = e/32 takes the low (t even) or high nibble of
+ * qs[32*(t/2) + l] and bit t of qh[l]: QCU:1068-1087 */
+static int q5k_level(const co_block_q5_k *b, int e) {
+    const int t = e / 32, l = e % 32;
+    const uint8_t q = b->qs[32 * (t / 2) + l];
+    return ((t & 1) ? (q >> 4) : (q & 0xF)) + (((b->qh[l] >> t) & 1) ? 16 : 0);
+}
+
+/* QCU:1054-1087: y = (dall*sc)*level - dmin*m with the (sc, m) of the sub-block (get_scale_min_k4) */
+static void dequant_q5_k(const co_block_q5_k *b, float *y) {
+    const float dall = co_fp16_to_f32(b->dm[0]), dmin = co_fp16_to_f32(b->dm[1]);
+    for (int t = 0; t < 8; ++t) {
+        uint8_t sc, m;
+        co_get_scale_min_k4(t, b->scales, &sc, &m);
+        const float d1 = dall * (float)sc, m1 = dmin * (float)m;
+        for (int l = 0; l < 32; ++l) y[32 * t + l] = d1 * (float)q5k_level(b, 32 * t + l) - m1;
+    }
+}
+
+/* QCU:1178-1199: y = q * d, d in f32 */
+static void dequant_q8_k(const co_block_q8_k *b, float *y) {
+    for (int e = 0; e < 256; ++e) y[e] = (float)b->qs[e] * b->d;
+}
+
 int co_dequantize(int fmt, const void *blocks, int64_t n_blocks, float *y) {
     switch (fmt) {
+    case CO_Q4_1:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q4_1((const co_block_q4_1 *)blocks + i, y + 32 * i);
+        return 0;
+    case CO_Q4_1_GGML:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q4_1_ggml((const co_block_q4_1 *)blocks + i, y + 32 * i);
+        return 0;
+    case CO_Q5_0:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q5_0((const co_block_q5_0 *)blocks + i, y + 32 * i);
+        return 0;
+    case CO_Q5_1:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q5_1((const co_block_q5_1 *)blocks + i, y + 32 * i);
+        return 0;
+    case CO_Q2_K:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q2_k((const co_block_q2_k *)blocks + i, y + 256 * i);
+        return 0;
+    case CO_Q3_K:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q3_k((const co_block_q3_k *)blocks + i, y + 256 * i);
+        return 0;
+    case CO_Q5_K:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q5_k((const co_block_q5_k *)blocks + i, y + 256 * i);
+        return 0;
+    case CO_Q8_K:
+        for (int64_t i = 0; i < n_blocks; ++i) dequant_q8_k((const co_block_q8_k *)blocks + i, y + 256 * i);
+        return 0;
     case CO_Q4_0:
         for (int64_t i = 0; i < n_blocks; ++i) dequant_q4_0((const co_block_q4_0 *)blocks + i, y + 32 * i);
         return 0;
@@ -627,9 +780,122 @@ static float vec_dot_q6_k(const co_block_q6_k *w, const co_block_q8_0 *x, int64_
     return acc;
 }
 
+static int32_t q8_block_sum(const co_block_q8_0 *x) {
+    int32_t s = 0;
+    for (int i = 0; i < 32; ++i) s += (int)x->qs[i];
+    return s;
+}
+
+/* QCU:1947-1975: sumi * (d4*d8) + m4 * s8, s8 = d8 * (sum of the block's quants), here with the exact integer sum.
+ * elem(j, hi) says which activation the low / high nibble of byte j pairs with (the two element orders). */
+static float vec_dot_q4_1(const co_block_q4_1 *w, const co_block_q8_0 *x, int64_t nb, int ggml_order) {
+    float acc = 0.0f;
+    for (int64_t b = 0; b < nb; ++b) {
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; ++j) {
+            sumi += (int)(w[b].qs[j] & 0xF) * (int)x[b].qs[ggml_order ? j : 2 * j];
+            sumi += (int)(w[b].qs[j] >> 4) * (int)x[b].qs[ggml_order ? j + 16 : 2 * j + 1];
+        }
+        const float d8 = co_fp16_to_f32(x[b].d);
+        acc += (co_fp16_to_f32(w[b].dm[0]) * d8) * (float)sumi + (co_fp16_to_f32(w[b].dm[1]) * d8) * (float)q8_block_sum(x + b);
+    }
+    return acc;
+}
+
+/* QCU:1982-2009: d5 * (sumi*d8 - 16*s8) = (d5*d8) * (sumi - 16*sum) with the exact integer sum */
+static float vec_dot_q5_0(const co_block_q5_0 *w, const co_block_q8_0 *x, int64_t nb) {
+    float acc = 0.0f;
+    for (int64_t b = 0; b < nb; ++b) {
+        int32_t sumi = 0;
+        for (int e = 0; e < 32; ++e) sumi += q5_level(w[b].qs, w[b].qh, e) * (int)x[b].qs[e];
+        sumi -= 16 * q8_block_sum(x + b);
+        acc += (co_fp16_to_f32(w[b].d) * co_fp16_to_f32(x[b].d)) * (float)sumi;
+    }
+    return acc;
+}
+
+/* QCU:2016-2053: sumi * (d5*d8) + m5 * s8 */
+static float vec_dot_q5_1(const co_block_q5_1 *w, const co_block_q8_0 *x, int64_t nb) {
+    float acc = 0.0f;
+    for (int64_t b = 0; b < nb; ++b) {
+        int32_t sumi = 0;
+        for (int e = 0; e < 32; ++e) sumi += q5_level(w[b].qs, w[b].qh, e) * (int)x[b].qs[e];
+        const float d8 = co_fp16_to_f32(x[b].d);
+        acc += (co_fp16_to_f32(w[b].dm[0]) * d8) * (float)sumi + (co_fp16_to_f32(w[b].dm[1]) * d8) * (float)q8_block_sum(x + b);
+    }
+    return acc;
+}
+
+/* QCU:2108-2135: per 16-value group sumf_d += d8*(dot*scale), sumf_m += d8*(sum*min); dall*sumf_d - dmin*sumf_m
+ * per super-block, groups in ascending order. */
+static float vec_dot_q2_k(const co_block_q2_k *w, const co_block_q8_0 *x, int64_t nsb) {
+    float acc = 0.0f;
+    for (int64_t s = 0; s < nsb; ++s) {
+        float sumf_d = 0.0f, sumf_m = 0.0f;
+        for (int g = 0; g < 16; ++g) {
+            const co_block_q8_0 *xb = x + 8 * s + g / 2;
+            int32_t dot = 0, sum = 0;
+            for (int i = 0; i < 16; ++i) {
+                const int e = 16 * g + i, n = e / 128, k = (e % 128) / 32, l = e % 32;
+                const int q = (w[s].qs[32 * n + l] >> (2 * k)) & 3;
+                dot += q * (int)xb->qs[e % 32];
+                sum += (int)xb->qs[e % 32];
+            }
+            const float d8 = co_fp16_to_f32(xb->d);
+            sumf_d += d8 * (float)(dot * (int)(w[s].scales[g] & 0xF));
+            sumf_m += d8 * (float)(sum * (int)(w[s].scales[g] >> 4));
+        }
+        acc += co_fp16_to_f32(w[s].dm[0]) * sumf_d - co_fp16_to_f32(w[s].dm[1]) * sumf_m;
+    }
+    return acc;
+}
+
+/* QCU:2177-2209: sumf += d8 * (dot * (scale - 32)) per 16-value group; d * sumf per super-block */
+static float vec_dot_q3_k(const co_block_q3_k *w, const co_block_q8_0 *x, int64_t nsb) {
+    float acc = 0.0f;
+    for (int64_t s = 0; s < nsb; ++s) {
+        float sumf = 0.0f;
+        for (int g = 0; g < 16; ++g) {
+            const co_block_q8_0 *xb = x + 8 * s + g / 2;
+            int32_t dot = 0;
+            for (int i = 0; i < 16; ++i) dot += q3k_level(w + s, 16 * g + i) * (int)xb->qs[(16 * g + i) % 32];
+            sumf += co_fp16_to_f32(xb->d) * (float)(dot * (q3k_scale(w[s].scales, g) - 32));
+        }
+        acc += co_fp16_to_f32(w[s].d) * sumf;
+    }
+    return acc;
+}
+
+/* QCU:2300-2331: as Q4_K with 5-bit levels */
+static float vec_dot_q5_k(const co_block_q5_k *w, const co_block_q8_0 *x, int64_t nsb) {
+    float acc = 0.0f;
+    for (int64_t s = 0; s < nsb; ++s) {
+        float sumf_d = 0.0f, sumf_m = 0.0f;
+        for (int t = 0; t < 8; ++t) {
+            const co_block_q8_0 *xb = x + 8 * s + t;
+            int32_t dot1 = 0;
+            for (int l = 0; l < 32; ++l) dot1 += q5k_level(w + s, 32 * t + l) * (int)xb->qs[l];
+            uint8_t sc, m;
+            co_get_scale_min_k4(t, w[s].scales, &sc, &m);
+            const float d8 = co_fp16_to_f32(xb->d);
+            sumf_d += d8 * (float)(dot1 * (int)sc);
+            sumf_m += d8 * (float)(q8_block_sum(xb) * (int)m);
+        }
+        acc += co_fp16_to_f32(w[s].dm[0]) * sumf_d - co_fp16_to_f32(w[s].dm[1]) * sumf_m;
+    }
+    return acc;
+}
+
 float co_vec_dot_q8_0(int fmt, const void *w_row, const void *x_q8_0, int64_t k) {
     const co_block_q8_0 *x = (const co_block_q8_0 *)x_q8_0;
     switch (fmt) {
+    case CO_Q4_1: return vec_dot_q4_1((const co_block_q4_1 *)w_row, x, k / 32, 0);
+    case CO_Q4_1_GGML: return vec_dot_q4_1((const co_block_q4_1 *)w_row, x, k / 32, 1);
+    case CO_Q5_0: return vec_dot_q5_0((const co_block_q5_0 *)w_row, x, k / 32);
+    case CO_Q5_1: return vec_dot_q5_1((const co_block_q5_1 *)w_row, x, k / 32);
+    case CO_Q2_K: return vec_dot_q2_k((const co_block_q2_k *)w_row, x, k / 256);
+    case CO_Q3_K: return vec_dot_q3_k((const co_block_q3_k *)w_row, x, k / 256);
+    case CO_Q5_K: return vec_dot_q5_k((const co_block_q5_k *)w_row, x, k / 256);
     case CO_Q4_0: return vec_dot_q4_0((const co_block_q4_0 *)w_row, x, k / 32);
     case CO_Q4_0_GGML: return vec_dot_q4_0_ggml((const co_block_q4_0 *)w_row, x, k / 32);
     case CO_Q8_0: return vec_dot_q8_0((const co_block_q8_0 *)w_row, x, k / 32);

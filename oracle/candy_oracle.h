@@ -29,11 +29,20 @@ enum {
     CO_Q8_0 = 8,
     CO_Q4_K = 12,
     CO_Q6_K = 14,
-    CO_Q4_0_GGML = 102 /* ggml/CUDA element order: y[j]=lo(qs[j]), y[j+16]=hi(qs[j]) */
+    CO_Q4_0_GGML = 102, /* ggml/CUDA element order: y[j]=lo(qs[j]), y[j+16]=hi(qs[j]) */
+    /* the reference's other block formats (numbers are ggml's type ids) */
+    CO_Q4_1 = 3,        /* candy CPU element order (QGO:107-116) */
+    CO_Q4_1_GGML = 103, /* ggml/CUDA element order (QCU:728-746) */
+    CO_Q5_0 = 6,
+    CO_Q5_1 = 7,
+    CO_Q2_K = 10,
+    CO_Q3_K = 11,
+    CO_Q5_K = 13,
+    CO_Q8_K = 15        /* dequantize only: the reference has no weight vec-dot for it */
 };
 
 int co_block_elems(int fmt);  /* 32 or 256; 0 for an unknown format */
-int co_block_bytes(int fmt);  /* 18, 34, 144, 210; 0 for an unknown format */
+int co_block_bytes(int fmt);  /* 18, 34, 144, 210, 20, 22, 24, 84, 110, 176, 292; 0 for an unknown format */
 
 float    co_fp16_to_f32(uint16_t h);
 uint16_t co_f32_to_fp16(float f);

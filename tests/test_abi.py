@@ -34,7 +34,10 @@ def test_format_tables():
     L = hip.lib()
     assert [L.candy_hip_block_bytes(f) for f in (hip.Q4_0, hip.Q8_0, hip.Q4_K, hip.Q6_K, hip.Q4_0_GGML)] == [18, 34, 144, 210, 18]
     assert [L.candy_hip_block_elems(f) for f in (hip.Q4_0, hip.Q8_0, hip.Q4_K, hip.Q6_K)] == [32, 32, 256, 256]
-    assert L.candy_hip_block_bytes(7) == 0
+    # the reference's other formats, by ggml type id (Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K, Q8_K) and Q4_1 in ggml order
+    assert [L.candy_hip_block_bytes(f) for f in (3, 6, 7, 10, 11, 13, 15, 103)] == [20, 22, 24, 84, 110, 176, 292, 20]
+    assert [L.candy_hip_block_elems(f) for f in (3, 6, 7, 10, 11, 13, 15, 103)] == [32, 32, 32, 256, 256, 256, 256, 32]
+    assert L.candy_hip_block_bytes(9) == 0 and L.candy_hip_block_bytes(16) == 0
     # sizes the hot-path shapes must have
     assert L.candy_hip_qweight_bytes(hip.Q4_K, 4096, 11008) == 25362432
     assert L.candy_hip_qweight_bytes(hip.Q8_0, 32000, 4096) == 139264000

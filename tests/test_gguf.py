@@ -171,13 +171,14 @@ def test_header_validation(tmp_path):
         gguf.GGUFFile(variant("trunc", lambda b: b.__delitem__(slice(len(b) - 1000, len(b)))))
     with pytest.raises(gguf.GGUFError, match="ends inside"):
         gguf.GGUFFile(variant("short", lambda b: b.__delitem__(slice(200, len(b)))))
-    # a tensor of a ggml type that exists but has no kernels here (Q5_K = 13)
-    p = str(tmp_path / "q5k.gguf")
-    gguf.write_gguf(p, {}, [("w", 13, (256, 2), np.zeros(2 * 176, np.uint8))])
+    # a tensor of a ggml type that exists but has no kernels here (Q8_1 = 9); Q5_K = 13 has
+    p = str(tmp_path / "q81.gguf")
+    gguf.write_gguf(p, {}, [("w", 9, (32, 2), np.zeros(2 * 36, np.uint8)), ("v", 13, (256, 2), np.zeros(2 * 176, np.uint8))])
     g = gguf.GGUFFile(p)
-    assert g.tensors["w"].nbytes == 352
+    assert g.tensors["w"].nbytes == 72 and g.tensors["v"].nbytes == 352
     with pytest.raises(gguf.GGUFError, match="no device kernels"):
         g.blocks("w")
+    assert g.blocks("v")[:3] == (synth.Q5_K, 2, 256)
     with pytest.raises(gguf.GGUFError, match="no tensor named"):
         g.raw("missing")
     with pytest.raises(gguf.GGUFError, match="multiple of the block size"):

@@ -64,6 +64,11 @@ def rel(got, want):
     ("small-mixed", dict(n_layers=3, d_model=512, n_heads=8, n_kv_heads=2, head_dim=64, d_ffn=1024, vocab=512,
                          max_pos=16, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q8_0, "gate": synth.Q4_0, "down": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q4_K}),
+    # the formats without fused decode kernels: every Linear falls back to quantize + general matvec (+ add)
+    ("other-formats", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=4, head_dim=64, d_ffn=1024, vocab=512,
+                           max_pos=16, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q5_K, "q": synth.Q5_0, "k": synth.Q4_1, "v": synth.Q5_1, "gate": synth.Q3_K, "up": synth.Q2_K,
+      "head": synth.Q4_1_GGML, "embed": synth.Q8_K}),
 ])
 def test_decode_steps_match_cpu_composition(dev, name, cfg, fmts):
     host, model = build(dev, cfg, fmts, seed=3)
@@ -102,6 +107,10 @@ PROMPT_CASES = [
     ("gqa-hd128-long", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=2, head_dim=128, d_ffn=512, vocab=256,
                             max_pos=224, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}, 203, 1e-3),
+    ("other-formats", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=4, head_dim=64, d_ffn=1024, vocab=256,
+                           max_pos=32, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q5_K, "q": synth.Q5_0, "k": synth.Q4_1, "v": synth.Q5_1, "gate": synth.Q3_K, "up": synth.Q2_K,
+      "head": synth.Q4_1_GGML, "embed": synth.Q8_K}, 21, 1e-3),
     ("short-prompt", dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=64, d_ffn=512, vocab=128,
                           max_pos=16, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q8_0, "gate": synth.Q4_0, "head": synth.Q6_K, "embed": synth.Q4_K}, 5, 1e-3),
