@@ -93,34 +93,31 @@ __device__ __forceinline__ int64_t src_block(int64_t b, const int64_t *__restric
     return ids ? ids[b / bpr] * bpr + b % bpr : b;
 }
 
-// quantized.go:85-93: y[2j] = d*(lo(qs[j])-8), y[2j+1] = d*(hi(qs[j])-8). 4 lanes per block.
+// quantized.go:85-93: y[2j] = d*(lo(qs[j])-8), y[2j+1] = d*(hi(qs[j])-8). 8 lanes per block, one float4 each
+// (a lane that wrote two float4 32 bytes apart left every store instruction half-filling its lines: 2.9 TB/s).
 __global__ __launch_bounds__(256) void k_dequant_q4_0(const BlockQ4_0 *__restrict__ blocks, int64_t nb,
         const int64_t *__restrict__ ids, int64_t bpr,
                                                       float4 *__restrict__ y, int ggml_order) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t b = t >> 2;
+    const int64_t b = t >> 3;
     if (b >= nb) return;
-    const int j = (int)(t & 3);  // bytes 4j..4j+3
+    const int j = (int)(t & 7);  // values 4j..4j+3
     const BlockQ4_0 *blk = blocks + src_block(b, ids, bpr);
     const float d = half_bits_to_float(blk->d);
-    const uint32_t q = *(const u32_a2 *)(blk->qs + 4 * j);
-    float lo[4], hi[4];
-    const float dm = -8.0f * d;
+    float v[4];
+    if (ggml_order) {  // quantized.cu:862-866: low nibbles fill y[0..15], high nibbles y[16..31]; d*q + (-8 d)
+        const uint32_t q = *(const u32_a2 *)(blk->qs + 4 * (j & 3)) >> (j >= 4 ? 4 : 0);
+        const float dm = -8.0f * d;
 #pragma unroll
-    for (int l = 0; l < 4; ++l) {
-        const float ql = (float)((q >> (8 * l)) & 0xF), qh = (float)((q >> (8 * l + 4)) & 0xF);
-        // the two reference forms agree everywhere except the sign of a zero result
-        lo[l] = ggml_order ? d * ql + dm : d * (ql - 8.0f);
-        hi[l] = ggml_order ? d * qh + dm : d * (qh - 8.0f);
+        for (int l = 0; l < 4; ++l) v[l] = d * (float)((q >> (8 * l)) & 0xF) + dm;
+    } else {  // the two reference forms agree everywhere except the sign of a zero result
+        const uint32_t q = *(const uint16_t *)(blk->qs + 2 * j);
+        v[0] = d * ((float)(q & 0xF) - 8.0f);
+        v[1] = d * ((float)((q >> 4) & 0xF) - 8.0f);
+        v[2] = d * ((float)((q >> 8) & 0xF) - 8.0f);
+        v[3] = d * ((float)(q >> 12) - 8.0f);
     }
-    float4 *out = y + b * 8;
-    if (ggml_order) {  // quantized.cu:862-866: low nibbles fill y[0..15], high nibbles y[16..31]
-        out[j] = make_float4(lo[0], lo[1], lo[2], lo[3]);
-        out[4 + j] = make_float4(hi[0], hi[1], hi[2], hi[3]);
-    } else {
-        out[2 * j] = make_float4(lo[0], hi[0], lo[1], hi[1]);
-        out[2 * j + 1] = make_float4(lo[2], hi[2], lo[3], hi[3]);
-    }
+    y[t] = make_float4(v[0], v[1], v[2], v[3]);
 }
 
 // quantized.go:131-136: y[i] = d*qs[i]. 8 lanes per block.
@@ -261,7 +258,7 @@ static int dequantize_impl(candy_hip_device *dev, int fmt, const void *dev_block
     case CANDY_HIP_Q8_K: return launch_dequant_more<FmtQ8K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
     default: break;
     }
-    const int lanes_per_block = fmt == CANDY_HIP_Q4_K ? 32 : fmt == CANDY_HIP_Q6_K ? 16 : fmt == CANDY_HIP_Q8_0 ? 8 : 4;
+    const int lanes_per_block = fmt == CANDY_HIP_Q4_K ? 32 : fmt == CANDY_HIP_Q6_K ? 16 : 8;
     const int64_t grid = (n_blocks * lanes_per_block + 255) / 256;
     CANDY_REQUIRE(grid <= 0x7FFFFFFF, "too many blocks");
     dim3 g((unsigned)grid), blk(256);
