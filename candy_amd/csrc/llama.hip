@@ -48,6 +48,7 @@ struct candy_hip_llama {
     hipGraph_t graph = nullptr;                   // the captured step (layers + head + argmax)
     hipGraphExec_t graph_exec = nullptr;
     bool graph_dirty = true;
+    bool tables_dirty = true;  // a weight, a norm or the choice of path changed since the persistent step's tables were built
     bool use_graph = true;
     std::vector<void *> owned;
     // prompt buffers, grown on demand to the longest prompt seen: [n][width] activations
@@ -214,7 +215,7 @@ int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const 
     case CANDY_HIP_W_EMBED: rows = c.vocab; cols = c.d_model; break;
     default: return fail(CANDY_HIP_ERR_INVALID, "weight kind %d is not a quantized matrix", which);
     }
-    m->graph_dirty = true;
+    m->graph_dirty = m->tables_dirty = true;
     CANDY_REQUIRE(w->rows == rows && w->cols == cols, "weight kind %d must be %lld x %lld, got %lld x %lld", which,
                   (long long)rows, (long long)cols, (long long)w->rows, (long long)w->cols);
     if (which == CANDY_HIP_W_HEAD) { m->head = w; return CANDY_HIP_OK; }
@@ -235,7 +236,7 @@ int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const 
 
 int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const float *dev_alpha) {
     CANDY_REQUIRE(m && dev_alpha, "nil argument");
-    m->graph_dirty = true;
+    m->graph_dirty = m->tables_dirty = true;
     if (which == CANDY_HIP_W_OUT_NORM) { m->out_norm = dev_alpha; return CANDY_HIP_OK; }
     CANDY_REQUIRE(which == CANDY_HIP_W_ATTN_NORM || which == CANDY_HIP_W_FFN_NORM, "weight kind %d is not a norm", which);
     CANDY_REQUIRE(layer >= 0 && layer < m->cfg.n_layers, "layer %d out of range", layer);
@@ -253,7 +254,7 @@ int candy_hip_llama_set_graph(candy_hip_llama *m, int enable) {
 int candy_hip_llama_set_persistent(candy_hip_llama *m, int enable) {
     CANDY_REQUIRE(m, "model is nil");
     m->persist_wanted = enable != 0;
-    m->graph_dirty = true;
+    m->graph_dirty = m->tables_dirty = true;
     return CANDY_HIP_OK;
 }
 
@@ -388,7 +389,9 @@ static int persist_enqueue(candy_hip_llama *m) {
     a.x_act = p; p += 2 * F;
     a.x_best = p;
     a.logits = m->logits; a.next_tok = m->next_tok; a.fail = m->next_tok + 1;
-    a.spin_limit = 1 << 15;
+    // polls before a workgroup gives up (about 50 ms); CANDY_HIP_PERSIST_SPIN_LIMIT overrides, negative = give up at once
+    const char *spin_env = getenv("CANDY_HIP_PERSIST_SPIN_LIMIT");
+    a.spin_limit = spin_env ? atoi(spin_env) : 1 << 15;
     a.prof = m->p_prof;
     return launch_decode_step(dev, a);
 }
@@ -456,10 +459,11 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
     } else {
         if ((rc = candy_hip_qindex_select(dev, m->embed, m->tok_id, 1, m->h))) return rc;
     }
-    if (m->graph_dirty || !m->use_graph) {
+    if (m->tables_dirty) {
         m->persist_ready = false;
         if (m->persist_wanted && !m->persist_broken && persist_covers(m))
             if ((rc = persist_prepare(m))) return rc;
+        m->tables_dirty = false;
     }
     if (m->use_graph) {
         if (m->graph_dirty) {
@@ -488,7 +492,7 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
             // step is trusted; clear the flag and redo it kernel by kernel, from now on
             m->persist_broken = true;
             m->persist_ready = false;
-            m->graph_dirty = true;
+            m->graph_dirty = m->tables_dirty = true;
             if ((rc = candy_hip_zero(dev, m->next_tok + 1, sizeof(uint32_t)))) return rc;
             return llama_step(m, pos, token, dev_hidden, dev_logits, next_token);
         }

@@ -233,6 +233,24 @@ def test_persistent_step_equals_kernel_by_kernel(dev, name, cfg, head, n):
     assert rel(bufs[0], bufs[2].astype(np.float64)) <= 1e-3 and rel(bufs[1], bufs[3].astype(np.float64)) <= 1e-3
 
 
+def test_persistent_step_time_out_falls_back(dev, monkeypatch):
+    # the host asks the kernel for its time-out path (every workgroup raises the flag and leaves at once, nothing
+    # hangs): the step is redone kernel by kernel, gives that path's result, and the model stays on it
+    cfg = dict(n_layers=2, d_model=512, n_heads=4, n_kv_heads=4, head_dim=128, d_ffn=768, vocab=300, max_pos=8,
+               rms_eps=1e-5, rope_base=10000.0)
+    fm = {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}
+    _, one = build(dev, cfg, fm, seed=33)
+    _, many = build(dev, cfg, fm, seed=33)
+    monkeypatch.setenv("CANDY_HIP_PERSIST_SPIN_LIMIT", "-1")
+    one.set_persistent(True)
+    for pos, tok in enumerate([7, 250, 31]):
+        ot, ol = one.decode(tok, pos)
+        mt, ml = many.decode(tok, pos)
+        assert one.decode_path() == 0
+        assert np.array_equal(ol, ml) and ot == mt
+    monkeypatch.delenv("CANDY_HIP_PERSIST_SPIN_LIMIT")
+
+
 def test_decode_errors(dev):
     cfg = dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, head_dim=128, d_ffn=256, vocab=64, max_pos=4,
                rms_eps=1e-5, rope_base=10000.0)
