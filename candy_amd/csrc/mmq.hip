@@ -18,6 +18,7 @@
 // 1e-4 (max-norm) of the CPU contraction, inside the 1e-3 bar (tests/test_gpu_mmq.py).
 // Bound: HBM (weights read once) for m = 16..32, MFMA for m >= 128.
 #include "blocks.h"
+#include "formats_more.h"
 #include "internal.h"
 
 namespace candy {
@@ -150,6 +151,27 @@ struct MmqQ6K {
                 const uint32_t hi2 = (qh[il >> 2] >> (8 * (il & 3) + 2 * qd)) & 3;
                 v[l] = (g < 2 ? s0 : s1) * (float)((int)(lo4 | (hi2 << 4)) - 32);
             }
+            out[g] = to_half8(v);
+        }
+    }
+};
+
+// The other formats (formats_more.h): the 32 weights are dequantized with the format's own quad() straight from
+// memory when the tile is built (no raw-byte stage ahead of it: these formats are not on the headline path).
+template <class F>
+struct MmqMore {
+    struct Raw { const uint8_t *blk; int j0; };
+    __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K / F::ELEMS) * F::BYTES; }
+    __device__ static __forceinline__ void load(const uint8_t *row, int kb, Raw &r) {
+        const int e = kb * 32;
+        r.blk = row + (size_t)(e / F::ELEMS) * F::BYTES;
+        r.j0 = (e % F::ELEMS) >> 2;
+    }
+    __device__ static __forceinline__ void dequant(const Raw &r, int, half8 (&out)[4]) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const float4 a = F::quad(r.blk, r.j0 + 2 * g), b = F::quad(r.blk, r.j0 + 2 * g + 1);
+            const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
             out[g] = to_half8(v);
         }
     }
@@ -317,10 +339,7 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     const int64_t K = w->cols;
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && K <= 0x7FFFFFFF && m <= 0x7FFFFFFF, "matrix too large");
     if (K % 64 != 0) return launch_matvec(dev, w, qs, scales, m, y);  // odd block counts: small-batch kernel in slices
-    switch (w->fmt) {  // the formats with tile kernels; the others contract in slices of the small-batch kernel
-    case CANDY_HIP_Q4_K: case CANDY_HIP_Q6_K: case CANDY_HIP_Q8_0: case CANDY_HIP_Q4_0: case CANDY_HIP_Q4_0_GGML: break;
-    default: return launch_matvec(dev, w, qs, scales, m, y);
-    }
+    if (w->fmt == CANDY_HIP_Q8_K) return launch_matvec(dev, w, qs, scales, m, y);  // reports that Q8_K does not contract
     // prompt-sized batches of Q4_K: big fp16 tiles (the integer kernel is bound by its per-sub-block rescale there);
     // smaller batches of Q4_K and Q6_K: int8 matrix cores (exact); the fp16 tile kernel below serves the rest
     const bool force_fp16 = force_old_fp16();
@@ -347,6 +366,13 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     case CANDY_HIP_Q4_0: return launch_fmt<MmqQ4_0<false>>(dev, w, xh, m, y);
     case CANDY_HIP_Q4_0_GGML: return launch_fmt<MmqQ4_0<true>>(dev, w, xh, m, y);
     case CANDY_HIP_Q6_K: return launch_fmt<MmqQ6K>(dev, w, xh, m, y);
+    case CANDY_HIP_Q4_1: return launch_fmt<MmqMore<FmtQ4_1<false>>>(dev, w, xh, m, y);
+    case CANDY_HIP_Q4_1_GGML: return launch_fmt<MmqMore<FmtQ4_1<true>>>(dev, w, xh, m, y);
+    case CANDY_HIP_Q5_0: return launch_fmt<MmqMore<FmtQ5<false>>>(dev, w, xh, m, y);
+    case CANDY_HIP_Q5_1: return launch_fmt<MmqMore<FmtQ5<true>>>(dev, w, xh, m, y);
+    case CANDY_HIP_Q2_K: return launch_fmt<MmqMore<FmtQ2K>>(dev, w, xh, m, y);
+    case CANDY_HIP_Q3_K: return launch_fmt<MmqMore<FmtQ3K>>(dev, w, xh, m, y);
+    case CANDY_HIP_Q5_K: return launch_fmt<MmqMore<FmtQ5K>>(dev, w, xh, m, y);
     default: return fail(CANDY_HIP_ERR_INVALID, "unknown quantized format %d", w->fmt);
     }
 }
