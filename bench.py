@@ -312,7 +312,35 @@ def main():
             sweep.append({"fmt": name, "rows": r, "cols": k, "us": round(ms * 1e3, 3), "GBps": round(gb, 1),
                           "frac": round(gb / HBM_PEAK_GBPS, 4)})
             log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
+        # the reference's other formats through the general kernel (no per-length batch-1 variants)
+        for f in (synth.Q4_1, synth.Q5_0, synth.Q5_1, synth.Q2_K, synth.Q3_K, synth.Q5_K):
+            r, k, name = 4096, 11008, synth.FORMAT_NAMES[f]
+            ms, _ = time_matvec(dev, f, r, k, s_steps, s_warm, quantize_each=False, seed=r + k + f)
+            gb = algorithmic_bytes(f, r, k) / (ms * 1e-3) / 1e9
+            sweep.append({"fmt": name, "rows": r, "cols": k, "us": round(ms * 1e3, 3), "GBps": round(gb, 1),
+                          "frac": round(gb / HBM_PEAK_GBPS, 4)})
+            log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
         out["sweep"] = sweep
+
+    if not args.no_sweep:
+        # weight quantizers from f32 (load-time): 4096x11008, one launch each
+        wq = []
+        r, k = 4096, 11008
+        xw = dev.from_numpy((np.random.default_rng(77).standard_normal((r, k)) * 0.02).astype(np.float32))
+        for f in (synth.Q4_0, synth.Q8_0, synth.Q4_K, synth.Q6_K):
+            dst = dev.alloc(synth.weight_nbytes(f, r, k))
+            for rep in range(2):
+                dev.synchronize()
+                t0 = time.perf_counter()
+                hip._check(hip.lib().candy_hip_quantize(dev.handle, f, xw.ptr, r, k, dst.ptr))
+                dev.synchronize()
+                dt = time.perf_counter() - t0
+            wq.append({"op": "quantize", "fmt": synth.FORMAT_NAMES[f], "rows": r, "cols": k, "ms": round(dt * 1e3, 3),
+                       "Gvalues_s": round(r * k / dt / 1e9, 1)})
+            log(f"  quantize {synth.FORMAT_NAMES[f]} {r}x{k}: {dt * 1e3:.2f} ms")
+            dst.free()
+        xw.free()
+        out["weight_quantizers"] = wq
 
     if not args.no_sweep:
         # the two conversions, both HBM-bound: dequantize writes 4 B per weight, quantize reads 4 B per value
