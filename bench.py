@@ -98,8 +98,17 @@ def cpu_baseline(rows, cols, budget_s=12.0):
             "ms_per_step": round(per_full * 1e3, 3)}
 
 
+def quantized_normal(dev, fmt, rows, cols, seed, std=0.02):
+    """Blocks of a [rows, cols] matrix drawn from N(0, std) and quantized by the library's own quantizer on the device."""
+    rng = np.random.Generator(np.random.Philox(seed))
+    x = rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(std)
+    return dev.quantize(fmt, x)
+
+
 def build_7b(dev, n_layers=32, max_pos=2176, seed=4000):
-    """Random-init Llama-7B-shaped decoder: Q4_K linears, Q6_K head, Q8_0 embedding rows."""
+    """Random-init Llama-7B-shaped decoder: Q4_K linears, Q6_K head, Q8_0 embedding rows; weights drawn from
+    N(0, 0.02) and then quantized on the device.  One draw per shape; the layers take it with its blocks rotated
+    (distinct contents, same distribution) so that building the model stays a matter of seconds."""
     from candy_amd import hip, synth
     cfg = dict(n_layers=n_layers, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=11008, vocab=32000,
                max_pos=max_pos, rms_eps=1e-5, rope_base=10000.0)
@@ -107,21 +116,21 @@ def build_7b(dev, n_layers=32, max_pos=2176, seed=4000):
     shapes = [(hip.W_Q, 4096, 4096), (hip.W_K, 4096, 4096), (hip.W_V, 4096, 4096), (hip.W_O, 4096, 4096),
               (hip.W_GATE, 11008, 4096), (hip.W_UP, 11008, 4096), (hip.W_DOWN, 4096, 11008)]
     ones = np.ones(4096, np.float32)
-    sc = synth.unit_scale(synth.Q4_K)
     t0 = time.perf_counter()
+    base = {(r, k): quantized_normal(dev, synth.Q4_K, r, k, seed + r + k).reshape(-1, synth.BLOCK_BYTES[synth.Q4_K])
+            for r, k in {(r, k) for _, r, k in shapes}}
+    shift = 0
     for l in range(n_layers):
         for kind, r, k in shapes:
-            seed += 1
-            model.set_qweight(kind, l, dev.qtensor(synth.Q4_K, r, k, synth.random_weight(synth.Q4_K, r, k, seed, sc)))
+            shift += 1
+            model.set_qweight(kind, l, dev.qtensor(synth.Q4_K, r, k, np.roll(base[(r, k)], 977 * shift, axis=0).reshape(-1)))
         model.set_norm(hip.W_ATTN_NORM, l, ones)
         model.set_norm(hip.W_FFN_NORM, l, ones)
         if l % 8 == 7:
             log(f"  built layer {l + 1}/{n_layers} ({time.perf_counter() - t0:.0f} s)")
     model.set_norm(hip.W_OUT_NORM, -1, ones)
-    model.set_qweight(hip.W_HEAD, -1, dev.qtensor(synth.Q6_K, 32000, 4096, synth.random_weight(
-        synth.Q6_K, 32000, 4096, seed + 1, synth.unit_scale(synth.Q6_K))))
-    model.set_qweight(hip.W_EMBED, -1, dev.qtensor(synth.Q8_0, 32000, 4096, synth.random_weight(
-        synth.Q8_0, 32000, 4096, seed + 2, synth.unit_scale(synth.Q8_0))))
+    model.set_qweight(hip.W_HEAD, -1, dev.qtensor(synth.Q6_K, 32000, 4096, quantized_normal(dev, synth.Q6_K, 32000, 4096, seed + 1)))
+    model.set_qweight(hip.W_EMBED, -1, dev.qtensor(synth.Q8_0, 32000, 4096, quantized_normal(dev, synth.Q8_0, 32000, 4096, seed + 2)))
     return cfg, model
 
 
@@ -213,7 +222,7 @@ def prefill_kv(dev, model, cfg, n_pos, seed=9):
 
 def decode_leg(dev, steps, warmup):
     from candy_amd import synth
-    log("building random-init 7B (Q4_K, Q6_K head) ...")
+    log("building random-init 7B (N(0, 0.02) quantized to Q4_K, Q6_K head) ...")
     n_pos = 2048
     cfg, model = build_7b(dev, max_pos=n_pos + steps + warmup + 8)
     prefill_kv(dev, model, cfg, n_pos)

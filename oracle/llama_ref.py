@@ -25,10 +25,14 @@ def rope_tables(max_pos: int, head_dim: int, base: float):
 
 
 class LlamaRef:
-    def __init__(self, cfg: dict, weights: dict):
-        """weights: {(kind, layer): (fmt, blocks) | f32 array}; kinds as in candy_hip.h."""
+    def __init__(self, cfg: dict, weights: dict, f32_activations: bool = False):
+        """weights: {(kind, layer): (fmt, blocks) | f32 array}; kinds as in candy_hip.h.
+        f32_activations: every Linear is dequantize + f32 matmul (candy's literal CPU composition, conv.go:373-389)
+        instead of the Q8_0-activation vec-dot: the same model without the activation quantizer, against which the
+        size of that quantizer's noise can be measured."""
         self.c = cfg
         self.w = weights
+        self.f32_activations = f32_activations
         c = cfg
         self.k_cache = np.zeros((c["n_layers"], c["n_kv_heads"], c["max_pos"], c["head_dim"]), np.float32)
         self.v_cache = np.zeros_like(self.k_cache)
@@ -36,6 +40,8 @@ class LlamaRef:
 
     def _lin(self, kind, layer, x, rows, cols):
         fmt, blocks = self.w[(kind, layer)]
+        if self.f32_activations:
+            return o.matmul_dequant_f32(fmt, blocks, rows, cols, np.asarray(x, np.float32).reshape(1, -1)).reshape(-1)
         return o.qmatmul(fmt, blocks, rows, cols, x).reshape(-1)
 
     def embed(self, token: int) -> np.ndarray:
