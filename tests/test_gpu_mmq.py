@@ -83,7 +83,7 @@ def test_contraction_length_not_a_multiple_of_64(dev, fmt, rows, cols):
 
 @pytest.mark.parametrize("m", [16, 128, 512])
 def test_config_prefill_q4k_14336x4096(dev, m):
-    # BASELINE config 2 at full size; the oracle runs on a strided subset of the weight rows
+    # the batched-prefill configuration (Q4_K 14336x4096, M in {16, 128, 512}) at full size; the oracle runs on a strided subset of the weight rows
     rows, cols = 14336, 4096
     w = synth.random_weight(synth.Q4_K, rows, cols, seed=77)
     x = synth.random_activations(m, cols, seed=78 + m)

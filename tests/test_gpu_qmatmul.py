@@ -50,7 +50,7 @@ def test_small_batch_matches_oracle(dev, fmt, m):
 
 
 def test_config_q4_0_4096x4096(dev):
-    # BASELINE config 0: Q4_0 4096x4096, one f32 N(0,1) vector, seeded
+    # the single-QMatMul configuration: Q4_0 4096x4096, one f32 N(0,1) vector, seeded
     rows = cols = 4096
     w = synth.random_weight(synth.Q4_0, rows, cols, seed=20240)
     x = synth.random_activations(1, cols, seed=20241)
@@ -70,7 +70,7 @@ def test_config_q4_0_4096x4096(dev):
 @pytest.mark.parametrize("fmt", [synth.Q8_0, synth.Q4_K])
 @pytest.mark.parametrize("rows,cols", [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)])
 def test_config_sweep_full_shapes(dev, fmt, rows, cols):
-    # BASELINE config 1 at full size: oracle on a strided row subset + linearity over the whole output
+    # the batch-1 sweep shapes at full size: oracle on a strided row subset + linearity over the whole output
     w = synth.random_weight(fmt, rows, cols, seed=rows + cols + fmt)
     x = synth.random_activations(1, cols, seed=3 * rows + fmt)
     q = dev.qtensor(fmt, rows, cols, w)
