@@ -55,44 +55,40 @@ struct TileQ4K {
     static constexpr int BLOCK = 144, SLOT = 144;
     typedef u32x4 GlobalChunk;  // rows are 16-byte aligned
     struct Exchange {
-        uint8_t sc[16 * 8];  // scale / min bytes [row][sub-block]
-        uint8_t mn[16 * 8];
-        float2 dd[16];       // {d, dmin} per row
+        float dsc[8][16];  // d * scale    [sub-block][row]
+        float dmf[8][16];  // dmin * min
     };
     template <int TM>
     static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &ex,
                                                       const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
         const uint8_t *wl = slice + j * pitch + SLOT * b;  // the row this lane feeds into the A operand
-        {   // lane (row j, pair c) unpacks one pair of 6-bit scales and parks it for the C-layout owners
+        {   // lane (row j, pair c) unpacks one pair of 6-bit scales / mins, folds the row's d / dmin in and parks
+            // the four factors for the lanes that own the row in the C layout
             const u32x4 h = *(const u32x4 *)wl;
             uint32_t sc2, m2;
             q4k_scale_min_pair(h.y, h.z, h.w, c, sc2, m2);
-            *(uint16_t *)&ex.sc[j * 8 + 2 * c] = (uint16_t)sc2;
-            *(uint16_t *)&ex.mn[j * 8 + 2 * c] = (uint16_t)m2;
-            if (c == 0)
-                ex.dd[j] = make_float2(half_bits_to_float((uint16_t)(h.x & 0xFFFF)), half_bits_to_float((uint16_t)(h.x >> 16)));
+            const float d = half_bits_to_float((uint16_t)(h.x & 0xFFFF)), dmin = half_bits_to_float((uint16_t)(h.x >> 16));
+            ex.dsc[2 * c][j] = d * (float)(sc2 & 0xFF);
+            ex.dsc[2 * c + 1][j] = d * (float)(sc2 >> 8);
+            ex.dmf[2 * c][j] = dmin * (float)(m2 & 0xFF);
+            ex.dmf[2 * c + 1][j] = dmin * (float)(m2 >> 8);
         }
         wave_lds_fence();
-        // my four C rows are 4c .. 4c+3: 8 scale bytes, 8 min bytes, {d, dmin} each
-        const u32x4 scA = *(const u32x4 *)&ex.sc[32 * c], scB = *(const u32x4 *)&ex.sc[32 * c + 16];
-        const u32x4 mnA = *(const u32x4 *)&ex.mn[32 * c], mnB = *(const u32x4 *)&ex.mn[32 * c + 16];
-        const float4 dd0 = *(const float4 *)&ex.dd[4 * c], dd1 = *(const float4 *)&ex.dd[4 * c + 2];
+        float4 dsq[8], dmq[8];  // my four C rows 4c .. 4c+3, per sub-block
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            dsq[t] = *(const float4 *)&ex.dsc[t][4 * c];
+            dmq[t] = *(const float4 *)&ex.dmf[t][4 * c];
+        }
         wave_lds_fence();  // the slots are rewritten by the next super-block
-        const uint32_t scw[8] = {scA.x, scA.y, scA.z, scA.w, scB.x, scB.y, scB.z, scB.w};
-        const uint32_t mnw[8] = {mnA.x, mnA.y, mnA.z, mnA.w, mnB.x, mnB.y, mnB.z, mnB.w};
-        const float dw[4] = {dd0.x, dd0.z, dd1.x, dd1.z}, dmn[4] = {dd0.y, dd0.w, dd1.y, dd1.w};
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             const u32x2 qa = *(const u32x2 *)(wl + 16 + 32 * (t >> 1) + 8 * c);
             const int sh = (t & 1) * 4;
             const uint32_t lo = (qa.x >> sh) & 0x0F0F0F0Fu, hi = (qa.y >> sh) & 0x0F0F0F0Fu;
             const long afrag = (long)(((uint64_t)hi << 32) | lo);
-            float dsc[4], dmf[4];  // d * sc and dmin * m of my four weight rows for this sub-block
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                dsc[i] = dw[i] * (float)((scw[2 * i + (t >> 2)] >> (8 * (t & 3))) & 0xFF);
-                dmf[i] = dmn[i] * (float)((mnw[2 * i + (t >> 2)] >> (8 * (t & 3))) & 0xFF);
-            }
+            const float dsc[4] = {dsq[t].x, dsq[t].y, dsq[t].z, dsq[t].w};  // d * sc and dmin * m of my four weight rows
+            const float dmf[4] = {dmq[t].x, dmq[t].y, dmq[t].z, dmq[t].w};
             int4v d[TM];  // all tiles of the sub-block first, so the matrix pipe runs under the rescale
 #pragma unroll
             for (int a = 0; a < TM; ++a) {
@@ -196,8 +192,11 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
     // slice pitch: an odd multiple of 16 bytes, so the 16 rows of an 8-byte pick fall in distinct banks
     constexpr int WPITCH = STG * F::SLOT + (((STG * F::SLOT / 16) & 1) ? 32 : 16);
     static_assert((WPITCH / 16) % 2 == 1, "pitch must be an odd number of 16-byte units");
-    __shared__ __align__(16) int8_t s_xq[BM * XROW];
-    __shared__ __align__(16) float2 s_xs[BM * 8];          // {d, d * bsum} per (row, block)
+    // few activation rows (TM <= 2): a super-block's work is too short to cover the latency of the next one's
+    // activation loads, so the tile holds a whole stage and is refilled once per stage, a stage ahead
+    constexpr int XS = TM <= 2 ? STG : 1;                       // super-blocks of activations in the tile
+    __shared__ __align__(16) int8_t s_xq[XS * BM * XROW];
+    __shared__ __align__(16) float2 s_xs[XS * BM * 8];          // {d, d * bsum} per (row, block)
     __shared__ __align__(16) uint8_t s_w[4][16 * WPITCH];  // per wavefront: the current stage's weight rows
     __shared__ __align__(16) typename F::Exchange s_ex[4];
 
@@ -230,26 +229,39 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
         }
     };
     // activations of one super-block: registers first (loaded a super-block ahead), then LDS
-    u32x4 xr[TM];
-    float xsd[XSC];
-    int xsb[XSC];
-    auto load_x = [&](int s) {
+    u32x4 xr[XS][TM];
+    float xsd[XS][XSC];
+    int xsb[XS][XSC];
+    auto load_x = [&](int s, int slot) __attribute__((always_inline)) {
         const int sb = min(s, nsb - 1);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int q = tid + i * 256, row = q >> 4, col = q & 15;
-            xr[i] = *(const u32x4 *)(xq + (size_t)min(m0 + row, M - 1) * K + (size_t)sb * 256 + col * 16);
+            xr[slot][i] = *(const u32x4 *)(xq + (size_t)min(m0 + row, M - 1) * K + (size_t)sb * 256 + col * 16);
         }
 #pragma unroll
         for (int i = 0; i < XSC; ++i) {
             const int e = min(tid + i * 256, BM * 8 - 1), row = e >> 3, t = e & 7;
             const Q8Scale v = xs[(size_t)min(m0 + row, M - 1) * (K >> 5) + sb * 8 + t];
-            xsd[i] = v.d;
-            xsb[i] = v.bsum;
+            xsd[slot][i] = v.d;
+            xsb[slot][i] = v.bsum;
+        }
+    };
+    auto park_x = [&](int slot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int q = tid + i * 256, row = q >> 4, col = q & 15;
+            *(u32x4 *)&s_xq[slot * BM * XROW + row * XROW + col * 16] = xr[slot][i];
+        }
+#pragma unroll
+        for (int i = 0; i < XSC; ++i) {
+            const int e = tid + i * 256;
+            if (BM * 8 % 256 == 0 || e < BM * 8) s_xs[slot * BM * 8 + e] = make_float2(xsd[slot][i], xsd[slot][i] * (float)xsb[slot][i]);
         }
     };
 
-    load_x(0);
+#pragma unroll
+    for (int b = 0; b < XS; ++b) load_x(b, b);
     load_stage(0);
 
     float acc[TM][4];
@@ -263,24 +275,28 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
         park_stage();
         load_stage(s0 + STG);
         wave_lds_fence();
+        if constexpr (XS > 1) {
 #pragma unroll
-        for (int b = 0; b < STG; ++b) {
-            const int s = s0 + b;
-            if (s < nsb) {  // uniform
+            for (int b = 0; b < STG; ++b) park_x(b);
+            __syncthreads();
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const int q = tid + i * 256, row = q >> 4, col = q & 15;
-                    *(u32x4 *)&s_xq[row * XROW + col * 16] = xr[i];
+            for (int b = 0; b < STG; ++b) load_x(s0 + STG + b, b);  // the next stage's activations fly under this stage
+#pragma unroll
+            for (int b = 0; b < STG; ++b)
+                if (s0 + b < nsb)  // uniform
+                    F::template superblock<TM>(s_w[wave], WPITCH, b, j, c, s_ex[wave], s_xq + b * BM * XROW, s_xs + b * BM * 8, acc);
+            __syncthreads();  // the activation tile is rewritten next
+        } else {
+#pragma unroll
+            for (int b = 0; b < STG; ++b) {
+                const int s = s0 + b;
+                if (s < nsb) {  // uniform
+                    park_x(0);
+                    __syncthreads();
+                    load_x(s + 1, 0);  // the next super-block's activations fly under this one's MFMAs
+                    F::template superblock<TM>(s_w[wave], WPITCH, b, j, c, s_ex[wave], s_xq, s_xs, acc);
+                    __syncthreads();  // the activation tile is rewritten next
                 }
-#pragma unroll
-                for (int i = 0; i < XSC; ++i) {
-                    const int e = tid + i * 256;
-                    if (BM * 8 % 256 == 0 || e < BM * 8) s_xs[e] = make_float2(xsd[i], xsd[i] * (float)xsb[i]);
-                }
-                __syncthreads();
-                load_x(s + 1);  // the next super-block's activations fly under this one's MFMAs
-                F::template superblock<TM>(s_w[wave], WPITCH, b, j, c, s_ex[wave], s_xq, s_xs, acc);
-                __syncthreads();  // the activation tile is rewritten next
             }
         }
     }
