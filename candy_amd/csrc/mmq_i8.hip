@@ -30,6 +30,8 @@
 //     super-block ahead into registers and parked in LDS between two barriers.
 // The rescale costs 16 VALU instructions per 16x16x32 tile (convert, multiply and two fused
 // multiply-adds per result register), which is what bounds the large-m rate.
+#include <cstdlib>
+
 #include "blocks.h"
 #include "internal.h"
 
@@ -183,10 +185,28 @@ struct TileQ6K {
 };
 
 // ---------------------------------------------------------------------------------------------
-template <class F, int TM, int STG>
-__global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
-                                                const Q8Scale *__restrict__ xs, float *__restrict__ y, int N, int M,
-                                                int K) {
+// LDS carve-up of k_mmq_i8 (dynamic: the K-split variant needs more than the 64 KB a static layout may take)
+template <class F, int TM, int STG, int KS>
+struct MmqI8Lds {
+    static constexpr int BM = 16 * TM;
+    static constexpr int WPITCH = STG * F::SLOT + (((STG * F::SLOT / 16) & 1) ? 32 : 16);
+    static constexpr int XS = TM <= 2 ? STG : 1;
+    static constexpr int XQ = XS * BM * XROW;                         // activation quants of one K group
+    static constexpr int XSS = XS * BM * 8 * (int)sizeof(float2);     // their {d, d * bsum}
+    static constexpr int SW = 16 * WPITCH;                            // one wavefront's weight slice
+    static constexpr int EX = ((int)sizeof(typename F::Exchange) + 15) & ~15;
+    static constexpr int PART = KS > 1 ? 4 * 64 * TM * 4 * (int)sizeof(float) : 0;
+    static constexpr int BYTES = KS * (XQ + XSS) + 4 * KS * (SW + EX) + PART;
+};
+
+// KS = 2: eight wavefronts, the second four walk the second half of K for the same 64 weight rows (a grid of
+// few workgroups leaves one wavefront per SIMD, which waits out every latency of its own instruction stream);
+// the halves are added through LDS, first half + second half.
+template <class F, int TM, int STG, int KS>
+__global__ __launch_bounds__(256 * KS) void k_mmq_i8(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
+                                                     const Q8Scale *__restrict__ xs, float *__restrict__ y, int N, int M,
+                                                     int K) {
+    typedef MmqI8Lds<F, TM, STG, KS> L;
     constexpr int BM = 16 * TM;
     constexpr int XSC = (BM * 8 + 255) / 256;  // activation scales per thread per super-block
     // slice pitch: an odd multiple of 16 bytes, so the 16 rows of an 8-byte pick fall in distinct banks
@@ -195,16 +215,24 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
     // few activation rows (TM <= 2): a super-block's work is too short to cover the latency of the next one's
     // activation loads, so the tile holds a whole stage and is refilled once per stage, a stage ahead
     constexpr int XS = TM <= 2 ? STG : 1;                       // super-blocks of activations in the tile
-    __shared__ __align__(16) int8_t s_xq[XS * BM * XROW];
-    __shared__ __align__(16) float2 s_xs[XS * BM * 8];          // {d, d * bsum} per (row, block)
-    __shared__ __align__(16) uint8_t s_w[4][16 * WPITCH];  // per wavefront: the current stage's weight rows
-    __shared__ __align__(16) typename F::Exchange s_ex[4];
+    static_assert(KS == 1 || XS > 1, "the K split goes with the stage-wide activation tile");
+    static_assert(WPITCH == L::WPITCH && XS == L::XS, "layout");
+    extern __shared__ __align__(16) uint8_t smem_i8[];
+    const int kg = threadIdx.x >> 8;                     // K group of this thread
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6, gw = threadIdx.x >> 6;
+    int8_t *s_xq = (int8_t *)smem_i8 + kg * L::XQ;                                  // [XS][BM][XROW]
+    float2 *s_xs = (float2 *)(smem_i8 + KS * L::XQ + kg * L::XSS);                  // {d, d * bsum} [XS][BM][8]
+    uint8_t *s_wm = smem_i8 + KS * (L::XQ + L::XSS) + gw * L::SW;                   // this wavefront's weight rows
+    typename F::Exchange &s_exm = *(typename F::Exchange *)(smem_i8 + KS * (L::XQ + L::XSS) + 4 * KS * L::SW + gw * L::EX);
+    float *s_part = (float *)(smem_i8 + KS * (L::XQ + L::XSS) + 4 * KS * (L::SW + L::EX));
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 15, c = lane >> 4;
     const int n0 = blockIdx.x * 64 + wave * 16, m0 = blockIdx.y * BM;
     const int nsb = K >> 8;
     const size_t rb = (size_t)nsb * F::BLOCK;
+    // the super-blocks of this K group: [sb_lo, sb_hi), `per` (whole stages) for every group
+    const int per = ((nsb + KS - 1) / KS + STG - 1) / STG * STG;
+    const int sb_lo = kg * per, sb_hi = min(nsb, sb_lo + per);
 
     // weights of one stage: 16 rows x STG blocks as 16-byte chunks along the rows, in registers
     // while in flight, then parked in the wavefront's LDS slice
@@ -225,7 +253,7 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
 #pragma unroll
         for (int i = 0; i < WCH; ++i) {
             const int q = lane + 64 * i, row = q / CPR, col = q % CPR;
-            if ((16 * CPR) % 64 == 0 || q < 16 * CPR) *(u32x4 *)&s_w[wave][row * WPITCH + col * 16] = wr[i];
+            if ((16 * CPR) % 64 == 0 || q < 16 * CPR) *(u32x4 *)&s_wm[row * WPITCH + col * 16] = wr[i];
         }
     };
     // activations of one super-block: registers first (loaded a super-block ahead), then LDS
@@ -261,8 +289,8 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
     };
 
 #pragma unroll
-    for (int b = 0; b < XS; ++b) load_x(b, b);
-    load_stage(0);
+    for (int b = 0; b < XS; ++b) load_x(sb_lo + b, b);
+    load_stage(sb_lo);
 
     float acc[TM][4];
 #pragma unroll
@@ -270,7 +298,8 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[a][i] = 0.0f;
 
-    for (int s0 = 0; s0 < nsb; s0 += STG) {
+    for (int it = 0; it < per; it += STG) {  // the same trip count in every K group: the barriers are workgroup-wide
+        const int s0 = sb_lo + it;
         wave_lds_fence();  // this wavefront is done reading the previous stage
         park_stage();
         load_stage(s0 + STG);
@@ -283,24 +312,38 @@ __global__ __launch_bounds__(256) void k_mmq_i8(const uint8_t *__restrict__ W, c
             for (int b = 0; b < STG; ++b) load_x(s0 + STG + b, b);  // the next stage's activations fly under this stage
 #pragma unroll
             for (int b = 0; b < STG; ++b)
-                if (s0 + b < nsb)  // uniform
-                    F::template superblock<TM>(s_w[wave], WPITCH, b, j, c, s_ex[wave], s_xq + b * BM * XROW, s_xs + b * BM * 8, acc);
+                if (s0 + b < sb_hi)  // uniform over the wavefront
+                    F::template superblock<TM>(s_wm, WPITCH, b, j, c, s_exm, s_xq + b * BM * XROW, s_xs + b * BM * 8, acc);
             __syncthreads();  // the activation tile is rewritten next
         } else {
 #pragma unroll
             for (int b = 0; b < STG; ++b) {
                 const int s = s0 + b;
-                if (s < nsb) {  // uniform
+                if (s < sb_hi) {  // uniform
                     park_x(0);
                     __syncthreads();
                     load_x(s + 1, 0);  // the next super-block's activations fly under this one's MFMAs
-                    F::template superblock<TM>(s_w[wave], WPITCH, b, j, c, s_ex[wave], s_xq, s_xs, acc);
+                    F::template superblock<TM>(s_wm, WPITCH, b, j, c, s_exm, s_xq, s_xs, acc);
                     __syncthreads();  // the activation tile is rewritten next
                 }
             }
         }
     }
 
+    if constexpr (KS > 1) {  // second half of K handed to the first through LDS
+        float4 *slot = (float4 *)s_part + (wave * 64 + lane) * TM;
+        if (kg == 1) {
+#pragma unroll
+            for (int a = 0; a < TM; ++a) slot[a] = make_float4(acc[a][0], acc[a][1], acc[a][2], acc[a][3]);
+        }
+        __syncthreads();
+        if (kg == 1) return;
+#pragma unroll
+        for (int a = 0; a < TM; ++a) {
+            const float4 o = slot[a];
+            acc[a][0] += o.x; acc[a][1] += o.y; acc[a][2] += o.z; acc[a][3] += o.w;
+        }
+    }
     // C layout: lane holds activation row j of each m-tile and weight rows 4c .. 4c+3
 #pragma unroll
     for (int a = 0; a < TM; ++a) {
@@ -323,15 +366,22 @@ static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const in
     const int N = (int)w->rows, K = (int)w->cols, M = (int)m;
     const unsigned gx = (unsigned)((N + 63) / 64);
     constexpr int DEEP = F::SLOT == 144 ? 4 : 2;  // super-blocks per stage where m is small (LDS budget)
-#define CANDY_MMQ_I8(TMV, STGV)                                                                                       \
-    hipLaunchKernelGGL((k_mmq_i8<F, TMV, STGV>), dim3(gx, (unsigned)((M + 16 * TMV - 1) / (16 * TMV))), dim3(256), 0, \
-                       dev->stream, (const uint8_t *)w->data, qs, scales, y, N, M, K)
+#define CANDY_MMQ_I8(TMV, STGV, KSV)                                                                            \
+    do {                                                                                                        \
+        constexpr int lds = MmqI8Lds<F, TMV, STGV, KSV>::BYTES;                                                 \
+        auto kern = k_mmq_i8<F, TMV, STGV, KSV>;                                                                \
+        CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds)); \
+        hipLaunchKernelGGL(kern, dim3(gx, (unsigned)((M + 16 * TMV - 1) / (16 * TMV))), dim3(256 * KSV), lds,   \
+                           dev->stream, (const uint8_t *)w->data, qs, scales, y, N, M, K);                      \
+    } while (0)
     // the largest tile height that still leaves about 1.5 wavefronts per SIMD: a wavefront walks the
     // whole contraction on its own, so a grid below that leaves load latency exposed
     const int64_t strips = (N + 15) / 16, want = 1536;
-    if (M > 32 && strips * ((M + 63) / 64) >= want) CANDY_MMQ_I8(4, 2);
-    else if (M > 16 && strips * ((M + 31) / 32) >= want) CANDY_MMQ_I8(2, DEEP);
-    else CANDY_MMQ_I8(1, DEEP);
+    static const bool no_ks = getenv("CANDY_HIP_MMQ_I8_NO_KSPLIT") != nullptr;
+    if (M > 32 && strips * ((M + 63) / 64) >= want) CANDY_MMQ_I8(4, 2, 1);
+    else if (M > 16 && strips * ((M + 31) / 32) >= want) CANDY_MMQ_I8(2, DEEP, 1);
+    else if (!no_ks && (int64_t)gx * ((M + 15) / 16) < 2 * dev->num_cus && (K >> 8) >= 2 * DEEP) CANDY_MMQ_I8(1, DEEP, 2);
+    else CANDY_MMQ_I8(1, DEEP, 1);
 #undef CANDY_MMQ_I8
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
