@@ -9,14 +9,18 @@ from candy_amd import gguf, synth
 from oracle import oracle as o
 
 
-def tiny_model(seed=1, tied=False):
+OTHER_FORMATS = {"attn_q": synth.Q5_K, "attn_k": synth.Q5_0, "attn_v": synth.Q5_1, "attn_output": synth.Q4_1,
+                 "ffn_gate": synth.Q3_K, "ffn_up": synth.Q2_K, "ffn_down": synth.Q5_K}
+
+
+def tiny_model(seed=1, tied=False, fmts=None):
     cfg = dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=64, d_ffn=512, vocab=96, max_pos=32,
                rms_eps=1e-6, rope_base=50000.0)
     qd, kvd = 256, 128
     shapes = {"attn_q": (qd, 256), "attn_k": (kvd, 256), "attn_v": (kvd, 256), "attn_output": (256, qd),
               "ffn_gate": (512, 256), "ffn_up": (512, 256), "ffn_down": (256, 512)}
-    fmts = {"attn_q": synth.Q4_K, "attn_k": synth.Q8_0, "attn_v": synth.Q6_K, "attn_output": synth.Q4_K,
-            "ffn_gate": synth.Q4_0, "ffn_up": synth.Q4_K, "ffn_down": synth.Q6_K}
+    fmts = fmts or {"attn_q": synth.Q4_K, "attn_k": synth.Q8_0, "attn_v": synth.Q6_K, "attn_output": synth.Q4_K,
+                    "ffn_gate": synth.Q4_0, "ffn_up": synth.Q4_K, "ffn_down": synth.Q6_K}
     rng = np.random.default_rng(seed)
     orig, tensors, s = {}, [], seed * 100
     for l in range(cfg["n_layers"]):
