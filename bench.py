@@ -204,20 +204,21 @@ def llama3_leg(dev, n_prompt=512, n_decode=128):
 
 
 def prefill_kv(dev, model, cfg, n_pos, seed=9):
-    """KV cache positions [0, n_pos) <- N(0,1) f32."""
+    """KV cache positions [0, n_pos) <- N(0,1), in the cache's element type (f32, or fp16 after set_kv_f16)."""
     from candy_amd import hip
     kptr, vptr, nbytes = model.kv_cache()
     rng = np.random.Generator(np.random.Philox(seed))
     per_head = cfg["max_pos"] * cfg["head_dim"]
-    rows = cfg["n_layers"] * cfg["n_kv_heads"]
+    elem = nbytes // (cfg["n_layers"] * cfg["n_kv_heads"] * per_head)
+    dt = {4: np.float32, 2: np.float16}[elem]
     chunk = np.empty((cfg["n_kv_heads"], n_pos, cfg["head_dim"]), np.float32)
     for base in (kptr, vptr):
         for l in range(cfg["n_layers"]):
             rng.standard_normal(chunk.shape, dtype=np.float32, out=chunk)
+            rows = chunk.astype(dt)
             for h in range(cfg["n_kv_heads"]):
-                off = ((l * cfg["n_kv_heads"] + h) * per_head) * 4
-                hip._check(hip.lib().candy_hip_h2d(dev.handle, base + off, chunk[h].ctypes.data, chunk[h].nbytes))
-    del rows
+                off = ((l * cfg["n_kv_heads"] + h) * per_head) * elem
+                hip._check(hip.lib().candy_hip_h2d(dev.handle, base + off, rows[h].ctypes.data, rows[h].nbytes))
 
 
 def decode_leg(dev, steps, warmup):
@@ -225,31 +226,39 @@ def decode_leg(dev, steps, warmup):
     log("building random-init 7B (N(0, 0.02) quantized to Q4_K, Q6_K head) ...")
     n_pos = 2048
     cfg, model = build_7b(dev, max_pos=n_pos + steps + warmup + 8)
-    prefill_kv(dev, model, cfg, n_pos)
-    rng = np.random.default_rng(1234)
-    prompt = rng.integers(0, cfg["vocab"], 128)
-    tok = int(prompt[-1])
-    pos = n_pos
-    for _ in range(warmup):
-        tok, _ = model.decode(tok, pos, want_logits=False)
-        pos += 1
-    dev.synchronize()
-    t0 = time.perf_counter()
-    toks = []
-    for _ in range(steps):
-        tok, _ = model.decode(tok, pos, want_logits=False)
-        toks.append(tok)
-        pos += 1
-    dev.synchronize()
-    dt = time.perf_counter() - t0
     layer_bytes = 4 * synth.weight_nbytes(synth.Q4_K, 4096, 4096) + 3 * synth.weight_nbytes(synth.Q4_K, 11008, 4096)
-    kv_bytes = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * n_pos * cfg["head_dim"] * 4
-    bpt = cfg["n_layers"] * layer_bytes + synth.weight_nbytes(synth.Q6_K, 32000, 4096) + kv_bytes
-    ms = dt / steps * 1e3
+    weight_bytes = cfg["n_layers"] * layer_bytes + synth.weight_nbytes(synth.Q6_K, 32000, 4096)
+
+    def run(kv_elem_bytes):
+        prefill_kv(dev, model, cfg, n_pos)
+        tok = int(np.random.default_rng(1234).integers(0, cfg["vocab"], 128)[-1])
+        pos = n_pos
+        for _ in range(warmup):
+            tok, _ = model.decode(tok, pos, want_logits=False)
+            pos += 1
+        dev.synchronize()
+        t0 = time.perf_counter()
+        toks = []
+        for _ in range(steps):
+            tok, _ = model.decode(tok, pos, want_logits=False)
+            toks.append(tok)
+            pos += 1
+        dev.synchronize()
+        dt = time.perf_counter() - t0
+        kv_bytes = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * n_pos * cfg["head_dim"] * kv_elem_bytes
+        bpt = weight_bytes + kv_bytes
+        ms = dt / steps * 1e3
+        return {"tok_s": round(steps / dt, 2), "ms_per_token": round(ms, 4), "steps": steps, "kv_positions": n_pos,
+                "bytes_per_token": bpt, "hbm_GBps": round(bpt / (ms * 1e-3) / 1e9, 1),
+                "hbm_frac": round(bpt / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "tokens": toks[:8]}
+
+    out = run(4)  # candy's cache is f32: this is the figure quoted
+    # the optional half-size cache, beside it (k and v rounded to fp16 on entry; not what the reference computes)
+    model.set_kv_f16(True)
+    half = run(2)
+    out["fp16_kv_cache"] = {k: half[k] for k in ("tok_s", "ms_per_token", "bytes_per_token", "hbm_GBps", "hbm_frac")}
     model.free()
-    return {"tok_s": round(steps / dt, 2), "ms_per_token": round(ms, 4), "steps": steps, "kv_positions": n_pos,
-            "bytes_per_token": bpt, "hbm_GBps": round(bpt / (ms * 1e-3) / 1e9, 1),
-            "hbm_frac": round(bpt / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "tokens": toks[:8]}
+    return out
 
 
 def main():

@@ -37,8 +37,8 @@ struct AttnArgs {
     const float *v_new;    // optional [n_kv_heads, hd]
     const float *cos_t;    // [max_pos, hd/2] (only with k_new)
     const float *sin_t;
-    float *k_cache;        // [n_kv_heads, *, hd], cache_stride elements between heads
-    float *v_cache;
+    void *k_cache;         // [n_kv_heads, *, hd] of f32 or fp16 (the kernel's KV type), cache_stride elements between heads
+    void *v_cache;
     const int *pos_ptr;    // optional: position of the new token in device memory
     int n_pos;             // used when pos_ptr is null: positions 0..n_pos-1 are in the cache
     int64_t cache_stride;
@@ -51,11 +51,14 @@ struct AttnArgs {
     Q8Scale *os;
 };
 
-template <int GROUP, int VEC>
+// KV: float (candy's cache) or _Float16 (optional: half the bytes of the step's largest stream; the rows are
+// rounded once, when they enter the cache, and every product and sum stays f32).
+template <int GROUP, int VEC, class KV>
 __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
     constexpr int HD = 32 * VEC;
     constexpr int UNR = 4;
     typedef float vecf __attribute__((ext_vector_type(VEC)));
+    typedef KV veckv __attribute__((ext_vector_type(VEC)));
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hw = lane >> 5, hl = lane & 31;
     const int kvh = blockIdx.x, split = blockIdx.y;
@@ -64,8 +67,8 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
     const int n_cached = fresh ? pos : pos + 1;               // rows to read from the cache
     const int per = (n_cached + a.n_splits - 1) / a.n_splits;
     const int p0 = split * per, p1 = min(n_cached, p0 + per);
-    float *kh = a.k_cache + (size_t)kvh * a.cache_stride;
-    float *vh = a.v_cache + (size_t)kvh * a.cache_stride;
+    KV *kh = (KV *)a.k_cache + (size_t)kvh * a.cache_stride;
+    KV *vh = (KV *)a.v_cache + (size_t)kvh * a.cache_stride;
 
     // Rope pairs (i, i + HD/2) sit 16 lanes apart inside the half-wavefront
     vecf cs, sn;
@@ -140,8 +143,8 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
             valid[u] = p < p1;
             const size_t off = (size_t)max(min(p, p1 - 1), 0) * HD + hl * VEC;
             // every cache byte is read once, by one instruction: stream it past the caches
-            kv[u] = __builtin_nontemporal_load((const vecf *)(kh + off));
-            vv[u] = __builtin_nontemporal_load((const vecf *)(vh + off));
+            kv[u] = __builtin_convertvector(__builtin_nontemporal_load((const veckv *)(kh + off)), vecf);
+            vv[u] = __builtin_convertvector(__builtin_nontemporal_load((const veckv *)(vh + off)), vecf);
         }
     };
     {
@@ -168,11 +171,14 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
     // the new token: Rope its key, append both rows to the cache, attend to them from registers
     if (fresh && split == a.n_splits - 1 && wave == 0) {
         vecf kn = rope(*(const vecf *)(a.k_new + (size_t)kvh * HD + hl * VEC));
-        const vecf vn = *(const vecf *)(a.v_new + (size_t)kvh * HD + hl * VEC);
+        vecf vn = *(const vecf *)(a.v_new + (size_t)kvh * HD + hl * VEC);
+        const veckv kc = __builtin_convertvector(kn, veckv), vc = __builtin_convertvector(vn, veckv);
         if (hw == 0) {
-            *(vecf *)(kh + (size_t)pos * HD + hl * VEC) = kn;
-            *(vecf *)(vh + (size_t)pos * HD + hl * VEC) = vn;
+            *(veckv *)(kh + (size_t)pos * HD + hl * VEC) = kc;
+            *(veckv *)(vh + (size_t)pos * HD + hl * VEC) = vc;
         }
+        kn = __builtin_convertvector(kc, vecf);  // attend to the rows as the cache holds them
+        vn = __builtin_convertvector(vc, vecf);
         vecf kv[UNR], vv[UNR];
         bool valid[UNR];
 #pragma unroll
@@ -284,19 +290,19 @@ size_t attention_scratch_bytes(int n_heads, int n_kv_heads, int head_dim, int n_
     return ((size_t)n_heads * n_splits * (head_dim + 2) + 64) * sizeof(float);
 }
 
-template <int GROUP>
+template <int GROUP, class KV>
 static int launch_group(candy_hip_device *dev, const AttnArgs &a, int n_kv_heads, int head_dim) {
     dim3 grid((unsigned)n_kv_heads, (unsigned)a.n_splits);
     const unsigned n_heads = (unsigned)(n_kv_heads * GROUP);
     switch (head_dim) {
     case 64:
-        hipLaunchKernelGGL((k_attn_decode<GROUP, 2>), grid, dim3(256), 0, dev->stream, a);
+        hipLaunchKernelGGL((k_attn_decode<GROUP, 2, KV>), grid, dim3(256), 0, dev->stream, a);
         CANDY_LAUNCH_CHECK();
         hipLaunchKernelGGL((k_attn_merge<64>), dim3(n_heads), dim3(64), 0, dev->stream, a.part_o, a.part_ml, a.n_splits,
                            a.out, a.oq, a.os);
         break;
     case 128:
-        hipLaunchKernelGGL((k_attn_decode<GROUP, 4>), grid, dim3(256), 0, dev->stream, a);
+        hipLaunchKernelGGL((k_attn_decode<GROUP, 4, KV>), grid, dim3(256), 0, dev->stream, a);
         CANDY_LAUNCH_CHECK();
         hipLaunchKernelGGL((k_attn_merge<128>), dim3(n_heads), dim3(128), 0, dev->stream, a.part_o, a.part_ml,
                            a.n_splits, a.out, a.oq, a.os);
@@ -315,11 +321,19 @@ int launch_attention(candy_hip_device *dev, const AttnLaunch &L) {
     a.part_o = (float *)L.scratch;
     a.part_ml = a.part_o + (size_t)L.n_heads * L.n_splits * L.head_dim;
     a.out = L.out; a.oq = L.oq; a.os = L.os;
-    switch (L.n_heads / L.n_kv_heads) {
-    case 1: return launch_group<1>(dev, a, L.n_kv_heads, L.head_dim);
-    case 2: return launch_group<2>(dev, a, L.n_kv_heads, L.head_dim);
-    case 4: return launch_group<4>(dev, a, L.n_kv_heads, L.head_dim);
-    case 8: return launch_group<8>(dev, a, L.n_kv_heads, L.head_dim);
+    const int group = L.n_heads / L.n_kv_heads;
+    if (L.kv_f16) switch (group) {
+        case 1: return launch_group<1, _Float16>(dev, a, L.n_kv_heads, L.head_dim);
+        case 2: return launch_group<2, _Float16>(dev, a, L.n_kv_heads, L.head_dim);
+        case 4: return launch_group<4, _Float16>(dev, a, L.n_kv_heads, L.head_dim);
+        case 8: return launch_group<8, _Float16>(dev, a, L.n_kv_heads, L.head_dim);
+        default: return fail(CANDY_HIP_ERR_UNSUPPORTED, "query heads per kv head must be 1, 2, 4 or 8");
+        }
+    switch (group) {
+    case 1: return launch_group<1, float>(dev, a, L.n_kv_heads, L.head_dim);
+    case 2: return launch_group<2, float>(dev, a, L.n_kv_heads, L.head_dim);
+    case 4: return launch_group<4, float>(dev, a, L.n_kv_heads, L.head_dim);
+    case 8: return launch_group<8, float>(dev, a, L.n_kv_heads, L.head_dim);
     default: return fail(CANDY_HIP_ERR_UNSUPPORTED, "query heads per kv head must be 1, 2, 4 or 8");
     }
 }

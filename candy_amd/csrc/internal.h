@@ -168,8 +168,9 @@ struct AttnLaunch {
     const float *v_new = nullptr;
     const float *cos_t = nullptr;  // Rope tables [max_pos, head_dim/2] (with k_new)
     const float *sin_t = nullptr;
-    float *k_cache = nullptr;      // this layer's cache, cache_stride elements between kv heads
-    float *v_cache = nullptr;
+    void *k_cache = nullptr;       // this layer's cache (f32, or fp16 with kv_f16), cache_stride elements between kv heads
+    void *v_cache = nullptr;
+    bool kv_f16 = false;
     const int *pos_ptr = nullptr;  // position of the new token in device memory, or
     int n_pos = 0;                 // number of cached positions to attend when pos_ptr is null
     int64_t cache_stride = 0;
@@ -199,9 +200,10 @@ int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int
                     int64_t m, float *y, const _Float16 *xh_ready = nullptr, const float *res = nullptr);
 // prefill.hip: prompt stages of the decoder (n tokens at positions pos0 ..).
 int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, const float *v, const float *cos_t,
-                           const float *sin_t, float *k_cache, float *v_cache, int n, int pos0, int n_heads,
+                           const float *sin_t, void *k_cache, void *v_cache, bool kv_f16, int n, int pos0, int n_heads,
                            int n_kv_heads, int head_dim, int64_t cache_stride);
-int launch_attn_prefill(candy_hip_device *dev, const float *q, const float *k_cache, const float *v_cache, float *out,
-                        int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride, float scale);
+int launch_attn_prefill(candy_hip_device *dev, const float *q, const void *k_cache, const void *v_cache, bool kv_f16,
+                        float *out, int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride,
+                        float scale);
 
 }  // namespace candy

@@ -25,7 +25,8 @@ struct candy_hip_llama {
     const float *out_norm = nullptr;
     const candy_hip_qtensor *head = nullptr, *embed = nullptr;
     // device buffers
-    float *k_cache = nullptr, *v_cache = nullptr;  // [n_layers][n_kv_heads][max_pos][head_dim]
+    float *k_cache = nullptr, *v_cache = nullptr;  // [n_layers][n_kv_heads][max_pos][head_dim], f32 or (kv_f16) fp16 in the same memory
+    bool kv_f16 = false;
     float *cos_t = nullptr, *sin_t = nullptr;      // [max_pos][head_dim/2]
     float *h = nullptr, *q = nullptr, *k = nullptr, *v = nullptr;
     float *gate_o = nullptr, *up_o = nullptr, *logits = nullptr;
@@ -269,8 +270,19 @@ int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, s
     if (dev_k) *dev_k = m->k_cache;
     if (dev_v) *dev_v = m->v_cache;
     if (bytes_each)
-        *bytes_each = (size_t)m->cfg.n_layers * m->cfg.n_kv_heads * m->cfg.max_pos * m->cfg.head_dim * sizeof(float);
+        *bytes_each = (size_t)m->cfg.n_layers * m->cfg.n_kv_heads * m->cfg.max_pos * m->cfg.head_dim * (m->kv_f16 ? 2 : 4);
     return CANDY_HIP_OK;
+}
+
+int candy_hip_llama_set_kv_f16(candy_hip_llama *m, int enable) {
+    CANDY_REQUIRE(m, "model is nil");
+    if (int rc = use_device(m->dev)) return rc;
+    m->kv_f16 = enable != 0;
+    m->graph_dirty = m->tables_dirty = true;
+    // the cache's contents do not survive a change of element type
+    const size_t kv = (size_t)m->cfg.n_layers * m->cfg.n_kv_heads * m->cfg.max_pos * m->cfg.head_dim;
+    if (int rc = candy_hip_zero(m->dev, m->k_cache, kv * sizeof(float))) return rc;
+    return candy_hip_zero(m->dev, m->v_cache, kv * sizeof(float));
 }
 
 static int llama_check_complete(const candy_hip_llama *m) {
@@ -288,6 +300,12 @@ static int llama_check_complete(const candy_hip_llama *m) {
 // synchronises, so the sequence can be captured once and replayed for every token.
 // y_i = W_i . q8(rmsnorm(h) * alpha) for up to three weights: one fused launch, or
 // RMSNorm+quantize then the batch-1 kernel when no fused instantiation covers the shape.
+// Layer l's part of a cache array (elements are 4 bytes, or 2 with the fp16 cache).
+static void *layer_cache(const candy_hip_llama *m, float *base, int l) {
+    const size_t layer_kv = (size_t)m->cfg.n_kv_heads * m->cfg.max_pos * m->cfg.head_dim;
+    return (uint8_t *)base + (size_t)l * layer_kv * (m->kv_f16 ? 2 : 4);
+}
+
 static int norm_linear(candy_hip_llama *m, const float *alpha, const candy_hip_qtensor *const *ws, float *const *ys,
                        int n) {
     const candy_hip_llama_config &c = m->cfg;
@@ -323,7 +341,7 @@ static int linear_residual(candy_hip_llama *m, const candy_hip_qtensor *w) {
 static bool persist_covers(const candy_hip_llama *m) {
     const candy_hip_llama_config &c = m->cfg;
     const int G = m->dev->num_cus;
-    if (c.head_dim != 128 || c.n_heads != c.n_kv_heads || c.n_heads * c.head_dim != c.d_model) return false;
+    if (m->kv_f16 || c.head_dim != 128 || c.n_heads != c.n_kv_heads || c.n_heads * c.head_dim != c.d_model) return false;
     if (c.d_model > 4096 || c.d_model % 256 || c.d_ffn > 16384 || c.d_ffn % 256 || 6 * c.n_layers + 2 >= 4096) return false;
     if (G % c.n_heads) return false;
     const int S = G / c.n_heads;
@@ -405,7 +423,7 @@ static int llama_enqueue_step(candy_hip_llama *m) {
     int rc;
     for (int l = 0; l < c.n_layers; ++l) {
         const candy_hip_llama::Layer &L = m->layers[l];
-        float *kc = m->k_cache + (size_t)l * layer_kv, *vc = m->v_cache + (size_t)l * layer_kv;
+        void *kc = layer_cache(m, m->k_cache, l), *vc = layer_cache(m, m->v_cache, l);
         {   // RMSNorm + quantize + q/k/v
             const candy_hip_qtensor *ws[3] = {L.wq, L.wk, L.wv};
             float *ys[3] = {m->q, m->k, m->v};
@@ -414,7 +432,7 @@ static int llama_enqueue_step(candy_hip_llama *m) {
         {   // Rope on q and the new k, append k/v to the cache, attention; the merge quantizes for Wo
             AttnLaunch A;
             A.q = m->q; A.k_new = m->k; A.v_new = m->v; A.cos_t = m->cos_t; A.sin_t = m->sin_t;
-            A.k_cache = kc; A.v_cache = vc; A.pos_ptr = m->d_pos;
+            A.k_cache = kc; A.v_cache = vc; A.kv_f16 = m->kv_f16; A.pos_ptr = m->d_pos;
             A.cache_stride = (int64_t)c.max_pos * c.head_dim; A.scale = scale;
             A.n_heads = c.n_heads; A.n_kv_heads = c.n_kv_heads; A.head_dim = c.head_dim; A.n_splits = m->n_splits;
             A.scratch = m->attn_scratch;
@@ -545,7 +563,7 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
     if ((rc = candy_hip_qindex_select(dev, m->embed, P.ids, n, P.h))) return rc;
     for (int l = 0; l < c.n_layers; ++l) {
         const candy_hip_llama::Layer &L = m->layers[l];
-        float *kc = m->k_cache + (size_t)l * layer_kv, *vc = m->v_cache + (size_t)l * layer_kv;
+        void *kc = layer_cache(m, m->k_cache, l), *vc = layer_cache(m, m->v_cache, l);
         // Where a projection runs on the fp16 tiles, the kernel that quantizes its input also writes the
         // fp16 expansion (one conversion for q/k/v, one for gate/up), and the residual add rides in the
         // projection's epilogue.
@@ -560,10 +578,10 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
         if ((rc = launch_contract(dev, L.wq, P.xq, P.xs, n, P.q, xh_for(L.wq)))) return rc;
         if ((rc = launch_contract(dev, L.wk, P.xq, P.xs, n, P.k, xh_for(L.wk)))) return rc;
         if ((rc = launch_contract(dev, L.wv, P.xq, P.xs, n, P.v, xh_for(L.wv)))) return rc;
-        if ((rc = launch_prefill_rope_kv(dev, P.q, P.k, P.v, m->cos_t, m->sin_t, kc, vc, n, pos0, c.n_heads,
+        if ((rc = launch_prefill_rope_kv(dev, P.q, P.k, P.v, m->cos_t, m->sin_t, kc, vc, m->kv_f16, n, pos0, c.n_heads,
                                          c.n_kv_heads, c.head_dim, cache_stride)))
             return rc;
-        if ((rc = launch_attn_prefill(dev, P.q, kc, vc, P.att, n, pos0, c.n_heads, c.n_kv_heads, c.head_dim,
+        if ((rc = launch_attn_prefill(dev, P.q, kc, vc, m->kv_f16, P.att, n, pos0, c.n_heads, c.n_kv_heads, c.head_dim,
                                       cache_stride, scale)))
             return rc;
         if ((rc = launch_quantize_q8(dev, P.att, n, qd, P.xq, P.xs, nullptr, xh_for(L.wo)))) return rc;

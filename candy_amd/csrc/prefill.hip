@@ -16,11 +16,24 @@
 
 namespace candy {
 
+// Four consecutive cache values as f32; KV is float (candy's cache) or _Float16 (the optional half-size cache).
+template <class KV>
+__device__ __forceinline__ float4 kv_load4(const KV *p);
+template <>
+__device__ __forceinline__ float4 kv_load4<float>(const float *p) { return *(const float4 *)p; }
+template <>
+__device__ __forceinline__ float4 kv_load4<_Float16>(const _Float16 *p) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 v = *(const h4 *)p;
+    return make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
+}
+
+template <class KV>
 __global__ __launch_bounds__(256) void k_prefill_rope_kv(float *__restrict__ q, const float *__restrict__ k,
                                                          const float *__restrict__ v,
                                                          const float *__restrict__ cos_t,
-                                                         const float *__restrict__ sin_t, float *__restrict__ k_cache,
-                                                         float *__restrict__ v_cache, int n, int pos0, int n_heads,
+                                                         const float *__restrict__ sin_t, KV *__restrict__ k_cache,
+                                                         KV *__restrict__ v_cache, int n, int pos0, int n_heads,
                                                          int n_kv_heads, int head_dim, int64_t cache_stride) {
     const int half = head_dim >> 1;
     const int slots = n_heads + 2 * n_kv_heads;  // q heads, then k heads, then v heads
@@ -40,25 +53,25 @@ __global__ __launch_bounds__(256) void k_prefill_rope_kv(float *__restrict__ q, 
     } else if (slot < n_heads + n_kv_heads) {
         const int h = slot - n_heads;
         const float *p = k + ((size_t)i * n_kv_heads + h) * head_dim + j;
-        float *dst = k_cache + (size_t)h * cache_stride + (size_t)pos * head_dim + j;
+        KV *dst = k_cache + (size_t)h * cache_stride + (size_t)pos * head_dim + j;
         const float a = p[0], b = p[half];
-        dst[0] = a * c - b * s;
-        dst[half] = a * s + b * c;
+        dst[0] = (KV)(a * c - b * s);
+        dst[half] = (KV)(a * s + b * c);
     } else {
         const int h = slot - n_heads - n_kv_heads;
         const float *p = v + ((size_t)i * n_kv_heads + h) * head_dim + j;
-        float *dst = v_cache + (size_t)h * cache_stride + (size_t)pos * head_dim + j;
-        dst[0] = p[0];
-        dst[half] = p[half];
+        KV *dst = v_cache + (size_t)h * cache_stride + (size_t)pos * head_dim + j;
+        dst[0] = (KV)p[0];
+        dst[half] = (KV)p[half];
     }
 }
 
 // grid (n_heads, ceil(n / 32)), 256 threads. Thread t serves query row t/8 throughout: in the score
 // phase it owns keys {t%8 + 8r}, in the output phase columns {4*(t%8) + 32r .. +3}; the 8 threads of
 // a row sit in adjacent lanes, so the row maximum and sum are three xor-shuffles.
-template <int HD>
-__global__ __launch_bounds__(256) void k_attn_prefill(const float *__restrict__ q, const float *__restrict__ k_cache,
-                                                      const float *__restrict__ v_cache, float *__restrict__ out,
+template <int HD, class KV>
+__global__ __launch_bounds__(256) void k_attn_prefill(const float *__restrict__ q, const KV *__restrict__ k_cache,
+                                                      const KV *__restrict__ v_cache, float *__restrict__ out,
                                                       int n, int pos0, int n_heads, int n_kv_heads,
                                                       int64_t cache_stride, float scale) {
     constexpr int QT = 32, KT = 32, PITCH = HD + 4;  // pitch = 4 mod 64 banks: the 8 rows of a read never collide
@@ -69,7 +82,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill(const float *__restrict__ 
     const int tid = threadIdx.x, qi = tid >> 3, sub = tid & 7;
     const int head = blockIdx.x, i0 = blockIdx.y * QT;
     const int kvh = head / (n_heads / n_kv_heads);
-    const float *kh = k_cache + (size_t)kvh * cache_stride, *vh = v_cache + (size_t)kvh * cache_stride;
+    const KV *kh = k_cache + (size_t)kvh * cache_stride, *vh = v_cache + (size_t)kvh * cache_stride;
     const int rows = min(QT, n - i0);
     const int n_keys = pos0 + i0 + rows;    // the tile's last query sees this many positions
     const int my_last = pos0 + i0 + qi;     // last position query row qi may attend
@@ -90,8 +103,8 @@ __global__ __launch_bounds__(256) void k_attn_prefill(const float *__restrict__ 
         for (int e = tid; e < KT * F4; e += 256) {
             const int r = e / F4, c4 = e % F4;
             const size_t p = (size_t)min(p0 + r, n_keys - 1);
-            *(float4 *)&s_k[r * PITCH + 4 * c4] = *(const float4 *)(kh + p * HD + 4 * c4);
-            *(float4 *)&s_v[r * HD + 4 * c4] = *(const float4 *)(vh + p * HD + 4 * c4);
+            *(float4 *)&s_k[r * PITCH + 4 * c4] = kv_load4(kh + p * HD + 4 * c4);
+            *(float4 *)&s_v[r * HD + 4 * c4] = kv_load4(vh + p * HD + 4 * c4);
         }
         __syncthreads();
         // scores of (row qi, keys sub + 8r)
@@ -190,8 +203,9 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-__global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restrict__ q, const float *__restrict__ k_cache,
-                                                           const float *__restrict__ v_cache, float *__restrict__ out,
+template <class KV>
+__global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restrict__ q, const KV *__restrict__ k_cache,
+                                                           const KV *__restrict__ v_cache, float *__restrict__ out,
                                                            int n, int pos0, int n_heads, int n_kv_heads,
                                                            int64_t cache_stride, float scale) {
     constexpr int HD = 128, QT = 64, KT = 32;
@@ -205,7 +219,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
     const int r16 = lane & 15, c4 = lane >> 4;
     const int head = blockIdx.x, i0 = blockIdx.y * QT;
     const int kvh = head / (n_heads / n_kv_heads);
-    const float *kh = k_cache + (size_t)kvh * cache_stride, *vh = v_cache + (size_t)kvh * cache_stride;
+    const KV *kh = k_cache + (size_t)kvh * cache_stride, *vh = v_cache + (size_t)kvh * cache_stride;
     const int n_keys = pos0 + min(i0 + QT, n);   // positions the tile's last query may see
     const int wave_last = pos0 + i0 + 16 * wave + 15;  // last position any row of this wavefront may see
 
@@ -241,13 +255,13 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
             const int e = tid + it * 256, key = e >> 5, d4 = e & 31;
-            kreg[it] = *(const float4 *)(kh + (size_t)min(p0 + key, n_keys - 1) * HD + 4 * d4);
+            kreg[it] = kv_load4(kh + (size_t)min(p0 + key, n_keys - 1) * HD + 4 * d4);
         }
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int e = tid + it * 256, kp = e >> 5, d4 = e & 31;
-            vreg[it][0] = *(const float4 *)(vh + (size_t)min(p0 + 2 * kp, n_keys - 1) * HD + 4 * d4);
-            vreg[it][1] = *(const float4 *)(vh + (size_t)min(p0 + 2 * kp + 1, n_keys - 1) * HD + 4 * d4);
+            vreg[it][0] = kv_load4(vh + (size_t)min(p0 + 2 * kp, n_keys - 1) * HD + 4 * d4);
+            vreg[it][1] = kv_load4(vh + (size_t)min(p0 + 2 * kp + 1, n_keys - 1) * HD + 4 * d4);
         }
     };
     request(0);
@@ -367,30 +381,48 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
 }
 
 int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, const float *v, const float *cos_t,
-                           const float *sin_t, float *k_cache, float *v_cache, int n, int pos0, int n_heads,
+                           const float *sin_t, void *k_cache, void *v_cache, bool kv_f16, int n, int pos0, int n_heads,
                            int n_kv_heads, int head_dim, int64_t cache_stride) {
     const int64_t total = (int64_t)n * (n_heads + 2 * n_kv_heads) * (head_dim / 2);
-    hipLaunchKernelGGL(k_prefill_rope_kv, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream, q, k, v,
-                       cos_t, sin_t, k_cache, v_cache, n, pos0, n_heads, n_kv_heads, head_dim, cache_stride);
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (kv_f16)
+        hipLaunchKernelGGL(k_prefill_rope_kv<_Float16>, grid, dim3(256), 0, dev->stream, q, k, v, cos_t, sin_t,
+                           (_Float16 *)k_cache, (_Float16 *)v_cache, n, pos0, n_heads, n_kv_heads, head_dim, cache_stride);
+    else
+        hipLaunchKernelGGL(k_prefill_rope_kv<float>, grid, dim3(256), 0, dev->stream, q, k, v, cos_t, sin_t,
+                           (float *)k_cache, (float *)v_cache, n, pos0, n_heads, n_kv_heads, head_dim, cache_stride);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
 
-int launch_attn_prefill(candy_hip_device *dev, const float *q, const float *k_cache, const float *v_cache, float *out,
-                        int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride, float scale) {
-    CANDY_REQUIRE(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
-    CANDY_REQUIRE(n > 0 && pos0 >= 0 && n_heads % n_kv_heads == 0, "invalid attention shape");
+template <class KV>
+static void launch_attn_prefill_kv(candy_hip_device *dev, const float *q, const KV *k_cache, const KV *v_cache, float *out,
+                                   int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride,
+                                   float scale) {
     const dim3 grid((unsigned)n_heads, (unsigned)((n + 31) / 32));
     static const bool valu_only = getenv("CANDY_HIP_ATTN_PREFILL_VALU") != nullptr;  // comparison runs
     if (head_dim == 128 && !valu_only)
-        hipLaunchKernelGGL(k_attn_prefill_mfma, dim3((unsigned)n_heads, (unsigned)((n + 63) / 64)), dim3(256), 0, dev->stream,
-                           q, k_cache, v_cache, out, n, pos0, n_heads, n_kv_heads, cache_stride, scale);
+        hipLaunchKernelGGL(k_attn_prefill_mfma<KV>, dim3((unsigned)n_heads, (unsigned)((n + 63) / 64)), dim3(256), 0,
+                           dev->stream, q, k_cache, v_cache, out, n, pos0, n_heads, n_kv_heads, cache_stride, scale);
     else if (head_dim == 128)
-        hipLaunchKernelGGL(k_attn_prefill<128>, grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n, pos0,
+        hipLaunchKernelGGL((k_attn_prefill<128, KV>), grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n, pos0,
                            n_heads, n_kv_heads, cache_stride, scale);
     else
-        hipLaunchKernelGGL(k_attn_prefill<64>, grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n, pos0,
+        hipLaunchKernelGGL((k_attn_prefill<64, KV>), grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n, pos0,
                            n_heads, n_kv_heads, cache_stride, scale);
+}
+
+int launch_attn_prefill(candy_hip_device *dev, const float *q, const void *k_cache, const void *v_cache, bool kv_f16,
+                        float *out, int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride,
+                        float scale) {
+    CANDY_REQUIRE(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
+    CANDY_REQUIRE(n > 0 && pos0 >= 0 && n_heads % n_kv_heads == 0, "invalid attention shape");
+    if (kv_f16)
+        launch_attn_prefill_kv(dev, q, (const _Float16 *)k_cache, (const _Float16 *)v_cache, out, n, pos0, n_heads,
+                               n_kv_heads, head_dim, cache_stride, scale);
+    else
+        launch_attn_prefill_kv(dev, q, (const float *)k_cache, (const float *)v_cache, out, n, pos0, n_heads, n_kv_heads,
+                               head_dim, cache_stride, scale);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }

@@ -86,6 +86,7 @@ SIGNATURES = {
     "candy_hip_llama_set_norm": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "candy_hip_llama_set_graph": (c_int, [c_void_p, c_int]),
     "candy_hip_llama_set_persistent": (c_int, [c_void_p, c_int]),
+    "candy_hip_llama_set_kv_f16": (c_int, [c_void_p, c_int]),
     "candy_hip_llama_decode_path": (c_int, [c_void_p, POINTER(c_int)]),
     "candy_hip_llama_kv_cache": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_size_t)]),
     "candy_hip_llama_decode": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
@@ -440,6 +441,10 @@ class Llama:
 
     def set_graph(self, enable: bool):
         _check(lib().candy_hip_llama_set_graph(self.handle, int(enable)))
+
+    def set_kv_f16(self, enable: bool):
+        """fp16 KV cache (clears the cache); kv_cache() then reports half the bytes."""
+        _check(lib().candy_hip_llama_set_kv_f16(self.handle, int(enable)))
 
     def set_persistent(self, enable: bool):
         _check(lib().candy_hip_llama_set_persistent(self.handle, int(enable)))

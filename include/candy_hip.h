@@ -222,7 +222,13 @@ int candy_hip_llama_set_graph(candy_hip_llama *m, int enable);
 int candy_hip_llama_set_persistent(candy_hip_llama *m, int enable);
 /* How the last decode step ran: 0 = kernel by kernel, 1 = the persistent kernel. */
 int candy_hip_llama_decode_path(candy_hip_llama *m, int *path);
-/* f32 KV cache, [n_layers][n_kv_heads][max_pos][head_dim] for K and the same for V. */
+/* Optional fp16 KV cache (off by default: candy's tensors are f32).  The new token's k (after Rope) and v are
+ * rounded to fp16 once, as they enter the cache; attention reads them back as f32 and every product and sum
+ * stays f32.  Halves the largest stream of a long-context decode step.  Changing the setting clears the cache.
+ * No counterpart in the reference. */
+int candy_hip_llama_set_kv_f16(candy_hip_llama *m, int enable);
+/* KV cache, [n_layers][n_kv_heads][max_pos][head_dim] for K and the same for V: f32, or fp16 after
+ * candy_hip_llama_set_kv_f16(m, 1) (bytes_each tells which). */
 int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, size_t *bytes_each);
 /* One decode step: token id at position pos -> logits [vocab] (device pointer owned by the
  * model, valid until the next step) and the greedy next token.  Either output may be NULL. */

@@ -25,14 +25,17 @@ def rope_tables(max_pos: int, head_dim: int, base: float):
 
 
 class LlamaRef:
-    def __init__(self, cfg: dict, weights: dict, f32_activations: bool = False):
+    def __init__(self, cfg: dict, weights: dict, f32_activations: bool = False, kv_f16: bool = False):
         """weights: {(kind, layer): (fmt, blocks) | f32 array}; kinds as in candy_hip.h.
         f32_activations: every Linear is dequantize + f32 matmul (candy's literal CPU composition, conv.go:373-389)
         instead of the Q8_0-activation vec-dot: the same model without the activation quantizer, against which the
-        size of that quantizer's noise can be measured."""
+        size of that quantizer's noise can be measured.
+        kv_f16: k (after Rope) and v are rounded to fp16 (nearest even) as they enter the cache; attention reads the
+        rounded values as f32.  candy's cache is f32: this models the device's optional half-size cache, nothing else."""
         self.c = cfg
         self.w = weights
         self.f32_activations = f32_activations
+        self.kv_f16 = kv_f16
         c = cfg
         self.k_cache = np.zeros((c["n_layers"], c["n_kv_heads"], c["max_pos"], c["head_dim"]), np.float32)
         self.v_cache = np.zeros_like(self.k_cache)
@@ -60,6 +63,8 @@ class LlamaRef:
             v = self._lin("v", l, xn, nkv * hd, d)
             q = o.rope(q, self.cos[pos], self.sin[pos], nh, hd, hd)
             k = o.rope(k, self.cos[pos], self.sin[pos], nkv, hd, hd)
+            if self.kv_f16:
+                k, v = k.astype(np.float16).astype(np.float32), v.astype(np.float16).astype(np.float32)
             self.k_cache[l, :, pos, :] = k.reshape(nkv, hd)
             self.v_cache[l, :, pos, :] = v.reshape(nkv, hd)
             att = o.attention_decode(q, self.k_cache[l], self.v_cache[l], nh, nkv, hd, pos + 1,

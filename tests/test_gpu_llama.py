@@ -254,6 +254,95 @@ def test_prompt_pass_matches_token_by_token_cpu(dev, name, cfg, fmts, n, bar):
         tok = rt
 
 
+def read_cache(dev, model, shape):
+    """Both device caches as f32 arrays, whichever element type they hold."""
+    kptr, vptr, nbytes = model.kv_cache()
+    n = int(np.prod(shape))
+    dt = {4 * n: np.float32, 2 * n: np.float16}[nbytes]
+    out = []
+    for ptr in (kptr, vptr):
+        got = np.empty(n, dt)
+        hip._check(hip.lib().candy_hip_d2h(dev.handle, got.ctypes.data, ptr, nbytes))
+        out.append(got.astype(np.float32).reshape(shape))
+    return out
+
+
+@pytest.mark.parametrize("layers", [1, 2])
+@pytest.mark.parametrize("case", [0, 1, 2])
+def test_fp16_kv_cache_matches_cpu_composition_with_rounded_cache(dev, case, layers):
+    # The optional half-size cache: k and v rounded to fp16 once, on entry; the CPU composition rounds the same
+    # values the same way.
+    # One layer: k and v come straight from the first projections, device and CPU agree to 1e-7 before rounding,
+    # nearly every stored number is the same fp16 value, and the f32 cache's 1e-3 bar holds as it is.
+    # Two layers: the second layer's k and v are 1e-4 apart before rounding, one value in ten straddles an fp16
+    # rounding boundary and is stored a whole fp16 step apart, so the two runs differ by a fraction of the noise
+    # the rounding itself adds.  That noise is measured here (CPU composition with the rounded cache against the
+    # same with candy's f32 cache; large on these random-block models, whose softmax is close to an argmax) and is
+    # the bar wherever it exceeds 1e-3.
+    # Cases: head_dim 64 (vector-ALU prompt attention, GQA), head_dim 128 MHA and GQA (matrix-core prompt
+    # attention), decode continuing from each.
+    name, cfg, fmts, n, bar = PROMPT_CASES[case]
+    cfg = dict(cfg, n_layers=layers)
+    host, model = build(dev, cfg, fmts, seed=21)
+    model.set_kv_f16(True)
+    ref = llama_ref.LlamaRef(cfg, host, kv_f16=True)
+    plain = llama_ref.LlamaRef(cfg, host)
+    tokens = [int(t) for t in np.random.default_rng(22).integers(0, cfg["vocab"], n)]
+
+    def cpu_step(tok, pos):
+        rt, rlogits, _ = ref.step(ref.embed(tok), pos)
+        _, plogits, _ = plain.step(plain.embed(tok), pos)
+        noise = rel(rlogits, plogits.astype(np.float64))
+        return rt, rlogits, bar if layers == 1 else max(bar, noise)
+
+    for pos, tok in enumerate(tokens):
+        rt, rlogits, lim = cpu_step(tok, pos)
+    nt, logits = model.prefill(tokens, 0)
+    assert rel(logits, rlogits) <= lim, name
+    assert model.kv_cache()[2] == ref.k_cache.size * 2
+    for got, want in zip(read_cache(dev, model, ref.k_cache.shape), (ref.k_cache, ref.v_cache)):
+        assert rel(got[:, :, :n], want[:, :, :n].astype(np.float64)) <= bar + 2.0 ** -10  # one fp16 step more
+        assert np.mean(got[:, :, :n] == want[:, :, :n]) > 0.8  # and most are the same fp16 number
+        assert np.mean(got[0, :, :n] == want[0, :, :n]) > 0.99  # the first layer's, all but stray straddles
+        assert not got[:, :, n:].any()
+    tok = nt
+    for pos in range(n, n + 3):
+        rt, rlogits, lim = cpu_step(tok, pos)
+        gt, glogits = model.decode(tok, pos)
+        assert rel(glogits, rlogits) <= lim, (name, pos)
+        assert model.decode_path() == 0
+        tok = rt
+    # token by token from an empty cache gives what the prompt pass gave (to the same bar); switching back to f32
+    # clears the cache and restores candy's cache to the f32 bar
+    _, other = build(dev, cfg, fmts, seed=21)
+    other.set_kv_f16(True)
+    for pos, t in enumerate(tokens[:12]):
+        ot, ologits = other.decode(t, pos)
+    pt, plogits = model.prefill(tokens[:12], 0)
+    assert rel(plogits, ologits.astype(np.float64)) <= lim
+    model.set_kv_f16(False)
+    assert model.kv_cache()[2] == ref.k_cache.size * 4
+    assert not any(c.any() for c in read_cache(dev, model, ref.k_cache.shape))
+    again = llama_ref.LlamaRef(cfg, host)
+    for pos, t in enumerate(tokens[:6]):
+        rt, rlogits, _ = again.step(again.embed(t), pos)
+        gt, glogits = model.decode(t, pos)
+    assert rel(glogits, rlogits) <= bar
+
+
+def test_fp16_kv_cache_differs_from_f32_cache_by_its_rounding_only(dev):
+    # how far the half-size cache moves the logits: well under the activation quantizer's own 1e-2, and not zero
+    name, cfg, fmts, n, _ = PROMPT_CASES[1]
+    host, a = build(dev, cfg, fmts, seed=23)
+    _, b = build(dev, cfg, fmts, seed=23)
+    b.set_kv_f16(True)
+    tokens = [int(t) for t in np.random.default_rng(24).integers(0, cfg["vocab"], n)]
+    _, la = a.prefill(tokens, 0)
+    _, lb = b.prefill(tokens, 0)
+    d = rel(lb, la.astype(np.float64))
+    assert 0 < d < 1e-2, d
+
+
 @pytest.mark.parametrize("case,n,cut", [(0, 50, 19), (2, 150, 77)])
 def test_prompt_in_two_chunks_equals_one_pass(dev, case, n, cut):
     # a prompt continued at pos0 > 0 attends the positions already in the cache (head_dim 64: vector-ALU
