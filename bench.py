@@ -221,7 +221,7 @@ def prefill_kv(dev, model, cfg, n_pos, seed=9):
                 hip._check(hip.lib().candy_hip_h2d(dev.handle, base + off, rows[h].ctypes.data, rows[h].nbytes))
 
 
-def decode_leg(dev, steps, warmup):
+def decode_leg(dev, steps, warmup, fp16_kv=True):
     from candy_amd import synth
     log("building random-init 7B (N(0, 0.02) quantized to Q4_K, Q6_K head) ...")
     n_pos = 2048
@@ -254,9 +254,10 @@ def decode_leg(dev, steps, warmup):
 
     out = run(4)  # candy's cache is f32: this is the figure quoted
     # the optional half-size cache, beside it (k and v rounded to fp16 on entry; not what the reference computes)
-    model.set_kv_f16(True)
-    half = run(2)
-    out["fp16_kv_cache"] = {k: half[k] for k in ("tok_s", "ms_per_token", "bytes_per_token", "hbm_GBps", "hbm_frac")}
+    if fp16_kv:
+        model.set_kv_f16(True)
+        half = run(2)
+        out["fp16_kv_cache"] = {k: half[k] for k in ("tok_s", "ms_per_token", "bytes_per_token", "hbm_GBps", "hbm_frac")}
     model.free()
     return out
 
@@ -272,6 +273,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the batched-prefill (MFMA) leg")
     ap.add_argument("--no-llama3", action="store_true", help="skip the Llama-3-8B-shaped prefill + decode leg")
     ap.add_argument("--decode-steps", type=int, default=32)
+    ap.add_argument("--no-fp16-kv", action="store_true", help="skip the decode leg's second figure (fp16 KV cache)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for counter runs)")
     args = ap.parse_args()
@@ -407,7 +409,7 @@ def main():
         out["prefill"] = pre
 
     if not args.no_decode:
-        out["decode"] = decode_leg(dev, args.decode_steps, 4)
+        out["decode"] = decode_leg(dev, args.decode_steps, 4, fp16_kv=not args.no_fp16_kv)
         log("decode:", out["decode"])
 
     if not args.no_llama3:

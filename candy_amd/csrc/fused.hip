@@ -9,6 +9,9 @@
 //   epilogue RES:   residual Add (backend.go:21) on the output.
 // The contraction itself is the batch-1 kernel of matvec.hip (same units, same exact load
 // counting: inputs first, then every weight load, nothing branches around a memory operation).
+#include <cstdlib>
+#include <type_traits>
+
 #include "blocks.h"
 #include "internal.h"
 #include "units.h"
@@ -29,6 +32,9 @@ struct FusedArgs {
     // PAIR epilogue output: planar Q8_0 of silu(gate.x) * (up.x)
     int8_t *oq;
     Q8Scale *os;
+    // PAIR workgroups that own less than a 32-value block: their f32 results and one counter per block
+    float *pair_act;
+    unsigned *pair_tickets;
     int K;
 };
 
@@ -169,7 +175,13 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
             if (lane == 0 && row0 + r < N) y[row0 + r] = res ? res[row0 + r] + v : v;
         }
     } else {
-        static_assert(EPI != EPI_PAIR || R * WAVES == 32, "a PAIR workgroup owns one 32-value block");
+        // A PAIR workgroup owns S = 32, 16 or 8 consecutive outputs: a whole Q8_0 block, or a part of one.  Parts
+        // exist so that the grid divides evenly over the CUs (344 whole blocks of a 11008-wide layer leave 88 CUs
+        // with twice the bytes of the others).  A part leaves its f32 values in pair_act and takes a ticket of its
+        // block; whoever draws the last ticket quantizes the block from pair_act (the same 32 values whichever
+        // workgroup that is, so the result does not depend on the order) and puts the counter back to zero.
+        constexpr int S = R * WAVES;
+        static_assert(EPI != EPI_PAIR || S == 32 || S == 16 || S == 8 || S == 4, "a PAIR workgroup owns a 32-value block or a part");
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float g = wave_sum(acc[0][r]), u = wave_sum(acc[1][r]);
@@ -177,10 +189,27 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
         }
         __syncthreads();
         if (wave == 0) {
+            const int blk = (wg * S) >> 5;  // N % 32 == 0
+            float mine;
+            if constexpr (S == 32) {
+                mine = s_act[lane & 31];
+            } else {
+                if (lane < S) __hip_atomic_store(a.pair_act + wg * S + lane, s_act[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // The values are out before the ticket is drawn: agent-scope atomic stores write through to where
+                // every XCD sees them, and the store counter reaches zero when they have arrived.  (A release fence
+                // would also write the whole L2 back and an acquire fence invalidate it: 17 us per launch, measured.)
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                unsigned old = 0;
+                if (lane == 0) old = __hip_atomic_fetch_add(a.pair_tickets + blk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
+                if (old != 32 / S - 1) return;  // a later workgroup finishes the block
+                asm volatile("" ::: "memory");  // agent-scope atomic loads below: they do not hit a stale cache line
+                mine = __hip_atomic_load(a.pair_act + blk * 32 + (lane & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (lane == 0) __hip_atomic_store(a.pair_tickets + blk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             __half h;
             int bsum;
-            const int q = quantize_q8_lane1(s_act[lane & 31], h, bsum);
-            const int blk = wg;  // N % 32 == 0: every workgroup holds a whole block
+            const int q = quantize_q8_lane1(mine, h, bsum);
             if (lane < 32) a.oq[(size_t)blk * 32 + lane] = (int8_t)q;
             if (lane == 0) {
                 Q8Scale sc;
@@ -203,7 +232,7 @@ static int launch_fused_cfg(candy_hip_device *dev, FusedArgs a) {
     const int rows_per_wg = R * WAVES;
     int total = 0;
     if (EPI == EPI_PAIR) {
-        total = a.jobs.j[0].N / 32;
+        total = a.jobs.j[0].N / rows_per_wg;
     } else {
         for (int i = 0; i < 3; ++i) {
             if (i < a.jobs.n) total += (a.jobs.j[i].N + rows_per_wg - 1) / rows_per_wg;
@@ -215,22 +244,52 @@ static int launch_fused_cfg(candy_hip_device *dev, FusedArgs a) {
     return CANDY_HIP_OK;
 }
 
+// Rows per PAIR workgroup, out of hi, hi/2, ... lo: the largest that leaves the fullest CU the fewest rows.  A
+// kernel whose workgroups all start at once lasts as long as its fullest CU streams (about 26 bytes per nanosecond
+// each), so 1.34 workgroups per CU cost as much as 2.  Measured on the 7B decode step (d_ffn 11008): 32 rows 1.914,
+// 16 rows (16 wavefronts x 1) 1.859, 8 rows (8 x 1) 1.855 ms per token; 4 rows 1.960; with four rows per wavefront
+// the 16-row shape is slower than whole blocks (2.036).  d_ffn 14336: 32 rows 1.983, 8 rows 1.957.  The same choice
+// for the plain RMSNorm-prologue kernel (16 or 8 rows) did not pay: 8 rows lose more to the repeated prologue than
+// the even split wins.  `env` names an override for comparison runs.
+static int balanced_rows(int rows, int cus, int hi, int lo, const char *env) {
+    if (const char *e = getenv(env)) {
+        const int v = atoi(e);
+        for (int s = hi; s >= lo; s >>= 1)
+            if (v == s) return s;
+    }
+    int best = hi;
+    long best_cost = -1;
+    for (int s = hi; s >= lo; s >>= 1) {
+        const long wgs = (rows + s - 1) / s, cost = (wgs + cus - 1) / cus * s;
+        if (best_cost < 0 || cost < best_cost) { best = s; best_cost = cost; }
+    }
+    return best;
+}
+
 // Tile shapes: PLAIN keeps the batch-1 kernel's one row per wavefront when the input is already
 // quantized; with the RMSNorm prologue a workgroup takes 16 rows so that the (redundant) prologue
-// is amortised; PAIR is 8 wavefronts x 4 rows of each of the two weights.
+// is amortised; PAIR is 8 wavefronts x 4 rows of each of the two weights (a whole 32-value block), or
+// 16 x 1 / 8 x 1 (half a block, a quarter) where that divides the rows more evenly over the CUs and the caller
+// has given the scratch the parts need.
 template <class U, int ITER>
 static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro, int epi) {
     if (epi == EPI_PAIR) {
         if constexpr (ITER <= 2) {  // two weights x 4 rows x ITER units must stay in registers
-            return pro == PRO_RMS ? launch_fused_cfg<U, ITER, 4, 8, PRO_RMS, EPI_PAIR>(dev, a)
-                                  : launch_fused_cfg<U, ITER, 4, 8, PRO_Q8, EPI_PAIR>(dev, a);
+            if (pro != PRO_RMS) return launch_fused_cfg<U, ITER, 4, 8, PRO_Q8, EPI_PAIR>(dev, a);
+            const int s = a.pair_act && a.pair_tickets ? balanced_rows(a.jobs.j[0].N, dev->num_cus, 32, 8, "CANDY_HIP_PAIR_ROWS") : 32;
+            if (s == 16) return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
+            if (s == 8) return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
+            return launch_fused_cfg<U, ITER, 4, 8, PRO_RMS, EPI_PAIR>(dev, a);
         } else {
             return CANDY_HIP_ERR_UNSUPPORTED;
         }
     }
     if (pro == PRO_RMS) {
-        if constexpr (ITER <= 2) return launch_fused_cfg<U, ITER, 4, 4, PRO_RMS, EPI_PLAIN>(dev, a);
-        else return launch_fused_cfg<U, ITER, 2, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+        if constexpr (ITER <= 2) {
+            return launch_fused_cfg<U, ITER, 4, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+        } else {
+            return launch_fused_cfg<U, ITER, 2, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+        }
     }
     return launch_fused_cfg<U, ITER, 1, 4, PRO_Q8, EPI_PLAIN>(dev, a);
 }
@@ -268,6 +327,7 @@ int launch_matvec_fused(candy_hip_device *dev, const FusedLaunch &L) {
         a.jobs.j[i].N = (int)L.w[i]->rows;
     }
     a.xq = L.xq; a.xs = L.xs; a.x = L.x; a.alpha = L.alpha; a.eps = L.eps; a.oq = L.oq; a.os = L.os;
+    a.pair_act = L.pair_act; a.pair_tickets = L.pair_tickets;
     a.K = (int)w0->cols;
     switch (w0->fmt) {
     case CANDY_HIP_Q4_K: return launch_fused_fmt<UnitQ4K>(dev, a, pro, epi);

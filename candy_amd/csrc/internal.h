@@ -159,6 +159,10 @@ struct FusedLaunch {
     bool pair = false;
     int8_t *oq = nullptr;
     Q8Scale *os = nullptr;
+    // pair only, optional: rows floats and rows / 32 counters (zero before the first launch; every launch leaves
+    // them zero) that let a workgroup own part of a 32-value output block where that spreads the rows evenly
+    float *pair_act = nullptr;
+    unsigned *pair_tickets = nullptr;
 };
 int launch_matvec_fused(candy_hip_device *dev, const FusedLaunch &launch);
 // attention.hip

@@ -30,6 +30,7 @@ struct candy_hip_llama {
     float *cos_t = nullptr, *sin_t = nullptr;      // [max_pos][head_dim/2]
     float *h = nullptr, *q = nullptr, *k = nullptr, *v = nullptr;
     float *gate_o = nullptr, *up_o = nullptr, *logits = nullptr;
+    unsigned *pair_tickets = nullptr;  // one counter per 32 FFN rows (fused gate/up kernel), zero between launches
     float *proj = nullptr;  // [d_model]: a projection's output before the residual add, for formats without that epilogue
     int8_t *xq = nullptr;           // planar Q8_0 quants of the current activation
     candy::Q8Scale *xs = nullptr;
@@ -131,6 +132,8 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
     if (!rc) rc = dev_alloc(m, &m->k, (size_t)cfg->n_kv_heads * cfg->head_dim);
     if (!rc) rc = dev_alloc(m, &m->v, (size_t)cfg->n_kv_heads * cfg->head_dim);
     if (!rc) rc = dev_alloc(m, &m->gate_o, (size_t)cfg->d_ffn);
+    if (!rc) rc = dev_alloc(m, &m->pair_tickets, (size_t)cfg->d_ffn / 32 + 1);
+    if (!rc) rc = candy_hip_zero(dev, m->pair_tickets, ((size_t)cfg->d_ffn / 32 + 1) * sizeof(unsigned));
     if (!rc) rc = dev_alloc(m, &m->proj, (size_t)cfg->d_model);
     if (!rc) rc = dev_alloc(m, &m->up_o, (size_t)cfg->d_ffn);
     if (!rc) rc = dev_alloc(m, &m->logits, (size_t)cfg->vocab);
@@ -418,7 +421,6 @@ static int llama_enqueue_step(candy_hip_llama *m) {
     if (m->persist_ready) return persist_enqueue(m);
     const candy_hip_llama_config &c = m->cfg;
     candy_hip_device *dev = m->dev;
-    const size_t layer_kv = (size_t)c.n_kv_heads * c.max_pos * c.head_dim;
     const float scale = 1.0f / std::sqrt((float)c.head_dim);
     int rc;
     for (int l = 0; l < c.n_layers; ++l) {
@@ -444,6 +446,7 @@ static int llama_enqueue_step(candy_hip_llama *m) {
             FusedLaunch F;
             F.n = 2; F.w[0] = L.gate; F.w[1] = L.up; F.pair = true;
             F.x = m->h; F.alpha = L.ffn_norm; F.eps = c.rms_eps; F.oq = m->xq; F.os = m->xs;
+            F.pair_act = m->gate_o; F.pair_tickets = m->pair_tickets;
             rc = launch_matvec_fused(dev, F);
             if (rc == CANDY_HIP_ERR_UNSUPPORTED) {
                 const candy_hip_qtensor *ws[2] = {L.gate, L.up};
@@ -555,7 +558,6 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
     const candy_hip_llama_config &c = m->cfg;
     candy_hip_device *dev = m->dev;
     candy_hip_llama::Prompt &P = m->pf;
-    const size_t layer_kv = (size_t)c.n_kv_heads * c.max_pos * c.head_dim;
     const int64_t cache_stride = (int64_t)c.max_pos * c.head_dim;
     const int64_t qd = (int64_t)c.n_heads * c.head_dim;
     const float scale = 1.0f / std::sqrt((float)c.head_dim);

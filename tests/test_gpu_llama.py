@@ -361,6 +361,28 @@ def test_prompt_in_two_chunks_equals_one_pass(dev, case, n, cut):
         a.prefill([], 0)
 
 
+@pytest.mark.parametrize("d_ffn", [11008, 1024 + 256])
+def test_gate_up_block_parts_give_the_same_bits(dev, monkeypatch, d_ffn):
+    # the fused gate/up kernel lets a workgroup own a whole 32-value block of the FFN activation or a half / quarter
+    # of one (whichever divides the rows evenly over the CUs); the block is quantized from the same 32 f32 values
+    # either way, so the logits are the same bits, step after step (the per-block counters return to zero)
+    cfg = dict(n_layers=2, d_model=4096 if d_ffn > 4096 else 512, n_heads=8, n_kv_heads=8,
+               head_dim=512 // 8 if d_ffn <= 4096 else 128, d_ffn=d_ffn, vocab=512, max_pos=16, rms_eps=1e-5, rope_base=10000.0)
+    if d_ffn > 4096:
+        cfg.update(n_heads=32, n_kv_heads=32)
+    fmts = {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}
+    tokens = [int(t) for t in np.random.default_rng(31).integers(0, cfg["vocab"], 5)]
+    runs = {}
+    for rows in ("32", "16", "8"):
+        monkeypatch.setenv("CANDY_HIP_PAIR_ROWS", rows)
+        _, model = build(dev, cfg, fmts, seed=30)
+        runs[rows] = [model.decode(t, pos)[1].copy() for pos, t in enumerate(tokens)]
+        model.free()
+    for rows in ("16", "8"):
+        for a, b in zip(runs["32"], runs[rows]):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), rows
+
+
 def test_graph_replay_equals_eager_launches(dev):
     # the captured step is replayed for every token; every replay must give what one-by-one
     # launches give, with other work and synchronisations in between
