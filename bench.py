@@ -341,6 +341,15 @@ def main():
                           "frac": round(gb / HBM_PEAK_GBPS, 4)})
             log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
         out["sweep"] = sweep
+        # small batches (mul_mat_vec_q serves 1..8 rows in the reference): f32 in -> f32 out, quantization included
+        small = []
+        for f, r, k in ((synth.Q4_K, 4096, 11008), (synth.Q4_K, 11008, 4096), (synth.Q6_K, 32000, 4096)):
+            for m in (2, 4, 8, 15):
+                ms, _ = time_matvec(dev, f, r, k, s_steps, s_warm, quantize_each=True, seed=r + k + f + m, m=m)
+                small.append({"fmt": synth.FORMAT_NAMES[f], "rows": r, "cols": k, "m": m, "us": round(ms * 1e3, 2),
+                              "GBps": round(algorithmic_bytes(f, r, k, m) / (ms * 1e-3) / 1e9, 1)})
+                log(f"  {synth.FORMAT_NAMES[f]} {r}x{k} m={m}: {ms * 1e3:.2f} us")
+        out["small_batch"] = small
 
     if not args.no_sweep:
         # weight quantizers from f32 (load-time): 4096x11008, one launch each

@@ -330,6 +330,134 @@ static int launch_jobs(candy_hip_device *dev, int fmt, const MatvecJobs &jobs, i
     }
 }
 
+// A unit's dot product in two parts where the unit offers them (U::P, U::prep, U::dot_p), in one otherwise.
+template <class U, class = void>
+struct Prepped {
+    typedef typename U::W P;
+    __device__ static __forceinline__ void prep(const typename U::W &w, int, P &p) { p = w; }
+    __device__ static __forceinline__ float dot(const P &p, int u, const int8_t *sq, const Q8Scale *ss) { return U::dot(p, u, sq, ss); }
+};
+template <class U>
+struct Prepped<U, std::void_t<typename U::P>> {
+    typedef typename U::P P;
+    __device__ static __forceinline__ void prep(const typename U::W &w, int u, P &p) { U::prep(w, u, p); }
+    __device__ static __forceinline__ float dot(const P &p, int u, const int8_t *sq, const Q8Scale *ss) { return U::dot_p(p, u, sq, ss); }
+};
+
+// Small batches (2 <= m <= 8 rows of activations per pass).  One workgroup of 16 wavefronts per CU holds all NB
+// quantized activation rows in LDS (up to 150 KB: staged once per CU, not once per 8 weight rows) and walks its
+// share of the weight rows, one row per wavefront at a time, every load of the row in flight before the first
+// dot, as in the batch-1 kernel; a lane dots its unit against each activation row in turn.  The weights are read
+// once whatever the batch; past m = 2 the kernel is bound by the dots (NB times the batch-1 arithmetic) and by the
+// LDS reads of the activation images, not by HBM.  Rows of the batch beyond m are a copy of row m - 1 and are not
+// stored.  No barrier after the staging: the wavefronts drift apart and cover each other's load latency.
+template <class U, int ITER, int NB>
+__global__ __launch_bounds__(1024) void k_matvec_mb(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
+                                                    const Q8Scale *__restrict__ xs, float *__restrict__ y, int N, int K,
+                                                    int m) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int units = K / U::ELEMS;
+    const size_t rb = U::row_bytes(K);
+    const int q_bytes = skewed(K), blocks_per_row = K >> 5;
+    int8_t *sq = (int8_t *)smem;
+    Q8Scale *ss = (Q8Scale *)(smem + NB * q_bytes);
+
+    const int step = gridDim.x * 16;
+    int row = blockIdx.x * 16 + wave;
+    typename U::W w[ITER];
+    {   // the first row's weights are requested before the activations are staged
+        const uint8_t *rp = W + (size_t)min(row, N - 1) * rb;
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) U::load(rp, min(it * 64 + lane, units - 1), w[it]);
+    }
+    {
+        const int chunks = K >> 4;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int src_row = min(nb, m - 1);
+            const uint4 *src = (const uint4 *)(xq + (size_t)src_row * K);
+            uint4 *dst = (uint4 *)(sq + nb * q_bytes);
+            for (int c = tid; c < chunks; c += 1024) dst[c + (c >> 4)] = src[c];
+            const uint2 *s2 = (const uint2 *)(xs + (size_t)src_row * blocks_per_row);
+            uint2 *d2 = (uint2 *)(ss + nb * blocks_per_row);
+            for (int i = tid; i < blocks_per_row; i += 1024) d2[i] = s2[i];
+        }
+    }
+    __syncthreads();
+
+    while (row < N) {
+        typename Prepped<U>::P pw[ITER];  // the weight-only part of the dots, once per weight row
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) Prepped<U>::prep(w[it], min(it * 64 + lane, units - 1), pw[it]);
+        // one activation row at a time (not unrolled: a lane's share of NB rows at once does not fit the registers)
+#pragma unroll 1
+        for (int nb = 0; nb < NB; ++nb) {
+            const int8_t *q = sq + nb * q_bytes;
+            const Q8Scale *sc = ss + nb * blocks_per_row;
+            float acc = 0.0f;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                const int u = it * 64 + lane;
+                const bool live = u < units;
+                const float v = Prepped<U>::dot(pw[it], live ? u : units - 1, q, sc);
+                acc += live ? v : 0.0f;
+            }
+            acc = wave_sum(acc);
+            if (lane == 0 && nb < m) y[(size_t)nb * N + row] = acc;
+        }
+        row += step;
+        if (row < N) {  // wavefront-uniform
+            const uint8_t *rp = W + (size_t)row * rb;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) U::load(rp, min(it * 64 + lane, units - 1), w[it]);
+        }
+    }
+}
+
+// LDS the small-batch kernel needs for NB activation rows of length K
+static size_t mb_lds_bytes(int nb, int64_t K) {
+    return (size_t)nb * ((size_t)K + (((size_t)K >> 8) << 4) + (size_t)(K >> 5) * sizeof(Q8Scale));
+}
+constexpr size_t MB_LDS_MAX = 160 * 1024;
+
+template <class U, int ITER, int NB>
+static int launch_mb_cfg(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int m,
+                         float *y) {
+    const int N = (int)w->rows, K = (int)w->cols;
+    const size_t smem = mb_lds_bytes(NB, K);
+    auto kern = k_matvec_mb<U, ITER, NB>;
+    CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    const int groups = (N + 15) / 16;
+    hipLaunchKernelGGL(kern, dim3((unsigned)std::min(groups, dev->num_cus)), dim3(1024), smem, dev->stream,
+                       (const uint8_t *)w->data, qs, scales, y, N, K, m);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+// One pass of up to 8 activation rows; CANDY_HIP_ERR_UNSUPPORTED (no error text) when the row is too long for it.
+template <class U>
+static int launch_mb(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int m,
+                     float *y) {
+    const int64_t K = w->cols;
+    const int iter = (int)((K / U::ELEMS + 63) / 64);
+    const bool wide = m > 4 && mb_lds_bytes(8, K) <= MB_LDS_MAX;
+    // rounds of 64 units the kernel holds in registers without spilling, per format (Q6_K: none so far)
+    constexpr int max_iter = std::is_same<U, UnitQ4K>::value ? 4 : std::is_same<U, UnitQ6K>::value ? 0 : 8;
+    if (iter > max_iter || (!wide && (m > 4 || mb_lds_bytes(4, K) > MB_LDS_MAX))) return CANDY_HIP_ERR_UNSUPPORTED;
+#define CANDY_MB(IT)                                                                  \
+    return wide ? launch_mb_cfg<U, IT, 8>(dev, w, qs, scales, m, y) : launch_mb_cfg<U, IT, 4>(dev, w, qs, scales, m, y)
+    switch (iter) {
+    case 1: CANDY_MB(1);
+    case 2: CANDY_MB(2);
+    case 3: CANDY_MB(3);
+    case 4: CANDY_MB(4);
+    case 5: case 6: CANDY_MB(6);
+    default: CANDY_MB(8);
+    }
+#undef CANDY_MB
+}
+
 template <class U, int NB, int R, int WAVES>
 static int launch_one(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                       float *y) {
@@ -370,12 +498,27 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
         }
     }
     int64_t done = 0;
+    const bool old_small = getenv("CANDY_HIP_OLD_SMALL_BATCH") != nullptr;  // comparison runs and tests
     while (done < m) {
         const int64_t left = m - done;
         const int8_t *q = qs + done * K;
         const Q8Scale *s = scales + done * sstride;
         float *yo = y + done * N;
         int rc;
+        if constexpr (!general_only<U>()) {
+            // The looping kernel below takes 8, 4, 2 or 1 rows per launch (fewer the longer the row is); where that
+            // covers what is left in as few launches as this kernel's 8 per pass, it is as fast or a little faster
+            // (short rows, up to about 16K of them), and two rows cost less there than as half of a 4-row pass.
+            int old_launches = 0;
+            for (int64_t l = left; l > 0; ++old_launches) l -= (l >= 8 && K <= 5632) ? 8 : (l >= 4 && K <= 11264) ? 4 : (l >= 2 && K <= 16384) ? 2 : 1;
+            const bool old_is_fine = left == 2 || (K <= 5632 && N <= 16384 && old_launches == (left + 7) / 8);
+            if (left >= 2 && !old_small && !old_is_fine) {  // up to 8 rows per pass, or 4 where 8 do not fit LDS
+                const int take = (int)std::min<int64_t>(left, mb_lds_bytes(8, K) <= MB_LDS_MAX ? 8 : 4);
+                rc = launch_mb<U>(dev, w, q, s, take, yo);
+                if (rc == CANDY_HIP_OK) { done += take; continue; }
+                if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+            }
+        }
         // LDS holds NB activation rows; keep the workgroup's share under 64 KB
         if (left >= 8 && K <= 5632) { rc = launch_one<U, 8, 2, 4>(dev, w, q, s, yo); done += 8; }
         else if (left >= 4 && K <= 11264) { rc = launch_one<U, 4, 2, 4>(dev, w, q, s, yo); done += 4; }
@@ -429,6 +572,19 @@ int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quan
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                   int64_t m, float *y) {
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && w->cols <= 0x7FFFFFFF, "matrix too large");
+    if (m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K) && mmq_i8_covers(w, qs)) {
+        // 5 .. 15 rows: the vector kernels below (one or two passes of up to 8 rows) or one pass of the int8 tile
+        // kernel with a 16-row tile, whichever a fit to measurements on this chip says is shorter, in us.  The tile
+        // kernel's time follows the length of the row (a wavefront walks it alone): 4096x4096 17.9, 11008x4096 19.2,
+        // 4096x11008 40.4 for Q4_K whatever m; the vector kernels' follows rows x columns x batch.
+        const bool q6 = w->fmt == CANDY_HIP_Q6_K;
+        const double kk = (double)w->cols / 1024.0, mnk = (double)w->rows * (double)w->cols * 1e-6;
+        const int m_pad = q6 ? (int)m : (int)((m + 3) / 4 * 4);
+        const double t_tiles = 3.5 + (q6 ? 4.7 : 3.5) * kk;
+        const double t_vector = 4.0 + (m > 8 ? 2.0 : 0.0) + (q6 ? 0.1 : 0.052) * mnk * m_pad;
+        const char *e = getenv("CANDY_HIP_I8_MIN_M");  // comparison runs: tiles from this batch size on
+        if (e ? m >= atoi(e) : t_tiles < t_vector) return launch_mmq_i8(dev, w, qs, scales, m, y);
+    }
     switch (w->fmt) {
     case CANDY_HIP_Q4_K: return launch_fmt<UnitQ4K>(dev, w, qs, scales, m, y);
     case CANDY_HIP_Q8_0: return launch_fmt<UnitQ8_0>(dev, w, qs, scales, m, y);

@@ -59,6 +59,40 @@ struct UnitQ4K {
         const float sm = s0.d * (float)__mul24(s0.bsum, (int)(m2 & 0xFF)) + s1.d * (float)__mul24(s1.bsum, (int)(m2 >> 8));
         return d * sd - dmin * sm;
     }
+    // The same dot in two parts for kernels that contract one unit with several activation rows: what depends on
+    // the weights only (nibbles spread to bytes, the two 6-bit scale / min pairs, d and dmin) is done once.
+    struct P { uint32_t lo[8], hi[8]; int sc_lo, sc_hi, m_lo, m_hi; float d, dmin; };
+    __device__ static __forceinline__ void prep(const W &w, int u, P &p) {
+        const uint32_t M = 0x0F0F0F0Fu;
+        const uint32_t q[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            p.lo[i] = q[i] & M;
+            p.hi[i] = (q[i] >> 4) & M;
+        }
+        uint32_t sc2, m2;
+        q4k_scale_min_pair(w.hdr.y, w.hdr.z, w.hdr.w, u & 3, sc2, m2);
+        p.sc_lo = (int)(sc2 & 0xFF); p.sc_hi = (int)(sc2 >> 8);
+        p.m_lo = (int)(m2 & 0xFF); p.m_hi = (int)(m2 >> 8);
+        p.d = half_bits_to_float((uint16_t)(w.hdr.x & 0xFFFF));
+        p.dmin = half_bits_to_float((uint16_t)(w.hdr.x >> 16));
+    }
+    __device__ static __forceinline__ float dot_p(const P &p, int u, const int8_t *sq, const Q8Scale *ss) {
+        const uint4 *xa = (const uint4 *)(sq + skewed(u * 64));
+        const uint4 x0 = xa[0], x1 = xa[1], x2 = xa[2], x3 = xa[3];
+        const Q8Scale s0 = ss[2 * u], s1 = ss[2 * u + 1];
+        const uint32_t xl[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+        const uint32_t xh[8] = {x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
+        int lo = 0, hi = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            lo = dot4_i8(p.lo[i], xl[i], lo);
+            hi = dot4_i8(p.hi[i], xh[i], hi);
+        }
+        const float sd = s0.d * (float)__mul24(lo, p.sc_lo) + s1.d * (float)__mul24(hi, p.sc_hi);
+        const float sm = s0.d * (float)__mul24(s0.bsum, p.m_lo) + s1.d * (float)__mul24(s1.bsum, p.m_hi);
+        return p.d * sd - p.dmin * sm;
+    }
 };
 
 struct UnitQ8_0 {

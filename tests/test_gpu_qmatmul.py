@@ -49,6 +49,36 @@ def test_small_batch_matches_oracle(dev, fmt, m):
     assert rel_err(got, want) <= 2e-5
 
 
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML, synth.Q6_K])
+@pytest.mark.parametrize("rows,cols", [(50, 11008), (4099, 1280), (600, 6144)])
+def test_small_batch_one_pass_per_eight_rows(dev, monkeypatch, fmt, rows, cols):
+    # 3 .. 15 activation rows against long or many weight rows: one workgroup per CU holds up to eight quantized
+    # rows in LDS and walks the weight rows (Q6_K: the looping kernel), or the int8 tile kernel takes the batch as
+    # one 16-row tile.  The vector kernels add a lane's units in the same order as the looping kernel: same bits;
+    # the tile kernel differs by f32 summation order only.  Row counts off the 16-row groups and more groups than
+    # CUs (4099 rows) are in.
+    w = synth.random_weight(fmt, rows, cols, seed=rows + fmt)
+    q = dev.qtensor(fmt, rows, cols, w)
+    for m in (3, 4, 5, 7, 8, 9, 13, 15):
+        x = synth.random_activations(m, cols, seed=m * 5 + fmt)
+        got = dev.qmatmul(q, x)
+        assert got.shape == (m, rows)
+        if m in (3, 8, 15):
+            assert rel_err(got, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5, m
+        monkeypatch.setenv("CANDY_HIP_OLD_SMALL_BATCH", "1")
+        monkeypatch.setenv("CANDY_HIP_I8_MIN_M", "99")
+        old = dev.qmatmul(q, x)
+        monkeypatch.setenv("CANDY_HIP_I8_MIN_M", "2")  # tiles wherever they apply (Q4_K, Q6_K)
+        tiles = dev.qmatmul(q, x)
+        monkeypatch.delenv("CANDY_HIP_OLD_SMALL_BATCH")
+        monkeypatch.setenv("CANDY_HIP_I8_MIN_M", "99")
+        vector = dev.qmatmul(q, x)
+        monkeypatch.delenv("CANDY_HIP_I8_MIN_M")
+        assert np.array_equal(vector.view(np.uint32), old.view(np.uint32)), m
+        assert rel_err(tiles, old) <= 2e-6, m
+        assert rel_err(got, old) <= 2e-6, m
+
+
 def test_config_q4_0_4096x4096(dev):
     # the single-QMatMul configuration: Q4_0 4096x4096, one f32 N(0,1) vector, seeded
     rows = cols = 4096
