@@ -101,6 +101,8 @@ int use_device(const candy_hip_device *dev);
 int workspace(candy_hip_device *dev, size_t bytes, void **out);
 // Second buffer, for the split-K partial sums (lives beside the activation workspace).
 int splitk_workspace(candy_hip_device *dev, size_t bytes, void **out);
+// mmq_f16.hip: y[i] = (res[i] +) part[0][i] + part[1][i] + ... in that order (count floats per part)
+int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split);
 // Formats with the per-length batch-1 kernels (residual epilogue, several weights per launch) and the fused
 // decode kernels; the others contract through the general small-batch kernel.
 inline bool format_has_batch1_kernel(int fmt) {

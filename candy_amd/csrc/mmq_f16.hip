@@ -287,6 +287,13 @@ __global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ pa
     }
 }
 
+int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split) {
+    hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((count / 4 + 256) / 256)), dim3(256), 0, dev->stream, part, y, res,
+                       count, n_split);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
 template <class F, int BN, int BM, int WN, int WM>
 static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                       const float *res) {

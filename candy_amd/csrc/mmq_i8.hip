@@ -30,6 +30,7 @@
 //     super-block ahead into registers and parked in LDS between two barriers.
 // The rescale costs 16 VALU instructions per 16x16x32 tile (convert, multiply and two fused
 // multiply-adds per result register), which is what bounds the large-m rate.
+#include <algorithm>
 #include <cstdlib>
 
 #include "blocks.h"
@@ -205,7 +206,7 @@ struct MmqI8Lds {
 template <class F, int TM, int STG, int KS>
 __global__ __launch_bounds__(256 * KS) void k_mmq_i8(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
                                                      const Q8Scale *__restrict__ xs, float *__restrict__ y, int N, int M,
-                                                     int K) {
+                                                     int K, int sb_split) {
     typedef MmqI8Lds<F, TM, STG, KS> L;
     constexpr int BM = 16 * TM;
     constexpr int XSC = (BM * 8 + 255) / 256;  // activation scales per thread per super-block
@@ -231,8 +232,11 @@ __global__ __launch_bounds__(256 * KS) void k_mmq_i8(const uint8_t *__restrict__
     const int nsb = K >> 8;
     const size_t rb = (size_t)nsb * F::BLOCK;
     // the super-blocks of this K group: [sb_lo, sb_hi), `per` (whole stages) for every group
-    const int per = ((nsb + KS - 1) / KS + STG - 1) / STG * STG;
-    const int sb_lo = kg * per, sb_hi = min(nsb, sb_lo + per);
+    // blockIdx.z walks super-blocks [z * sb_split, ...) and writes its own copy of the output (summed afterwards)
+    const int sb_first = blockIdx.z * sb_split, sb_end = min(nsb, sb_first + sb_split);
+    const int per = ((sb_end - sb_first + KS - 1) / KS + STG - 1) / STG * STG;
+    const int sb_lo = sb_first + kg * per, sb_hi = min(sb_end, sb_lo + per);
+    y += (size_t)blockIdx.z * M * N;
 
     // weights of one stage: 16 rows x STG blocks as 16-byte chunks along the rows, in registers
     // while in flight, then parked in the wavefront's LDS slice
@@ -371,19 +375,38 @@ static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const in
         constexpr int lds = MmqI8Lds<F, TMV, STGV, KSV>::BYTES;                                                 \
         auto kern = k_mmq_i8<F, TMV, STGV, KSV>;                                                                \
         CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds)); \
-        hipLaunchKernelGGL(kern, dim3(gx, (unsigned)((M + 16 * TMV - 1) / (16 * TMV))), dim3(256 * KSV), lds,   \
-                           dev->stream, (const uint8_t *)w->data, qs, scales, y, N, M, K);                      \
+        const unsigned gy = (unsigned)((M + 16 * TMV - 1) / (16 * TMV));                                          \
+        /* a wavefront walks its share of K alone, about 1.3 us per super-block, and LDS lets two of them share a */ \
+        /* SIMD: a grid of at most one per SIMD splits K over workgroups up to two per SIMD, at least one stage   */ \
+        /* per K group each; the copies are added in a fixed order by k_splitk_sum                                 */ \
+        const int64_t waves = (int64_t)gx * gy * 4 * KSV, simds = 4 * (int64_t)dev->num_cus;                       \
+        if (!no_gs && waves <= simds) n_split = (int)std::min<int64_t>(2 * simds / waves, nsb / (STGV * KSV));     \
+        if (n_split < 1) n_split = 1;                                                                             \
+        sb_split = (nsb + n_split - 1) / n_split;                                                                 \
+        n_split = (nsb + sb_split - 1) / sb_split;                                                                \
+        if (n_split > 1) {                                                                                        \
+            void *p = nullptr;                                                                                    \
+            if (int rc = splitk_workspace(dev, (size_t)n_split * (size_t)M * N * sizeof(float), &p)) return rc;   \
+            out = (float *)p;                                                                                     \
+        }                                                                                                         \
+        hipLaunchKernelGGL(kern, dim3(gx, gy, (unsigned)n_split), dim3(256 * KSV), lds, dev->stream,              \
+                           (const uint8_t *)w->data, qs, scales, out, N, M, K, sb_split);                         \
     } while (0)
-    // the largest tile height that still leaves about 1.5 wavefronts per SIMD: a wavefront walks the
-    // whole contraction on its own, so a grid below that leaves load latency exposed
-    const int64_t strips = (N + 15) / 16, want = 1536;
+    // Tile height: 64 activation rows per workgroup from 33 rows on (a weight fragment serves four MFMAs), 16 below
+    // that; where the grid is at most one wavefront per SIMD the launch macro splits K over workgroups, and for at
+    // most 16 rows on such a grid the workgroup has eight wavefronts that split K among themselves first.  Measured
+    // on 4096x11008, 11008x4096, 4096x4096 and 14336x4096 at 16 .. 192 rows; 32-row tiles won nowhere.
     static const bool no_ks = getenv("CANDY_HIP_MMQ_I8_NO_KSPLIT") != nullptr;
-    if (M > 32 && strips * ((M + 63) / 64) >= want) CANDY_MMQ_I8(4, 2, 1);
-    else if (M > 16 && strips * ((M + 31) / 32) >= want) CANDY_MMQ_I8(2, DEEP, 1);
-    else if (!no_ks && (int64_t)gx * ((M + 15) / 16) < 2 * dev->num_cus && (K >> 8) >= 2 * DEEP) CANDY_MMQ_I8(1, DEEP, 2);
+    const bool no_gs = getenv("CANDY_HIP_MMQ_I8_NO_GRID_SPLIT") != nullptr;  // comparison runs and tests
+    const int nsb = K >> 8;
+    int n_split = 1, sb_split = nsb;
+    float *out = y;
+    if (M > 32) CANDY_MMQ_I8(4, 2, 1);
+    else if (M <= 16 && !no_ks && (int64_t)gx < 2 * dev->num_cus && nsb >= 2 * DEEP) CANDY_MMQ_I8(1, DEEP, 2);
     else CANDY_MMQ_I8(1, DEEP, 1);
 #undef CANDY_MMQ_I8
     CANDY_LAUNCH_CHECK();
+    if (n_split > 1) return launch_splitk_sum(dev, out, y, nullptr, (size_t)M * N, n_split);
     return CANDY_HIP_OK;
 }
 

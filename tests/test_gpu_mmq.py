@@ -55,6 +55,26 @@ def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K])
+@pytest.mark.parametrize("rows,cols", [(200, 11008), (64, 4352), (1000, 2560)])
+def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, rows, cols):
+    # few weight rows and a long contraction: the grid is at most one wavefront per SIMD, so K is split over
+    # workgroups (and, up to 16 rows, over the wavefronts of a workgroup first) and the copies are summed in a
+    # fixed order: the answer moves by f32 summation order only, and is the same from call to call
+    w = synth.random_weight(fmt, rows, cols, seed=rows + cols + fmt)
+    q = dev.qtensor(fmt, rows, cols, w)
+    for m in (16, 24, 33, 64, 130):
+        x = synth.random_activations(m, cols, seed=m * 7 + fmt)
+        got = dev.qmatmul(q, x)
+        assert np.array_equal(got.view(np.uint32), dev.qmatmul(q, x).view(np.uint32))
+        if m in (16, 33):
+            assert rel_err(got, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5, m
+        monkeypatch.setenv("CANDY_HIP_MMQ_I8_NO_GRID_SPLIT", "1")
+        whole = dev.qmatmul(q, x)
+        monkeypatch.delenv("CANDY_HIP_MMQ_I8_NO_GRID_SPLIT")
+        assert rel_err(got, whole) <= 2e-6, m
+
+
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K])
 @pytest.mark.parametrize("m", [256, 257, 300, 512, 700])
 @pytest.mark.parametrize("rows,cols", [(1, 256), (127, 512), (129, 1024), (300, 2304), (1030, 768), (130, 4352)])
 def test_big_fp16_tiles(dev, fmt, m, rows, cols):
