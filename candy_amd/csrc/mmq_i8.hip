@@ -84,6 +84,32 @@ struct TileQ4K {
             dmq[t] = *(const float4 *)&ex.dmf[t][4 * c];
         }
         wave_lds_fence();  // the slots are rewritten by the next super-block
+        if constexpr (TM == 1) {
+            // one tile per sub-block: nothing else in the wavefront covers an MFMA's latency, so all eight products
+            // of the super-block are issued first and rescaled afterwards
+            int4v d8[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const u32x2 qa = *(const u32x2 *)(wl + 16 + 32 * (t >> 1) + 8 * c);
+                const int sh = (t & 1) * 4;
+                const uint32_t lo = (qa.x >> sh) & 0x0F0F0F0Fu, hi = (qa.y >> sh) & 0x0F0F0F0Fu;
+                const long afrag = (long)(((uint64_t)hi << 32) | lo);
+                const long bfrag = *(const long *)&s_xq[j * XROW + 32 * t + 8 * c];
+                d8[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const float dsc[4] = {dsq[t].x, dsq[t].y, dsq[t].z, dsq[t].w};
+                const float dmf[4] = {dmq[t].x, dmq[t].y, dmq[t].z, dmq[t].w};
+                const float2 sx = s_xs[j * 8 + t];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[0][i] += sx.x * ((float)d8[t][i] * dsc[i]);
+                    acc[0][i] -= dmf[i] * sx.y;
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             const u32x2 qa = *(const u32x2 *)(wl + 16 + 32 * (t >> 1) + 8 * c);
