@@ -332,7 +332,7 @@ def main():
             sweep.append({"fmt": name, "rows": r, "cols": k, "us": round(ms * 1e3, 3), "GBps": round(gb, 1),
                           "frac": round(gb / HBM_PEAK_GBPS, 4)})
             log(f"  {name} {r}x{k}: {ms * 1e3:.2f} us, {gb:.0f} GB/s")
-        # the reference's other formats through the general kernel (no per-length batch-1 variants)
+        # the reference's other formats (same batch-1 kernel template, no span staging, no fused decode kernels)
         for f in (synth.Q4_1, synth.Q5_0, synth.Q5_1, synth.Q2_K, synth.Q3_K, synth.Q5_K):
             r, k, name = 4096, 11008, synth.FORMAT_NAMES[f]
             ms, _ = time_matvec(dev, f, r, k, s_steps, s_warm, quantize_each=False, seed=r + k + f)

@@ -48,7 +48,6 @@ struct FmtQ4_1 {
 template <bool GGML_ORDER>
 struct UnitQ4_1 {
     static constexpr int ELEMS = 32, ROW_ALIGN = 4, SPAN = 0;
-    static constexpr bool GENERAL_ONLY = true;
     struct W { u32x4 q; uint32_t dm; };
     __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * 20; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
@@ -108,7 +107,6 @@ struct FmtQ5 {
 template <bool HAS_MIN>
 struct UnitQ5 {
     static constexpr int ELEMS = 32, ROW_ALIGN = 2, SPAN = 0;
-    static constexpr bool GENERAL_ONLY = true;
     static constexpr int BYTES = HAS_MIN ? 24 : 22;
     struct W { u32x4 q; uint32_t qh, dm; };
     __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 5) * BYTES; }
@@ -162,7 +160,6 @@ struct FmtQ2K {
 // unit = the 8 bytes qs[32n + 8j ..]: elements 128n + 32k + 8j + i (k = 0..3, i = 0..7)
 struct UnitQ2K {
     static constexpr int ELEMS = 32, ROW_ALIGN = 4, SPAN = 0;
-    static constexpr bool GENERAL_ONLY = true;
     struct W { u32x2 q; uint32_t sc, dm; };
     __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 84; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
@@ -220,7 +217,6 @@ struct FmtQ3K {
 // unit as for Q2_K, plus the 8 mask bytes hmask[8j ..] (bit 4n + k) and the 6-bit scales of its four groups
 struct UnitQ3K {
     static constexpr int ELEMS = 32, ROW_ALIGN = 2, SPAN = 0;
-    static constexpr bool GENERAL_ONLY = true;
     struct W { u32x2 q, h; uint32_t sc; uint16_t d; };
     __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 110; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
@@ -274,7 +270,6 @@ struct FmtQ5K {
 // unit = two sub-blocks sharing 32 nibble bytes (as UnitQ4K) plus the 32 bytes of 5th bits
 struct UnitQ5K {
     static constexpr int ELEMS = 64, ROW_ALIGN = 16, SPAN = 0;
-    static constexpr bool GENERAL_ONLY = true;
     struct W { u32x4 hdr, h0, h1, q0, q1; };
     __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return (size_t)(K >> 8) * 176; }
     __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {

@@ -443,7 +443,7 @@ static int launch_mb(candy_hip_device *dev, const candy_hip_qtensor *w, const in
     const int iter = (int)((K / U::ELEMS + 63) / 64);
     const bool wide = m > 4 && mb_lds_bytes(8, K) <= MB_LDS_MAX;
     // rounds of 64 units the kernel holds in registers without spilling, per format (Q6_K: none so far)
-    constexpr int max_iter = std::is_same<U, UnitQ4K>::value ? 4 : std::is_same<U, UnitQ6K>::value ? 0 : 8;
+    constexpr int max_iter = std::is_same<U, UnitQ4K>::value ? 4 : (std::is_same<U, UnitQ8_0>::value || std::is_same<U, UnitQ4_0<false>>::value || std::is_same<U, UnitQ4_0<true>>::value) ? 8 : 0;
     if (iter > max_iter || (!wide && (m > 4 || mb_lds_bytes(4, K) > MB_LDS_MAX))) return CANDY_HIP_ERR_UNSUPPORTED;
 #define CANDY_MB(IT)                                                                  \
     return wide ? launch_mb_cfg<U, IT, 8>(dev, w, qs, scales, m, y) : launch_mb_cfg<U, IT, 4>(dev, w, qs, scales, m, y)
@@ -473,29 +473,19 @@ static int launch_one(candy_hip_device *dev, const candy_hip_qtensor *w, const i
     return CANDY_HIP_OK;
 }
 
-// Units of the secondary formats go through the general kernel only (no per-length batch-1 variants).
-template <class U, class = void>
-struct GeneralOnly { static constexpr bool value = false; };
-template <class U>
-struct GeneralOnly<U, std::enable_if_t<U::GENERAL_ONLY>> { static constexpr bool value = true; };
-template <class U>
-static constexpr bool general_only() { return GeneralOnly<U>::value; }
-
 template <class U>
 static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                       int64_t m, float *y) {
     const int64_t K = w->cols, N = w->rows;
     const int64_t sstride = K >> 5;
-    if constexpr (!general_only<U>()) {
-        if (m == 1) {
-            MatvecJobs jobs{};
-            jobs.n = 1;
-            jobs.j[0].W = (const uint8_t *)w->data;
-            jobs.j[0].y = y;
-            jobs.j[0].N = (int)N;
-            const int rc = launch_jobs_fmt<U>(dev, jobs, K, qs, scales);
-            if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
-        }
+    if (m == 1) {
+        MatvecJobs jobs{};
+        jobs.n = 1;
+        jobs.j[0].W = (const uint8_t *)w->data;
+        jobs.j[0].y = y;
+        jobs.j[0].N = (int)N;
+        const int rc = launch_jobs_fmt<U>(dev, jobs, K, qs, scales);
+        if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     }
     int64_t done = 0;
     const bool old_small = getenv("CANDY_HIP_OLD_SMALL_BATCH") != nullptr;  // comparison runs and tests
@@ -505,7 +495,7 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
         const Q8Scale *s = scales + done * sstride;
         float *yo = y + done * N;
         int rc;
-        if constexpr (!general_only<U>()) {
+        {
             // The looping kernel below takes 8, 4, 2 or 1 rows per launch (fewer the longer the row is); where that
             // covers what is left in as few launches as this kernel's 8 per pass, it is as fast or a little faster
             // (short rows, up to about 16K of them), and two rows cost less there than as half of a 4-row pass.
