@@ -103,11 +103,17 @@ int workspace(candy_hip_device *dev, size_t bytes, void **out);
 int splitk_workspace(candy_hip_device *dev, size_t bytes, void **out);
 // mmq_f16.hip: y[i] = (res[i] +) part[0][i] + part[1][i] + ... in that order (count floats per part)
 int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split);
-// Formats with the per-length batch-1 kernels (residual epilogue, several weights per launch) and the fused
-// decode kernels; the others contract through the general small-batch kernel.
+// Formats the batch-1 kernel contracts (residual epilogue, several weights per launch): all that have a vec-dot.
+// The fused decode kernels exist for Q4_K, Q6_K, Q8_0 and the two Q4_0 orders only.
 inline bool format_has_batch1_kernel(int fmt) {
-    return fmt == CANDY_HIP_Q4_K || fmt == CANDY_HIP_Q6_K || fmt == CANDY_HIP_Q8_0 || fmt == CANDY_HIP_Q4_0 ||
-           fmt == CANDY_HIP_Q4_0_GGML;
+    switch (fmt) {
+    case CANDY_HIP_Q4_K: case CANDY_HIP_Q6_K: case CANDY_HIP_Q8_0: case CANDY_HIP_Q4_0: case CANDY_HIP_Q4_0_GGML:
+    case CANDY_HIP_Q4_1: case CANDY_HIP_Q4_1_GGML: case CANDY_HIP_Q5_0: case CANDY_HIP_Q5_1: case CANDY_HIP_Q2_K:
+    case CANDY_HIP_Q3_K: case CANDY_HIP_Q5_K:
+        return true;
+    default:
+        return false;
+    }
 }
 
 // quant.hip: x[rows, cols] -> planar int8 quants + scales; optionally also 34-byte blocks.

@@ -331,8 +331,11 @@ static int linear_residual(candy_hip_llama *m, const candy_hip_qtensor *w) {
     const candy_hip_qtensor *ws[1] = {w};
     float *ys[1] = {m->h};
     const float *res[1] = {m->h};
-    if (format_has_batch1_kernel(w->fmt)) return launch_matvec_multi(m->dev, ws, ys, res, 1, m->xq, m->xs);
-    // the other formats: general kernel into a buffer of its own, then the add
+    if (format_has_batch1_kernel(w->fmt)) {
+        rc = launch_matvec_multi(m->dev, ws, ys, res, 1, m->xq, m->xs);
+        if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+    }
+    // rows too long for the batch-1 kernel: looping kernel into a buffer of its own, then the add
     if ((rc = launch_matvec(m->dev, w, m->xq, m->xs, 1, m->proj))) return rc;
     return candy_hip_add(m->dev, m->h, m->proj, w->rows, m->h);
 }

@@ -324,8 +324,15 @@ static int launch_jobs(candy_hip_device *dev, int fmt, const MatvecJobs &jobs, i
     case CANDY_HIP_Q4_0: return launch_jobs_fmt<UnitQ4_0<false>>(dev, jobs, K, qs, scales);
     case CANDY_HIP_Q4_0_GGML: return launch_jobs_fmt<UnitQ4_0<true>>(dev, jobs, K, qs, scales);
     case CANDY_HIP_Q6_K: return launch_jobs_fmt<UnitQ6K>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q4_1: return launch_jobs_fmt<UnitQ4_1<false>>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q4_1_GGML: return launch_jobs_fmt<UnitQ4_1<true>>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q5_0: return launch_jobs_fmt<UnitQ5<false>>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q5_1: return launch_jobs_fmt<UnitQ5<true>>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q2_K: return launch_jobs_fmt<UnitQ2K>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q3_K: return launch_jobs_fmt<UnitQ3K>(dev, jobs, K, qs, scales);
+    case CANDY_HIP_Q5_K: return launch_jobs_fmt<UnitQ5K>(dev, jobs, K, qs, scales);
     default:
-        if (format_info(fmt).elems != 0) return CANDY_HIP_ERR_UNSUPPORTED;  // the other formats: one launch per weight
+        if (format_info(fmt).elems != 0) return CANDY_HIP_ERR_UNSUPPORTED;  // Q8_K: no vec-dot
         return fail(CANDY_HIP_ERR_INVALID, "unknown quantized format %d", fmt);
     }
 }
@@ -541,7 +548,7 @@ int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *w
         if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     }
     for (int i = 0; i < n; ++i) {
-        if (res && res[i]) return fail(CANDY_HIP_ERR_UNSUPPORTED, "residual epilogue needs the batch-1 kernel");
+        if (res && res[i]) return CANDY_HIP_ERR_UNSUPPORTED;  // rows too long for the batch-1 kernel: the caller adds the residual itself
         if (int rc = launch_matvec(dev, ws[i], qs, scales, 1, ys[i])) return rc;
     }
     return CANDY_HIP_OK;

@@ -144,6 +144,31 @@ def test_decode_with_weights_quantized_from_normal(dev):
     assert rel(kc[0, :, :3], ref.k_cache[0, :, :3].astype(np.float64)) <= 1e-3
 
 
+def test_decode_with_rows_too_long_for_the_batch1_kernels(dev):
+    # FFN rows longer than the batch-1 kernels hold in registers (16640 > 8 x 64 units of 32 values): the down
+    # projection takes the looping kernel into a buffer of its own and the residual is added afterwards.  A row of
+    # 16640 re-quantized activations is where f32 summation order shows first (the op itself is 3e-7 from the CPU),
+    # so the bar is the activation quantizer's noise, as above; the first step's first-layer k/v hold 1e-3.
+    cfg = dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=64, d_ffn=16640, vocab=256,
+               max_pos=16, rms_eps=1e-5, rope_base=10000.0)
+    fmts = {"default": synth.Q8_0, "down": synth.Q6_K, "head": synth.Q6_K, "embed": synth.Q8_0}
+    host, model = build(dev, cfg, fmts, seed=50)
+    ref = llama_ref.LlamaRef(cfg, host)
+    plain = llama_ref.LlamaRef(cfg, host, f32_activations=True)
+    for pos, tok in enumerate([3, 200, 57]):
+        nt, logits = model.decode(tok, pos)
+        rt, rlogits, _ = ref.step(ref.embed(tok), pos)
+        _, plogits, _ = plain.step(plain.embed(tok), pos)
+        noise = rel(rlogits, plogits.astype(np.float64))
+        assert rel(logits, rlogits) <= max(1e-3, 0.5 * noise), (pos, rel(logits, rlogits), noise)
+        assert nt == int(np.argmax(logits))
+    kptr, _, nbytes = model.kv_cache()
+    kc = np.empty(nbytes // 4, np.float32)
+    hip._check(hip.lib().candy_hip_d2h(dev.handle, kc.ctypes.data, kptr, nbytes))
+    kc = kc.reshape(ref.k_cache.shape)
+    assert rel(kc[0, :, :1], ref.k_cache[0, :, :1].astype(np.float64)) <= 1e-3
+
+
 def test_full_depth_7b_step_within_activation_noise(dev):
     # The benchmark's model at its full depth: 32 layers 4096 / 11008, 32 heads x 128, vocab 32000, every matrix
     # N(0, 0.02) quantized on the device (one draw per shape, blocks rotated per layer), KV cache pre-filled with
