@@ -60,12 +60,13 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
     const int units = K / U::ELEMS;
     const size_t rb = U::row_bytes(K);
 
-    int ji = 0, wg = blockIdx.x;
-    if (EPI == EPI_PLAIN) {
-        ji = (int)(blockIdx.x >= (unsigned)a.jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)a.jobs.j[1].wg_end);
-        wg = blockIdx.x - (ji > 0 ? a.jobs.j[ji - 1].wg_end : 0);
-    }
-    const int N = a.jobs.j[ji].N;
+    // PLAIN: the (up to three) weights form one run of rows, wg_end holding each weight's END ROW in that run, and
+    // a workgroup takes R * WAVES consecutive rows of the run wherever they fall, so that the run divides over the
+    // CUs evenly whatever the single row counts are (6144 rows of an 8B q/k/v = 256 workgroups of 24).  A wavefront
+    // resolves each of its rows to a weight and a row of that weight (wavefront-uniform).  PAIR: blockIdx is the
+    // group of S row pairs.
+    const int wg = blockIdx.x;
+    const int N = a.jobs.j[0].N;  // PAIR: both weights have N rows
 
     // ---- inputs first (oldest entries of the in-order return queue)
     uint4 aq[AQ];
@@ -90,12 +91,21 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
     // ---- every weight load of the wavefront
     const int row0 = (wg * WAVES + wave) * R;
     typename U::W w[NW][R][ITER];
+    int job[R], jrow[R];  // PLAIN: weight and row within it, -1 past the end of the run
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int g = row0 + r;
+        const int e0 = a.jobs.j[0].wg_end, e1 = a.jobs.j[1].wg_end, e2 = a.jobs.j[2].wg_end;
+        const int ji = (int)(g >= e0) + (int)(g >= e1);
+        job[r] = g < e2 ? ji : -1;
+        jrow[r] = g < e2 ? g - (ji == 0 ? 0 : ji == 1 ? e0 : e1) : 0;
+    }
 #pragma unroll
     for (int m = 0; m < NW; ++m) {
-        const uint8_t *Wm = EPI == EPI_PAIR ? a.jobs.j[m].W : a.jobs.j[ji].W;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint8_t *row = Wm + (size_t)min(row0 + r, N - 1) * rb;
+            const uint8_t *row = EPI == EPI_PAIR ? a.jobs.j[m].W + (size_t)min(row0 + r, N - 1) * rb
+                                                 : a.jobs.j[max(job[r], 0)].W + (size_t)jrow[r] * rb;
 #pragma unroll
             for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
         }
@@ -167,12 +177,14 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
     }
 
     if (EPI == EPI_PLAIN) {
-        float *y = a.jobs.j[ji].y;  // may alias res (h += W.x)
-        const float *res = a.jobs.j[ji].res;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float v = wave_sum(acc[0][r]);
-            if (lane == 0 && row0 + r < N) y[row0 + r] = res ? res[row0 + r] + v : v;
+            if (lane == 0 && job[r] >= 0) {
+                float *y = a.jobs.j[job[r]].y;  // may alias res (h += W.x)
+                const float *res = a.jobs.j[job[r]].res;
+                y[jrow[r]] = res ? res[jrow[r]] + v : v;
+            }
         }
     } else {
         // A PAIR workgroup owns S = 32, 16 or 8 consecutive outputs: a whole Q8_0 block, or a part of one.  Parts
@@ -234,10 +246,12 @@ static int launch_fused_cfg(candy_hip_device *dev, FusedArgs a) {
     if (EPI == EPI_PAIR) {
         total = a.jobs.j[0].N / rows_per_wg;
     } else {
+        int rows = 0;
         for (int i = 0; i < 3; ++i) {
-            if (i < a.jobs.n) total += (a.jobs.j[i].N + rows_per_wg - 1) / rows_per_wg;
-            a.jobs.j[i].wg_end = total;
+            if (i < a.jobs.n) rows += a.jobs.j[i].N;
+            a.jobs.j[i].wg_end = rows;  // end row in the run; unused slots end where the last real one does
         }
+        total = (rows + rows_per_wg - 1) / rows_per_wg;
     }
     hipLaunchKernelGGL((k_matvec_fused<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)total), dim3(T), smem, dev->stream, a);
     CANDY_LAUNCH_CHECK();
@@ -250,7 +264,8 @@ static int launch_fused_cfg(candy_hip_device *dev, FusedArgs a) {
 // 16 rows (16 wavefronts x 1) 1.859, 8 rows (8 x 1) 1.855 ms per token; 4 rows 1.960; with four rows per wavefront
 // the 16-row shape is slower than whole blocks (2.036).  d_ffn 14336: 32 rows 1.983, 8 rows 1.957.  The same choice
 // for the plain RMSNorm-prologue kernel (16 or 8 rows) did not pay: 8 rows lose more to the repeated prologue than
-// the even split wins.  `env` names an override for comparison runs.
+// the even split wins (24-row workgroups over the weights' rows as one run do).  `env` names an override for
+// comparison runs.
 static int balanced_rows(int rows, int cus, int hi, int lo, const char *env) {
     if (const char *e = getenv(env)) {
         const int v = atoi(e);
@@ -286,6 +301,13 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
     }
     if (pro == PRO_RMS) {
         if constexpr (ITER <= 2) {
+            // 16 rows per workgroup (4 x 4), or 24 (8 wavefronts x 3) where that leaves the fullest CU fewer rows
+            int rows = 0;
+            for (int i = 0; i < a.jobs.n; ++i) rows += a.jobs.j[i].N;
+            const int cus = dev->num_cus;
+            const long c16 = (long)((rows + 15) / 16 + cus - 1) / cus * 16, c24 = (long)((rows + 23) / 24 + cus - 1) / cus * 24;
+            const char *e = getenv("CANDY_HIP_RMS_ROWS");  // comparison runs
+            if (e ? atoi(e) == 24 : c24 < c16) return launch_fused_cfg<U, ITER, 3, 8, PRO_RMS, EPI_PLAIN>(dev, a);
             return launch_fused_cfg<U, ITER, 4, 4, PRO_RMS, EPI_PLAIN>(dev, a);
         } else {
             return launch_fused_cfg<U, ITER, 2, 4, PRO_RMS, EPI_PLAIN>(dev, a);
