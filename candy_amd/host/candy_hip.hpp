@@ -293,7 +293,31 @@ public:
             return {nullptr, e};
         return {Ptr(new QTensor(dev, h, f, rows, cols)), Ok()};
     }
-    ~QTensor() { candy_hip_qtensor_free(h_); }
+    // Quantize f32 [rows, cols] on the device into blocks of f (the kernels candy only names,
+    // tensor/internal/metal/kernels/kernels.go:563-592); the QTensor owns the block buffer.
+    static Result<Ptr> Quantize(const DevicePtr &dev, QFormat f, const HipStorage<float>::Ptr &x, int rows, int cols) {
+        if (!x) return {nullptr, Errorf("quantize: input must live on the HIP device")};
+        if (rows <= 0 || cols <= 0 || (size_t)rows * cols != x->Len()) return {nullptr, Errorf("quantize: shape mismatch")};
+        const size_t nbytes = candy_hip_qweight_bytes((int)f, rows, cols);
+        if (nbytes == 0) return {nullptr, Errorf("quantize: cols is not a multiple of the block size")};
+        void *blocks = nullptr;
+        if (Error e = last_error(candy_hip_alloc(dev->handle(), nbytes, &blocks), "quantize")) return {nullptr, e};
+        int rc = (int)f == CANDY_HIP_Q8_0 ? candy_hip_quantize_q8_0(dev->handle(), (const float *)x->ptr(), rows, cols, blocks)
+                                          : candy_hip_quantize(dev->handle(), (int)f, (const float *)x->ptr(), rows, cols, blocks);
+        candy_hip_qtensor *h = nullptr;
+        if (!rc) rc = candy_hip_qtensor_wrap(dev->handle(), (int)f, rows, cols, blocks, nbytes, &h);
+        if (Error e = last_error(rc, "quantize")) {
+            candy_hip_free(dev->handle(), blocks);
+            return {nullptr, e};
+        }
+        Ptr q(new QTensor(dev, h, f, rows, cols));
+        q->owned_blocks_ = blocks;
+        return {q, Ok()};
+    }
+    ~QTensor() {
+        candy_hip_qtensor_free(h_);
+        if (owned_blocks_) candy_hip_free(dev_->handle(), owned_blocks_);
+    }
     QTensor(const QTensor &) = delete;
     int Rows() const { return rows_; }
     int Cols() const { return cols_; }
@@ -329,6 +353,7 @@ private:
     candy_hip_qtensor *h_;
     QFormat f_;
     int rows_, cols_;
+    void *owned_blocks_ = nullptr;
 };
 
 }  // namespace candy

@@ -171,6 +171,24 @@ int main() {
             CHECK(q.value->QMatMul(xs, &lbad).err.msg.rfind("qmatmul: shape mismatch", 0) == 0, "qmatmul shape error");
         }
         CHECK((bool)QTensor::New(dev, QFormat::Q4_K, 4, 100, std::vector<uint8_t>(10)).err, "cols not a multiple of the block");
+        // ---- QTensor::Quantize: the device's blocks dequantize to what the CPU restatement's blocks do, bit for bit
+        struct Qm { QFormat f; int id; } qfm[] = {{QFormat::Q4_0, CO_Q4_0}, {QFormat::Q8_0, CO_Q8_0}, {QFormat::Q4_K, CO_Q4_K}, {QFormat::Q6_K, CO_Q6_K}};
+        for (auto fm : qfm) {
+            const int rows = 6, cols = 768;
+            std::vector<float> xw((size_t)rows * cols);
+            for (auto &v : xw) v = 0.02f * nd(rng);
+            std::vector<uint8_t> cpu_blocks((size_t)rows * (cols / co_block_elems(fm.id)) * co_block_bytes(fm.id));
+            CHECK(co_quantize(fm.id, xw.data(), rows, cols, cpu_blocks.data()) == 0, "co_quantize fmt %d", fm.id);
+            std::vector<float> want((size_t)rows * cols);
+            co_dequantize(fm.id, cpu_blocks.data(), rows * cols / co_block_elems(fm.id), want.data());
+            auto q = QTensor::Quantize(dev, fm.f, F::FromSlice(dev, xw).value, rows, cols);
+            CHECK(q.ok(), "QTensor::Quantize fmt %d", fm.id);
+            if (q.ok()) {
+                auto got = q.value->Dequantize().value->Data();
+                CHECK(std::memcmp(got.data(), want.data(), got.size() * 4) == 0, "Quantize -> Dequantize bit-exact fmt %d", fm.id);
+            }
+        }
+        CHECK((bool)QTensor::Quantize(dev, QFormat::Q4_K, F::FromSlice(dev, std::vector<float>(300)).value, 3, 100).err, "quantize: cols off the block");
     }
     CHECK(!dev->Synchronize(), "Synchronize");
     std::printf(g_fail ? "host mirror: %d check(s) FAILED\n" : "host mirror: all checks passed\n", g_fail);
