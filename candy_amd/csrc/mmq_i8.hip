@@ -211,6 +211,49 @@ struct TileQ6K {
     }
 };
 
+// Q8_0: the weights are int8 already.  A super-block is eight 34-byte blocks (272 bytes = 17 chunks, no overrun);
+// the A operand of sub-block t is 8 of the block's 32 quants as they lie (2-byte aligned in the slice), and the
+// rescale is acc += (d_w * d_x) * dot as vec_dot_q8_0_q8_1 does (quantized.cu:2058-2073).  The fp16 scales of a row
+// are widened once per super-block by the lane that feeds the row into the A operand (row j, blocks 2c and 2c + 1)
+// and handed through LDS to the lanes that own the row in the C layout, like Q4_K's factors.
+struct TileQ8_0 {
+    static constexpr int BLOCK = 272, SLOT = 272;
+    typedef u32x4_a2 GlobalChunk;  // rows sit on 2-byte boundaries
+    struct Exchange {
+        float dw[8][16];  // block scale [sub-block][row]
+    };
+    template <int TM>
+    static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &ex,
+                                                      const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        const uint8_t *wl = slice + j * pitch + SLOT * b;
+        ex.dw[2 * c][j] = half_bits_to_float(*(const uint16_t *)(wl + 34 * (2 * c)));
+        ex.dw[2 * c + 1][j] = half_bits_to_float(*(const uint16_t *)(wl + 34 * (2 * c + 1)));
+        wave_lds_fence();
+        float4 dq[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) dq[t] = *(const float4 *)&ex.dw[t][4 * c];
+        wave_lds_fence();  // the slots are rewritten by the next super-block
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const u32x2 qa = *(const u32x2_a2 *)(wl + 34 * t + 2 + 8 * c);
+            const long afrag = (long)(((uint64_t)qa.y << 32) | qa.x);
+            const float dw[4] = {dq[t].x, dq[t].y, dq[t].z, dq[t].w};
+            int4v d[TM];
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
+                d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const float dx = s_xs[(16 * a + j) * 8 + t].x;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[a][i] += (dw[i] * dx) * (float)d[a][i];
+            }
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // LDS carve-up of k_mmq_i8 (dynamic: the K-split variant needs more than the 64 KB a static layout may take)
 template <class F, int TM, int STG, int KS>
@@ -442,11 +485,13 @@ bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs) {
     // the last chunk of a Q6_K row runs 14 bytes past the block: only buffers allocated by the library
     // (which pads them) are known to have that room after the last row
     if (w->fmt == CANDY_HIP_Q6_K) return w->owned && ((uintptr_t)w->data & 1) == 0;
+    if (w->fmt == CANDY_HIP_Q8_0) return ((uintptr_t)w->data & 1) == 0;
     return false;
 }
 
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                   int64_t m, float *y) {
+    if (w->fmt == CANDY_HIP_Q8_0) return launch_i8<TileQ8_0>(dev, w, qs, scales, m, y);
     return w->fmt == CANDY_HIP_Q4_K ? launch_i8<TileQ4K>(dev, w, qs, scales, m, y)
                                     : launch_i8<TileQ6K>(dev, w, qs, scales, m, y);
 }
