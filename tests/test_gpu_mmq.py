@@ -91,6 +91,16 @@ def test_big_fp16_tiles(dev, fmt, m, rows, cols):
         assert np.max(per_row) <= 2 * TOL
 
 
+def test_q8_0_wide_prompt_grid_takes_the_fp16_tiles(dev):
+    # many weight rows and a prompt-sized batch: Q8_0 leaves the int8 tiles for the 128 x 128 fp16 tiles
+    rows, cols, m = 8192, 256, 352
+    w = synth.random_weight(synth.Q8_0, rows, cols, seed=9)
+    x = synth.random_activations(m, cols, seed=10)
+    got = dev.qmatmul(dev.qtensor(synth.Q8_0, rows, cols, w), x)
+    err = rel_err(got, o.qmatmul(synth.Q8_0, w, rows, cols, x))
+    assert 2e-6 < err <= TOL  # fp16 operands: not the integer-exact kernel
+
+
 @pytest.mark.parametrize("fmt,rows,cols", [(synth.Q8_0, 70, 96), (synth.Q4_0, 33, 160), (synth.Q8_0, 64, 32)])
 def test_contraction_length_not_a_multiple_of_64(dev, fmt, rows, cols):
     # odd block counts take the small-batch kernel in slices: same result, integer-exact dots
