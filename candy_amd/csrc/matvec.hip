@@ -569,8 +569,9 @@ int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quan
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                   int64_t m, float *y) {
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && w->cols <= 0x7FFFFFFF, "matrix too large");
-    // Q8_0: the vector kernel matches the tile kernel up to 8 rows (one pass); from 9 rows on it needs two
-    if (m >= 9 && w->fmt == CANDY_HIP_Q8_0 && getenv("CANDY_HIP_I8_MIN_M") == nullptr && mmq_i8_covers(w, qs))
+    // Q8_0, Q4_0: the vector kernel matches the tile kernel up to 8 rows (one pass); from 9 rows on it needs two
+    if (m >= 9 && (w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML) &&
+        getenv("CANDY_HIP_I8_MIN_M") == nullptr && mmq_i8_covers(w, qs))
         return launch_mmq_i8(dev, w, qs, scales, m, y);
     if (m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K) && mmq_i8_covers(w, qs)) {
         // 5 .. 15 rows: the vector kernels below (one or two passes of up to 8 rows) or one pass of the int8 tile

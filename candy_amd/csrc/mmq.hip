@@ -347,7 +347,8 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     // Q8_0 on the int8 tiles as well, except where the 128 x 128 fp16 tiles below fill the chip (many weight rows and
     // a prompt-sized batch; measured: 11008x4096 m = 256 127 against 123 us, m = 512 228 against 134; 32000x4096
     // m = 128 165 against 129; but 4096x11008 m = 128 68 against 313, 4096x4096 m = 512 88 against 121)
-    const bool q8_wide = w->fmt == CANDY_HIP_Q8_0 && w->rows >= 8192 && (double)m * (double)w->rows >= 2.8e6;
+    const bool q8_wide = (w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML) && w->rows >= 8192 &&
+                         (double)m * (double)w->rows >= 2.8e6;
     if (!force_fp16 && !big && !q8_wide && mmq_i8_covers(w, qs)) return launch_mmq_i8(dev, w, qs, scales, m, y);
     if (big && xh_ready) {
         *res_done = res != nullptr;

@@ -254,6 +254,64 @@ struct TileQ8_0 {
     }
 };
 
+// Q4_0: eight 18-byte blocks per super-block (144 bytes = 9 chunks, no overrun).  A lane's 8 values of a
+// sub-block are the two nibbles of 4 consecutive bytes in candy's element order (quantized.go:85-93: y[2j] low,
+// y[2j+1] high) or one nibble of 8 consecutive bytes in ggml's (low nibbles are values 0-15, high 16-31).  The
+// -8 offset is applied through the activation block sum: acc += d_w * (d_x * dot - 8 * d_x * bsum), the integer
+// form of vec_dot_q4_0_q8_1 (quantized.cu:1919-1941) with the exact sum in place of Q8_1's rounded one.
+template <bool GGML>
+struct TileQ4_0 {
+    static constexpr int BLOCK = 144, SLOT = 144;
+    typedef u32x4_a2 GlobalChunk;
+    struct Exchange {
+        float dw[8][16];
+    };
+    template <int TM>
+    static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &ex,
+                                                      const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        const uint8_t *wl = slice + j * pitch + SLOT * b;
+        ex.dw[2 * c][j] = half_bits_to_float(*(const uint16_t *)(wl + 18 * (2 * c)));
+        ex.dw[2 * c + 1][j] = half_bits_to_float(*(const uint16_t *)(wl + 18 * (2 * c + 1)));
+        wave_lds_fence();
+        float4 dq[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) dq[t] = *(const float4 *)&ex.dw[t][4 * c];
+        wave_lds_fence();  // the slots are rewritten by the next super-block
+        const uint32_t M = 0x0F0F0F0Fu;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            uint32_t lo, hi;  // values 8c .. 8c+3 and 8c+4 .. 8c+7 of the sub-block, one per byte
+            if (GGML) {
+                const u32x2 q = *(const u32x2_a2 *)(wl + 18 * t + 2 + 8 * (c & 1));
+                const int sh = (c >> 1) * 4;
+                lo = (q.x >> sh) & M;
+                hi = (q.y >> sh) & M;
+            } else {
+                uint32_t q;
+                __builtin_memcpy(&q, wl + 18 * t + 2 + 4 * c, 4);
+                const uint32_t l = q & M, h = (q >> 4) & M;
+                lo = __builtin_amdgcn_perm(h, l, 0x05010400u);  // l0 h0 l1 h1
+                hi = __builtin_amdgcn_perm(h, l, 0x07030602u);  // l2 h2 l3 h3
+            }
+            const long afrag = (long)(((uint64_t)hi << 32) | lo);
+            const float dw[4] = {dq[t].x, dq[t].y, dq[t].z, dq[t].w};
+            int4v d[TM];
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
+                d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int a = 0; a < TM; ++a) {
+                const float2 sx = s_xs[(16 * a + j) * 8 + t];
+                const float off = -8.0f * sx.y;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[a][i] += dw[i] * (sx.x * (float)d[a][i] + off);
+            }
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // LDS carve-up of k_mmq_i8 (dynamic: the K-split variant needs more than the 64 KB a static layout may take)
 template <class F, int TM, int STG, int KS>
@@ -485,13 +543,15 @@ bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs) {
     // the last chunk of a Q6_K row runs 14 bytes past the block: only buffers allocated by the library
     // (which pads them) are known to have that room after the last row
     if (w->fmt == CANDY_HIP_Q6_K) return w->owned && ((uintptr_t)w->data & 1) == 0;
-    if (w->fmt == CANDY_HIP_Q8_0) return ((uintptr_t)w->data & 1) == 0;
+    if (w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML) return ((uintptr_t)w->data & 1) == 0;
     return false;
 }
 
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                   int64_t m, float *y) {
     if (w->fmt == CANDY_HIP_Q8_0) return launch_i8<TileQ8_0>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q4_0) return launch_i8<TileQ4_0<false>>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q4_0_GGML) return launch_i8<TileQ4_0<true>>(dev, w, qs, scales, m, y);
     return w->fmt == CANDY_HIP_Q4_K ? launch_i8<TileQ4K>(dev, w, qs, scales, m, y)
                                     : launch_i8<TileQ6K>(dev, w, qs, scales, m, y);
 }
