@@ -344,11 +344,12 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     // smaller batches of Q4_K and Q6_K: int8 matrix cores (exact); the fp16 tile kernel below serves the rest
     const bool force_fp16 = force_old_fp16();
     const bool big = !force_fp16 && mmq_f16_big_covers(w, m);
-    // Q8_0 on the int8 tiles as well, except where the 128 x 128 fp16 tiles below fill the chip (many weight rows and
+    // the 32-value formats (Q8_0, Q4_0, Q4_1, Q5_0, Q5_1) on the int8 tiles as well, except where the 128 x 128 fp16 tiles below fill the chip (many weight rows and
     // a prompt-sized batch; measured: 11008x4096 m = 256 127 against 123 us, m = 512 228 against 134; 32000x4096
     // m = 128 165 against 129; but 4096x11008 m = 128 68 against 313, 4096x4096 m = 512 88 against 121)
-    const bool q8_wide = (w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML) && w->rows >= 8192 &&
-                         (double)m * (double)w->rows >= 2.8e6;
+    const bool is_q32 = w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML ||
+                        w->fmt == CANDY_HIP_Q4_1 || w->fmt == CANDY_HIP_Q4_1_GGML || w->fmt == CANDY_HIP_Q5_0 || w->fmt == CANDY_HIP_Q5_1;
+    const bool q8_wide = is_q32 && w->rows >= 8192 && (double)m * (double)w->rows >= 2.8e6;
     if (!force_fp16 && !big && !q8_wide && mmq_i8_covers(w, qs)) return launch_mmq_i8(dev, w, qs, scales, m, y);
     if (big && xh_ready) {
         *res_done = res != nullptr;

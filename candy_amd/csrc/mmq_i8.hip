@@ -35,6 +35,7 @@
 
 #include "blocks.h"
 #include "internal.h"
+#include "formats_more.h"
 
 namespace candy {
 
@@ -54,86 +55,111 @@ __device__ __forceinline__ void wave_lds_fence() {
 //   slice   the wavefront's LDS slice, row r's super-block b at slice + r * pitch + b * SLOT
 //   s_xq    activation tile [16*TM][XROW] int8, s_xs {d, d*bsum} [16*TM][8]
 //   acc     lane (j = lane%16, c = lane/16) holds activation row 16a+j, weight rows 4c+i
+// Q4_K and Q5_K share everything but the fifth bit: a Q5_K block is a Q4_K block with 32 bytes of high bits
+// between the header and the nibbles (bit t of byte l belongs to value l of sub-block t, quantized.cu:1044-1080).
+struct ExchangeK {
+    float dsc[8][16];  // d * scale    [sub-block][row]
+    float dmf[8][16];  // dmin * min
+};
+template <int TM, bool FIVE>
+__device__ __forceinline__ void superblock_q45k(const uint8_t *wl, int j, int c, ExchangeK &ex, const int8_t *s_xq,
+                                                const float2 *s_xs, float (&acc)[TM][4]) {
+    constexpr int QS = FIVE ? 48 : 16;  // where the nibbles start
+    {   // lane (row j, pair c) unpacks one pair of 6-bit scales / mins, folds the row's d / dmin in and parks
+        // the four factors for the lanes that own the row in the C layout
+        const u32x4 h = *(const u32x4 *)wl;
+        uint32_t sc2, m2;
+        q4k_scale_min_pair(h.y, h.z, h.w, c, sc2, m2);
+        const float d = half_bits_to_float((uint16_t)(h.x & 0xFFFF)), dmin = half_bits_to_float((uint16_t)(h.x >> 16));
+        ex.dsc[2 * c][j] = d * (float)(sc2 & 0xFF);
+        ex.dsc[2 * c + 1][j] = d * (float)(sc2 >> 8);
+        ex.dmf[2 * c][j] = dmin * (float)(m2 & 0xFF);
+        ex.dmf[2 * c + 1][j] = dmin * (float)(m2 >> 8);
+    }
+    wave_lds_fence();
+    float4 dsq[8], dmq[8];  // my four C rows 4c .. 4c+3, per sub-block
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        dsq[t] = *(const float4 *)&ex.dsc[t][4 * c];
+        dmq[t] = *(const float4 *)&ex.dmf[t][4 * c];
+    }
+    wave_lds_fence();  // the slots are rewritten by the next super-block
+    u32x2 qh = {0u, 0u};
+    if (FIVE) qh = *(const u32x2 *)(wl + 16 + 8 * c);  // fifth bits of values 8c .. 8c+7 of every sub-block
+    auto afrag_of = [&](int t) __attribute__((always_inline)) {
+        const u32x2 qa = *(const u32x2 *)(wl + QS + 32 * (t >> 1) + 8 * c);
+        const int sh = (t & 1) * 4;
+        uint32_t lo = (qa.x >> sh) & 0x0F0F0F0Fu, hi = (qa.y >> sh) & 0x0F0F0F0Fu;
+        if (FIVE) {
+            lo |= ((qh.x >> t) & 0x01010101u) << 4;
+            hi |= ((qh.y >> t) & 0x01010101u) << 4;
+        }
+        return (long)(((uint64_t)hi << 32) | lo);
+    };
+    if constexpr (TM == 1) {
+        // one tile per sub-block: nothing else in the wavefront covers an MFMA's latency, so all eight products
+        // of the super-block are issued first and rescaled afterwards
+        int4v d8[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const long bfrag = *(const long *)&s_xq[j * XROW + 32 * t + 8 * c];
+            d8[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag_of(t), bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const float dsc[4] = {dsq[t].x, dsq[t].y, dsq[t].z, dsq[t].w};
+            const float dmf[4] = {dmq[t].x, dmq[t].y, dmq[t].z, dmq[t].w};
+            const float2 sx = s_xs[j * 8 + t];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[0][i] += sx.x * ((float)d8[t][i] * dsc[i]);
+                acc[0][i] -= dmf[i] * sx.y;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const long afrag = afrag_of(t);
+        const float dsc[4] = {dsq[t].x, dsq[t].y, dsq[t].z, dsq[t].w};  // d * sc and dmin * m of my four weight rows
+        const float dmf[4] = {dmq[t].x, dmq[t].y, dmq[t].z, dmq[t].w};
+        int4v d[TM];  // all tiles of the sub-block first, so the matrix pipe runs under the rescale
+#pragma unroll
+        for (int a = 0; a < TM; ++a) {
+            const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
+            d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+        }
+#pragma unroll
+        for (int a = 0; a < TM; ++a) {
+            const float2 sx = s_xs[(16 * a + j) * 8 + t];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[a][i] += sx.x * ((float)d[a][i] * dsc[i]);  // d8 * d * sc * dot
+                acc[a][i] -= dmf[i] * sx.y;                     // d8 * bsum * dmin * m
+            }
+        }
+    }
+}
+
 struct TileQ4K {
     static constexpr int BLOCK = 144, SLOT = 144;
     typedef u32x4 GlobalChunk;  // rows are 16-byte aligned
-    struct Exchange {
-        float dsc[8][16];  // d * scale    [sub-block][row]
-        float dmf[8][16];  // dmin * min
-    };
+    typedef ExchangeK Exchange;
     template <int TM>
     static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &ex,
                                                       const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
-        const uint8_t *wl = slice + j * pitch + SLOT * b;  // the row this lane feeds into the A operand
-        {   // lane (row j, pair c) unpacks one pair of 6-bit scales / mins, folds the row's d / dmin in and parks
-            // the four factors for the lanes that own the row in the C layout
-            const u32x4 h = *(const u32x4 *)wl;
-            uint32_t sc2, m2;
-            q4k_scale_min_pair(h.y, h.z, h.w, c, sc2, m2);
-            const float d = half_bits_to_float((uint16_t)(h.x & 0xFFFF)), dmin = half_bits_to_float((uint16_t)(h.x >> 16));
-            ex.dsc[2 * c][j] = d * (float)(sc2 & 0xFF);
-            ex.dsc[2 * c + 1][j] = d * (float)(sc2 >> 8);
-            ex.dmf[2 * c][j] = dmin * (float)(m2 & 0xFF);
-            ex.dmf[2 * c + 1][j] = dmin * (float)(m2 >> 8);
-        }
-        wave_lds_fence();
-        float4 dsq[8], dmq[8];  // my four C rows 4c .. 4c+3, per sub-block
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            dsq[t] = *(const float4 *)&ex.dsc[t][4 * c];
-            dmq[t] = *(const float4 *)&ex.dmf[t][4 * c];
-        }
-        wave_lds_fence();  // the slots are rewritten by the next super-block
-        if constexpr (TM == 1) {
-            // one tile per sub-block: nothing else in the wavefront covers an MFMA's latency, so all eight products
-            // of the super-block are issued first and rescaled afterwards
-            int4v d8[8];
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                const u32x2 qa = *(const u32x2 *)(wl + 16 + 32 * (t >> 1) + 8 * c);
-                const int sh = (t & 1) * 4;
-                const uint32_t lo = (qa.x >> sh) & 0x0F0F0F0Fu, hi = (qa.y >> sh) & 0x0F0F0F0Fu;
-                const long afrag = (long)(((uint64_t)hi << 32) | lo);
-                const long bfrag = *(const long *)&s_xq[j * XROW + 32 * t + 8 * c];
-                d8[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
-            }
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                const float dsc[4] = {dsq[t].x, dsq[t].y, dsq[t].z, dsq[t].w};
-                const float dmf[4] = {dmq[t].x, dmq[t].y, dmq[t].z, dmq[t].w};
-                const float2 sx = s_xs[j * 8 + t];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc[0][i] += sx.x * ((float)d8[t][i] * dsc[i]);
-                    acc[0][i] -= dmf[i] * sx.y;
-                }
-            }
-            return;
-        }
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const u32x2 qa = *(const u32x2 *)(wl + 16 + 32 * (t >> 1) + 8 * c);
-            const int sh = (t & 1) * 4;
-            const uint32_t lo = (qa.x >> sh) & 0x0F0F0F0Fu, hi = (qa.y >> sh) & 0x0F0F0F0Fu;
-            const long afrag = (long)(((uint64_t)hi << 32) | lo);
-            const float dsc[4] = {dsq[t].x, dsq[t].y, dsq[t].z, dsq[t].w};  // d * sc and dmin * m of my four weight rows
-            const float dmf[4] = {dmq[t].x, dmq[t].y, dmq[t].z, dmq[t].w};
-            int4v d[TM];  // all tiles of the sub-block first, so the matrix pipe runs under the rescale
-#pragma unroll
-            for (int a = 0; a < TM; ++a) {
-                const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
-                d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
-            }
-#pragma unroll
-            for (int a = 0; a < TM; ++a) {
-                const float2 sx = s_xs[(16 * a + j) * 8 + t];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc[a][i] += sx.x * ((float)d[a][i] * dsc[i]);  // d8 * d * sc * dot
-                    acc[a][i] -= dmf[i] * sx.y;                     // d8 * bsum * dmin * m
-                }
-            }
-        }
+        superblock_q45k<TM, false>(slice + j * pitch + SLOT * b, j, c, ex, s_xq, s_xs, acc);
+    }
+};
+
+struct TileQ5K {
+    static constexpr int BLOCK = 176, SLOT = 176;
+    typedef u32x4 GlobalChunk;
+    typedef ExchangeK Exchange;
+    template <int TM>
+    static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &ex,
+                                                      const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        superblock_q45k<TM, true>(slice + j * pitch + SLOT * b, j, c, ex, s_xq, s_xs, acc);
     }
 };
 
@@ -254,47 +280,69 @@ struct TileQ8_0 {
     }
 };
 
-// Q4_0: eight 18-byte blocks per super-block (144 bytes = 9 chunks, no overrun).  A lane's 8 values of a
-// sub-block are the two nibbles of 4 consecutive bytes in candy's element order (quantized.go:85-93: y[2j] low,
-// y[2j+1] high) or one nibble of 8 consecutive bytes in ggml's (low nibbles are values 0-15, high 16-31).  The
-// -8 offset is applied through the activation block sum: acc += d_w * (d_x * dot - 8 * d_x * bsum), the integer
-// form of vec_dot_q4_0_q8_1 (quantized.cu:1919-1941) with the exact sum in place of Q8_1's rounded one.
-template <bool GGML>
-struct TileQ4_0 {
-    static constexpr int BLOCK = 144, SLOT = 144;
+// The 32-value formats with 4- or 5-bit levels: Q4_0 (18 bytes: d, 16 bytes of nibbles), Q4_1 (20: d, m, nibbles),
+// Q5_0 (22: d, 32 fifth bits, nibbles) and Q5_1 (24: d, m, fifth bits, nibbles).  Eight blocks make a super-block
+// (144 / 160 / 176 / 192 bytes: whole 16-byte chunks, no overrun).  A lane's 8 values of a sub-block are the two
+// nibbles of 4 consecutive bytes in candy's element order (quantized.go:85-93, 107-116: y[2j] low, y[2j+1] high) or
+// one nibble of 8 consecutive bytes in ggml's (low nibbles are values 0-15, high 16-31; the only order of Q5_0 and
+// Q5_1).  The level offset (-8, -16) or the block minimum goes through the activation block sum:
+//   acc += d_w * (d_x * dot - OFF * d_x * bsum)        Q4_0, Q5_0   (quantized.cu:1919-1941, 2001-2025)
+//   acc += d_w * (d_x * dot) + m_w * (d_x * bsum)      Q4_1, Q5_1   (quantized.cu:1947-1975, 2027-2053)
+// with the exact integer sum in place of Q8_1's rounded one, like the vector kernels.
+template <int BYTES, bool HAS_MIN, bool HAS_HIGH, bool GGML>
+struct TileQ32 {
+    static constexpr int BLOCK = 8 * BYTES, SLOT = 8 * BYTES;
+    static constexpr int QH = 2 + 2 * HAS_MIN, QS = QH + 4 * HAS_HIGH;
     typedef u32x4_a2 GlobalChunk;
     struct Exchange {
         float dw[8][16];
+        float mw[HAS_MIN ? 8 : 1][16];
     };
     template <int TM>
     static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &ex,
                                                       const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        static_assert(!HAS_HIGH || GGML, "Q5_0 / Q5_1 exist in ggml's element order only");
         const uint8_t *wl = slice + j * pitch + SLOT * b;
-        ex.dw[2 * c][j] = half_bits_to_float(*(const uint16_t *)(wl + 18 * (2 * c)));
-        ex.dw[2 * c + 1][j] = half_bits_to_float(*(const uint16_t *)(wl + 18 * (2 * c + 1)));
-        wave_lds_fence();
-        float4 dq[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) dq[t] = *(const float4 *)&ex.dw[t][4 * c];
+        for (int h = 0; h < 2; ++h) {
+            ex.dw[2 * c + h][j] = half_bits_to_float(*(const uint16_t *)(wl + BYTES * (2 * c + h)));
+            if (HAS_MIN) ex.mw[2 * c + h][j] = half_bits_to_float(*(const uint16_t *)(wl + BYTES * (2 * c + h) + 2));
+        }
+        wave_lds_fence();
+        float4 dq[8], mq[HAS_MIN ? 8 : 1];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            dq[t] = *(const float4 *)&ex.dw[t][4 * c];
+            if (HAS_MIN) mq[t] = *(const float4 *)&ex.mw[t][4 * c];
+        }
         wave_lds_fence();  // the slots are rewritten by the next super-block
         const uint32_t M = 0x0F0F0F0Fu;
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
+            const uint8_t *blk = wl + BYTES * t;
             uint32_t lo, hi;  // values 8c .. 8c+3 and 8c+4 .. 8c+7 of the sub-block, one per byte
             if (GGML) {
-                const u32x2 q = *(const u32x2_a2 *)(wl + 18 * t + 2 + 8 * (c & 1));
+                const u32x2 q = *(const u32x2_a2 *)(blk + QS + 8 * (c & 1));
                 const int sh = (c >> 1) * 4;
                 lo = (q.x >> sh) & M;
                 hi = (q.y >> sh) & M;
+                if (HAS_HIGH) {
+                    uint32_t qh;
+                    __builtin_memcpy(&qh, blk + QH, 4);
+                    lo |= q5_high4(qh, 8 * c);
+                    hi |= q5_high4(qh, 8 * c + 4);
+                }
             } else {
                 uint32_t q;
-                __builtin_memcpy(&q, wl + 18 * t + 2 + 4 * c, 4);
+                __builtin_memcpy(&q, blk + QS + 4 * c, 4);
                 const uint32_t l = q & M, h = (q >> 4) & M;
                 lo = __builtin_amdgcn_perm(h, l, 0x05010400u);  // l0 h0 l1 h1
                 hi = __builtin_amdgcn_perm(h, l, 0x07030602u);  // l2 h2 l3 h3
             }
             const long afrag = (long)(((uint64_t)hi << 32) | lo);
             const float dw[4] = {dq[t].x, dq[t].y, dq[t].z, dq[t].w};
+            const float4 mt = HAS_MIN ? mq[t] : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float mw[4] = {mt.x, mt.y, mt.z, mt.w};
             int4v d[TM];
 #pragma unroll
             for (int a = 0; a < TM; ++a) {
@@ -304,13 +352,20 @@ struct TileQ4_0 {
 #pragma unroll
             for (int a = 0; a < TM; ++a) {
                 const float2 sx = s_xs[(16 * a + j) * 8 + t];
-                const float off = -8.0f * sx.y;
+                const float off = (HAS_HIGH ? -16.0f : -8.0f) * sx.y;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[a][i] += dw[i] * (sx.x * (float)d[a][i] + off);
+                for (int i = 0; i < 4; ++i) {
+                    if (HAS_MIN) acc[a][i] += dw[i] * (sx.x * (float)d[a][i]) + mw[i] * sx.y;
+                    else acc[a][i] += dw[i] * (sx.x * (float)d[a][i] + off);
+                }
             }
         }
     }
 };
+template <bool GGML> using TileQ4_0 = TileQ32<18, false, false, GGML>;
+template <bool GGML> using TileQ4_1 = TileQ32<20, true, false, GGML>;
+using TileQ5_0 = TileQ32<22, false, true, true>;
+using TileQ5_1 = TileQ32<24, true, true, true>;
 
 // ---------------------------------------------------------------------------------------------
 // LDS carve-up of k_mmq_i8 (dynamic: the K-split variant needs more than the 64 KB a static layout may take)
@@ -539,19 +594,30 @@ static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const in
 
 bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs) {
     if (((uintptr_t)qs & 15) != 0 || w->cols % 256 != 0) return false;
-    if (w->fmt == CANDY_HIP_Q4_K) return ((uintptr_t)w->data & 15) == 0;
+    if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
     // the last chunk of a Q6_K row runs 14 bytes past the block: only buffers allocated by the library
     // (which pads them) are known to have that room after the last row
     if (w->fmt == CANDY_HIP_Q6_K) return w->owned && ((uintptr_t)w->data & 1) == 0;
-    if (w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML) return ((uintptr_t)w->data & 1) == 0;
+    switch (w->fmt) {
+    case CANDY_HIP_Q8_0: case CANDY_HIP_Q4_0: case CANDY_HIP_Q4_0_GGML: case CANDY_HIP_Q4_1: case CANDY_HIP_Q4_1_GGML:
+    case CANDY_HIP_Q5_0: case CANDY_HIP_Q5_1:
+        return ((uintptr_t)w->data & 1) == 0;
+    default:
+        break;
+    }
     return false;
 }
 
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                   int64_t m, float *y) {
     if (w->fmt == CANDY_HIP_Q8_0) return launch_i8<TileQ8_0>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q5_K) return launch_i8<TileQ5K>(dev, w, qs, scales, m, y);
     if (w->fmt == CANDY_HIP_Q4_0) return launch_i8<TileQ4_0<false>>(dev, w, qs, scales, m, y);
     if (w->fmt == CANDY_HIP_Q4_0_GGML) return launch_i8<TileQ4_0<true>>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q4_1) return launch_i8<TileQ4_1<false>>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q4_1_GGML) return launch_i8<TileQ4_1<true>>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q5_0) return launch_i8<TileQ5_0>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q5_1) return launch_i8<TileQ5_1>(dev, w, qs, scales, m, y);
     return w->fmt == CANDY_HIP_Q4_K ? launch_i8<TileQ4K>(dev, w, qs, scales, m, y)
                                     : launch_i8<TileQ6K>(dev, w, qs, scales, m, y);
 }
