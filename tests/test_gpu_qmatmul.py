@@ -50,13 +50,13 @@ def test_small_batch_matches_oracle(dev, fmt, m):
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML, synth.Q6_K])
-@pytest.mark.parametrize("rows,cols", [(50, 11008), (4099, 1280), (600, 6144)])
+@pytest.mark.parametrize("rows,cols", [(50, 11008), (4099, 1280), (600, 6144), (40, 15360)])
 def test_small_batch_one_pass_per_eight_rows(dev, monkeypatch, fmt, rows, cols):
     # 3 .. 15 activation rows against long or many weight rows: one workgroup per CU holds up to eight quantized
     # rows in LDS and walks the weight rows (Q6_K: the looping kernel), or the int8 tile kernel takes the batch as
     # one 16-row tile.  The vector kernels add a lane's units in the same order as the looping kernel: same bits;
     # the tile kernel differs by f32 summation order only.  Row counts off the 16-row groups and more groups than
-    # CUs (4099 rows) are in.
+    # CUs (4099 rows) are in, and the longest row whose eight images still fit LDS (15360: 158 KB).
     w = synth.random_weight(fmt, rows, cols, seed=rows + fmt)
     q = dev.qtensor(fmt, rows, cols, w)
     for m in (3, 4, 5, 7, 8, 9, 13, 15):
