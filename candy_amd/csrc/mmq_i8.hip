@@ -367,6 +367,119 @@ template <bool GGML> using TileQ4_1 = TileQ32<20, true, false, GGML>;
 using TileQ5_0 = TileQ32<22, false, true, true>;
 using TileQ5_1 = TileQ32<24, true, true, true>;
 
+// Q2_K (84 bytes: 16 bytes of {4-bit scale, 4-bit min} per 16-value group, 64 bytes of 2-bit levels, d, dmin;
+// quantized.cu:902-935).  A 32-value sub-block spans two groups with their own scale and min, but a level times
+// its scale is at most 3 * 15 and fits the int8 operand: one MFMA contracts scale * level with the activations,
+// a second one contracts the group's min (every value of the group carries it) with them, and the rescale is
+//   acc += d * (d_x * dot) - dmin * (d_x * dot_min)
+// which is vec_dot_q2_K_q8_1 (quantized.cu:2108-2135) with the sums over the group taken by the matrix core.
+// Blocks are not a whole number of 16-byte chunks: the slot is 96 bytes and the last chunk runs 12 bytes into
+// the next block (past the tensor's end on the last row: library-owned, padded buffers only).
+struct TileQ2K {
+    static constexpr int BLOCK = 84, SLOT = 96;
+    typedef u32x4_a2 GlobalChunk;
+    struct Exchange {};
+    template <int TM>
+    static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &,
+                                                      const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        const uint8_t *wl = slice + j * pitch + SLOT * b;
+        float dw[4], mw[4];  // d and dmin of my four C rows
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t dm = *(const uint32_t *)(slice + (4 * c + i) * pitch + SLOT * b + 80);
+            dw[i] = half_bits_to_float((uint16_t)(dm & 0xFFFF));
+            mw[i] = half_bits_to_float((uint16_t)(dm >> 16));
+        }
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            const u32x2 q = *(const u32x2 *)(wl + 16 + 32 * n + 8 * c);  // levels of values 8c .. 8c+7 of four sub-blocks
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int t = 4 * n + k;
+                const uint32_t sm = wl[2 * t + (c >> 1)];  // my group's {scale, min}
+                const uint32_t sc = sm & 0xF, mn = (sm >> 4) * 0x01010101u;
+                const uint32_t lo = ((q.x >> (2 * k)) & 0x03030303u) * sc, hi = ((q.y >> (2 * k)) & 0x03030303u) * sc;
+                const long afrag = (long)(((uint64_t)hi << 32) | lo), mfrag = (long)(((uint64_t)mn << 32) | mn);
+                int4v d[TM], dm[TM];
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
+                    d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+                    dm[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(mfrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+                }
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    const float dx = s_xs[(16 * a + j) * 8 + t].x;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[a][i] += dw[i] * (dx * (float)d[a][i]) - mw[i] * (dx * (float)dm[a][i]);
+                }
+            }
+        }
+    }
+};
+
+// Q3_K (110 bytes: 32 mask bytes, 64 bytes of 2-bit levels, 12 bytes of 6-bit scales, d; quantized.cu:938-990).
+// A value is d * (scale - 32) * (level - 4) with level = two bits | mask bit << 2.  (32 - scale) * (level - 4) lies
+// in [-128, 124] and fits the int8 operand ((scale - 32) * (level - 4) would reach +128), so one MFMA per sub-block
+// contracts it with the activations and the rescale is acc -= d * (d_x * dot): vec_dot_q3_K_q8_1
+// (quantized.cu:2177-2209) with the scale folded into the operand.  The four signed bytes of a word are multiplied
+// by the group's factor as two pairs of 16-bit lanes.  Slot of 112 bytes: the last chunk runs 2 bytes into the next
+// block (library-owned, padded buffers only).
+typedef short short2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t mul_s8x4(uint32_t w, int f) {  // four signed bytes times f, products within int8
+    short2v ws;
+    __builtin_memcpy(&ws, &w, 4);
+    const short2v sh8 = {8, 8}, ff = {(short)f, (short)f};
+    const short2v pe = ((ws << sh8) >> sh8) * ff, po = (ws >> sh8) * ff;  // bytes 0 and 2, bytes 1 and 3
+    uint32_t e, o;
+    __builtin_memcpy(&e, &pe, 4);
+    __builtin_memcpy(&o, &po, 4);
+    return __builtin_amdgcn_perm(o, e, 0x06020400u);
+}
+struct TileQ3K {
+    static constexpr int BLOCK = 110, SLOT = 112;
+    typedef u32x4_a2 GlobalChunk;
+    struct Exchange {};
+    template <int TM>
+    static __device__ __forceinline__ void superblock(const uint8_t *slice, int pitch, int b, int j, int c, Exchange &,
+                                                      const int8_t *s_xq, const float2 *s_xs, float (&acc)[TM][4]) {
+        const uint8_t *wl = slice + j * pitch + SLOT * b;
+        float dw[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dw[i] = half_bits_to_float(*(const uint16_t *)(slice + (4 * c + i) * pitch + SLOT * b + 108));
+        const u32x2 hm = *(const u32x2 *)(wl + 8 * c);  // mask bytes of values 8c .. 8c+7: bit t belongs to sub-block t
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            const u32x2 q = *(const u32x2 *)(wl + 32 + 32 * n + 8 * c);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int t = 4 * n + k;
+                const int f = 32 - q3k_scale6(wl + 96, 2 * t + (c >> 1));
+                uint32_t lev[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const uint32_t raw = ((q[e] >> (2 * k)) & 0x03030303u) | (((hm[e] >> t) & 0x01010101u) << 2);  // 0 .. 7
+                    lev[e] = ((raw | 0x80808080u) - 0x04040404u) ^ 0x80808080u;                                 // - 4, bytewise
+                }
+                const uint32_t lo = mul_s8x4(lev[0], f), hi = mul_s8x4(lev[1], f);
+                const long afrag = (long)(((uint64_t)hi << 32) | lo);
+                int4v d[TM];
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    const long bfrag = *(const long *)&s_xq[(16 * a + j) * XROW + 32 * t + 8 * c];
+                    d[a] = __builtin_amdgcn_mfma_i32_16x16x32_i8(afrag, bfrag, int4v{0, 0, 0, 0}, 0, 0, 0);
+                }
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    const float dx = s_xs[(16 * a + j) * 8 + t].x;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[a][i] -= dw[i] * (dx * (float)d[a][i]);
+                }
+            }
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // LDS carve-up of k_mmq_i8 (dynamic: the K-split variant needs more than the 64 KB a static layout may take)
 template <class F, int TM, int STG, int KS>
@@ -597,7 +710,7 @@ bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs) {
     if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
     // the last chunk of a Q6_K row runs 14 bytes past the block: only buffers allocated by the library
     // (which pads them) are known to have that room after the last row
-    if (w->fmt == CANDY_HIP_Q6_K) return w->owned && ((uintptr_t)w->data & 1) == 0;
+    if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q2_K || w->fmt == CANDY_HIP_Q3_K) return w->owned && ((uintptr_t)w->data & 1) == 0;
     switch (w->fmt) {
     case CANDY_HIP_Q8_0: case CANDY_HIP_Q4_0: case CANDY_HIP_Q4_0_GGML: case CANDY_HIP_Q4_1: case CANDY_HIP_Q4_1_GGML:
     case CANDY_HIP_Q5_0: case CANDY_HIP_Q5_1:
@@ -612,6 +725,8 @@ int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
                   int64_t m, float *y) {
     if (w->fmt == CANDY_HIP_Q8_0) return launch_i8<TileQ8_0>(dev, w, qs, scales, m, y);
     if (w->fmt == CANDY_HIP_Q5_K) return launch_i8<TileQ5K>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q2_K) return launch_i8<TileQ2K>(dev, w, qs, scales, m, y);
+    if (w->fmt == CANDY_HIP_Q3_K) return launch_i8<TileQ3K>(dev, w, qs, scales, m, y);
     if (w->fmt == CANDY_HIP_Q4_0) return launch_i8<TileQ4_0<false>>(dev, w, qs, scales, m, y);
     if (w->fmt == CANDY_HIP_Q4_0_GGML) return launch_i8<TileQ4_0<true>>(dev, w, qs, scales, m, y);
     if (w->fmt == CANDY_HIP_Q4_1) return launch_i8<TileQ4_1<false>>(dev, w, qs, scales, m, y);

@@ -245,7 +245,7 @@ PROMPT_CASES = [
     ("other-formats", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=4, head_dim=64, d_ffn=1024, vocab=256,
                            max_pos=32, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q5_K, "q": synth.Q5_0, "k": synth.Q4_1, "v": synth.Q5_1, "gate": synth.Q3_K, "up": synth.Q2_K,
-      "head": synth.Q4_1_GGML, "embed": synth.Q8_K}, 21, 3e-3),  # fp16 tiles: 3e-4 per Linear, compounding over the layers
+      "head": synth.Q4_1_GGML, "embed": synth.Q8_K}, 21, 1e-3),  # every one of them on the integer-exact tiles
     ("short-prompt", dict(n_layers=2, d_model=256, n_heads=4, n_kv_heads=2, head_dim=64, d_ffn=512, vocab=128,
                           max_pos=16, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q8_0, "gate": synth.Q4_0, "head": synth.Q6_K, "embed": synth.Q4_K}, 5, 1e-3),

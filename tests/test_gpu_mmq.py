@@ -41,7 +41,7 @@ def test_tile_kernel_matches_oracle(dev, fmt, m):
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML, synth.Q4_1,
-                                 synth.Q4_1_GGML, synth.Q5_0, synth.Q5_1, synth.Q5_K])
+                                 synth.Q4_1_GGML, synth.Q5_0, synth.Q5_1, synth.Q5_K, synth.Q2_K, synth.Q3_K])
 @pytest.mark.parametrize("m", [16, 31, 32, 48, 65, 129, 300])
 @pytest.mark.parametrize("rows,cols", [(1, 256), (15, 768), (67, 1280), (130, 2304), (1030, 512)])
 def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
