@@ -15,6 +15,7 @@
 #include "blocks.h"
 #include "internal.h"
 #include "units.h"
+#include "formats_more.h"
 
 namespace candy {
 
@@ -288,32 +289,51 @@ static int balanced_rows(int rows, int cus, int hi, int lo, const char *env) {
 // has given the scratch the parts need.
 template <class U, int ITER>
 static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro, int epi) {
-    if (epi == EPI_PAIR) {
-        if constexpr (ITER <= 2) {  // two weights x 4 rows x ITER units must stay in registers
-            if (pro != PRO_RMS) return launch_fused_cfg<U, ITER, 4, 8, PRO_Q8, EPI_PAIR>(dev, a);
-            const int s = a.pair_act && a.pair_tickets ? balanced_rows(a.jobs.j[0].N, dev->num_cus, 32, 8, "CANDY_HIP_PAIR_ROWS") : 32;
-            if (s == 16) return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
-            if (s == 8) return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
-            return launch_fused_cfg<U, ITER, 4, 8, PRO_RMS, EPI_PAIR>(dev, a);
-        } else {
-            return CANDY_HIP_ERR_UNSUPPORTED;
+    // Q5_K holds 80 bytes of registers per unit: one row (pair) per wavefront, or two with the RMSNorm prologue
+    if constexpr (sizeof(typename U::W) > 48) {
+        if (epi == EPI_PAIR) {
+            if constexpr (ITER <= 2) {
+                if (pro != PRO_RMS || !a.pair_act || !a.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
+                if (balanced_rows(a.jobs.j[0].N, dev->num_cus, 16, 8, "CANDY_HIP_PAIR_ROWS") == 8)
+                    return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
+                return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
+            } else {
+                return CANDY_HIP_ERR_UNSUPPORTED;
+            }
         }
-    }
-    if (pro == PRO_RMS) {
-        if constexpr (ITER <= 2) {
-            // 16 rows per workgroup (4 x 4), or 24 (8 wavefronts x 3) where that leaves the fullest CU fewer rows
-            int rows = 0;
-            for (int i = 0; i < a.jobs.n; ++i) rows += a.jobs.j[i].N;
-            const int cus = dev->num_cus;
-            const long c16 = (long)((rows + 15) / 16 + cus - 1) / cus * 16, c24 = (long)((rows + 23) / 24 + cus - 1) / cus * 24;
-            const char *e = getenv("CANDY_HIP_RMS_ROWS");  // comparison runs
-            if (e ? atoi(e) == 24 : c24 < c16) return launch_fused_cfg<U, ITER, 3, 8, PRO_RMS, EPI_PLAIN>(dev, a);
-            return launch_fused_cfg<U, ITER, 4, 4, PRO_RMS, EPI_PLAIN>(dev, a);
-        } else {
-            return launch_fused_cfg<U, ITER, 2, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+        if (pro == PRO_RMS) {
+            if constexpr (ITER <= 2) return launch_fused_cfg<U, ITER, 2, 8, PRO_RMS, EPI_PLAIN>(dev, a);
+            else return CANDY_HIP_ERR_UNSUPPORTED;
         }
+        return launch_fused_cfg<U, ITER, 1, 4, PRO_Q8, EPI_PLAIN>(dev, a);
+    } else {
+        if (epi == EPI_PAIR) {
+            if constexpr (ITER <= 2) {  // two weights x 4 rows x ITER units must stay in registers
+                if (pro != PRO_RMS) return launch_fused_cfg<U, ITER, 4, 8, PRO_Q8, EPI_PAIR>(dev, a);
+                const int s = a.pair_act && a.pair_tickets ? balanced_rows(a.jobs.j[0].N, dev->num_cus, 32, 8, "CANDY_HIP_PAIR_ROWS") : 32;
+                if (s == 16) return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
+                if (s == 8) return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
+                return launch_fused_cfg<U, ITER, 4, 8, PRO_RMS, EPI_PAIR>(dev, a);
+            } else {
+                return CANDY_HIP_ERR_UNSUPPORTED;
+            }
+        }
+        if (pro == PRO_RMS) {
+            if constexpr (ITER <= 2) {
+                // 16 rows per workgroup (4 x 4), or 24 (8 wavefronts x 3) where that leaves the fullest CU fewer rows
+                int rows = 0;
+                for (int i = 0; i < a.jobs.n; ++i) rows += a.jobs.j[i].N;
+                const int cus = dev->num_cus;
+                const long c16 = (long)((rows + 15) / 16 + cus - 1) / cus * 16, c24 = (long)((rows + 23) / 24 + cus - 1) / cus * 24;
+                const char *e = getenv("CANDY_HIP_RMS_ROWS");  // comparison runs
+                if (e ? atoi(e) == 24 : c24 < c16) return launch_fused_cfg<U, ITER, 3, 8, PRO_RMS, EPI_PLAIN>(dev, a);
+                return launch_fused_cfg<U, ITER, 4, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+            } else {
+                return launch_fused_cfg<U, ITER, 2, 4, PRO_RMS, EPI_PLAIN>(dev, a);
+            }
+        }
+        return launch_fused_cfg<U, ITER, 1, 4, PRO_Q8, EPI_PLAIN>(dev, a);
     }
-    return launch_fused_cfg<U, ITER, 1, 4, PRO_Q8, EPI_PLAIN>(dev, a);
 }
 
 template <class U>
@@ -357,6 +377,7 @@ int launch_matvec_fused(candy_hip_device *dev, const FusedLaunch &L) {
     case CANDY_HIP_Q4_0: return launch_fused_fmt<UnitQ4_0<false>>(dev, a, pro, epi);
     case CANDY_HIP_Q4_0_GGML: return launch_fused_fmt<UnitQ4_0<true>>(dev, a, pro, epi);
     case CANDY_HIP_Q6_K: return launch_fused_fmt<UnitQ6K>(dev, a, pro, epi);
+    case CANDY_HIP_Q5_K: return launch_fused_fmt<UnitQ5K>(dev, a, pro, epi);
     default: return CANDY_HIP_ERR_UNSUPPORTED;
     }
 }

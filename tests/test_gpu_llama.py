@@ -78,6 +78,10 @@ def rel(got, want):
     ("small-mixed", dict(n_layers=3, d_model=512, n_heads=8, n_kv_heads=2, head_dim=64, d_ffn=1024, vocab=512,
                          max_pos=16, rms_eps=1e-5, rope_base=10000.0),
      {"default": synth.Q8_0, "gate": synth.Q4_0, "down": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q4_K}),
+    # Q5_K_M-like: Q5_K linears on the fused kernels' lighter shapes (one row, or row pair, per wavefront)
+    ("q5_k-q6k-down", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=4, head_dim=64, d_ffn=1536, vocab=512,
+                           max_pos=16, rms_eps=1e-5, rope_base=10000.0),
+     {"default": synth.Q5_K, "down": synth.Q6_K, "head": synth.Q6_K, "embed": synth.Q8_0}),
     # the formats without fused decode kernels: every Linear falls back to quantize + general matvec (+ add)
     ("other-formats", dict(n_layers=2, d_model=512, n_heads=8, n_kv_heads=4, head_dim=64, d_ffn=1024, vocab=512,
                            max_pos=16, rms_eps=1e-5, rope_base=10000.0),
