@@ -69,6 +69,37 @@ struct BigQ4K {
     }
 };
 
+// Q5_K: Q4_K's layout with 32 bytes of fifth bits between the header and the nibbles (quantized.cu:1044-1080):
+// bit t of byte l is the fifth bit of value l of sub-block t.
+struct BigQ5K {
+    static constexpr int BLOCK = 176;
+    struct Raw { u32x4 hdr; u32x2 qh; u32x2 q[4]; };
+    __device__ static __forceinline__ void load(const uint8_t *blk, int c, Raw &r) {
+        r.hdr = *(const u32x4 *)blk;
+        r.qh = *(const u32x2 *)(blk + 16 + c * 8);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) r.q[g] = *(const u32x2 *)(blk + 48 + g * 32 + c * 8);
+    }
+    __device__ static __forceinline__ void dequant(const Raw &r, int g, int c, half8 &o0, half8 &o1, int &k0, int &k1) {
+        uint32_t sc2, m2;
+        q4k_scale_min_pair(r.hdr.y, r.hdr.z, r.hdr.w, g, sc2, m2);
+        const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
+        const float d_lo = d * (float)(sc2 & 0xFF), d_hi = d * (float)((sc2 >> 8) & 0xFF);
+        const float m_lo = dmin * (float)(m2 & 0xFF), m_hi = dmin * (float)((m2 >> 8) & 0xFF);
+        const u32x2 q = r.q[g];
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+            const uint32_t byte = ((l < 4 ? q.x : q.y) >> (8 * (l & 3))) & 0xFF;
+            const uint32_t hb = ((l < 4 ? r.qh.x : r.qh.y) >> (8 * (l & 3))) & 0xFF;
+            o0[l] = (_Float16)(d_lo * (float)((byte & 0xF) | (((hb >> (2 * g)) & 1) << 4)) - m_lo);
+            o1[l] = (_Float16)(d_hi * (float)((byte >> 4) | (((hb >> (2 * g + 1)) & 1) << 4)) - m_hi);
+        }
+        k0 = c * 8;
+        k1 = 32 + c * 8;
+    }
+};
+
 struct BigQ6K {
     static constexpr int BLOCK = 210;
     // per half ip: ql bytes 64ip+16c..+15 (low nibbles: quarters 0/1, high nibbles: quarters 2/3) and qh bytes
@@ -335,7 +366,7 @@ static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
     static const int min_m = getenv("CANDY_HIP_MMQ_BIG_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_BIG_MIN_M")) : 256;
     if (m < min_m || w->cols % 256 != 0) return false;
-    if (w->fmt == CANDY_HIP_Q4_K) return ((uintptr_t)w->data & 15) == 0;
+    if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
     if (w->fmt == CANDY_HIP_Q6_K) return ((uintptr_t)w->data & 1) == 0;
     return false;
 }
@@ -344,6 +375,7 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                        const float *res) {
     if (w->fmt == CANDY_HIP_Q6_K) return launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
+    if (w->fmt == CANDY_HIP_Q5_K) return launch_big<BigQ5K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
     return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
 }
 
