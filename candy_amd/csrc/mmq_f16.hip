@@ -131,6 +131,52 @@ struct BigQ8_0 {
     }
 };
 
+// Q4_0: eight 18-byte blocks per "super-block" (144 bytes).  The task's 16 values of block 2g + c/2 are the two
+// nibbles of 8 consecutive bytes in candy's element order (quantized.go:85-93) or one nibble of all 16 bytes in
+// ggml's.  d * (q - 8) is exact in f32, one rounding to fp16.
+template <bool GGML>
+struct BigQ4_0 {
+    static constexpr int BLOCK = 144;
+    struct Raw { u32x4 q[4]; uint32_t d01, d23; };
+    __device__ static __forceinline__ void load(const uint8_t *blk, int c, Raw &r) {
+        uint32_t d[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint8_t *b = blk + 18 * (2 * g + (c >> 1));
+            d[g] = *(const uint16_t *)b;
+            if (GGML) {
+                r.q[g] = *(const u32x4_a2 *)(b + 2);
+            } else {
+                const u32x2 h = *(const u32x2_a2 *)(b + 2 + 8 * (c & 1));
+                r.q[g] = u32x4{h.x, h.y, 0u, 0u};
+            }
+        }
+        r.d01 = d[0] | (d[1] << 16);
+        r.d23 = d[2] | (d[3] << 16);
+    }
+    __device__ static __forceinline__ void dequant(const Raw &r, int g, int c, half8 &o0, half8 &o1, int &k0, int &k1) {
+        const uint32_t dd = g < 2 ? r.d01 : r.d23;
+        const float d = half_bits_to_float((uint16_t)((dd >> (16 * (g & 1))) & 0xFFFF));
+        const uint32_t w[4] = {r.q[g].x, r.q[g].y, r.q[g].z, r.q[g].w};
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+            int q0, q1;  // values l and 8 + l of the task's sixteen
+            if (GGML) {
+                const int sh = 4 * (c & 1);
+                q0 = (int)((w[l >> 2] >> (8 * (l & 3) + sh)) & 0xF);
+                q1 = (int)((w[2 + (l >> 2)] >> (8 * (l & 3) + sh)) & 0xF);
+            } else {
+                q0 = (int)((w[0] >> (8 * (l >> 1) + 4 * (l & 1))) & 0xF);
+                q1 = (int)((w[1] >> (8 * (l >> 1) + 4 * (l & 1))) & 0xF);
+            }
+            o0[l] = (_Float16)(d * (float)(q0 - 8));
+            o1[l] = (_Float16)(d * (float)(q1 - 8));
+        }
+        k0 = 32 * (c >> 1) + 16 * (c & 1);
+        k1 = k0 + 8;
+    }
+};
+
 struct BigQ6K {
     static constexpr int BLOCK = 210;
     // per half ip: ql bytes 64ip+16c..+15 (low nibbles: quarters 0/1, high nibbles: quarters 2/3) and qh bytes
@@ -398,7 +444,8 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
     static const int min_m = getenv("CANDY_HIP_MMQ_BIG_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_BIG_MIN_M")) : 256;
     if (m < min_m || w->cols % 256 != 0) return false;
     if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
-    if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q8_0) return ((uintptr_t)w->data & 1) == 0;
+    if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML)
+        return ((uintptr_t)w->data & 1) == 0;
     return false;
 }
 
@@ -408,6 +455,8 @@ int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const 
     if (w->fmt == CANDY_HIP_Q6_K) return launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
     if (w->fmt == CANDY_HIP_Q5_K) return launch_big<BigQ5K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
     if (w->fmt == CANDY_HIP_Q8_0) return launch_big<BigQ8_0, 128, 256, 2, 4>(dev, w, xh, m, y, res);
+    if (w->fmt == CANDY_HIP_Q4_0) return launch_big<BigQ4_0<false>, 128, 256, 2, 4>(dev, w, xh, m, y, res);
+    if (w->fmt == CANDY_HIP_Q4_0_GGML) return launch_big<BigQ4_0<true>, 128, 256, 2, 4>(dev, w, xh, m, y, res);
     return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
 }
 

@@ -52,7 +52,7 @@ def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
     want = o.qmatmul(fmt, w, rows, cols, x)
     assert got.shape == (m, rows)
     # 256 activation rows or more run on the fp16 tiles (operands rounded to fp16)
-    assert rel_err(got, want) <= (5e-4 if m >= 256 and fmt in (synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0) else 2e-5)
+    assert rel_err(got, want) <= (5e-4 if m >= 256 and fmt in (synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML) else 2e-5)
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K])
@@ -75,7 +75,7 @@ def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, 
         assert rel_err(got, whole) <= 2e-6, m
 
 
-@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0])
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML])
 @pytest.mark.parametrize("m", [256, 257, 300, 512, 700])
 @pytest.mark.parametrize("rows,cols", [(1, 256), (127, 512), (129, 1024), (300, 2304), (1030, 768), (130, 4352)])
 def test_big_fp16_tiles(dev, fmt, m, rows, cols):
