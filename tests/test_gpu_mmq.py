@@ -1,6 +1,6 @@
 """GPU parity of the batched (m >= 16) QMatMul, the MFMA tile kernels, against the CPU oracle.
-Bar: max|gpu - ref| / max|ref| <= 1e-3. The fp16 tile kernels (Q4_K / Q6_K from 256 activation rows
-up, Q8_0 / Q4_0 on wide prompt-sized grids) round their operands to fp16 and land near 3e-4;
+Bar: max|gpu - ref| / max|ref| <= 1e-3. The fp16 tile kernels (Q4_K / Q5_K / Q6_K / Q8_0 / Q4_0 from 256
+activation rows up, the 32-value formats on wide prompt-sized grids) round their operands to fp16 and land near 3e-4;
 the Q4_K / Q6_K / Q8_0 / Q4_0 int8 kernel multiplies integers on the matrix cores and differs from the oracle's
 integer dots only by f32 summation order, so it is held to 2e-5."""
 import numpy as np
