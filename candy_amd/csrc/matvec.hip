@@ -23,22 +23,24 @@
 
 namespace candy {
 
+// m <= NB rows exist; the images past them are copies of row m - 1 (their results are not stored)
 template <int NB, int THREADS>
 __device__ __forceinline__ void stage_activations(const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs,
-                                                  int K, uint8_t *smem, int8_t *&sq, Q8Scale *&ss) {
+                                                  int K, int m, uint8_t *smem, int8_t *&sq, Q8Scale *&ss) {
     const int q_bytes = skewed(K);  // per activation row, a multiple of 16
     sq = (int8_t *)smem;
     ss = (Q8Scale *)(smem + NB * q_bytes);
     const int chunks = K >> 4;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        const uint4 *src = (const uint4 *)(xq + (size_t)nb * K);
+        const int row = min(nb, m - 1);
+        const uint4 *src = (const uint4 *)(xq + (size_t)row * K);
         uint4 *dst = (uint4 *)(sq + nb * q_bytes);
         for (int c = threadIdx.x; c < chunks; c += THREADS) dst[c + (c >> 4)] = src[c];
+        const uint2 *s2 = (const uint2 *)xs + (size_t)row * (K >> 5);
+        uint2 *d2 = (uint2 *)ss + (size_t)nb * (K >> 5);
+        for (int i = threadIdx.x; i < (K >> 5); i += THREADS) d2[i] = s2[i];
     }
-    const uint2 *s2 = (const uint2 *)xs;
-    uint2 *d2 = (uint2 *)ss;
-    for (int i = threadIdx.x; i < NB * (K >> 5); i += THREADS) d2[i] = s2[i];
     __syncthreads();
 }
 
@@ -203,11 +205,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1_span(const MatvecJobs jo
 template <class U, int NB, int R, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
                                                        const Q8Scale *__restrict__ xs, float *__restrict__ y,
-                                                       int N, int K) {
+                                                       int N, int K, int m) {
     extern __shared__ __align__(16) uint8_t smem[];
     int8_t *sq;
     Q8Scale *ss;
-    stage_activations<NB, WAVES * 64>(xq, xs, K, smem, sq, ss);
+    stage_activations<NB, WAVES * 64>(xq, xs, K, m, smem, sq, ss);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int row0 = (blockIdx.x * WAVES + wave) * R;
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             const float v = wave_sum(acc[r][nb]);
-            if (lane == 0 && row0 + r < N) y[(size_t)nb * N + row0 + r] = v;
+            if (lane == 0 && row0 + r < N && nb < m) y[(size_t)nb * N + row0 + r] = v;
         }
 }
 
@@ -467,7 +469,7 @@ static int launch_mb(candy_hip_device *dev, const candy_hip_qtensor *w, const in
 
 template <class U, int NB, int R, int WAVES>
 static int launch_one(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                      float *y) {
+                      float *y, int m = NB) {
     const int N = (int)w->rows, K = (int)w->cols;
     const size_t q_bytes = (size_t)K + (((size_t)K >> 8) << 4);
     const size_t smem = NB * (q_bytes + (size_t)(K >> 5) * sizeof(Q8Scale));
@@ -475,9 +477,19 @@ static int launch_one(candy_hip_device *dev, const candy_hip_qtensor *w, const i
     const int rows_per_wg = R * WAVES;
     const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
     hipLaunchKernelGGL((k_matvec<U, NB, R, WAVES>), dim3(grid), dim3(WAVES * 64), smem, dev->stream,
-                       (const uint8_t *)w->data, qs, scales, y, N, K);
+                       (const uint8_t *)w->data, qs, scales, y, N, K, m);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
+}
+
+// Activation images per launch of the looping kernel: the smallest of 1, 2, 4, 8 that covers what is left (three rows
+// ride in a four-image launch, the fourth image a copy nobody stores), capped so that the images stay under 64 KB
+// of LDS.
+static int looping_rows(int64_t left, int64_t K) {
+    const int cap = K <= 5632 ? 8 : K <= 11264 ? 4 : K <= 16384 ? 2 : 1;
+    int nb = 1;
+    while (nb < left && nb < cap) nb <<= 1;
+    return nb;
 }
 
 template <class U>
@@ -503,11 +515,11 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
         float *yo = y + done * N;
         int rc;
         {
-            // The looping kernel below takes 8, 4, 2 or 1 rows per launch (fewer the longer the row is); where that
+            // The looping kernel below takes up to 8, 4, 2 or 1 rows per launch (fewer the longer the row is); where that
             // covers what is left in as few launches as this kernel's 8 per pass, it is as fast or a little faster
             // (short rows, up to about 16K of them), and two rows cost less there than as half of a 4-row pass.
             int old_launches = 0;
-            for (int64_t l = left; l > 0; ++old_launches) l -= (l >= 8 && K <= 5632) ? 8 : (l >= 4 && K <= 11264) ? 4 : (l >= 2 && K <= 16384) ? 2 : 1;
+            for (int64_t l = left; l > 0; ++old_launches) l -= std::min<int64_t>(l, looping_rows(l, K));
             const bool old_is_fine = left == 2 || (K <= 5632 && N <= 16384 && old_launches == (left + 7) / 8);
             if (left >= 2 && !old_small && !old_is_fine) {  // up to 8 rows per pass, or 4 where 8 do not fit LDS
                 const int take = (int)std::min<int64_t>(left, mb_lds_bytes(8, K) <= MB_LDS_MAX ? 8 : 4);
@@ -516,12 +528,15 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
                 if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
             }
         }
-        // LDS holds NB activation rows; keep the workgroup's share under 64 KB
-        if (left >= 8 && K <= 5632) { rc = launch_one<U, 8, 2, 4>(dev, w, q, s, yo); done += 8; }
-        else if (left >= 4 && K <= 11264) { rc = launch_one<U, 4, 2, 4>(dev, w, q, s, yo); done += 4; }
-        else if (left >= 2 && K <= 16384) { rc = launch_one<U, 2, 2, 4>(dev, w, q, s, yo); done += 2; }
-        else { rc = launch_one<U, 1, 2, 4>(dev, w, q, s, yo); done += 1; }
+        const int nb = looping_rows(left, K), take = (int)std::min<int64_t>(left, nb);
+        switch (nb) {
+        case 8: rc = launch_one<U, 8, 2, 4>(dev, w, q, s, yo, take); break;
+        case 4: rc = launch_one<U, 4, 2, 4>(dev, w, q, s, yo, take); break;
+        case 2: rc = launch_one<U, 2, 2, 4>(dev, w, q, s, yo, take); break;
+        default: rc = launch_one<U, 1, 2, 4>(dev, w, q, s, yo, take); break;
+        }
         if (rc) return rc;
+        done += take;
     }
     return CANDY_HIP_OK;
 }
