@@ -591,14 +591,14 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
     if (m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q5_K) && mmq_i8_covers(w, qs)) {
         // 5 .. 15 rows: the vector kernels below (one or two passes of up to 8 rows) or one pass of the int8 tile
         // kernel with a 16-row tile, whichever a fit to measurements on this chip says is shorter, in us.  The tile
-        // kernel's time hardly depends on m: Q4_K 4096x4096 14.7, 11008x4096 19.2, 4096x11008 21.5, 32000x4096 39;
-        // Q6_K 14.1, 25.4, 23.3, 49.5 (short rows: a few us per super-block); the vector kernels' follows rows x
+        // kernel's time hardly depends on m: Q4_K 4096x4096 12.7, 11008x4096 19.6, 4096x11008 19.3, 32000x4096 31.5;
+        // Q6_K 14.0, 23.2, 21.5, 41.3 (short rows: a few us per super-block); the vector kernels' follows rows x
         // columns x batch.
         const bool q6 = w->fmt != CANDY_HIP_Q4_K;  // Q6_K and Q5_K: the looping vector kernel, a heavier tile
         const double nsb = (double)(w->cols >> 8), mnk = (double)w->rows * (double)w->cols * 1e-6;
         const int m_pad = q6 ? (int)m : (int)((m + 3) / 4 * 4);
-        const double t_tiles = q6 ? std::min(3.5 + 2.5 * nsb * (1.0 + mnk / 40.0), 11.0 + 0.29 * mnk)
-                                  : std::min(3.5 + 2.0 * nsb * (1.0 + mnk / 40.0), 11.5 + 0.21 * mnk);
+        const double t_tiles = q6 ? std::min(3.5 + 2.5 * nsb * (1.0 + mnk / 40.0), 11.5 + 0.23 * mnk)
+                                  : std::min(3.5 + 2.0 * nsb * (1.0 + mnk / 40.0), 11.0 + 0.16 * mnk);
         const double t_vector = 4.0 + (m > 8 ? 2.0 : 0.0) + (q6 ? 0.1 : 0.052) * mnk * m_pad;
         const char *e = getenv("CANDY_HIP_I8_MIN_M");  // comparison runs: tiles from this batch size on
         if (e ? m >= atoi(e) : t_tiles < t_vector) return launch_mmq_i8(dev, w, qs, scales, m, y);

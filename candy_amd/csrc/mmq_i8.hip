@@ -664,7 +664,6 @@ static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const in
                      int64_t m, float *y) {
     const int N = (int)w->rows, K = (int)w->cols, M = (int)m;
     const unsigned gx = (unsigned)((N + 63) / 64);
-    constexpr int DEEP = F::SLOT == 144 ? 4 : 2;  // super-blocks per stage where m is small (LDS budget)
 #define CANDY_MMQ_I8(TMV, STGV, KSV)                                                                            \
     do {                                                                                                        \
         constexpr int lds = MmqI8Lds<F, TMV, STGV, KSV>::BYTES;                                                 \
@@ -688,17 +687,17 @@ static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const in
                            (const uint8_t *)w->data, qs, scales, out, N, M, K, sb_split);                         \
     } while (0)
     // Tile height: 64 activation rows per workgroup from 33 rows on (a weight fragment serves four MFMAs), 16 below
-    // that; where the grid is at most one wavefront per SIMD the launch macro splits K over workgroups, and for at
-    // most 16 rows on such a grid the workgroup has eight wavefronts that split K among themselves first.  Measured
-    // on 4096x11008, 11008x4096, 4096x4096 and 14336x4096 at 16 .. 192 rows; 32-row tiles won nowhere.
-    static const bool no_ks = getenv("CANDY_HIP_MMQ_I8_NO_KSPLIT") != nullptr;
+    // that; one super-block per stage and four wavefronts per workgroup throughout.  Where the grid is at most one
+    // wavefront per SIMD the launch macro splits K over workgroups.  Measured on 4096x11008, 11008x4096, 4096x4096
+    // and 14336x4096 at 8 .. 255 rows for Q4_K, Q6_K and Q8_0: deeper stages (2 or 4 super-blocks in flight per
+    // wavefront) and a K split inside an eight-wavefront workgroup, both of which helped before the split over
+    // workgroups existed, now cost 1-10 % (Q6_K at 64-row tiles: 25 %); 32-row tiles won nowhere.
     const bool no_gs = getenv("CANDY_HIP_MMQ_I8_NO_GRID_SPLIT") != nullptr;  // comparison runs and tests
     const int nsb = K >> 8;
     int n_split = 1, sb_split = nsb;
     float *out = y;
-    if (M > 32) CANDY_MMQ_I8(4, 2, 1);
-    else if (M <= 16 && !no_ks && (int64_t)gx < 2 * dev->num_cus && nsb >= 2 * DEEP) CANDY_MMQ_I8(1, DEEP, 2);
-    else CANDY_MMQ_I8(1, DEEP, 1);
+    if (M > 32) CANDY_MMQ_I8(4, 1, 1);
+    else CANDY_MMQ_I8(1, 1, 1);
 #undef CANDY_MMQ_I8
     CANDY_LAUNCH_CHECK();
     if (n_split > 1) return launch_splitk_sum(dev, out, y, nullptr, (size_t)M * N, n_split);
