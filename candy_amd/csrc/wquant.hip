@@ -7,8 +7,9 @@
 // blocks come out bit for bit as a CPU evaluation of the same steps gives them.  This file is compiled
 // with -ffp-contract=off for that reason (a fused multiply-add rounds once where the steps round twice).
 //
-// A load-time operation: one thread per block (32 values) or super-block (256 values), the candidate
-// search of the K formats running serially in that thread.  Inputs must be finite.
+// A load-time operation: one thread per block of 32 values (Q4_0, and the sub-blocks of Q4_K, whose eight
+// lanes settle the super-block's header with shuffles) or per super-block (Q6_K), the candidate search
+// running serially in that thread.  Inputs must be finite.
 #include "blocks.h"
 #include "internal.h"
 
@@ -68,9 +69,10 @@ __global__ __launch_bounds__(256) void k_wquant_q4_0(const float *__restrict__ x
 // rdelta 0.1, 20 steps, squared error): min/max rounding first, then 21 nearby scales, each followed by
 // the weighted least-squares fit of (scale, min) to the levels it yields; the best weighted error wins.
 // Returns the scale; neg_min receives -min.
-__device__ float search_affine32(const float *x, const float *w, uint8_t *L, float &neg_min) {
+__device__ __forceinline__ float search_affine32(const float (&x)[32], const float (&w)[32], int (&L)[32], float &neg_min) {
     float lo = x[0], hi = x[0];
     float sum_w = w[0], sum_x = sum_w * x[0];
+#pragma unroll
     for (int i = 1; i < 32; ++i) {
         if (x[i] < lo) lo = x[i];
         if (x[i] > hi) hi = x[i];
@@ -79,6 +81,7 @@ __device__ float search_affine32(const float *x, const float *w, uint8_t *L, flo
     }
     if (lo > 0.0f) lo = 0.0f;
     if (hi == lo) {
+#pragma unroll
         for (int i = 0; i < 32; ++i) L[i] = 0;
         neg_min = -lo;
         return 0.0f;
@@ -86,20 +89,23 @@ __device__ float search_affine32(const float *x, const float *w, uint8_t *L, flo
     float iscale = 15.0f / (hi - lo);
     float scale = 1.0f / iscale;
     float best = 0.0f;
+#pragma unroll
     for (int i = 0; i < 32; ++i) {
         const int l = clampi(rne_int(iscale * (x[i] - lo)), 0, 15);
-        L[i] = (uint8_t)l;
+        L[i] = l;
         float diff = scale * (float)l + lo - x[i];
         diff = diff * diff;
         best += w[i] * diff;
     }
-    uint8_t cand[32];
+    int cand[32];
+#pragma unroll 1
     for (int is = 0; is <= 20; ++is) {
-        iscale = (-1.0f + 0.1f * (float)is + 15.0f) / (hi - lo);
+        iscale = (-1.0f + 0.1f * (float)is + 15.0f) / (hi - lo);  // lo: the best minimum so far
         float sum_l = 0.0f, sum_l2 = 0.0f, sum_xl = 0.0f;
+#pragma unroll
         for (int i = 0; i < 32; ++i) {
             const int l = clampi(rne_int(iscale * (x[i] - lo)), 0, 15);
-            cand[i] = (uint8_t)l;
+            cand[i] = l;
             sum_l += w[i] * (float)l;
             sum_l2 += w[i] * (float)l * (float)l;
             sum_xl += w[i] * (float)l * x[i];
@@ -113,12 +119,14 @@ __device__ float search_affine32(const float *x, const float *w, uint8_t *L, flo
                 s = sum_xl / sum_l2;
             }
             float err = 0.0f;
+#pragma unroll
             for (int i = 0; i < 32; ++i) {
                 float diff = s * (float)cand[i] + m - x[i];
                 diff = diff * diff;
                 err += w[i] * diff;
             }
             if (err < best) {
+#pragma unroll
                 for (int i = 0; i < 32; ++i) L[i] = cand[i];
                 best = err;
                 scale = s;
@@ -130,56 +138,82 @@ __device__ float search_affine32(const float *x, const float *w, uint8_t *L, flo
     return scale;
 }
 
-// One super-block: per-sub-block (scale, min) with weights rms + |x|, both stored in 6 bits relative to
-// their maxima (d, dmin in fp16, packed as get_scale_min_k4 of quantized.cu:993-1005 unpacks them), then
-// the levels assigned again with the STORED scales (a sub-block whose stored scale is 0 keeps the search's).
-__global__ __launch_bounds__(64) void k_wquant_q4_k(const float *__restrict__ x, int64_t nb, BlockQ4K *__restrict__ out) {
-    const int64_t b = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (b >= nb) return;
-    const float *xb = x + 256 * b;
-    uint8_t L[256];
-    float scales[8], mins[8];
-    float max_scale = 0.0f, max_min = 0.0f;
-    for (int j = 0; j < 8; ++j) {
-        float xs[32], w[32];
-        float sum_x2 = 0.0f;
-        for (int l = 0; l < 32; ++l) {
-            xs[l] = xb[32 * j + l];
-            sum_x2 += xs[l] * xs[l];
+// One super-block per eight neighbouring lanes, one 32-value sub-block per lane (values, weights and levels
+// in registers): per-sub-block (scale, min) with weights rms + |x|, both stored in 6 bits relative to their
+// maxima over the eight lanes (d, dmin in fp16, packed as get_scale_min_k4 of quantized.cu:993-1005 unpacks
+// them), then the levels assigned again with the STORED scales (a sub-block whose stored scale is 0 keeps the
+// search's).  Lanes past the last super-block work on zeros and store nothing, so every shuffle is full.
+__global__ __launch_bounds__(256) void k_wquant_q4_k(const float *__restrict__ x, int64_t nb, BlockQ4K *__restrict__ out) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = t >> 3;
+    const int j = (int)(t & 7);
+    const bool live = b < nb;
+    float xs[32], w[32];
+    {
+        const float4 *src = (const float4 *)(x + 256 * b + 32 * j);
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+            const float4 v = live ? src[l] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            xs[4 * l] = v.x, xs[4 * l + 1] = v.y, xs[4 * l + 2] = v.z, xs[4 * l + 3] = v.w;
         }
-        const float av = sqrtf(sum_x2 / 32.0f);
-        for (int l = 0; l < 32; ++l) w[l] = av + fabsf(xs[l]);
-        scales[j] = search_affine32(xs, w, L + 32 * j, mins[j]);
-        if (scales[j] > max_scale) max_scale = scales[j];
-        if (mins[j] > max_min) max_min = mins[j];
     }
+    float sum_x2 = 0.0f;
+#pragma unroll
+    for (int l = 0; l < 32; ++l) sum_x2 += xs[l] * xs[l];
+    const float av = sqrtf(sum_x2 / 32.0f);
+#pragma unroll
+    for (int l = 0; l < 32; ++l) w[l] = av + fabsf(xs[l]);
+    int L[32];
+    float neg_min;
+    const float scale = search_affine32(xs, w, L, neg_min);
+    float max_scale = scale, max_min = neg_min;
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) {
+        max_scale = fmaxf(max_scale, __shfl_xor(max_scale, o));
+        max_min = fmaxf(max_min, __shfl_xor(max_min, o));
+    }
+    if (!(max_scale > 0.0f)) max_scale = 0.0f;  // the serial maximum starts from +0
+    if (!(max_min > 0.0f)) max_min = 0.0f;
     const float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
     const float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
-    uint8_t sc6[8], mn6[8], packed[12];
-    for (int j = 0; j < 8; ++j) {
-        const int ls = rne_int(inv_scale * scales[j]), lm = rne_int(inv_min * mins[j]);
-        sc6[j] = (uint8_t)(ls < 63 ? ls : 63);
-        mn6[j] = (uint8_t)(lm < 63 ? lm : 63);
-    }
-    for (int j = 0; j < 4; ++j) {
-        packed[j] = (uint8_t)(sc6[j] | ((sc6[j + 4] >> 4) << 6));
-        packed[j + 4] = (uint8_t)(mn6[j] | ((mn6[j + 4] >> 4) << 6));
-        packed[j + 8] = (uint8_t)((sc6[j + 4] & 0xF) | ((mn6[j + 4] & 0xF) << 4));
-    }
-    BlockQ4K *y = out + b;
+    const int ls = rne_int(inv_scale * scale), lm = rne_int(inv_min * neg_min);
+    const int sc6 = ls < 63 ? ls : 63, mn6 = lm < 63 ? lm : 63;
+    const int sc6_hi = __shfl_down(sc6, 4), mn6_hi = __shfl_down(mn6, 4);  // lanes 0-3: sub-block j + 4
     const uint16_t dh = f32_to_half_bits(max_scale / 63.0f), mh = f32_to_half_bits(max_min / 63.0f);
-    y->d = dh;
-    y->dmin = mh;
-    for (int j = 0; j < 12; ++j) y->scales[j] = packed[j];
-    const float df = half_bits_to_float(dh), mf = half_bits_to_float(mh);
-    for (int j = 0; j < 8; ++j) {
-        const float d = df * (float)sc6[j];
-        if (d == 0.0f) continue;
-        const float dm = mf * (float)mn6[j];
-        for (int i = 0; i < 32; ++i) L[32 * j + i] = (uint8_t)clampi(rne_int((xb[32 * j + i] + dm) / d), 0, 15);
+    BlockQ4K *y = out + b;
+    if (live && j < 4) {
+        y->scales[j] = (uint8_t)(sc6 | ((sc6_hi >> 4) << 6));
+        y->scales[j + 4] = (uint8_t)(mn6 | ((mn6_hi >> 4) << 6));
+        y->scales[j + 8] = (uint8_t)((sc6_hi & 0xF) | ((mn6_hi & 0xF) << 4));
     }
-    for (int g = 0; g < 4; ++g)
-        for (int l = 0; l < 32; ++l) y->qs[32 * g + l] = (uint8_t)(L[64 * g + l] | (L[64 * g + 32 + l] << 4));
+    if (live && j == 0) {
+        y->d = dh;
+        y->dmin = mh;
+    }
+    const float d = half_bits_to_float(dh) * (float)sc6;
+    if (d != 0.0f) {
+        const float dm = half_bits_to_float(mh) * (float)mn6;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) L[i] = clampi(rne_int((xs[i] + dm) / d), 0, 15);
+    }
+    // Byte l of a 64-value group = level l of its even sub-block | level l of the odd one << 4: the two lanes
+    // exchange their levels, four to a word, and each stores 16 of the 32 bytes.
+    uint32_t mine[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mine[i] = (uint32_t)(L[4 * i] | (L[4 * i + 1] << 8) | (L[4 * i + 2] << 16) | (L[4 * i + 3] << 24));
+    const int odd = j & 1;
+    uint16_t *dst = (uint16_t *)(y->qs + 32 * (j >> 1) + 16 * odd);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t give = odd ? mine[i] : mine[4 + i];       // the half the other lane stores
+        const uint32_t keep = odd ? mine[4 + i] : mine[i];
+        const uint32_t got = (uint32_t)__shfl_xor((int)give, 1);
+        const uint32_t word = odd ? (got | (keep << 4)) : (keep | (got << 4));
+        if (live) {
+            dst[2 * i] = (uint16_t)word;
+            dst[2 * i + 1] = (uint16_t)(word >> 16);
+        }
+    }
 }
 
 // ------------------------------------------------------------------ Q6_K
@@ -292,7 +326,7 @@ int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64
     CANDY_REQUIRE(((uintptr_t)dev_out_blocks & 1) == 0, "output blocks must be 2-byte aligned");
     if (int rc = use_device(dev)) return rc;
     const int64_t nb = rows * cols / qk;
-    const int per = qk == 32 ? 256 : 64;
+    const int per = qk == 32 ? 256 : (fmt == CANDY_HIP_Q4_K ? 32 : 64);
     const int64_t grid = (nb + per - 1) / per;
     CANDY_REQUIRE(grid <= 0x7FFFFFFF, "matrix too large");
     switch (fmt) {
@@ -302,7 +336,7 @@ int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64
                            (BlockQ4_0 *)dev_out_blocks, fmt == CANDY_HIP_Q4_0_GGML ? 1 : 0);
         break;
     case CANDY_HIP_Q4_K:
-        hipLaunchKernelGGL(k_wquant_q4_k, dim3((unsigned)grid), dim3(64), 0, dev->stream, dev_x, nb, (BlockQ4K *)dev_out_blocks);
+        hipLaunchKernelGGL(k_wquant_q4_k, dim3((unsigned)grid), dim3(256), 0, dev->stream, dev_x, nb, (BlockQ4K *)dev_out_blocks);
         break;
     case CANDY_HIP_Q6_K:
         hipLaunchKernelGGL(k_wquant_q6_k, dim3((unsigned)grid), dim3(64), 0, dev->stream, dev_x, nb, (BlockQ6K *)dev_out_blocks);
