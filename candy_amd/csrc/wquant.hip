@@ -8,8 +8,8 @@
 // with -ffp-contract=off for that reason (a fused multiply-add rounds once where the steps round twice).
 //
 // A load-time operation: one thread per block of 32 values (Q4_0, and the sub-blocks of Q4_K, whose eight
-// lanes settle the super-block's header with shuffles) or per super-block (Q6_K), the candidate search
-// running serially in that thread.  Inputs must be finite.
+// lanes settle the super-block's header with shuffles) or of 16 (Q6_K's groups), the candidate search running
+// serially in that thread.  Inputs must be finite.
 #include "blocks.h"
 #include "internal.h"
 
@@ -220,40 +220,48 @@ __global__ __launch_bounds__(256) void k_wquant_q4_k(const float *__restrict__ x
 // Symmetric levels -32..31 for 16 values (make_qx_quants, weights x^2): the value of largest magnitude
 // maps to -32, then 18 nearby scales are tried and the largest (sum w x l)^2 / (sum w l^2) wins.
 // L receives level + 32.
-__device__ float search_symmetric16(const float *x, int8_t *L) {
+__device__ __forceinline__ float search_symmetric16(const float (&x)[16], int (&L)[16]) {
     float vmax = 0.0f, amax = 0.0f;
+#pragma unroll
     for (int i = 0; i < 16; ++i) {
         const float a = fabsf(x[i]);
         if (a > amax) { amax = a; vmax = x[i]; }
     }
     if (amax < 1e-15f) {
+#pragma unroll
         for (int i = 0; i < 16; ++i) L[i] = 0;
         return 0.0f;
     }
     float iscale = -32.0f / vmax;
     float sumlx = 0.0f, suml2 = 0.0f;
+#pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int l = clampi(rne_int(iscale * x[i]), -32, 31);
-        L[i] = (int8_t)(l + 32);
+        L[i] = l + 32;
         const float w = x[i] * x[i];
         sumlx += w * x[i] * (float)l;
         suml2 += w * (float)l * (float)l;
     }
     float scale = suml2 != 0.0f ? sumlx / suml2 : 0.0f;
     float best = scale * sumlx;
+#pragma unroll 1
     for (int is = -9; is <= 9; ++is) {
         if (is == 0) continue;
         iscale = -(32.0f + 0.1f * (float)is) / vmax;
         sumlx = 0.0f;
         suml2 = 0.0f;
+        int cand[16];
+#pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int l = clampi(rne_int(iscale * x[i]), -32, 31);
+            cand[i] = l + 32;
             const float w = x[i] * x[i];
             sumlx += w * x[i] * (float)l;
             suml2 += w * (float)l * (float)l;
         }
         if (suml2 > 0.0f && sumlx * sumlx > best * suml2) {
-            for (int i = 0; i < 16; ++i) L[i] = (int8_t)(32 + clampi(rne_int(iscale * x[i]), -32, 31));
+#pragma unroll
+            for (int i = 0; i < 16; ++i) L[i] = cand[i];
             scale = sumlx / suml2;
             best = scale * sumlx;
         }
@@ -261,52 +269,80 @@ __device__ float search_symmetric16(const float *x, int8_t *L) {
     return scale;
 }
 
-// One super-block: sixteen group scales, the one of largest magnitude mapping to -128 in int8 (d in
-// fp16 keeps its sign), levels assigned again with the STORED scales, packed as quantized.cu:1103-1128
-// reads them (ql: low nibbles of two quarters per byte, qh: the two high bits of four quarters).
-__global__ __launch_bounds__(64) void k_wquant_q6_k(const float *__restrict__ x, int64_t nb, BlockQ6K *__restrict__ out) {
-    const int64_t b = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (b >= nb) return;
-    const float *xb = x + 256 * b;
-    int8_t L[256];
-    float scales[16];
-    float max_scale = 0.0f, max_abs = 0.0f;
-    for (int g = 0; g < 16; ++g) {
-        float xs[16];
-        for (int i = 0; i < 16; ++i) xs[i] = xb[16 * g + i];
-        const float s = search_symmetric16(xs, L + 16 * g);
-        scales[g] = s;
-        if (fabsf(s) > max_abs) { max_abs = fabsf(s); max_scale = s; }
-    }
-    BlockQ6K *y = out + b;
-    if (max_abs < 1e-15f) {
-        uint16_t *z = (uint16_t *)y;  // 210 bytes, 2-byte aligned
-        for (int i = 0; i < 105; ++i) z[i] = 0;
-        return;
-    }
-    const float iscale = -128.0f / max_scale;
-    const uint16_t dh = f32_to_half_bits(1.0f / iscale);
-    int8_t sc8[16];
-    for (int g = 0; g < 16; ++g) {
-        const int v = rne_int(iscale * scales[g]);
-        sc8[g] = (int8_t)(v < 127 ? v : 127);
-    }
-    const float df = half_bits_to_float(dh);
-    for (int g = 0; g < 16; ++g) {
-        const float d = df * (float)sc8[g];
-        if (d == 0.0f) continue;
-        for (int i = 0; i < 16; ++i) L[16 * g + i] = (int8_t)(clampi(rne_int(xb[16 * g + i] / d), -32, 31) + 32);
-    }
-    y->d = dh;
-    for (int g = 0; g < 16; ++g) y->scales[g] = sc8[g];
-    for (int h = 0; h < 2; ++h)
-        for (int l = 0; l < 32; ++l) {
-            const uint32_t a0 = (uint8_t)L[128 * h + l], a1 = (uint8_t)L[128 * h + 32 + l];
-            const uint32_t a2 = (uint8_t)L[128 * h + 64 + l], a3 = (uint8_t)L[128 * h + 96 + l];
-            y->ql[64 * h + l] = (uint8_t)((a0 & 0xF) | ((a2 & 0xF) << 4));
-            y->ql[64 * h + 32 + l] = (uint8_t)((a1 & 0xF) | ((a3 & 0xF) << 4));
-            y->qh[32 * h + l] = (uint8_t)((a0 >> 4) | ((a1 >> 4) << 2) | ((a2 >> 4) << 4) | ((a3 >> 4) << 6));
+// One super-block per sixteen neighbouring lanes, one 16-value group per lane: sixteen group scales, the
+// first of largest magnitude mapping to -128 in int8 (d in fp16 keeps its sign), levels assigned again with
+// the STORED scales, handed over through LDS and packed as quantized.cu:1103-1128 reads them (ql: low
+// nibbles of two quarters per byte, qh: the two high bits of four quarters), each lane storing 8 bytes of
+// ql, 4 of qh and its scale.  Lanes past the last super-block work on zeros and store nothing.
+__global__ __launch_bounds__(256) void k_wquant_q6_k(const float *__restrict__ x, int64_t nb, BlockQ6K *__restrict__ out) {
+    __shared__ __align__(16) uint8_t s_levels[16][256];
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t b = t >> 4;
+    const int g = (int)(t & 15);
+    const bool live = b < nb;
+    float xs[16];
+    {
+        const float4 *src = (const float4 *)(x + 256 * b + 16 * g);
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const float4 v = live ? src[l] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            xs[4 * l] = v.x, xs[4 * l + 1] = v.y, xs[4 * l + 2] = v.z, xs[4 * l + 3] = v.w;
         }
+    }
+    int L[16];
+    const float scale = search_symmetric16(xs, L);
+    float max_abs = fabsf(scale), max_scale = scale;
+    int max_at = g;
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+        const float oa = __shfl_xor(max_abs, o), os = __shfl_xor(max_scale, o);
+        const int oi = __shfl_xor(max_at, o);
+        if (oa > max_abs || (oa == max_abs && oi < max_at)) max_abs = oa, max_scale = os, max_at = oi;
+    }
+    const bool zero = max_abs < 1e-15f;  // the whole super-block is stored as zero bytes
+    const float iscale = -128.0f / max_scale;
+    const uint16_t dh = zero ? (uint16_t)0 : f32_to_half_bits(1.0f / iscale);
+    const int v = rne_int(iscale * scale);
+    const int sc8 = zero ? 0 : (int)(int8_t)(v < 127 ? v : 127);
+    const float d = half_bits_to_float(dh) * (float)sc8;
+    if (d != 0.0f) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) L[i] = clampi(rne_int(xs[i] / d), -32, 31) + 32;
+    }
+    uint8_t *mine = s_levels[threadIdx.x >> 4];
+    {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            w[i] = (uint32_t)(L[4 * i] | (L[4 * i + 1] << 8) | (L[4 * i + 2] << 16) | (L[4 * i + 3] << 24));
+            if (zero) w[i] = 0;
+        }
+        *(uint4 *)(mine + 16 * g) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    __syncthreads();
+    if (!live) return;
+    BlockQ6K *y = out + b;
+    if (g == 0) y->d = dh;
+    y->scales[g] = (int8_t)sc8;
+    {  // ql bytes 8g .. 8g + 7: byte 64h + r = level (128h + r) low nibble | level (128h + 64 + r) low nibble << 4
+        const int h = g >> 3, r = (8 * g) & 63;
+        const uint2 lo = *(const uint2 *)(mine + 128 * h + r), hi = *(const uint2 *)(mine + 128 * h + 64 + r);
+        const uint32_t q0 = (lo.x & 0x0F0F0F0Fu) | ((hi.x & 0x0F0F0F0Fu) << 4);
+        const uint32_t q1 = (lo.y & 0x0F0F0F0Fu) | ((hi.y & 0x0F0F0F0Fu) << 4);
+        uint16_t *dst = (uint16_t *)(y->ql + 8 * g);
+        dst[0] = (uint16_t)q0, dst[1] = (uint16_t)(q0 >> 16), dst[2] = (uint16_t)q1, dst[3] = (uint16_t)(q1 >> 16);
+    }
+    {  // qh bytes 4g .. 4g + 3: byte 32h + l = bits 4-5 of levels 128h + 32q + l, q = 0..3, two bits each
+        const int h = g >> 3, l = (4 * g) & 31;
+        uint32_t q = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t a = *(const uint32_t *)(mine + 128 * h + 32 * k + l);
+            q |= ((a >> 4) & 0x03030303u) << (2 * k);
+        }
+        uint16_t *dst = (uint16_t *)(y->qh + 4 * g);
+        dst[0] = (uint16_t)q, dst[1] = (uint16_t)(q >> 16);
+    }
 }
 
 }  // namespace candy
@@ -326,7 +362,7 @@ int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64
     CANDY_REQUIRE(((uintptr_t)dev_out_blocks & 1) == 0, "output blocks must be 2-byte aligned");
     if (int rc = use_device(dev)) return rc;
     const int64_t nb = rows * cols / qk;
-    const int per = qk == 32 ? 256 : (fmt == CANDY_HIP_Q4_K ? 32 : 64);
+    const int per = qk == 32 ? 256 : (fmt == CANDY_HIP_Q4_K ? 32 : 16);
     const int64_t grid = (nb + per - 1) / per;
     CANDY_REQUIRE(grid <= 0x7FFFFFFF, "matrix too large");
     switch (fmt) {
@@ -339,7 +375,7 @@ int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64
         hipLaunchKernelGGL(k_wquant_q4_k, dim3((unsigned)grid), dim3(256), 0, dev->stream, dev_x, nb, (BlockQ4K *)dev_out_blocks);
         break;
     case CANDY_HIP_Q6_K:
-        hipLaunchKernelGGL(k_wquant_q6_k, dim3((unsigned)grid), dim3(64), 0, dev->stream, dev_x, nb, (BlockQ6K *)dev_out_blocks);
+        hipLaunchKernelGGL(k_wquant_q6_k, dim3((unsigned)grid), dim3(256), 0, dev->stream, dev_x, nb, (BlockQ6K *)dev_out_blocks);
         break;
     default: CANDY_REQUIRE(false, "no quantizer for format %d", fmt);
     }
