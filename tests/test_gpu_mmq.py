@@ -59,7 +59,7 @@ def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
 @pytest.mark.parametrize("rows,cols", [(200, 11008), (64, 4352), (1000, 2560)])
 def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, rows, cols):
     # few weight rows and a long contraction: the grid is at most one wavefront per SIMD, so K is split over
-    # workgroups (and, up to 16 rows, over the wavefronts of a workgroup first) and the copies are summed in a
+    # workgroups and the copies are summed in a
     # fixed order: the answer moves by f32 summation order only, and is the same from call to call
     w = synth.random_weight(fmt, rows, cols, seed=rows + cols + fmt)
     q = dev.qtensor(fmt, rows, cols, w)
