@@ -313,7 +313,7 @@ def main():
                    "device": dev.name},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MATVEC_TRAFFIC_BYTES,
-                     "kernel": "k_matvec<UnitQ4K>", "us_per_launch": round(ms_kernel * 1e3, 3)},
+                     "kernel": "k_matvec1<UnitQ4K,3,1,4>", "us_per_launch": round(ms_kernel * 1e3, 3)},
     }
 
     if not args.no_sweep:
@@ -410,7 +410,7 @@ def main():
             ms, _ = time_matvec(dev, synth.Q4_K, r, k, 200, 20, quantize_each=True, seed=m, m=m)
             flops = 2.0 * m * r * k
             byts = algorithmic_bytes(synth.Q4_K, r, k, m)
-            pre.append({"m": m, "kernel": "k_mmq_q4k_i8 (int8 MFMA)" if m < 256 else "k_mmq_f16<BigQ4K> (fp16 MFMA)",
+            pre.append({"m": m, "kernel": ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if m < 256 else "k_mmq_f16<BigQ4K,128,256,2,4> (fp16 MFMA)",
                         "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
                         "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
