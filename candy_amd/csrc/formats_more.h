@@ -19,8 +19,10 @@ __device__ __forceinline__ uint32_t load_u32_a2(const uint8_t *p) { return *(con
 
 // The 5th bits of four consecutive elements e0..e0+3 of a Q5_0 / Q5_1 block, moved to bit 4 of each byte.
 __device__ __forceinline__ uint32_t q5_high4(uint32_t qh, int e0) {
-    const uint32_t v = qh >> e0;
-    return ((v << 4) & 0x00000010u) | ((v << 11) & 0x00001000u) | ((v << 18) & 0x00100000u) | ((v << 25) & 0x10000000u);
+    // one 24-bit multiply copies the nibble to offsets 0, 7, 14 and 21 (no two copies of different bits meet, so
+    // nothing carries); bit i is then picked from the copy that puts it at 8i
+    const uint32_t n = (qh >> e0) & 0xFu;
+    return (__umul24(n, 0x00204081u) << 4) & 0x10101010u;
 }
 __device__ __forceinline__ int sum4_i8(uint32_t x, int acc) { return dot4_i8(0x01010101u, x, acc); }
 
