@@ -226,6 +226,8 @@ struct UnitQ3K {
         const int n = (u >> 2) & 1, j = u & 3;
         w.q = *(const u32x2_a2 *)(b->qs + 32 * n + 8 * j);
         w.h = *(const u32x2_a2 *)(b->hmask + 8 * j);
+        // eight single-byte loads: fetching the 12 scale bytes as two 8-byte loads and picking the fields with
+        // byte permutes was measured slower (4096x11008 batch 1: 14.1 against 11.6 us)
         uint32_t sc = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) sc |= (uint32_t)q3k_scale6(b->scales, 8 * n + 2 * k + (j >> 1)) << (8 * k);
