@@ -174,7 +174,8 @@ struct UnitQ6K {
         w.ql0 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 8 * j);
         w.ql1 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 32 + 8 * j);
         w.qh = *(const u32x2_a2 *)(blk->qh + 32 * ip + 8 * j);
-        // four single-byte loads: fetching the 16 scale bytes at once and permuting was measured slower
+        // four single-byte loads: fetching the 16 scale bytes at once and permuting was measured slower, and so was
+        // one 8-byte load with one v_perm_b32 picking the four (32000x4096 batch 1: 26.5 against 25.7 us)
         const int8_t *sc = blk->scales + 8 * ip + (j >> 1);
         w.sc = (uint32_t)(uint8_t)sc[0] | ((uint32_t)(uint8_t)sc[2] << 8) | ((uint32_t)(uint8_t)sc[4] << 16) |
                ((uint32_t)(uint8_t)sc[6] << 24);
