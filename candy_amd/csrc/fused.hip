@@ -265,14 +265,11 @@ static int launch_fused_cfg(candy_hip_device *dev, FusedArgs a) {
 // 16 rows (16 wavefronts x 1) 1.859, 8 rows (8 x 1) 1.855 ms per token; 4 rows 1.960; with four rows per wavefront
 // the 16-row shape is slower than whole blocks (2.036).  d_ffn 14336: 32 rows 1.983, 8 rows 1.957.  The same choice
 // for the plain RMSNorm-prologue kernel (16 or 8 rows) did not pay: 8 rows lose more to the repeated prologue than
-// the even split wins (24-row workgroups over the weights' rows as one run do).  `env` names an override for
-// comparison runs.
-static int balanced_rows(int rows, int cus, int hi, int lo, const char *env) {
-    if (const char *e = getenv(env)) {
-        const int v = atoi(e);
-        for (int s = hi; s >= lo; s >>= 1)
-            if (v == s) return s;
-    }
+// the even split wins (24-row workgroups over the weights' rows as one run do).  `forced` (the fused.pair_rows
+// option) overrides the choice for comparison runs.
+static int balanced_rows(int rows, int cus, int hi, int lo, int forced) {
+    for (int s = hi; s >= lo; s >>= 1)
+        if (forced == s) return s;
     int best = hi;
     long best_cost = -1;
     for (int s = hi; s >= lo; s >>= 1) {
@@ -294,7 +291,7 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
         if (epi == EPI_PAIR) {
             if constexpr (ITER <= 2) {
                 if (pro != PRO_RMS || !a.pair_act || !a.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
-                if (balanced_rows(a.jobs.j[0].N, dev->num_cus, 16, 8, "CANDY_HIP_PAIR_ROWS") == 8)
+                if (balanced_rows(a.jobs.j[0].N, dev->num_cus, 16, 8, dev->opt.pair_rows) == 8)
                     return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
                 return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
             } else {
@@ -310,7 +307,7 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
         if (epi == EPI_PAIR) {
             if constexpr (ITER <= 2) {  // two weights x 4 rows x ITER units must stay in registers
                 if (pro != PRO_RMS) return launch_fused_cfg<U, ITER, 4, 8, PRO_Q8, EPI_PAIR>(dev, a);
-                const int s = a.pair_act && a.pair_tickets ? balanced_rows(a.jobs.j[0].N, dev->num_cus, 32, 8, "CANDY_HIP_PAIR_ROWS") : 32;
+                const int s = a.pair_act && a.pair_tickets ? balanced_rows(a.jobs.j[0].N, dev->num_cus, 32, 8, dev->opt.pair_rows) : 32;
                 if (s == 16) return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
                 if (s == 8) return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
                 return launch_fused_cfg<U, ITER, 4, 8, PRO_RMS, EPI_PAIR>(dev, a);
@@ -325,8 +322,8 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
                 for (int i = 0; i < a.jobs.n; ++i) rows += a.jobs.j[i].N;
                 const int cus = dev->num_cus;
                 const long c16 = (long)((rows + 15) / 16 + cus - 1) / cus * 16, c24 = (long)((rows + 23) / 24 + cus - 1) / cus * 24;
-                const char *e = getenv("CANDY_HIP_RMS_ROWS");  // comparison runs
-                if (e ? atoi(e) == 24 : c24 < c16) return launch_fused_cfg<U, ITER, 3, 8, PRO_RMS, EPI_PLAIN>(dev, a);
+                const int forced = dev->opt.rms_rows;  // comparison runs
+                if (forced ? forced == 24 : c24 < c16) return launch_fused_cfg<U, ITER, 3, 8, PRO_RMS, EPI_PLAIN>(dev, a);
                 return launch_fused_cfg<U, ITER, 4, 4, PRO_RMS, EPI_PLAIN>(dev, a);
             } else {
                 return launch_fused_cfg<U, ITER, 2, 4, PRO_RMS, EPI_PLAIN>(dev, a);

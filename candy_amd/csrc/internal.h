@@ -45,10 +45,28 @@ struct Q8Scale {
     int32_t bsum;  // sum of the block's 32 quants (for the `min` term of Q4_K)
 };
 
+// Switches of one device handle, set with candy_hip_set_option (the keys are listed in runtime.hip and in
+// include/candy_hip.h).  The defaults are what the library is measured and shipped with; the others select a
+// kernel that the default dispatch would not pick, for comparison runs and for tests that want a given kernel.
+struct Options {
+    int matvec_span = 1;         // batch-1 kernel of the 2-byte aligned formats: aligned 16-byte spans through LDS
+    int small_batch_kernel = 1;  // 2..8 rows: the one-workgroup-per-CU kernel (0: the looping kernel only)
+    int i8_min_m = 0;            // 5..15 rows: int8 tiles from this batch on (0: whichever the fitted times say)
+    int mmq_min_m = 16;          // batch from which the tile kernels take over from the matvec family (>= 16)
+    int f16_big_min_m = 256;     // batch from which the fp16 big tiles take over from the int8 tiles
+    int mmq_fp16_only = 0;       // 1: every tile contraction on the single-buffered fp16 tiles
+    int i8_grid_split = 1;       // int8 tiles: split K over workgroups on small grids
+    int pair_rows = 0;           // fused gate/up: row pairs per workgroup, 32 / 16 / 8 (0: the most even split)
+    int rms_rows = 0;            // fused RMSNorm prologue: rows per workgroup, 16 / 24 (0: the most even split)
+    int prefill_attention_valu = 0;  // prompt attention for head_dim 128 on the vector ALU instead of the matrix cores
+    int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
+};
+
 }  // namespace candy
 
 struct candy_hip_device {
     int ordinal = 0;
+    candy::Options opt;
     hipStream_t stream = nullptr;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int num_cus = 0;
@@ -207,7 +225,7 @@ struct ActWorkspace {
 int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quants, ActWorkspace *out);
 // matvec.hip: y[m, rows] = x . W^T for any m from planar activations that live OUTSIDE the device
 // workspace (the tile kernel may carve its fp16 scratch from it).
-int mmq_min_m();
+int mmq_min_m(const candy_hip_device *dev);
 int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                     int64_t m, float *y, const _Float16 *xh_ready = nullptr, const float *res = nullptr);
 // prefill.hip: prompt stages of the decoder (n tokens at positions pos0 ..).

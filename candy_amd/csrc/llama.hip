@@ -9,9 +9,6 @@
 
 #include "blocks.h"
 #include "internal.h"
-#include <cstdio>
-
-#include "persist.h"
 
 struct candy_hip_llama {
     candy_hip_device *dev = nullptr;
@@ -34,23 +31,14 @@ struct candy_hip_llama {
     float *proj = nullptr;  // [d_model]: a projection's output before the residual add, for formats without that epilogue
     int8_t *xq = nullptr;           // planar Q8_0 quants of the current activation
     candy::Q8Scale *xs = nullptr;
-    uint32_t *next_tok = nullptr;   // [2]: greedy token, then the persistent kernel's time-out flag
+    uint32_t *next_tok = nullptr;   // greedy token of the last step
     int64_t *tok_id = nullptr;
     int *d_pos = nullptr;                         // position of the token being decoded (device copy)
     void *attn_scratch = nullptr;                 // attention split partials
     int n_splits = 1;
-    // the step as one persistent kernel (persist.hip), when the configuration is one it covers
-    bool persist_wanted = false, persist_broken = false, persist_ready = false;
-    int last_path = 0;
-    candy::u64 *p_prof = nullptr;  // phase stamps of the last persistent step (CANDY_HIP_PERSIST_PROF)
-    std::vector<candy::PersistLayer> p_host;
-    candy::PersistLayer *p_layers = nullptr;
-    unsigned *p_epoch = nullptr;
-    candy::u64 *p_xchg = nullptr;
     hipGraph_t graph = nullptr;                   // the captured step (layers + head + argmax)
     hipGraphExec_t graph_exec = nullptr;
     bool graph_dirty = true;
-    bool tables_dirty = true;  // a weight, a norm or the choice of path changed since the persistent step's tables were built
     bool use_graph = true;
     std::vector<void *> owned;
     // prompt buffers, grown on demand to the longest prompt seen: [n][width] activations
@@ -69,11 +57,9 @@ struct candy_hip_llama {
 namespace candy {
 
 // Parks the step's position and token id in device memory (read by the captured kernels).
-__global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok, unsigned *epoch) {
+__global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok) {
     *pos_dst = pos;
     if (tok >= 0) *tok_dst = tok;
-    const unsigned e = *epoch + 1;  // tags of the persistent kernel's exchange words: never 0, new every step
-    *epoch = e == 0 ? 1 : e;
 }
 
 }  // namespace candy
@@ -139,10 +125,8 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
     if (!rc) rc = dev_alloc(m, &m->logits, (size_t)cfg->vocab);
     if (!rc) rc = dev_alloc(m, &m->xq, widest);
     if (!rc) rc = dev_alloc(m, &m->xs, widest / 32);
-    if (!rc) rc = dev_alloc(m, &m->next_tok, 2);
-    if (!rc) rc = candy_hip_zero(dev, m->next_tok, 2 * sizeof(uint32_t));
-    if (!rc) rc = dev_alloc(m, &m->p_epoch, 1);
-    if (!rc) rc = candy_hip_zero(dev, m->p_epoch, sizeof(unsigned));
+    if (!rc) rc = dev_alloc(m, &m->next_tok, 1);
+    if (!rc) rc = candy_hip_zero(dev, m->next_tok, sizeof(uint32_t));
     if (!rc) rc = dev_alloc(m, &m->tok_id, 1);
     if (!rc) rc = dev_alloc(m, &m->d_pos, 1);
     m->n_splits = attention_splits(dev, cfg->n_kv_heads, cfg->max_pos);
@@ -151,8 +135,7 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
         rc = dev_alloc(m, &p, attention_scratch_bytes(cfg->n_heads, cfg->n_kv_heads, cfg->head_dim, m->n_splits));
         m->attn_scratch = p;
     }
-    m->use_graph = getenv("CANDY_HIP_NO_GRAPH") == nullptr;
-    m->persist_wanted = getenv("CANDY_HIP_PERSIST") != nullptr;  // opt-in: measured slower than the launches so far
+    m->use_graph = dev->opt.llama_graph != 0;
     if (!rc) rc = candy_hip_zero(dev, m->k_cache, kv * sizeof(float));
     if (!rc) rc = candy_hip_zero(dev, m->v_cache, kv * sizeof(float));
     if (!rc) {
@@ -179,20 +162,6 @@ int candy_hip_llama_free(candy_hip_llama *m) {
     if (!m) return CANDY_HIP_OK;
     (void)hipSetDevice(m->dev->ordinal);
     (void)hipStreamSynchronize(m->dev->stream);
-    if (m->p_prof) {  // the last step's phase stamps (100 MHz clock), one line per workgroup and layer
-        const size_t n = (size_t)m->dev->num_cus * (size_t)(m->cfg.n_layers + 1) * candy::PROF_SLOTS;
-        std::vector<candy::u64> h(n);
-        const char *path = getenv("CANDY_HIP_PERSIST_PROF");
-        FILE *f = path ? fopen(path, "w") : nullptr;
-        if (f && hipMemcpy(h.data(), m->p_prof, n * sizeof(candy::u64), hipMemcpyDeviceToHost) == hipSuccess)
-            for (size_t i = 0; i < n; i += candy::PROF_SLOTS) {
-                const size_t row = i / candy::PROF_SLOTS;
-                fprintf(f, "%zu %zu", row / (size_t)(m->cfg.n_layers + 1), row % (size_t)(m->cfg.n_layers + 1));
-                for (int j = 0; j < candy::PROF_SLOTS; ++j) fprintf(f, " %llu", h[i + j]);
-                fprintf(f, "\n");
-            }
-        if (f) fclose(f);
-    }
     if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
     if (m->graph) (void)hipGraphDestroy(m->graph);
     for (void *p : m->owned) (void)candy_hip_free(m->dev, p);
@@ -219,7 +188,7 @@ int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const 
     case CANDY_HIP_W_EMBED: rows = c.vocab; cols = c.d_model; break;
     default: return fail(CANDY_HIP_ERR_INVALID, "weight kind %d is not a quantized matrix", which);
     }
-    m->graph_dirty = m->tables_dirty = true;
+    m->graph_dirty = true;
     CANDY_REQUIRE(w->rows == rows && w->cols == cols, "weight kind %d must be %lld x %lld, got %lld x %lld", which,
                   (long long)rows, (long long)cols, (long long)w->rows, (long long)w->cols);
     if (which == CANDY_HIP_W_HEAD) { m->head = w; return CANDY_HIP_OK; }
@@ -240,7 +209,7 @@ int candy_hip_llama_set_qweight(candy_hip_llama *m, int which, int layer, const 
 
 int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const float *dev_alpha) {
     CANDY_REQUIRE(m && dev_alpha, "nil argument");
-    m->graph_dirty = m->tables_dirty = true;
+    m->graph_dirty = true;
     if (which == CANDY_HIP_W_OUT_NORM) { m->out_norm = dev_alpha; return CANDY_HIP_OK; }
     CANDY_REQUIRE(which == CANDY_HIP_W_ATTN_NORM || which == CANDY_HIP_W_FFN_NORM, "weight kind %d is not a norm", which);
     CANDY_REQUIRE(layer >= 0 && layer < m->cfg.n_layers, "layer %d out of range", layer);
@@ -252,19 +221,6 @@ int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const flo
 int candy_hip_llama_set_graph(candy_hip_llama *m, int enable) {
     CANDY_REQUIRE(m, "model is nil");
     m->use_graph = enable != 0;
-    return CANDY_HIP_OK;
-}
-
-int candy_hip_llama_set_persistent(candy_hip_llama *m, int enable) {
-    CANDY_REQUIRE(m, "model is nil");
-    m->persist_wanted = enable != 0;
-    m->graph_dirty = m->tables_dirty = true;
-    return CANDY_HIP_OK;
-}
-
-int candy_hip_llama_decode_path(candy_hip_llama *m, int *path) {
-    CANDY_REQUIRE(m && path, "model or output is nil");
-    *path = m->last_path;
     return CANDY_HIP_OK;
 }
 
@@ -281,7 +237,7 @@ int candy_hip_llama_set_kv_f16(candy_hip_llama *m, int enable) {
     CANDY_REQUIRE(m, "model is nil");
     if (int rc = use_device(m->dev)) return rc;
     m->kv_f16 = enable != 0;
-    m->graph_dirty = m->tables_dirty = true;
+    m->graph_dirty = true;
     // the cache's contents do not survive a change of element type
     const size_t kv = (size_t)m->cfg.n_layers * m->cfg.n_kv_heads * m->cfg.max_pos * m->cfg.head_dim;
     if (int rc = candy_hip_zero(m->dev, m->k_cache, kv * sizeof(float))) return rc;
@@ -343,85 +299,7 @@ static int linear_residual(candy_hip_llama *m, const candy_hip_qtensor *w) {
 // Enqueues one decode step (hidden state in m->h, position in *m->d_pos) on the stream: six
 // launches per layer. Everything it touches is owned by the model, nothing allocates or
 // synchronises, so the sequence can be captured once and replayed for every token.
-// Whether the persistent kernel covers this model on this device (persist.hip states what it covers).
-static bool persist_covers(const candy_hip_llama *m) {
-    const candy_hip_llama_config &c = m->cfg;
-    const int G = m->dev->num_cus;
-    if (m->kv_f16 || c.head_dim != 128 || c.n_heads != c.n_kv_heads || c.n_heads * c.head_dim != c.d_model) return false;
-    if (c.d_model > 4096 || c.d_model % 256 || c.d_ffn > 16384 || c.d_ffn % 256 || 6 * c.n_layers + 2 >= 4096) return false;
-    if (G % c.n_heads) return false;
-    const int S = G / c.n_heads;
-    if (S < 1 || S > 128 || 128 % S) return false;  // a split's merge uses S * (128 / S + 2) <= 384 threads
-    auto q4k = [](const candy_hip_qtensor *w) { return w->fmt == CANDY_HIP_Q4_K && ((uintptr_t)w->data & 15) == 0; };
-    for (const candy_hip_llama::Layer &L : m->layers)
-        if (!q4k(L.wq) || !q4k(L.wk) || !q4k(L.wv) || !q4k(L.wo) || !q4k(L.gate) || !q4k(L.up) || !q4k(L.down)) return false;
-    return q4k(m->head) || (m->head->fmt == CANDY_HIP_Q6_K && ((uintptr_t)m->head->data & 1) == 0);
-}
-
-// Exchange buffers (allocated and cleared once) and the layer table (uploaded again whenever a weight
-// changed).  Runs outside stream capture; the upload is ordered on the stream before the next step.
-static size_t persist_part_words(const candy_hip_llama *m) {
-    return (size_t)m->cfg.n_heads * (size_t)(m->dev->num_cus / m->cfg.n_heads) * (128 + 2);
-}
-
-static int persist_prepare(candy_hip_llama *m) {
-    const candy_hip_llama_config &c = m->cfg;
-    candy_hip_device *dev = m->dev;
-    const size_t D = (size_t)c.d_model, F = (size_t)c.d_ffn;
-    const size_t words = 2 * (D + D + 3 * D + persist_part_words(m) + D + F) + 2 * (size_t)dev->num_cus;
-    if (!m->p_xchg) {
-        if (int rc = dev_alloc(m, &m->p_xchg, words)) return rc;
-        if (int rc = candy_hip_zero(dev, m->p_xchg, words * sizeof(u64))) return rc;
-        if (int rc = dev_alloc(m, &m->p_layers, (size_t)c.n_layers)) return rc;
-    }
-    if (!m->p_prof && getenv("CANDY_HIP_PERSIST_PROF"))
-        if (int rc = dev_alloc(m, &m->p_prof, (size_t)dev->num_cus * (size_t)(c.n_layers + 1) * candy::PROF_SLOTS)) return rc;
-    CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));  // a step still in flight reads the table being replaced
-    m->p_host.resize((size_t)c.n_layers);
-    for (int l = 0; l < c.n_layers; ++l) {
-        const candy_hip_llama::Layer &L = m->layers[l];
-        PersistLayer &P = m->p_host[(size_t)l];
-        auto addr = [](const void *p) { return (candy::u64)(uintptr_t)p; };
-        P.wq = addr(L.wq->data); P.wk = addr(L.wk->data); P.wv = addr(L.wv->data); P.wo = addr(L.wo->data);
-        P.gate = addr(L.gate->data); P.up = addr(L.up->data); P.down = addr(L.down->data);
-        P.attn_norm = addr(L.attn_norm); P.ffn_norm = addr(L.ffn_norm);
-    }
-    if (int rc = candy_hip_h2d(dev, m->p_layers, m->p_host.data(), m->p_host.size() * sizeof(PersistLayer))) return rc;
-    m->persist_ready = true;
-    return CANDY_HIP_OK;
-}
-
-// The step as one launch (nothing here allocates or synchronises: it may be captured).
-static int persist_enqueue(candy_hip_llama *m) {
-    const candy_hip_llama_config &c = m->cfg;
-    candy_hip_device *dev = m->dev;
-    const size_t D = (size_t)c.d_model, F = (size_t)c.d_ffn;
-    const size_t part = persist_part_words(m);
-    PersistArgs a{};
-    a.layers = m->p_layers;
-    a.n_layers = c.n_layers; a.d_model = c.d_model; a.n_heads = c.n_heads; a.d_ffn = c.d_ffn; a.vocab = c.vocab;
-    a.max_pos = c.max_pos; a.eps = c.rms_eps; a.scale = 1.0f / std::sqrt((float)c.head_dim);
-    a.out_norm = m->out_norm; a.head = (const uint8_t *)m->head->data; a.head_is_q6k = m->head->fmt == CANDY_HIP_Q6_K;
-    a.cos_t = m->cos_t; a.sin_t = m->sin_t; a.k_cache = m->k_cache; a.v_cache = m->v_cache;
-    a.h_in = m->h; a.pos_ptr = m->d_pos; a.epoch_ptr = m->p_epoch;
-    u64 *p = m->p_xchg;
-    a.x_ha = p; p += 2 * D;
-    a.x_hb = p; p += 2 * D;
-    a.x_qkv = p; p += 6 * D;
-    a.x_part = p; p += 2 * part;
-    a.x_att = p; p += 2 * D;
-    a.x_act = p; p += 2 * F;
-    a.x_best = p;
-    a.logits = m->logits; a.next_tok = m->next_tok; a.fail = m->next_tok + 1;
-    // polls before a workgroup gives up (about 50 ms); CANDY_HIP_PERSIST_SPIN_LIMIT overrides, negative = give up at once
-    const char *spin_env = getenv("CANDY_HIP_PERSIST_SPIN_LIMIT");
-    a.spin_limit = spin_env ? atoi(spin_env) : 1 << 15;
-    a.prof = m->p_prof;
-    return launch_decode_step(dev, a);
-}
-
 static int llama_enqueue_step(candy_hip_llama *m) {
-    if (m->persist_ready) return persist_enqueue(m);
     const candy_hip_llama_config &c = m->cfg;
     candy_hip_device *dev = m->dev;
     const float scale = 1.0f / std::sqrt((float)c.head_dim);
@@ -470,24 +348,15 @@ static int llama_enqueue_step(candy_hip_llama *m) {
 }
 
 static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const float *dev_hidden,
-                      const float **dev_logits, int32_t *next_token);
-
-static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const float *dev_hidden,
                       const float **dev_logits, int32_t *next_token) {
     candy_hip_device *dev = m->dev;
     int rc;
-    hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token, m->p_epoch);
+    hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token);
     CANDY_LAUNCH_CHECK();
     if (dev_hidden) {
         if ((rc = candy_hip_d2d(dev, m->h, dev_hidden, (size_t)m->cfg.d_model * sizeof(float)))) return rc;
     } else {
         if ((rc = candy_hip_qindex_select(dev, m->embed, m->tok_id, 1, m->h))) return rc;
-    }
-    if (m->tables_dirty) {
-        m->persist_ready = false;
-        if (m->persist_wanted && !m->persist_broken && persist_covers(m))
-            if ((rc = persist_prepare(m))) return rc;
-        m->tables_dirty = false;
     }
     if (m->use_graph) {
         if (m->graph_dirty) {
@@ -508,21 +377,11 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
         if ((rc = llama_enqueue_step(m))) return rc;
     }
     if (dev_logits) *dev_logits = m->logits;
-    if (next_token || m->persist_ready) {
-        uint32_t t[2] = {0, 0};  // token, time-out flag of the persistent kernel
-        if ((rc = candy_hip_d2h(dev, t, m->next_tok, sizeof(t)))) return rc;
-        if (t[1] != 0) {
-            // a workgroup gave up waiting for another (the grid was not resident as a whole): nothing of the
-            // step is trusted; clear the flag and redo it kernel by kernel, from now on
-            m->persist_broken = true;
-            m->persist_ready = false;
-            m->graph_dirty = m->tables_dirty = true;
-            if ((rc = candy_hip_zero(dev, m->next_tok + 1, sizeof(uint32_t)))) return rc;
-            return llama_step(m, pos, token, dev_hidden, dev_logits, next_token);
-        }
-        if (next_token) *next_token = (int32_t)t[0];
+    if (next_token) {
+        uint32_t t = 0;
+        if ((rc = candy_hip_d2h(dev, &t, m->next_tok, sizeof(t)))) return rc;
+        *next_token = (int32_t)t;
     }
-    m->last_path = m->persist_ready ? 1 : 0;
     return CANDY_HIP_OK;
 }
 

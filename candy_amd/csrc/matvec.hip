@@ -13,7 +13,6 @@
 // consecutive bytes of the row; the R rows' loads are issued together to keep many bytes in
 // flight per wavefront.  Per-row partial sums are reduced across the 64 lanes at the end.
 #include <algorithm>
-#include <cstdlib>
 #include <type_traits>
 
 #include "blocks.h"
@@ -292,7 +291,7 @@ static int launch_jobs_fmt(candy_hip_device *dev, const MatvecJobs &jobs, int64_
                            const Q8Scale *scales) {
     const int iter = (int)((K / U::ELEMS + 63) / 64);
     if constexpr (U::SPAN > 0) {
-        bool aligned = U::row_bytes((int)K) % 16 == 0 && getenv("CANDY_HIP_NO_SPAN") == nullptr;
+        bool aligned = U::row_bytes((int)K) % 16 == 0 && dev->opt.matvec_span != 0;
         for (int i = 0; i < jobs.n; ++i) aligned = aligned && ((uintptr_t)jobs.j[i].W & 15) == 0;
         if (aligned) switch (iter) {
             case 1: return launch1_span<U, 1, 4>(dev, jobs, (int)K, qs, scales);
@@ -507,7 +506,7 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
         if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     }
     int64_t done = 0;
-    const bool old_small = getenv("CANDY_HIP_OLD_SMALL_BATCH") != nullptr;  // comparison runs and tests
+    const bool old_small = dev->opt.small_batch_kernel == 0;  // comparison runs and tests
     while (done < m) {
         const int64_t left = m - done;
         const int8_t *q = qs + done * K;
@@ -586,7 +585,7 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && w->cols <= 0x7FFFFFFF, "matrix too large");
     // the 32-value formats: the vector kernels match the tile kernel up to 8 rows (one pass); from 9 rows on they need two
     if (m >= 9 && w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K && w->fmt != CANDY_HIP_Q5_K &&
-        getenv("CANDY_HIP_I8_MIN_M") == nullptr && mmq_i8_covers(w, qs))
+        dev->opt.i8_min_m == 0 && mmq_i8_covers(w, qs))
         return launch_mmq_i8(dev, w, qs, scales, m, y);
     if (m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q5_K) && mmq_i8_covers(w, qs)) {
         // 5 .. 15 rows: the vector kernels below (one or two passes of up to 8 rows) or one pass of the int8 tile
@@ -600,8 +599,8 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
         const double t_tiles = q6 ? std::min(3.5 + 2.5 * nsb * (1.0 + mnk / 40.0), 11.5 + 0.23 * mnk)
                                   : std::min(3.5 + 2.0 * nsb * (1.0 + mnk / 40.0), 11.0 + 0.16 * mnk);
         const double t_vector = 4.0 + (m > 8 ? 2.0 : 0.0) + (q6 ? 0.1 : 0.052) * mnk * m_pad;
-        const char *e = getenv("CANDY_HIP_I8_MIN_M");  // comparison runs: tiles from this batch size on
-        if (e ? m >= atoi(e) : t_tiles < t_vector) return launch_mmq_i8(dev, w, qs, scales, m, y);
+        const int from = dev->opt.i8_min_m;  // comparison runs: tiles from this batch size on
+        if (from ? m >= from : t_tiles < t_vector) return launch_mmq_i8(dev, w, qs, scales, m, y);
     }
     switch (w->fmt) {
     case CANDY_HIP_Q4_K: return launch_fmt<UnitQ4K>(dev, w, qs, scales, m, y);
@@ -621,14 +620,11 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
     }
 }
 
-int mmq_min_m() {
-    static const int v = getenv("CANDY_HIP_MMQ_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_MIN_M")) : 16;
-    return v < 16 ? 16 : v;
-}
+int mmq_min_m(const candy_hip_device *dev) { return dev->opt.mmq_min_m < 16 ? 16 : dev->opt.mmq_min_m; }
 
 int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                     int64_t m, float *y, const _Float16 *xh_ready, const float *res) {
-    if (m < mmq_min_m()) {
+    if (m < mmq_min_m(dev)) {
         CANDY_REQUIRE(res != y, "internal: in-place residual needs the fused epilogue");
         if (int rc = launch_matvec(dev, w, qs, scales, m, y)) return rc;
         return res ? candy_hip_add(dev, res, y, m * w->rows, y) : CANDY_HIP_OK;
@@ -653,7 +649,7 @@ static int qmatmul_check(candy_hip_device *dev, const candy_hip_qtensor *w, int6
 }
 
 static int contract(candy_hip_device *dev, const candy_hip_qtensor *w, const ActWorkspace &a, int64_t m, float *y) {
-    return m < mmq_min_m() ? launch_matvec(dev, w, a.qs, a.scales, m, y) : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws);
+    return m < mmq_min_m(dev) ? launch_matvec(dev, w, a.qs, a.scales, m, y) : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws);
 }
 
 int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m, float *dev_y) {

@@ -316,13 +316,10 @@ int64_t mmq_m_pad(int64_t m) { return (m + 255) / 256 * 256; }  // a multiple of
 static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                         int64_t m, float *y, void *half_ws, const _Float16 *xh_ready, const float *res, bool *res_done);
 
-static bool force_old_fp16() {
-    static const bool v = getenv("CANDY_HIP_MMQ_FP16") != nullptr;
-    return v;
-}
+static bool force_old_fp16(const candy_hip_device *dev) { return dev->opt.mmq_fp16_only != 0; }
 
 bool mmq_fuses_residual(const candy_hip_qtensor *w, int64_t m) {
-    return m >= mmq_min_m() && w->cols % 64 == 0 && !force_old_fp16() && mmq_f16_big_covers(w, m);
+    return m >= mmq_min_m(w->dev) && w->cols % 64 == 0 && !force_old_fp16(w->dev) && mmq_f16_big_covers(w, m);
 }
 
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int64_t m,
@@ -342,7 +339,7 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     if (w->fmt == CANDY_HIP_Q8_K) return launch_matvec(dev, w, qs, scales, m, y);  // reports that Q8_K does not contract
     // prompt-sized batches of Q4_K: big fp16 tiles (the integer kernel is bound by its per-sub-block rescale there);
     // smaller batches of Q4_K and Q6_K: int8 matrix cores (exact); the fp16 tile kernel below serves the rest
-    const bool force_fp16 = force_old_fp16();
+    const bool force_fp16 = force_old_fp16(dev);
     const bool big = !force_fp16 && mmq_f16_big_covers(w, m);
     // the 32-value formats (Q8_0, Q4_0, Q4_1, Q5_0, Q5_1) on the int8 tiles as well, except where the 128 x 128 fp16 tiles below fill the chip (many weight rows and
     // a prompt-sized batch; measured: 11008x4096 m = 256 127 against 123 us, m = 512 228 against 134; 32000x4096

@@ -441,7 +441,7 @@ static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _
 }
 
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
-    static const int min_m = getenv("CANDY_HIP_MMQ_BIG_MIN_M") ? atoi(getenv("CANDY_HIP_MMQ_BIG_MIN_M")) : 256;
+    const int min_m = w->dev->opt.f16_big_min_m;
     if (m < min_m || w->cols % 256 != 0) return false;
     if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
     if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML)

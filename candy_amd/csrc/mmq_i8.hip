@@ -692,7 +692,7 @@ static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const in
     // and 14336x4096 at 8 .. 255 rows for Q4_K, Q6_K and Q8_0: deeper stages (2 or 4 super-blocks in flight per
     // wavefront) and a K split inside an eight-wavefront workgroup, both of which helped before the split over
     // workgroups existed, now cost 1-10 % (Q6_K at 64-row tiles: 25 %); 32-row tiles won nowhere.
-    const bool no_gs = getenv("CANDY_HIP_MMQ_I8_NO_GRID_SPLIT") != nullptr;  // comparison runs and tests
+    const bool no_gs = dev->opt.i8_grid_split == 0;  // comparison runs and tests
     const int nsb = K >> 8;
     int n_split = 1, sb_split = nsb;
     float *out = y;

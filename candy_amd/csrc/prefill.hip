@@ -400,7 +400,7 @@ static void launch_attn_prefill_kv(candy_hip_device *dev, const float *q, const 
                                    int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride,
                                    float scale) {
     const dim3 grid((unsigned)n_heads, (unsigned)((n + 31) / 32));
-    static const bool valu_only = getenv("CANDY_HIP_ATTN_PREFILL_VALU") != nullptr;  // comparison runs
+    const bool valu_only = dev->opt.prefill_attention_valu != 0;  // comparison runs
     if (head_dim == 128 && !valu_only)
         hipLaunchKernelGGL(k_attn_prefill_mfma<KV>, dim3((unsigned)n_heads, (unsigned)((n + 63) / 64)), dim3(256), 0,
                            dev->stream, q, k_cache, v_cache, out, n, pos0, n_heads, n_kv_heads, cache_stride, scale);

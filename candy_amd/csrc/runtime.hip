@@ -314,6 +314,50 @@ int candy_hip_qtensor_info(const candy_hip_qtensor *q, int *fmt, int64_t *rows, 
     return CANDY_HIP_OK;
 }
 
+namespace {
+struct OptionKey {
+    const char *key;
+    int candy::Options::*field;
+    int lo, hi;
+};
+// every key of candy_hip_set_option with the range it accepts
+const OptionKey OPTION_KEYS[] = {
+    {"matvec.span", &candy::Options::matvec_span, 0, 1},
+    {"matvec.small_batch_kernel", &candy::Options::small_batch_kernel, 0, 1},
+    {"mmq.i8_min_m", &candy::Options::i8_min_m, 0, 1 << 20},
+    {"mmq.min_m", &candy::Options::mmq_min_m, 16, 1 << 20},
+    {"mmq.f16_big_min_m", &candy::Options::f16_big_min_m, 16, 1 << 30},
+    {"mmq.fp16_only", &candy::Options::mmq_fp16_only, 0, 1},
+    {"mmq.i8_grid_split", &candy::Options::i8_grid_split, 0, 1},
+    {"fused.pair_rows", &candy::Options::pair_rows, 0, 32},
+    {"fused.rms_rows", &candy::Options::rms_rows, 0, 24},
+    {"prefill.attention_valu", &candy::Options::prefill_attention_valu, 0, 1},
+    {"llama.graph", &candy::Options::llama_graph, 0, 1},
+};
+const OptionKey *find_option(const char *key) {
+    for (const OptionKey &k : OPTION_KEYS)
+        if (strcmp(k.key, key) == 0) return &k;
+    return nullptr;
+}
+}  // namespace
+
+int candy_hip_set_option(candy_hip_device *dev, const char *key, int64_t value) {
+    CANDY_REQUIRE(dev && key, "nil argument");
+    const OptionKey *k = find_option(key);
+    CANDY_REQUIRE(k, "unknown option \"%s\"", key);
+    CANDY_REQUIRE(value >= k->lo && value <= k->hi, "option %s takes %d .. %d, got %lld", key, k->lo, k->hi, (long long)value);
+    dev->opt.*(k->field) = (int)value;
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_get_option(const candy_hip_device *dev, const char *key, int64_t *value) {
+    CANDY_REQUIRE(dev && key && value, "nil argument");
+    const OptionKey *k = find_option(key);
+    CANDY_REQUIRE(k, "unknown option \"%s\"", key);
+    *value = dev->opt.*(k->field);
+    return CANDY_HIP_OK;
+}
+
 int candy_hip_timer_start(candy_hip_device *dev) {
     if (int rc = use_device(dev)) return rc;
     CANDY_HIP_TRY(hipEventRecord(dev->ev_start, dev->stream));

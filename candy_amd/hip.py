@@ -43,6 +43,8 @@ SIGNATURES = {
     "candy_hip_device_ordinal": (c_int, [c_void_p, POINTER(c_int)]),
     "candy_hip_device_name": (c_int, [c_void_p, c_char_p, c_size_t]),
     "candy_hip_synchronize": (c_int, [c_void_p]),
+    "candy_hip_set_option": (c_int, [c_void_p, c_char_p, c_int64]),
+    "candy_hip_get_option": (c_int, [c_void_p, c_char_p, POINTER(c_int64)]),
     "candy_hip_alloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "candy_hip_free": (c_int, [c_void_p, c_void_p]),
     "candy_hip_zero": (c_int, [c_void_p, c_void_p, c_size_t]),
@@ -85,9 +87,7 @@ SIGNATURES = {
     "candy_hip_llama_set_qweight": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "candy_hip_llama_set_norm": (c_int, [c_void_p, c_int, c_int, c_void_p]),
     "candy_hip_llama_set_graph": (c_int, [c_void_p, c_int]),
-    "candy_hip_llama_set_persistent": (c_int, [c_void_p, c_int]),
     "candy_hip_llama_set_kv_f16": (c_int, [c_void_p, c_int]),
-    "candy_hip_llama_decode_path": (c_int, [c_void_p, POINTER(c_int)]),
     "candy_hip_llama_kv_cache": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_size_t)]),
     "candy_hip_llama_decode": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_llama_decode_hidden": (c_int, [c_void_p, c_void_p, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
@@ -223,6 +223,15 @@ class Device:
         if self.handle is not None:
             lib().candy_hip_close(self.handle)
             self.handle = None
+
+    # ---- switches (include/candy_hip.h lists the keys)
+    def set_option(self, key: str, value: int):
+        _check(lib().candy_hip_set_option(self.handle, key.encode(), int(value)))
+
+    def get_option(self, key: str) -> int:
+        v = c_int64(0)
+        _check(lib().candy_hip_get_option(self.handle, key.encode(), byref(v)))
+        return v.value
 
     # ---- memory
     def alloc(self, nbytes: int) -> Buffer:
@@ -445,15 +454,6 @@ class Llama:
     def set_kv_f16(self, enable: bool):
         """fp16 KV cache (clears the cache); kv_cache() then reports half the bytes."""
         _check(lib().candy_hip_llama_set_kv_f16(self.handle, int(enable)))
-
-    def set_persistent(self, enable: bool):
-        _check(lib().candy_hip_llama_set_persistent(self.handle, int(enable)))
-
-    def decode_path(self) -> int:
-        """0: the last decode step ran kernel by kernel; 1: as the persistent kernel."""
-        p = c_int(-1)
-        _check(lib().candy_hip_llama_decode_path(self.handle, byref(p)))
-        return p.value
 
     def kv_cache(self):
         k, v, n = c_void_p(), c_void_p(), c_size_t()

@@ -73,6 +73,27 @@ int candy_hip_device_ordinal(const candy_hip_device *dev, int *ordinal);
 int candy_hip_device_name(const candy_hip_device *dev, char *buf, size_t buf_len);
 int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchronize                */
 
+/* Switches of one device handle.  No environment variable is ever read: what selects a kernel is an argument
+ * or one of these, set from the thread that uses the handle.  The defaults are the measured, shipped choice;
+ * everything else exists so that comparison runs and tests can ask for a kernel the dispatch would not pick
+ * (results stay within the documented tolerance whichever is chosen).  Unknown keys and values out of range
+ * are CANDY_HIP_ERR_INVALID.  No counterpart in the reference.
+ *   key                          default  meaning
+ *   "llama.graph"                1        decoders created afterwards replay a captured HIP graph (0: eager)
+ *   "mmq.min_m"                  16       batch from which tile kernels replace the matvec family (>= 16)
+ *   "mmq.f16_big_min_m"          256      batch from which fp16 big tiles (3e-4 per matmul) replace the exact int8 tiles
+ *   -- comparison / test only --
+ *   "matvec.span"                1        batch-1 kernel of 2-byte aligned formats fetches aligned 16-byte spans
+ *   "matvec.small_batch_kernel"  1        2..8 rows on the one-workgroup-per-CU kernel (0: looping kernel)
+ *   "mmq.i8_min_m"               0        5..15 rows: int8 tiles from this batch on (0: by measured cost model)
+ *   "mmq.fp16_only"              0        every tile contraction on the single-buffered fp16 tiles
+ *   "mmq.i8_grid_split"          1        int8 tiles split K over workgroups on small grids
+ *   "fused.pair_rows"            0        fused gate/up: row pairs per workgroup 32 / 16 / 8 (0: most even split)
+ *   "fused.rms_rows"             0        fused RMSNorm prologue: rows per workgroup 16 / 24 (0: most even split)
+ *   "prefill.attention_valu"     0        prompt attention for head_dim 128 on the vector ALU */
+int candy_hip_set_option(candy_hip_device *dev, const char *key, int64_t value);
+int candy_hip_get_option(const candy_hip_device *dev, const char *key, int64_t *value);
+
 /* ------------------------------------------------------------------ raw device memory
  * Backs BackendStorage[T] (backend.go:4-16): Data() is a d2h copy, Clone() a d2d copy. */
 int candy_hip_alloc(candy_hip_device *dev, size_t bytes, void **dptr);
@@ -211,17 +232,6 @@ int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const flo
  * position and token travel through device memory); enable = 0 launches the kernels one by
  * one instead.  Results are identical either way. */
 int candy_hip_llama_set_graph(candy_hip_llama *m, int enable);
-/* Experimental, off by default: where the model's shape allows (head_dim 128, one kv head per query
- * head, Q4_K layer weights, d_model <= 4096, d_ffn <= 16384) the decode step can run as ONE persistent
- * kernel, one workgroup per compute unit, whose phases hand their results on through tagged words in
- * device memory, instead of six launches per layer.  enable = 1 selects it (so does the environment
- * variable CANDY_HIP_PERSIST); a model it does not cover, or a device on which its workgroups cannot
- * all be resident, keeps the launches.  Results agree to f32 summation order.  As measured on the 7B
- * shape it is the slower of the two.  No counterpart in the reference, which has no model code and runs
- * one op per call. */
-int candy_hip_llama_set_persistent(candy_hip_llama *m, int enable);
-/* How the last decode step ran: 0 = kernel by kernel, 1 = the persistent kernel. */
-int candy_hip_llama_decode_path(candy_hip_llama *m, int *path);
 /* Optional fp16 KV cache (off by default: candy's tensors are f32).  The new token's k (after Rope) and v are
  * rounded to fp16 once, as they enter the cache; attention reads them back as f32 and every product and sum
  * stays f32.  Halves the largest stream of a long-context decode step.  Changing the setting clears the cache.

@@ -103,7 +103,6 @@ def test_decode_steps_match_cpu_composition(dev, name, cfg, fmts):
         if top2[1] - top2[0] > 2e-3 * np.max(np.abs(rlogits)):
             assert nt == rt, (name, pos)
         assert nt == int(np.argmax(logits))
-        assert model.decode_path() == 0  # kernel by kernel unless the one-kernel step is asked for
     # the device KV cache holds what the CPU composition wrote
     kptr, vptr, nbytes = model.kv_cache()
     kc = np.empty(nbytes // 4, np.float32)
@@ -339,7 +338,6 @@ def test_fp16_kv_cache_matches_cpu_composition_with_rounded_cache(dev, case, lay
         rt, rlogits, lim = cpu_step(tok, pos)
         gt, glogits = model.decode(tok, pos)
         assert rel(glogits, rlogits) <= lim, (name, pos)
-        assert model.decode_path() == 0
         tok = rt
     # a short prompt (12 rows: one 16-row tile of the int8 kernel, whose sums run in another order than the batch-1
     # kernel's and the CPU's, so even the first layer's k and v straddle a rounding boundary here and there: the
@@ -408,10 +406,13 @@ def test_gate_up_block_parts_give_the_same_bits(dev, monkeypatch, d_ffn):
     tokens = [int(t) for t in np.random.default_rng(31).integers(0, cfg["vocab"], 5)]
     runs = {}
     for rows in ("32", "16", "8"):
-        monkeypatch.setenv("CANDY_HIP_PAIR_ROWS", rows)
-        _, model = build(dev, cfg, fmts, seed=30)
-        runs[rows] = [model.decode(t, pos)[1].copy() for pos, t in enumerate(tokens)]
-        model.free()
+        dev.set_option("fused.pair_rows", int(rows))
+        try:
+            _, model = build(dev, cfg, fmts, seed=30)
+            runs[rows] = [model.decode(t, pos)[1].copy() for pos, t in enumerate(tokens)]
+            model.free()
+        finally:
+            dev.set_option("fused.pair_rows", 0)
     for rows in ("16", "8"):
         for a, b in zip(runs["32"], runs[rows]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), rows
@@ -451,6 +452,11 @@ PERSIST_CASES = [
 ]
 
 
+PERSIST_SKIP = ("the one-kernel decode step measured slower than the launches (401 against 539 tokens/s on the 7B "
+                "shape) and was taken out of the library; its sources are no longer built")
+
+
+@pytest.mark.skip(reason=PERSIST_SKIP)
 @pytest.mark.parametrize("name,cfg,head,n", PERSIST_CASES)
 def test_persistent_step_equals_kernel_by_kernel(dev, name, cfg, head, n):
     # the same arithmetic in another summation order (RMS sums, attention splits): most steps come out bit for
@@ -488,6 +494,7 @@ def test_persistent_step_equals_kernel_by_kernel(dev, name, cfg, head, n):
     assert rel(bufs[0], bufs[2].astype(np.float64)) <= 1e-3 and rel(bufs[1], bufs[3].astype(np.float64)) <= 1e-3
 
 
+@pytest.mark.skip(reason=PERSIST_SKIP)
 def test_persistent_step_time_out_falls_back(dev, monkeypatch):
     # the host asks the kernel for its time-out path (every workgroup raises the flag and leaves at once, nothing
     # hangs): the step is redone kernel by kernel, gives that path's result, and the model stays on it

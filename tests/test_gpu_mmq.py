@@ -69,9 +69,11 @@ def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, 
         assert np.array_equal(got.view(np.uint32), dev.qmatmul(q, x).view(np.uint32))
         if m in (16, 33):
             assert rel_err(got, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5, m
-        monkeypatch.setenv("CANDY_HIP_MMQ_I8_NO_GRID_SPLIT", "1")
-        whole = dev.qmatmul(q, x)
-        monkeypatch.delenv("CANDY_HIP_MMQ_I8_NO_GRID_SPLIT")
+        dev.set_option("mmq.i8_grid_split", 0)
+        try:
+            whole = dev.qmatmul(q, x)
+        finally:
+            dev.set_option("mmq.i8_grid_split", 1)
         assert rel_err(got, whole) <= 2e-6, m
 
 

@@ -65,15 +65,18 @@ def test_small_batch_one_pass_per_eight_rows(dev, monkeypatch, fmt, rows, cols):
         assert got.shape == (m, rows)
         if m in (3, 8, 15):
             assert rel_err(got, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5, m
-        monkeypatch.setenv("CANDY_HIP_OLD_SMALL_BATCH", "1")
-        monkeypatch.setenv("CANDY_HIP_I8_MIN_M", "99")
-        old = dev.qmatmul(q, x)
-        monkeypatch.setenv("CANDY_HIP_I8_MIN_M", "2")  # tiles wherever they apply (Q4_K, Q6_K)
-        tiles = dev.qmatmul(q, x)
-        monkeypatch.delenv("CANDY_HIP_OLD_SMALL_BATCH")
-        monkeypatch.setenv("CANDY_HIP_I8_MIN_M", "99")
-        vector = dev.qmatmul(q, x)
-        monkeypatch.delenv("CANDY_HIP_I8_MIN_M")
+        try:
+            dev.set_option("matvec.small_batch_kernel", 0)
+            dev.set_option("mmq.i8_min_m", 99)
+            old = dev.qmatmul(q, x)
+            dev.set_option("mmq.i8_min_m", 2)  # tiles wherever they apply (Q4_K, Q6_K)
+            tiles = dev.qmatmul(q, x)
+            dev.set_option("matvec.small_batch_kernel", 1)
+            dev.set_option("mmq.i8_min_m", 99)
+            vector = dev.qmatmul(q, x)
+        finally:
+            dev.set_option("matvec.small_batch_kernel", 1)
+            dev.set_option("mmq.i8_min_m", 0)
         assert np.array_equal(vector.view(np.uint32), old.view(np.uint32)), m
         assert rel_err(tiles, old) <= 2e-6, m
         assert rel_err(got, old) <= 2e-6, m
