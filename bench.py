@@ -34,14 +34,65 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 MFMA rate
-# HBM bytes one launch of the Q4_K 4096x11008 matvec moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by a copy kernel of known size (profiles/matvec_q4k_4096x11008.md): 24985 KiB read + 32 KiB written
-MATVEC_TRAFFIC_BYTES = (24985 + 32) * 1024
+MFMA_I8_PEAK_TOPS = 5000.0  # MI355X published dense int8 MFMA rate
 ROTATE_BYTES = 640 << 20  # distinct weight bytes cycled through (last-level cache is 256 MB)
+# HBM bytes one launch of the Q4_K 4096x11008 matvec moves: written by `bench.py --write-traffic DIR` from the
+# two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) whose commands profiles/matvec_q4k_4096x11008.md gives
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "matvec_q4k_4096x11008_traffic.txt")
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def read_traffic():
+    """HBM bytes per launch of the headline kernel from the committed counter summary, or None."""
+    try:
+        kv = dict(line.split(None, 1) for line in open(TRAFFIC_FILE) if line.strip() and not line.startswith("#"))
+        return int(kv["traffic_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def write_traffic(prof_dir):
+    """Summarise DIR/fetch_counter_collection.csv and DIR/write_counter_collection.csv (rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE over `bench.py ... --calibrate-copy`) into TRAFFIC_FILE.  Each counter is scaled by what it reads for
+    the 256 MiB device-to-device copy of the same run."""
+    import csv
+    copy_kib = 256 * 1024
+
+    def means(path):
+        acc = {}
+        for r in csv.DictReader(open(path)):
+            acc.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+    out = {}
+    for tag, name in (("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")):
+        m = means(os.path.join(prof_dir, f"{tag}_counter_collection.csv"))
+        copy = [v for k, v in m.items() if "copyBuffer" in k]
+        mv = [(k, v) for k, v in m.items() if "k_matvec1<candy::UnitQ4K, 3, 1, 4>" in k or "k_matvec1<candy::UnitQ4K,3,1,4>" in k]
+        if not copy or not mv:
+            sys.exit(f"bench.py --write-traffic: no copy or matvec dispatches in the {name} run under {prof_dir}")
+        out[tag] = (mv[0][1], copy_kib / copy[0])
+    traffic = int(round((out["fetch"][0] * out["fetch"][1] + out["write"][0] * out["write"][1]) * 1024))
+    with open(TRAFFIC_FILE, "w") as f:
+        f.write("# k_matvec1<UnitQ4K,3,1,4>, Q4_K 4096x11008 batch 1: HBM bytes per launch from rocprofv3 --pmc\n")
+        f.write("# (KiB per dispatch, mean over dispatches; factor = 262144 KiB / what the counter reads for a 256 MiB copy)\n")
+        f.write(f"fetch_KiB_raw {out['fetch'][0]:.1f}\nfetch_factor {out['fetch'][1]:.4f}\n")
+        f.write(f"write_KiB_raw {out['write'][0]:.1f}\nwrite_factor {out['write'][1]:.4f}\n")
+        f.write(f"traffic_bytes {traffic}\n")
+    print(open(TRAFFIC_FILE).read())
+
+
+def stream_floor(dev, nbytes):
+    """What a kernel that only reads achieves on this device, measured now: GB/s for launches of `nbytes` rotating
+    over ROTATE_BYTES, GB/s for one pass over ROTATE_BYTES, and microseconds per launch of an empty kernel."""
+    span = ROTATE_BYTES // nbytes * nbytes
+    us_small = dev.stream_probe(nbytes, span, 400) / 400 * 1e3
+    us_big = dev.stream_probe(span, span, 10) / 10 * 1e3
+    us_empty = dev.stream_probe(0, 0, 1000) / 1000 * 1e3
+    return nbytes / us_small / 1e3, span / us_big / 1e3, us_empty, us_small
 
 
 def algorithmic_bytes(fmt, rows, cols, m=1):
@@ -276,7 +327,12 @@ def main():
     ap.add_argument("--no-fp16-kv", action="store_true", help="skip the decode leg's second figure (fp16 KV cache)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for counter runs)")
+    ap.add_argument("--write-traffic", metavar="DIR",
+                    help="no benchmark: summarise the FETCH_SIZE / WRITE_SIZE runs under DIR into " + TRAFFIC_FILE)
     args = ap.parse_args()
+    if args.write_traffic:
+        write_traffic(args.write_traffic)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE MI355X; --gpus must be 1 (no collectives, no sharding)")
 
@@ -301,6 +357,10 @@ def main():
     achieved = alg / (ms_kernel * 1e-3) / 1e9
     log(f"Q4_K {rows}x{cols}: path {ms_step * 1e3:.2f} us/step = {value:.0f} GB/s; "
         f"matvec kernel {ms_kernel * 1e3:.2f} us = {achieved:.0f} GB/s ({achieved / HBM_PEAK_GBPS:.1%} of 8 TB/s)")
+    # the same bytes through a kernel that only reads them, and an empty kernel: the floor under any launch
+    floor_small, floor_big, us_empty, us_floor = stream_floor(dev, synth.weight_nbytes(fmt, rows, cols))
+    log(f"read-only stream: {floor_small:.0f} GB/s at {synth.weight_nbytes(fmt, rows, cols)} B per launch ({us_floor:.2f} us), "
+        f"{floor_big:.0f} GB/s over {ROTATE_BYTES >> 20} MiB in one launch; empty kernel {us_empty:.2f} us per launch")
 
     out = {
         "metric": "Q4_K matvec GB/s (batch 1, 4096x11008, f32 in -> f32 out)",
@@ -310,10 +370,16 @@ def main():
         "config": {"workload": "configs[1]: Q4_K 4096x11008 (N x K) batch-1 matvec, activation quantized to Q8_0 "
                                "on device each step", "weight_bytes": synth.weight_nbytes(fmt, rows, cols),
                    "algorithmic_bytes_per_step": alg, "distinct_weight_copies": n_copies,
-                   "device": dev.name},
+                   "device": dev.name,
+                   "decode_model": "random-init 7B: one N(0, 0.02) draw per weight shape quantized on the device by "
+                                   "candy_hip_quantize (Q4_K / Q6_K quantizers restate ggml's published reference "
+                                   "quantizers; parity unpinned against ggml itself), each layer taking the draw "
+                                   "with its blocks rotated"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MATVEC_TRAFFIC_BYTES,
-                     "kernel": "k_matvec1<UnitQ4K,3,1,4>", "us_per_launch": round(ms_kernel * 1e3, 3)},
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": read_traffic(),
+                     "kernel": "k_matvec1<UnitQ4K,3,1,4>", "us_per_launch": round(ms_kernel * 1e3, 3),
+                     "achievable_GBps_25MB": round(floor_small, 1), "achievable_GBps_stream": round(floor_big, 1),
+                     "empty_launch_us": round(us_empty, 3), "frac_of_achievable": round(achieved / floor_small, 4)},
     }
 
     if not args.no_sweep:
@@ -402,19 +468,25 @@ def main():
 
     if not args.no_prefill:
         # batched prefill: Q4_K 14336x4096 x f32 [M, 4096], f32 in -> f32 out (activation quantization included).
-        # m < 256 runs on the int8 matrix cores (exact integer dots), m >= 256 on fp16 tiles; mfma_frac is quoted
-        # against the dense fp16 peak (2.5 PFLOP/s) for both (the int8 peak is twice that)
+        # m < 256 runs on the int8 matrix cores (exact integer dots; peak 5.0 POP/s), m >= 256 on fp16 tiles
+        # (peak 2.5 PFLOP/s).  roofline_us = the larger of the bytes at 8 TB/s and the contraction at that peak.
         pre = []
         r, k = 14336, 4096
+        big_min = dev.get_option("mmq.f16_big_min_m")
         for m in (16, 128, 512):
             ms, _ = time_matvec(dev, synth.Q4_K, r, k, 200, 20, quantize_each=True, seed=m, m=m)
             flops = 2.0 * m * r * k
             byts = algorithmic_bytes(synth.Q4_K, r, k, m)
-            pre.append({"m": m, "kernel": ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if m < 256 else "k_mmq_f16<BigQ4K,128,256,2,4> (fp16 MFMA)",
+            int8 = m < big_min
+            peak = MFMA_I8_PEAK_TOPS if int8 else MFMA_F16_PEAK_TFLOPS
+            roof_us = max(byts / (HBM_PEAK_GBPS * 1e9), flops / (peak * 1e12)) * 1e6
+            pre.append({"m": m, "kernel": ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else "k_mmq_f16<BigQ4K,128,256,2,4> (fp16 MFMA)",
                         "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
-                        "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                        "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
-            log(f"  prefill q4_k {r}x{k} M={m}: {ms * 1e3:.1f} us, {pre[-1]['TFLOPs']} TFLOP/s, {pre[-1]['GBps']} GB/s")
+                        "mfma_peak_TFLOPs": peak, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / peak, 4),
+                        "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                        "roofline_us": round(roof_us, 2), "roofline_frac": round(roof_us / (ms * 1e3), 4)})
+            log(f"  prefill q4_k {r}x{k} M={m}: {ms * 1e3:.1f} us, {pre[-1]['TFLOPs']} TFLOP/s, {pre[-1]['GBps']} GB/s, "
+                f"{pre[-1]['roofline_frac']:.1%} of its roofline")
         out["prefill"] = pre
 
     if not args.no_decode:

@@ -98,6 +98,7 @@ SIGNATURES = {
     "candy_hip_dequantize_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int, POINTER(c_float)]),
     "candy_hip_quantize_sweep": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p, c_int,
                                          POINTER(c_float)]),
+    "candy_hip_stream_probe": (c_int, [c_void_p, c_size_t, c_size_t, c_int, POINTER(c_float)]),
     "candy_hip_timer_start": (c_int, [c_void_p]),
     "candy_hip_timer_stop": (c_int, [c_void_p, POINTER(c_float)]),
 }
@@ -406,6 +407,12 @@ class Device:
         ms = c_float(0)
         _check(lib().candy_hip_quantize_sweep(self.handle, x_buf.ptr, x_stride, n_x, rows, cols, out_buf.ptr, iters,
                                               byref(ms)))
+        return ms.value
+
+    def stream_probe(self, bytes_per_launch: int, span_bytes: int, iters: int) -> float:
+        """Elapsed milliseconds of `iters` read-only launches (0 bytes: empty kernels)."""
+        ms = c_float(0)
+        _check(lib().candy_hip_stream_probe(self.handle, bytes_per_launch, span_bytes, iters, byref(ms)))
         return ms.value
 
     def timer_start(self):

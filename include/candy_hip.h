@@ -272,6 +272,14 @@ int candy_hip_dequantize_sweep(candy_hip_device *dev, const candy_hip_qtensor *c
                                float *dev_out, int iters, float *elapsed_ms);
 int candy_hip_quantize_sweep(candy_hip_device *dev, const float *dev_x, int64_t x_stride, int n_x, int64_t rows,
                              int64_t cols, void *dev_out_blocks, int iters, float *elapsed_ms);
+/* What the device delivers to a kernel that only reads (no counterpart in the reference; the matvec's bytes per
+ * second are quoted against it beside the published peak).  `iters` launches back to back, launch i reading
+ * bytes_per_launch bytes (a multiple of 16) with 16-byte loads from region i of a scratch buffer of span_bytes
+ * that the call allocates, zero-fills and frees; a span larger than the last-level cache makes every launch read
+ * HBM.  bytes_per_launch = 0 times launches of an empty kernel.  Returns the time between HIP events recorded
+ * on the handle's stream around the loop. */
+int candy_hip_stream_probe(candy_hip_device *dev, size_t bytes_per_launch, size_t span_bytes, int iters,
+                           float *elapsed_ms);
 int candy_hip_timer_start(candy_hip_device *dev);
 int candy_hip_timer_stop(candy_hip_device *dev, float *elapsed_ms);   /* synchronises */
 
