@@ -77,6 +77,9 @@ struct candy_hip_device {
     // Partial sums of the split-K tile kernel (same policy).
     void *ws_split = nullptr;
     size_t ws_split_bytes = 0;
+    // One word of pinned host memory that kernels raise when they meet an index outside its table (the condition
+    // the CPU path panics on); check_fault() reports and clears it after a synchronisation.
+    int *fault = nullptr;
 };
 
 struct candy_hip_qtensor {
@@ -115,6 +118,9 @@ namespace candy {
 
 // Makes dev's GPU current for the calling thread (cgo may move goroutines between threads).
 int use_device(const candy_hip_device *dev);
+// After the stream has been synchronised: CANDY_HIP_ERR_INVALID if a kernel since the last check met an
+// out-of-range index (the word is cleared), CANDY_HIP_OK otherwise.
+int check_fault(candy_hip_device *dev);
 // Returns a workspace of at least `bytes` bytes (256-byte aligned).
 int workspace(candy_hip_device *dev, size_t bytes, void **out);
 // Second buffer, for the split-K partial sums (lives beside the activation workspace).
@@ -142,8 +148,9 @@ int launch_quantize_q8(candy_hip_device *dev, const float *x, int64_t rows, int6
 int launch_q8_blocks_to_planar(candy_hip_device *dev, const void *blocks, int64_t n_blocks,
                                int8_t *qs, Q8Scale *scales);
 // matvec.hip: y[m, rows] for m in 1..15 from planar activations.
+// vector_only: never the int8 tile kernel (whose K split takes a workspace), whatever the batch.
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
-                  const Q8Scale *scales, int64_t m, float *y);
+                  const Q8Scale *scales, int64_t m, float *y, bool vector_only = false);
 // matvec.hip: one activation row against up to three weights in one launch, optional residuals.
 int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *ws, float *const *ys,
                         const float *const *res, int n, const int8_t *qs, const Q8Scale *scales);

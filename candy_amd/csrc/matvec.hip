@@ -581,13 +581,13 @@ int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quan
 }
 
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                  int64_t m, float *y) {
+                  int64_t m, float *y, bool vector_only) {
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && w->cols <= 0x7FFFFFFF, "matrix too large");
     // the 32-value formats: the vector kernels match the tile kernel up to 8 rows (one pass); from 9 rows on they need two
-    if (m >= 9 && w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K && w->fmt != CANDY_HIP_Q5_K &&
+    if (!vector_only && m >= 9 && w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K && w->fmt != CANDY_HIP_Q5_K &&
         dev->opt.i8_min_m == 0 && mmq_i8_covers(w, qs))
         return launch_mmq_i8(dev, w, qs, scales, m, y);
-    if (m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q5_K) && mmq_i8_covers(w, qs)) {
+    if (!vector_only && m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q5_K) && mmq_i8_covers(w, qs)) {
         // 5 .. 15 rows: the vector kernels below (one or two passes of up to 8 rows) or one pass of the int8 tile
         // kernel with a 16-row tile, whichever a fit to measurements on this chip says is shorter, in us.  The tile
         // kernel's time hardly depends on m: Q4_K 4096x4096 12.7, 11008x4096 19.6, 4096x11008 19.3, 32000x4096 31.5;

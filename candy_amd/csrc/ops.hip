@@ -143,12 +143,18 @@ __global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ src, 
 }
 
 // indexing.go:8-26 along dim 0 of a [n_src, width] table; id == MaxInt64 selects zeros.
-__global__ __launch_bounds__(256) void k_index_select(const float *__restrict__ table, int64_t width,
-                                                      const int64_t *__restrict__ ids, float *__restrict__ out) {
+// indexing.go:8-26: the MaxInt64 id selects a row of zeros.  Any other id outside [0, n_src) makes the CPU loop
+// panic on its bounds check; a kernel cannot, so the row is written as zeros, nothing is read, and the device
+// handle's fault word is raised for the next synchronising call to report.
+__global__ __launch_bounds__(256) void k_index_select(const float *__restrict__ table, int64_t n_src, int64_t width,
+                                                      const int64_t *__restrict__ ids, float *__restrict__ out,
+                                                      int *fault) {
     const int64_t id = ids[blockIdx.x];
+    const bool in_range = id >= 0 && id < n_src;
+    if (!in_range && id != 0x7FFFFFFFFFFFFFFFll && threadIdx.x == 0) *fault = 1;
     float *orow = out + (size_t)blockIdx.x * width;
     for (int64_t c = threadIdx.x; c < width; c += blockDim.x)
-        orow[c] = id == 0x7FFFFFFFFFFFFFFFll ? 0.0f : table[id * width + c];
+        orow[c] = in_range ? table[id * width + c] : 0.0f;
 }
 
 // conv.go:251-267 / :373-389: c[b,i,j] = sum_l a[b,i,l] * B[b,l,j]; one output per thread,
@@ -169,6 +175,20 @@ __global__ __launch_bounds__(256) void k_matmul_f32(const float *__restrict__ a,
         for (int64_t l = 0; l < k; ++l) sum += ar[l] * bm[l * n + j];
     }
     c[(bb * m + i) * n + j] = sum;
+}
+
+
+// conv.go:373-389 with the strides CpuStorage.MatMul hands it for one batch (cpu/storage.go:893-910: the last two
+// strides of each layout): c[i,j] = sum_l a[i*ars + l*acs] * b[l*brs + j*bcs], l ascending, one f32 accumulator.
+__global__ __launch_bounds__(256) void k_matmul_f32_strided(const float *__restrict__ a, const float *__restrict__ b,
+                                                            float *__restrict__ c, int64_t n, int64_t k, int64_t ars,
+                                                            int64_t acs, int64_t brs, int64_t bcs) {
+    const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = blockIdx.y;
+    if (j >= n) return;
+    float sum = 0.0f;
+    for (int64_t l = 0; l < k; ++l) sum += a[i * ars + l * acs] * b[l * brs + j * bcs];
+    c[i * n + j] = sum;
 }
 
 
@@ -304,6 +324,21 @@ int candy_hip_matmul_f32(candy_hip_device *dev, const float *a, const float *b, 
     return CANDY_HIP_OK;
 }
 
+int candy_hip_matmul_f32_strided(candy_hip_device *dev, const float *a, const float *b, float *c, int64_t m, int64_t n,
+                                 int64_t k, int64_t a_row_stride, int64_t a_col_stride, int64_t b_row_stride,
+                                 int64_t b_col_stride) {
+    CANDY_REQUIRE(m > 0 && n > 0 && k > 0, "invalid matrix dimensions");  // cpu/storage.go:877-879
+    CANDY_REQUIRE(a && b && c, "layouts cannot be nil");
+    CANDY_REQUIRE(m <= 65535, "matrix too large");
+    CANDY_REQUIRE(a_row_stride >= 0 && a_col_stride >= 0 && b_row_stride >= 0 && b_col_stride >= 0,
+                  "negative strides are not supported");
+    if (int rc = use_device(dev)) return rc;
+    hipLaunchKernelGGL(k_matmul_f32_strided, dim3(blocks_for(n), (unsigned)m), dim3(256), 0, dev->stream, a, b, c, n, k,
+                       a_row_stride, a_col_stride, b_row_stride, b_col_stride);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
 int candy_hip_rms_norm(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows, int64_t cols,
                        float *out) {
     CANDY_REQUIRE(rows >= 0 && cols >= 0 && cols <= 0x7FFFFFFF && rows <= 0x7FFFFFFF, "invalid dimensions");
@@ -368,7 +403,8 @@ int candy_hip_index_select(candy_hip_device *dev, const float *table, int64_t n_
     if (n_ids * width == 0) return CANDY_HIP_OK;
     CANDY_REQUIRE(table && dev_ids && out, "nil pointer");
     if (int rc = use_device(dev)) return rc;
-    hipLaunchKernelGGL(k_index_select, dim3((unsigned)n_ids), dim3(256), 0, dev->stream, table, width, dev_ids, out);
+    hipLaunchKernelGGL(k_index_select, dim3((unsigned)n_ids), dim3(256), 0, dev->stream, table, n_src, width, dev_ids, out,
+                       dev->fault);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }

@@ -89,20 +89,35 @@ int launch_q8_blocks_to_planar(candy_hip_device *dev, const void *blocks, int64_
 // Each lane writes whole float4 vectors so the (dominant) output stream is coalesced.
 // With `ids` set the kernels gather rows: output block b comes from row ids[b / bpr] of a
 // table with bpr blocks per row (embedding lookup, indexing.go:8-26 on a quantized table).
-__device__ __forceinline__ int64_t src_block(int64_t b, const int64_t *__restrict__ ids, int64_t bpr) {
-    return ids ? ids[b / bpr] * bpr + b % bpr : b;
+// An id outside [0, n_rows) cannot stop the kernel the way the CPU loop's bounds check stops the program: the
+// block is read from row 0 instead (a valid address) and the device handle's fault word is raised, which the
+// next synchronising call reports.
+struct Gather {
+    const int64_t *ids;  // null: no gather
+    int64_t bpr;         // blocks per table row
+    int64_t n_rows;      // rows of the table
+    int *fault;          // host-visible word of the device handle
+};
+__device__ __forceinline__ int64_t src_block(int64_t b, const Gather &g) {
+    if (!g.ids) return b;
+    int64_t row = g.ids[b / g.bpr];
+    if (row < 0 || row >= g.n_rows) {
+        *g.fault = 1;
+        row = 0;
+    }
+    return row * g.bpr + b % g.bpr;
 }
 
 // quantized.go:85-93: y[2j] = d*(lo(qs[j])-8), y[2j+1] = d*(hi(qs[j])-8). 8 lanes per block, one float4 each
 // (a lane that wrote two float4 32 bytes apart left every store instruction half-filling its lines: 2.9 TB/s).
 __global__ __launch_bounds__(256) void k_dequant_q4_0(const BlockQ4_0 *__restrict__ blocks, int64_t nb,
-        const int64_t *__restrict__ ids, int64_t bpr,
+        const Gather gather,
                                                       float4 *__restrict__ y, int ggml_order) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t b = t >> 3;
     if (b >= nb) return;
     const int j = (int)(t & 7);  // values 4j..4j+3
-    const BlockQ4_0 *blk = blocks + src_block(b, ids, bpr);
+    const BlockQ4_0 *blk = blocks + src_block(b, gather);
     const float d = half_bits_to_float(blk->d);
     float v[4];
     if (ggml_order) {  // quantized.cu:862-866: low nibbles fill y[0..15], high nibbles y[16..31]; d*q + (-8 d)
@@ -122,13 +137,13 @@ __global__ __launch_bounds__(256) void k_dequant_q4_0(const BlockQ4_0 *__restric
 
 // quantized.go:131-136: y[i] = d*qs[i]. 8 lanes per block.
 __global__ __launch_bounds__(256) void k_dequant_q8_0(const BlockQ8_0 *__restrict__ blocks, int64_t nb,
-        const int64_t *__restrict__ ids, int64_t bpr,
+        const Gather gather,
                                                       float4 *__restrict__ y) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t b = t >> 3;
     if (b >= nb) return;
     const int j = (int)(t & 7);
-    const BlockQ8_0 *blk = blocks + src_block(b, ids, bpr);
+    const BlockQ8_0 *blk = blocks + src_block(b, gather);
     const float d = half_bits_to_float(blk->d);
     const uint32_t q = *(const u32_a2 *)(blk->qs + 4 * j);
     y[t] = make_float4(d * (float)(int8_t)(q & 0xFF), d * (float)(int8_t)((q >> 8) & 0xFF),
@@ -138,14 +153,14 @@ __global__ __launch_bounds__(256) void k_dequant_q8_0(const BlockQ8_0 *__restric
 // quantized.cu:1008-1041: group il of 64 values, low nibbles with (sc, m) of sub-block 2il,
 // high nibbles with those of 2il+1; y = (d*sc)*q - (dmin*m). 32 lanes per super-block.
 __global__ __launch_bounds__(256) void k_dequant_q4_k(const BlockQ4K *__restrict__ blocks, int64_t nb,
-        const int64_t *__restrict__ ids, int64_t bpr,
+        const Gather gather,
                                                       float4 *__restrict__ y) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t b = t >> 5;
     if (b >= nb) return;
     const int il = (int)(t & 31) >> 3;  // 64-value group
     const int ir = (int)(t & 7);        // 4 bytes within the group's 32
-    const uint32_t *w = (const uint32_t *)(blocks + src_block(b, ids, bpr));  // 144-byte blocks keep 16-byte alignment
+    const uint32_t *w = (const uint32_t *)(blocks + src_block(b, gather));  // 144-byte blocks keep 16-byte alignment
     const uint32_t dm = w[0];
     const float dall = half_bits_to_float((uint16_t)(dm & 0xFFFF));
     const float dmin = half_bits_to_float((uint16_t)(dm >> 16));
@@ -167,14 +182,14 @@ __global__ __launch_bounds__(256) void k_dequant_q4_k(const BlockQ4K *__restrict
 
 // quantized.cu:1103-1128. 16 lanes per super-block, each 4 consecutive `il` of one half.
 __global__ __launch_bounds__(256) void k_dequant_q6_k(const BlockQ6K *__restrict__ blocks, int64_t nb,
-        const int64_t *__restrict__ ids, int64_t bpr,
+        const Gather gather,
                                                       float4 *__restrict__ y) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t b = t >> 4;
     if (b >= nb) return;
     const int ip = (int)(t & 15) >> 3;
     const int il0 = ((int)(t & 7)) * 4;
-    const BlockQ6K *blk = blocks + src_block(b, ids, bpr);
+    const BlockQ6K *blk = blocks + src_block(b, gather);
     const float d = half_bits_to_float(blk->d);
     const uint32_t ql0 = *(const u32_a2 *)(blk->ql + 64 * ip + il0);
     const uint32_t ql1 = *(const u32_a2 *)(blk->ql + 64 * ip + 32 + il0);
@@ -199,20 +214,20 @@ __global__ __launch_bounds__(256) void k_dequant_q6_k(const BlockQ6K *__restrict
 // The other formats: one lane per float4 of output, F::quad gives values 4j .. 4j+3 of a block.
 template <class F>
 __global__ __launch_bounds__(256) void k_dequant_more(const uint8_t *__restrict__ blocks, int64_t nb,
-                                                      const int64_t *__restrict__ ids, int64_t bpr, float4 *__restrict__ y) {
+                                                      const Gather gather, float4 *__restrict__ y) {
     constexpr int LPB = F::ELEMS / 4;
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t b = t / LPB;
     if (b >= nb) return;
-    y[t] = F::quad(blocks + src_block(b, ids, bpr) * F::BYTES, (int)(t - b * LPB));
+    y[t] = F::quad(blocks + src_block(b, gather) * F::BYTES, (int)(t - b * LPB));
 }
 
 template <class F>
-static int launch_dequant_more(candy_hip_device *dev, const void *blocks, int64_t nb, const int64_t *ids, int64_t bpr, float *out) {
+static int launch_dequant_more(candy_hip_device *dev, const void *blocks, int64_t nb, const Gather &gather, float *out) {
     const int64_t grid = (nb * (F::ELEMS / 4) + 255) / 256;
     CANDY_REQUIRE(grid <= 0x7FFFFFFF, "too many blocks");
-    hipLaunchKernelGGL(k_dequant_more<F>, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const uint8_t *)blocks, nb, ids,
-                       bpr, (float4 *)out);
+    hipLaunchKernelGGL(k_dequant_more<F>, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const uint8_t *)blocks, nb, gather,
+                       (float4 *)out);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
@@ -238,7 +253,7 @@ using namespace candy;
 extern "C" {
 
 static int dequantize_impl(candy_hip_device *dev, int fmt, const void *dev_blocks, int64_t n_blocks,
-                           const int64_t *ids, int64_t bpr, float *dev_out) {
+                           const int64_t *ids, int64_t bpr, int64_t n_rows, float *dev_out) {
     FormatInfo fi = format_info(fmt);
     CANDY_REQUIRE(fi.elems != 0, "unknown quantized format %d", fmt);
     CANDY_REQUIRE(n_blocks >= 0, "negative block count");
@@ -247,15 +262,16 @@ static int dequantize_impl(candy_hip_device *dev, int fmt, const void *dev_block
     CANDY_REQUIRE(((uintptr_t)dev_out & 15) == 0, "output must be 16-byte aligned");
     CANDY_REQUIRE(((uintptr_t)dev_blocks & (uintptr_t)(block_alignment(fmt) - 1)) == 0, "blocks are misaligned");
     if (int rc = use_device(dev)) return rc;
+    const Gather gather{ids, bpr, n_rows, dev->fault};
     switch (fmt) {
-    case CANDY_HIP_Q4_1: return launch_dequant_more<FmtQ4_1<false>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
-    case CANDY_HIP_Q4_1_GGML: return launch_dequant_more<FmtQ4_1<true>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
-    case CANDY_HIP_Q5_0: return launch_dequant_more<FmtQ5<false>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
-    case CANDY_HIP_Q5_1: return launch_dequant_more<FmtQ5<true>>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
-    case CANDY_HIP_Q2_K: return launch_dequant_more<FmtQ2K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
-    case CANDY_HIP_Q3_K: return launch_dequant_more<FmtQ3K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
-    case CANDY_HIP_Q5_K: return launch_dequant_more<FmtQ5K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
-    case CANDY_HIP_Q8_K: return launch_dequant_more<FmtQ8K>(dev, dev_blocks, n_blocks, ids, bpr, dev_out);
+    case CANDY_HIP_Q4_1: return launch_dequant_more<FmtQ4_1<false>>(dev, dev_blocks, n_blocks, gather, dev_out);
+    case CANDY_HIP_Q4_1_GGML: return launch_dequant_more<FmtQ4_1<true>>(dev, dev_blocks, n_blocks, gather, dev_out);
+    case CANDY_HIP_Q5_0: return launch_dequant_more<FmtQ5<false>>(dev, dev_blocks, n_blocks, gather, dev_out);
+    case CANDY_HIP_Q5_1: return launch_dequant_more<FmtQ5<true>>(dev, dev_blocks, n_blocks, gather, dev_out);
+    case CANDY_HIP_Q2_K: return launch_dequant_more<FmtQ2K>(dev, dev_blocks, n_blocks, gather, dev_out);
+    case CANDY_HIP_Q3_K: return launch_dequant_more<FmtQ3K>(dev, dev_blocks, n_blocks, gather, dev_out);
+    case CANDY_HIP_Q5_K: return launch_dequant_more<FmtQ5K>(dev, dev_blocks, n_blocks, gather, dev_out);
+    case CANDY_HIP_Q8_K: return launch_dequant_more<FmtQ8K>(dev, dev_blocks, n_blocks, gather, dev_out);
     default: break;
     }
     const int lanes_per_block = fmt == CANDY_HIP_Q4_K ? 32 : fmt == CANDY_HIP_Q6_K ? 16 : 8;
@@ -265,19 +281,19 @@ static int dequantize_impl(candy_hip_device *dev, int fmt, const void *dev_block
     switch (fmt) {
     case CANDY_HIP_Q4_0:
     case CANDY_HIP_Q4_0_GGML:
-        hipLaunchKernelGGL(k_dequant_q4_0, g, blk, 0, dev->stream, (const BlockQ4_0 *)dev_blocks, n_blocks, ids, bpr,
+        hipLaunchKernelGGL(k_dequant_q4_0, g, blk, 0, dev->stream, (const BlockQ4_0 *)dev_blocks, n_blocks, gather,
                            (float4 *)dev_out, fmt == CANDY_HIP_Q4_0_GGML ? 1 : 0);
         break;
     case CANDY_HIP_Q8_0:
-        hipLaunchKernelGGL(k_dequant_q8_0, g, blk, 0, dev->stream, (const BlockQ8_0 *)dev_blocks, n_blocks, ids, bpr,
+        hipLaunchKernelGGL(k_dequant_q8_0, g, blk, 0, dev->stream, (const BlockQ8_0 *)dev_blocks, n_blocks, gather,
                            (float4 *)dev_out);
         break;
     case CANDY_HIP_Q4_K:
-        hipLaunchKernelGGL(k_dequant_q4_k, g, blk, 0, dev->stream, (const BlockQ4K *)dev_blocks, n_blocks, ids, bpr,
+        hipLaunchKernelGGL(k_dequant_q4_k, g, blk, 0, dev->stream, (const BlockQ4K *)dev_blocks, n_blocks, gather,
                            (float4 *)dev_out);
         break;
     case CANDY_HIP_Q6_K:
-        hipLaunchKernelGGL(k_dequant_q6_k, g, blk, 0, dev->stream, (const BlockQ6K *)dev_blocks, n_blocks, ids, bpr,
+        hipLaunchKernelGGL(k_dequant_q6_k, g, blk, 0, dev->stream, (const BlockQ6K *)dev_blocks, n_blocks, gather,
                            (float4 *)dev_out);
         break;
     }
@@ -287,7 +303,7 @@ static int dequantize_impl(candy_hip_device *dev, int fmt, const void *dev_block
 
 int candy_hip_dequantize_blocks(candy_hip_device *dev, int fmt, const void *dev_blocks, int64_t n_blocks,
                                 float *dev_out) {
-    return dequantize_impl(dev, fmt, dev_blocks, n_blocks, nullptr, 1, dev_out);
+    return dequantize_impl(dev, fmt, dev_blocks, n_blocks, nullptr, 1, 0, dev_out);
 }
 
 int candy_hip_qindex_select(candy_hip_device *dev, const candy_hip_qtensor *q, const int64_t *dev_ids, int64_t n_ids,
@@ -298,7 +314,7 @@ int candy_hip_qindex_select(candy_hip_device *dev, const candy_hip_qtensor *q, c
     if (n_ids == 0) return CANDY_HIP_OK;
     CANDY_REQUIRE(dev_ids, "ids is nil");
     const int64_t bpr = q->cols / format_info(q->fmt).elems;
-    return dequantize_impl(dev, q->fmt, q->data, n_ids * bpr, dev_ids, bpr, out);
+    return dequantize_impl(dev, q->fmt, q->data, n_ids * bpr, dev_ids, bpr, q->rows, out);
 }
 
 int candy_hip_dequantize(candy_hip_device *dev, const candy_hip_qtensor *q, float *dev_out) {

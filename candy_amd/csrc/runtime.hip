@@ -53,6 +53,16 @@ int use_device(const candy_hip_device *dev) {
     return CANDY_HIP_OK;
 }
 
+int check_fault(candy_hip_device *dev) {
+    volatile int *f = dev->fault;
+    if (f && *f) {
+        *f = 0;
+        return fail(CANDY_HIP_ERR_INVALID, "an index-select on this device met an id outside its table (indexing.go:8-26 "
+                                           "panics there); the rows it selected are not valid");
+    }
+    return CANDY_HIP_OK;
+}
+
 int workspace(candy_hip_device *dev, size_t bytes, void **out) {
     if (bytes > dev->ws_bytes) {
         // Work already enqueued may still read the old buffer.
@@ -144,6 +154,8 @@ int candy_hip_open(int ordinal, candy_hip_device **out) {
     hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&dev->ev_start);
     if (e == hipSuccess) e = hipEventCreate(&dev->ev_stop);
+    if (e == hipSuccess) e = hipHostMalloc((void **)&dev->fault, 64, hipHostMallocDefault);  // pinned: kernels store to it
+    if (e == hipSuccess) *dev->fault = 0;
     if (e != hipSuccess) {
         candy_hip_close(dev);
         return fail(CANDY_HIP_ERR_HIP, "creating stream/events failed: %s", hipGetErrorString(e));
@@ -158,6 +170,7 @@ int candy_hip_close(candy_hip_device *dev) {
     if (dev->stream) (void)hipStreamSynchronize(dev->stream);
     if (dev->ws) (void)hipFree(dev->ws);
     if (dev->ws_split) (void)hipFree(dev->ws_split);
+    if (dev->fault) (void)hipHostFree(dev->fault);
     if (dev->ev_start) (void)hipEventDestroy(dev->ev_start);
     if (dev->ev_stop) (void)hipEventDestroy(dev->ev_stop);
     if (dev->stream) (void)hipStreamDestroy(dev->stream);
@@ -180,7 +193,7 @@ int candy_hip_device_name(const candy_hip_device *dev, char *buf, size_t buf_len
 int candy_hip_synchronize(candy_hip_device *dev) {
     if (int rc = use_device(dev)) return rc;
     CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
-    return CANDY_HIP_OK;
+    return check_fault(dev);
 }
 
 int candy_hip_alloc(candy_hip_device *dev, size_t bytes, void **dptr) {
@@ -231,7 +244,7 @@ int candy_hip_d2h(candy_hip_device *dev, void *dst_host, const void *src_dev, si
     if (int rc = use_device(dev)) return rc;
     CANDY_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, dev->stream));
     CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
-    return CANDY_HIP_OK;
+    return check_fault(dev);
 }
 
 int candy_hip_d2d(candy_hip_device *dev, void *dst_dev, const void *src_dev, size_t bytes) {

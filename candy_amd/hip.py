@@ -70,6 +70,8 @@ SIGNATURES = {
     "candy_hip_qact_quantize": (c_int, [c_void_p, c_void_p, c_int64, c_int64]),
     "candy_hip_qmatmul_qact": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "candy_hip_matmul_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int]),
+    "candy_hip_matmul_f32_strided": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                             c_int64, c_int64, c_int64]),
     "candy_hip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p]),
     "candy_hip_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "candy_hip_softmax": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
@@ -308,6 +310,14 @@ class Device:
         dc = self.alloc(max(batch * m * n * 4, 4))
         _check(lib().candy_hip_matmul_f32(self.handle, da.ptr, db.ptr, dc.ptr, batch, m, n, k, int(rhs_transposed)))
         return dc.download(np.float32, batch * m * n)
+
+    def matmul_f32_strided(self, a, b, m, n, k, a_strides, b_strides, a_offset=0, b_offset=0) -> np.ndarray:
+        """One batch; a_strides / b_strides are (row, column) element strides, the offsets the layouts' start offsets."""
+        da, db = self._f32(a), self._f32(b)
+        dc = self.alloc(m * n * 4)
+        _check(lib().candy_hip_matmul_f32_strided(self.handle, da.ptr + 4 * a_offset, db.ptr + 4 * b_offset, dc.ptr, m, n, k,
+                                                  a_strides[0], a_strides[1], b_strides[0], b_strides[1]))
+        return dc.download(np.float32, m * n)
 
     def rms_norm(self, x, cols: int, eps: float, alpha=None) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32).reshape(-1)

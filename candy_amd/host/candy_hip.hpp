@@ -153,21 +153,28 @@ public:
         if (!rhs) return {nullptr, Errorf("rhs storage must be HipStorage")};
         if (!lhsLayout || !rhsLayout) return {nullptr, Errorf("layouts cannot be nil")};
         if (m <= 0 || n <= 0 || k <= 0) return {nullptr, Errorf("invalid matrix dimensions")};
-        if (!lhsLayout->IsContiguous()) return {nullptr, Errorf("lhs must be contiguous on the HIP backend")};
-        int transposed = 0;
-        if (!rhsLayout->IsContiguous()) {
-            // the only strided rhs on the path: Linear's W^T view, strides {1, k} (nn/linear.go:65)
-            auto st = rhsLayout->Stride();
-            const int r = rhsLayout->Rank();
-            if (b != 1 || r < 2 || st[r - 2] != 1 || st[r - 1] != k)
-                return {nullptr, Errorf("rhs must be contiguous or a transposed [n, k] weight view")};
-            transposed = 1;
-        }
         auto out = Alloc(dev_, (size_t)b * m * n);
         if (!out.ok()) return out;
-        if (Error e = last_error(candy_hip_matmul_f32(dev_->handle(), (const float *)ptr_, (const float *)rhs->ptr_,
-                                                      (float *)out.value->ptr_, b, m, n, k, transposed), "matmul"))
-            return {nullptr, e};
+        const float *lp = (const float *)ptr_ + lhsLayout->StartOffset(), *rp = (const float *)rhs->ptr_ + rhsLayout->StartOffset();
+        int rc;
+        if (lhsLayout->IsContiguous() && rhsLayout->IsContiguous()) {
+            rc = candy_hip_matmul_f32(dev_->handle(), lp, rp, (float *)out.value->ptr_, b, m, n, k, 0);
+        } else if (b == 1) {
+            // one batch through the last two strides of each layout (cpu/storage.go:893-910); Linear's W^T view,
+            // strides {1, k} (nn/linear.go:65), is the case on the hot path
+            auto ls = lhsLayout->Stride(), rs = rhsLayout->Stride();
+            const int lr = lhsLayout->Rank(), rr = rhsLayout->Rank();
+            if (lr < 2 || rr < 2) return {nullptr, Errorf("MatMul operands must have at least two dimensions")};
+            if (ls[lr - 2] < 0 || ls[lr - 1] < 0 || rs[rr - 2] < 0 || rs[rr - 1] < 0)
+                return {nullptr, Errorf("negative strides are not supported on the HIP backend")};
+            rc = candy_hip_matmul_f32_strided(dev_->handle(), lp, rp, (float *)out.value->ptr_, m, n, k, ls[lr - 2], ls[lr - 1],
+                                              rs[rr - 2], rs[rr - 1]);
+        } else {
+            // cpu/storage.go:911-926 multiplies such operands as if they were contiguous; that is a wrong answer,
+            // not a behaviour to keep
+            return {nullptr, Errorf("batched MatMul needs contiguous operands on the HIP backend")};
+        }
+        if (Error e = last_error(rc, "matmul")) return {nullptr, e};
         return out;
     }
 

@@ -167,6 +167,14 @@ int candy_hip_qmatmul_qact(candy_hip_device *dev, const candy_hip_qtensor *w, co
  * rhs is [b,n,k] (the strided W^T view nn/linear.go:65 creates).  CONV:251-267 / :373-389. */
 int candy_hip_matmul_f32(candy_hip_device *dev, const float *a, const float *b, float *c,
                          int64_t batch, int64_t m, int64_t n, int64_t k, int rhs_transposed);
+/* The same MatMul for one batch with operands viewed through strides, in elements: a[i, l] sits at
+ * a[i * a_row_stride + l * a_col_stride], b[l, j] at b[l * b_row_stride + j * b_col_stride] -- what
+ * cpu/storage.go:889-910 passes to CONV:373-389 (the last two strides of each Layout).  The caller adds each
+ * Layout's StartOffset() to the pointer it passes (cpu/storage.go:889-927 forgets it; this boundary does not).
+ * c is contiguous [m, n].  Layouts with a batch dimension must be contiguous (candy_hip_matmul_f32). */
+int candy_hip_matmul_f32_strided(candy_hip_device *dev, const float *a, const float *b, float *c, int64_t m, int64_t n,
+                                 int64_t k, int64_t a_row_stride, int64_t a_col_stride, int64_t b_row_stride,
+                                 int64_t b_col_stride);
 /* backend.go:150 FastRmsNorm; reduce.go:3071-3092.  alpha may be NULL. */
 int candy_hip_rms_norm(candy_hip_device *dev, const float *x, const float *alpha, float eps,
                        int64_t rows, int64_t cols, float *out);
@@ -184,7 +192,10 @@ int candy_hip_mul(candy_hip_device *dev, const float *a, const float *b, int64_t
 int candy_hip_silu_mul(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *out);
 /* backend.go:129 FastArgmax; reduce.go:846-862 (first maximum wins). */
 int candy_hip_argmax(candy_hip_device *dev, const float *src, int64_t rows, int64_t cols, uint32_t *out);
-/* IndexSelect along dim 0 of a [n_src, width] f32 table; indexing.go:8-26. ids are int64 on the device. */
+/* IndexSelect along dim 0 of a [n_src, width] f32 table; indexing.go:8-26. ids are int64 on the device; the
+ * MaxInt64 id selects zeros, as there.  Any other id outside [0, n_src) -- where the CPU loop panics on its bounds
+ * check -- reads nothing (f32 table: the row is zeros; quantized table: row 0 is read) and makes the next
+ * candy_hip_synchronize or candy_hip_d2h on the handle fail with CANDY_HIP_ERR_INVALID. */
 int candy_hip_index_select(candy_hip_device *dev, const float *table, int64_t n_src, int64_t width,
                            const int64_t *dev_ids, int64_t n_ids, float *out);
 /* Row gather from a quantized table (embedding lookup): dequantizes rows ids[i] of q. */

@@ -61,6 +61,9 @@
  *   co_vec_dot_q8_0       QCU:2058-2073, 2239-2263, 2367-2389 (shape of the float
  *                         combination); integer parts pinned with Python ints, the float
  *                         result against exact-arithmetic sum of dequantized products.
+ *   co_set_block_order    test aid, no reference counterpart: the same terms of a row added in another order
+ *                         (descending, even then odd, second half first).  Pinned: equals the ascending sum to
+ *                         1e-6 per Linear; the terms themselves are the pinned ones.
  *   co_qmatmul            authored here (candy has no CPU QMatMul); pinned as above.
  *   co_matmul_dequant_f32 CONV:373-389 applied to dequantized weights.
  *   co_naive_batched_*    CONV:251-267, 373-389. Pinned: reference fixtures of
@@ -519,6 +522,15 @@ static float make_qkx2_quants(int n, int nmax, const float *x, const float *weig
     return scale;
 }
 
+/* Test hooks: the two searches on their own, so that a test can hold their answer against a brute-force
+ * evaluation of every candidate the published algorithms name. */
+float co_make_qkx2_quants(int n, int nmax, const float *x, const float *weights, uint8_t *L, float *the_min,
+                          float rmin, float rdelta, int nstep) {
+    uint8_t Laux[256];
+    if (n < 1 || n > 256) return NAN;
+    return make_qkx2_quants(n, nmax, x, weights, L, the_min, Laux, rmin, rdelta, nstep);
+}
+
 /* quantize_row_q4_K_ref for one super-block: eight 32-value sub-blocks get (scale, min) from
  * make_qkx2_quants with weights rms + |x|; scales and mins are stored in 6 bits relative to their
  * maxima (d, dmin in fp16), then the levels are assigned again with the STORED scales. */
@@ -621,6 +633,8 @@ static float make_qx_quants(int n, int nmax, const float *x, int8_t *L) {
     }
     return scale;
 }
+
+float co_make_qx_quants(int n, int nmax, const float *x, int8_t *L) { return make_qx_quants(n, nmax, x, L); }
 
 /* quantize_row_q6_K_ref for one super-block: sixteen 16-value groups, each with a make_qx_quants
  * scale; the scale of largest magnitude maps to -128 in int8 (d in fp16 carries its sign), then
@@ -886,7 +900,35 @@ static float vec_dot_q5_k(const co_block_q5_k *w, const co_block_q8_0 *x, int64_
     return acc;
 }
 
+/* Other, equally valid orders of the same f32 additions: 0 the blocks (super-blocks) of a row ascending, as
+ * everywhere else in this file; 1 descending; 2 the even-numbered blocks ascending, then the odd-numbered ones;
+ * 3 the second half of the row, then the first.  Nothing in the reference prescribes the order (QCU:2787-2871
+ * spreads the blocks of a row over the lanes of a warp and adds the lanes' partial sums in a tree); the others
+ * exist so that tests can measure, on the CPU alone, how far correct evaluations of one model drift apart. */
+static int g_block_order = 0;
+void co_set_block_order(int order) { g_block_order = (order >= 0 && order <= 3) ? order : 0; }
+
+static float vec_dot_ascending(int fmt, const void *w_row, const void *x_q8_0, int64_t k);
+
 float co_vec_dot_q8_0(int fmt, const void *w_row, const void *x_q8_0, int64_t k) {
+    if (g_block_order == 0) return vec_dot_ascending(fmt, w_row, x_q8_0, k);
+    const int qk = co_block_elems(fmt), bs = co_block_bytes(fmt);
+    if (qk == 0 || k % qk != 0) return NAN;
+    const int64_t nu = k / qk;
+    float acc = 0.0f;
+    for (int64_t i = 0; i < nu; ++i) {
+        int64_t u = i;
+        if (g_block_order == 1) u = nu - 1 - i;
+        else if (g_block_order == 2) u = i < (nu + 1) / 2 ? 2 * i : 2 * (i - (nu + 1) / 2) + 1;
+        else if (g_block_order == 3) u = (i + nu / 2) % nu;
+        /* one block at a time: 0.0f + its term is the term itself */
+        acc += vec_dot_ascending(fmt, (const uint8_t *)w_row + (size_t)u * (size_t)bs,
+                                 (const uint8_t *)x_q8_0 + (size_t)u * (size_t)(qk / 32) * 34, qk);
+    }
+    return acc;
+}
+
+static float vec_dot_ascending(int fmt, const void *w_row, const void *x_q8_0, int64_t k) {
     const co_block_q8_0 *x = (const co_block_q8_0 *)x_q8_0;
     switch (fmt) {
     case CO_Q4_1: return vec_dot_q4_1((const co_block_q4_1 *)w_row, x, k / 32, 0);

@@ -59,8 +59,18 @@ int co_quantize_q8_0(const float *x, int64_t rows, int64_t cols, void *out_block
  * above): x is rows*cols f32, cols a multiple of the block; out receives rows*cols/qk blocks. */
 int co_quantize(int fmt, const float *x, int64_t rows, int64_t cols, void *out_blocks);
 
+/* Test hooks on the scale searches inside co_quantize (Q4_K sub-blocks: n = 32, nmax = 15, rmin = -1,
+ * rdelta = 0.1, nstep = 20, weights rms + |x|; Q6_K groups: n = 16, nmax = 32). */
+float co_make_qkx2_quants(int n, int nmax, const float *x, const float *weights, uint8_t *L, float *the_min,
+                          float rmin, float rdelta, int nstep);
+float co_make_qx_quants(int n, int nmax, const float *x, int8_t *L);
+
 /* One weight row (k/qk blocks) against one activation row (k/32 Q8_0 blocks). */
 float co_vec_dot_q8_0(int fmt, const void *w_row, const void *x_q8_0, int64_t k);
+
+/* Test aid: the order in which co_vec_dot_q8_0 (and everything built on it) adds a row's blocks: 0 ascending
+ * (the default), 1 descending, 2 even-numbered then odd-numbered, 3 second half then first.  Process-wide. */
+void co_set_block_order(int order);
 
 /* y[m, rows] = x[m, cols] . W^T with activations quantized to Q8_0 first. */
 int co_qmatmul(int fmt, const void *w_blocks, int64_t rows, int64_t cols,

@@ -49,6 +49,12 @@ def lib() -> ctypes.CDLL:
         L.co_quantize.restype = ctypes.c_int
         L.co_vec_dot_q8_0.argtypes = [ctypes.c_int, vp, vp, i64]
         L.co_vec_dot_q8_0.restype = f32
+        L.co_make_qkx2_quants.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, f32, f32, ctypes.c_int]
+        L.co_make_qkx2_quants.restype = f32
+        L.co_make_qx_quants.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp]
+        L.co_make_qx_quants.restype = f32
+        L.co_set_block_order.argtypes = [ctypes.c_int]
+        L.co_set_block_order.restype = None
         L.co_qmatmul.argtypes = [ctypes.c_int, vp, i64, i64, vp, i64, vp]
         L.co_matmul_dequant_f32.argtypes = [ctypes.c_int, vp, i64, i64, vp, i64, vp]
         L.co_naive_batched_matmul_f32.argtypes = [i64, i64, i64, i64, vp, vp, vp]
@@ -150,8 +156,31 @@ def quantize(fmt: int, x, rows: int | None = None, cols: int | None = None) -> n
     return out
 
 
+def make_qkx2_quants(x, weights, nmax=15, rmin=-1.0, rdelta=0.1, nstep=20):
+    """Test hook: (scale, -min, levels) of the Q4_K sub-block search."""
+    x, weights = _f32(x).reshape(-1), _f32(weights).reshape(-1)
+    L = np.zeros(x.size, np.uint8)
+    the_min = np.zeros(1, np.float32)
+    scale = lib().co_make_qkx2_quants(x.size, nmax, _p(x), _p(weights), _p(L), _p(the_min), rmin, rdelta, nstep)
+    return float(scale), float(the_min[0]), L
+
+
+def make_qx_quants(x, nmax=32):
+    """Test hook: (scale, levels + nmax) of the Q6_K group search."""
+    x = _f32(x).reshape(-1)
+    L = np.zeros(x.size, np.int8)
+    scale = lib().co_make_qx_quants(x.size, nmax, _p(x), _p(L))
+    return float(scale), L
+
+
 def vec_dot_q8_0(fmt: int, w_row, x_q8_0, k: int) -> float:
     return lib().co_vec_dot_q8_0(fmt, _p(_u8(w_row)), _p(_u8(x_q8_0)), k)
+
+
+def set_block_order(order: int):
+    """Test aid: the order vec-dots add a row's blocks in (0 ascending, 1 descending, 2 even then odd, 3 second
+    half first); process-wide."""
+    lib().co_set_block_order(int(order))
 
 
 def qmatmul(fmt: int, w_blocks, rows: int, cols: int, x) -> np.ndarray:

@@ -90,6 +90,27 @@ int main() {
         auto r = xs->MatMul(&lx, ws, &lwt, 1, m, n, k);
         CHECK(r.ok() && rel_err(r.value->Data(), want) < 1e-5, "Linear-shaped MatMul");
     }
+    // ---- other strided views of one batch, with start offsets: a column-major lhs window inside a larger buffer
+    //      times a row-strided rhs window (cpu/storage.go:893-910 takes the last two strides; its missing
+    //      StartOffset is not reproduced); a batched strided operand is an error, not a silent contiguous read
+    {
+        std::mt19937 rng(2);
+        std::normal_distribution<float> nd;
+        const int m = 5, n = 9, k = 17, a_off = 3, b_off = 7;
+        std::vector<float> abuf(a_off + k * m + 4), bbuf(b_off + k * (2 * n) + 4), want(m * n);
+        for (auto &v : abuf) v = nd(rng);
+        for (auto &v : bbuf) v = nd(rng);
+        // a[i, l] at a_off + i + l * m (strides {1, m}); b[l, j] at b_off + l * 2n + j * 2 (strides {2n, 2})
+        const int64_t as[3] = {0, 1, m}, bs[3] = {0, 2 * n, 2}, cs[3] = {0, n, 1};
+        co_naive_batched_matmul_strided_f32(1, m, n, k, abuf.data() + a_off, bbuf.data() + b_off, want.data(), as, bs, cs);
+        auto sa = F::FromSlice(dev, abuf).value, sb = F::FromSlice(dev, bbuf).value;
+        Layout la({m, k}, {1, m}, a_off), lb({k, n}, {2 * n, 2}, b_off);
+        auto r = sa->MatMul(&la, sb, &lb, 1, m, n, k);
+        CHECK(r.ok() && r.value->Data() == want, "strided MatMul with start offsets equals the CPU loop bit for bit");
+        Layout l3({2, m, k}, {m * k, 1, m}, 0), r3 = Layout::Contiguous({2, k, n});
+        CHECK(sa->MatMul(&l3, sb, &r3, 2, m, n, k).err.msg == "batched MatMul needs contiguous operands on the HIP backend",
+              "batched strided MatMul is refused");
+    }
     // ---- FastRmsNorm: reduce_test.go:1909-1971
     {
         auto x = F::FromSlice(dev, {1, 2, 3, 4, 5, 6}).value;

@@ -6,7 +6,7 @@ import math
 import numpy as np
 import pytest
 
-from candy_amd import hip
+from candy_amd import hip, synth
 from oracle import oracle as o
 
 pytestmark = pytest.mark.gpu
@@ -40,6 +40,50 @@ def test_reference_vectors(dev, golden):
     for c in golden["silu_f32"]:
         want = [x / (1 + math.exp(-x)) for x in c["inp"]]
         assert close(dev.silu(c["inp"]), want, 0, 1e-6), c["name"]
+
+
+def test_matmul_f32_strided_views_match_the_cpu_loop_bitwise(dev):
+    # one batch through arbitrary (row, column) strides and start offsets: the call CpuStorage.MatMul makes for any
+    # non-contiguous layout (cpu/storage.go:893-910 -> conv.go:373-389)
+    rng = np.random.default_rng(11)
+    m, n, k = 7, 33, 50
+    abuf = rng.standard_normal(5 + m * k * 2).astype(np.float32)
+    bbuf = rng.standard_normal(9 + k * n * 3).astype(np.float32)
+    for (ast, bst, ao, bo) in (((k, 1), (1, k), 0, 0),           # Linear: contiguous x, W^T view
+                               ((1, m), (n, 1), 5, 0),           # transposed lhs with an offset
+                               ((2 * k, 2), (3, 3 * k), 3, 9),   # every-other-column lhs, strided W^T view, both offset
+                               ((k, 1), (0, 1), 0, 2)):          # broadcast rows of rhs (stride 0)
+        got = dev.matmul_f32_strided(abuf, bbuf, m, n, k, ast, bst, ao, bo)
+        want = o.naive_batched_matmul_strided_f32(1, m, n, k, abuf[ao:], bbuf[bo:], [0, ast[0], ast[1]],
+                                                  [0, bst[0], bst[1]], [0, n, 1], m * n)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (ast, bst)
+    with pytest.raises(hip.CandyHipError, match="negative strides"):
+        dev.matmul_f32_strided(abuf, bbuf, m, n, k, (k, -1), (n, 1))
+
+
+def test_index_select_out_of_range_ids_are_reported_not_read(dev):
+    # indexing.go:8-26 panics on an id outside the table (Go bounds check); the kernels read nothing there, write
+    # zeros, and the next synchronising call on the handle fails
+    table = np.arange(12, dtype=np.float32).reshape(4, 3)
+    ids = np.array([2, 0x7FFFFFFFFFFFFFFF, 0], np.int64)
+    assert np.array_equal(dev.index_select(table, ids), np.stack([table[2], np.zeros(3, np.float32), table[0]]))
+    for bad in (4, -1, 1 << 40):
+        dt, di = dev.from_numpy(table), dev.from_numpy(np.array([1, bad], np.int64))
+        out = dev.alloc(2 * 3 * 4)
+        hip._check(hip.lib().candy_hip_index_select(dev.handle, dt.ptr, 4, 3, di.ptr, 2, out.ptr))
+        with pytest.raises(hip.CandyHipError, match="outside its table"):
+            dev.synchronize()
+        dev.synchronize()  # reported once, then clear
+        got = out.download(np.float32, 6).reshape(2, 3)
+        assert np.array_equal(got[0], table[1]) and not got[1].any()
+    w = synth.random_weight(synth.Q8_0, 4, 64, seed=3)
+    q = dev.qtensor(synth.Q8_0, 4, 64, w)
+    di = dev.from_numpy(np.array([3, 4], np.int64))
+    out = dev.alloc(2 * 64 * 4)
+    hip._check(hip.lib().candy_hip_qindex_select(dev.handle, q.handle, di.ptr, 2, out.ptr))
+    with pytest.raises(hip.CandyHipError, match="outside its table"):
+        out.download(np.float32, 128)
+    dev.synchronize()
 
 
 def test_matmul_f32_matches_naive_loop_bitwise(dev):

@@ -129,6 +129,21 @@ def test_q6_k_head_shape(dev):
     assert rel_err(got[:, sub], o.qmatmul(synth.Q6_K, wb, len(sub), cols, x)) <= 2e-5
 
 
+def test_q6_k_llama3_head_shape(dev):
+    # the Llama-3 output head, 128256 x 4096 in Q6_K (431 MB), batch 1: oracle on a strided row subset, the exact
+    # scaling property over every row
+    rows, cols = 128256, 4096
+    w = synth.random_weight(synth.Q6_K, rows, cols, seed=808)
+    x = synth.random_activations(1, cols, seed=809)
+    q = dev.qtensor(synth.Q6_K, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    sub = np.arange(0, rows, 501)
+    wb = w.reshape(rows, -1)[sub].reshape(-1)
+    assert rel_err(got[:, sub], o.qmatmul(synth.Q6_K, wb, len(sub), cols, x)) <= 2e-5
+    assert np.array_equal(dev.qmatmul(q, 2 * x), 2 * got)
+    q.free()
+
+
 def test_qmatmul_from_prequantized_blocks(dev):
     rows, cols, m = 64, 1024, 3
     w = synth.random_weight(synth.Q4_K, rows, cols, seed=1)

@@ -173,3 +173,112 @@ def test_quantize_dispatch_and_shapes():
     a = o.dequantize(Q4_0, o.quantize(Q4_0, x))
     b = o.dequantize(Q4_0_GGML, o.quantize(Q4_0_GGML, x))
     assert np.array_equal(a, b)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The scale searches against a brute-force evaluation of every candidate the published algorithms name
+# (make_qkx2_quants: min/max rounding, then inverse scales (rmin + rdelta * is + nmax) / (max - min) for
+# is = 0 .. nstep, each followed by the weighted least-squares (scale, min) of the levels it yields, the smallest
+# weighted squared error wins; make_qx_quants: -(nmax + 0.1 * is) / max for is = -9 .. 9, the largest
+# (sum w x l)^2 / (sum w l^2) wins).  Evaluated here in float64, vectorised, from that description: a search that
+# tries one candidate too few, steps by another amount or fits differently picks a worse candidate on some input.
+# This pins the oracle to the stated candidate set; whether ggml's set is this one stays unpinned (no ggml here).
+
+def _round_half_even(v):
+    return np.rint(v)  # numpy rounds to nearest even, like the 1.5 * 2^23 trick
+
+
+def _qkx2_search(x32, w32, nmax=15, rmin=-1.0, rdelta=0.1, nstep=20):
+    """The published search, step by step: returns (error, levels, steps that improved the error, clear) where
+    clear says that no accept / reject decision was closer than 1e-3 (so f32 and f64 must agree on every one).
+    Note the published quirk: a step that improves the error also replaces `min`, which the following steps use
+    for their inverse scale and their level assignment."""
+    f32 = np.float32
+    x, w = x32.astype(np.float64), w32.astype(np.float64)
+    mn, mx = min(f32(x32.min()), f32(0)), f32(x32.max())
+
+    def levels(numerator, mn):  # the level assignment in f32, as stated; sums and errors in f64
+        isc = f32(numerator) / (mx - f32(mn))
+        return np.clip(_round_half_even(isc * (x32 - f32(mn))), 0, nmax).astype(np.float64), float(isc)
+
+    L, isc = levels(nmax, mn)
+    best = float(np.sum(w * ((1 / isc) * L + float(mn) - x) ** 2))
+    improved, clear = [], True
+    sw, sx = w.sum(), (w * x).sum()
+    for k in range(nstep + 1):
+        La, _ = levels(f32(rmin) + f32(rdelta) * f32(k) + f32(nmax), mn)
+        sl, sl2, sxl = (w * La).sum(), (w * La * La).sum(), (w * La * x).sum()
+        D = sw * sl2 - sl * sl
+        if D <= 0:
+            continue
+        sc, m = (sw * sxl - sx * sl) / D, (sl2 * sx - sl * sxl) / D
+        if m > 0:
+            m, sc = 0.0, sxl / sl2
+        mad = float(np.sum(w * (sc * La + m - x) ** 2))
+        if np.array_equal(La, L) and improved:
+            continue  # the levels of the best step so far: the same fit, the same error, no decision to take
+        if abs(mad - best) <= 1e-3 * best:
+            clear = False
+        if mad < best:
+            improved.append((k, (best - mad) / best))
+            best, L, mn = mad, La, m
+    return best, L, improved, clear
+
+
+def test_q4_k_sub_block_search_follows_the_published_steps():
+    # The search is a chain of f32 comparisons whose later steps depend on the earlier outcomes, so an f64
+    # re-evaluation can part ways with it on single blocks (a level on a rounding boundary, a near tie).  What is
+    # held: on the blocks where every decision has a margin the two agree almost always, and for every step k the
+    # blocks on which step k is the last one to cut the error, by 2 % or more, end at that lower error in the
+    # oracle too -- a search that stops one step early, steps by another width or fits differently loses them.
+    rng = np.random.default_rng(2024)
+    by_last_step = {}
+    n_clear = n_agree = 0
+    for trial in range(20000):
+        kind = trial % 3
+        x = (rng.standard_normal(32) * 0.02 if kind == 0 else rng.uniform(-1, 1, 32) if kind == 1
+             else rng.standard_normal(32) ** 3).astype(np.float32)
+        w = (np.sqrt(np.mean(x.astype(np.float64) ** 2)) + np.abs(x)).astype(np.float32)
+        scale, the_min, L = o.make_qkx2_quants(x, w)
+        got = float(np.sum(w.astype(np.float64) * (scale * L.astype(np.float64) - the_min - x) ** 2))
+        best, Lb, improved, clear = _qkx2_search(x, w)
+        if not clear:
+            continue
+        n_clear += 1
+        agree = abs(got - best) <= 1e-2 * best + 1e-12
+        n_agree += int(agree)
+        if improved and improved[-1][1] >= 0.02:
+            by_last_step.setdefault(improved[-1][0], []).append(agree)
+    assert n_clear > 10000 and n_agree > 0.97 * n_clear, (n_clear, n_agree)
+    for k in range(21):
+        hits = by_last_step.get(k, [])
+        assert len(hits) >= 3 and np.mean(hits) >= 0.8, (k, len(hits), float(np.mean(hits)) if hits else None)
+
+
+def test_q6_k_group_search_picks_the_best_published_candidate():
+    rng = np.random.default_rng(7)
+    winners = set()
+    for trial in range(6000):
+        x = (rng.standard_normal(16) * 0.02 if trial % 2 else rng.standard_normal(16) ** 3).astype(np.float32)
+        scale, L = o.make_qx_quants(x)
+        xd = x.astype(np.float64)
+        mx = xd[np.argmax(np.abs(xd))]
+        wt = xd * xd
+        by_levels = {}
+        for k in range(-9, 10):
+            isc = np.float32(-(np.float32(32) + np.float32(0.1) * np.float32(k))) / x[np.argmax(np.abs(xd))]
+            l = np.clip(_round_half_even(isc * x), -32, 31).astype(np.float64)  # level assignment in f32, as stated
+            slx, sl2 = float(np.sum(wt * xd * l)), float(np.sum(wt * l * l))
+            if sl2 > 0:
+                by_levels.setdefault(tuple(l), [slx * slx / sl2, l, set()])[2].add(k)
+        cands = sorted(by_levels.values(), key=lambda c: -c[0])
+        l_got = L.astype(np.float64) - 32
+        slx, sl2 = float(np.sum(wt * xd * l_got)), float(np.sum(wt * l_got * l_got))
+        assert slx * slx / sl2 >= cands[0][0] * (1 - 2e-6), trial  # the objective is flat: candidates differ by 1e-5
+        assert abs(scale - slx / sl2) <= 1e-5 * abs(scale)  # and the scale is the least-squares one of its levels
+        if len(cands) == 1 or cands[0][0] > cands[1][0] * (1 + 1e-5):
+            assert np.array_equal(l_got, cands[0][1]), trial
+            winners |= cands[0][2]
+    # every step -9 .. 9 reaches the best levels somewhere in the sample (neighbouring steps mostly share their
+    # levels, so this does not show that each single step is tried; the per-block maximum above is what is held)
+    assert winners >= set(range(-9, 10)), sorted(set(range(-9, 10)) - winners)
