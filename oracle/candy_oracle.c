@@ -957,6 +957,9 @@ int co_qmatmul(int fmt, const void *w_blocks, int64_t rows, int64_t cols,
     co_quantize_q8_0(x, m, cols, xq);
     size_t row_bytes = (size_t)(cols / qk) * (size_t)bs;
     size_t xrow_bytes = (size_t)(cols / 32) * 34;
+    /* every output is its own chain of operations: spreading the outputs over threads changes no bit
+     * (the candy CPU path itself is single-threaded; the timed baseline, co_matmul_dequant_f32, stays so) */
+    #pragma omp parallel for collapse(2) schedule(static)
     for (int64_t i = 0; i < m; ++i)
         for (int64_t n = 0; n < rows; ++n)
             y[i * rows + n] = co_vec_dot_q8_0(fmt, (const uint8_t *)w_blocks + (size_t)n * row_bytes,
