@@ -80,6 +80,8 @@ struct candy_hip_device {
     // One word of pinned host memory that kernels raise when they meet an index outside its table (the condition
     // the CPU path panics on); check_fault() reports and clears it after a synchronisation.
     int *fault = nullptr;
+    // This GPU's copy of the library's file-scope scratch array (matvec.hip), resolved when the handle is opened.
+    void *noalloc_scratch = nullptr;
 };
 
 struct candy_hip_qtensor {
@@ -151,6 +153,8 @@ int launch_q8_blocks_to_planar(candy_hip_device *dev, const void *blocks, int64_
 // vector_only: never the int8 tile kernel (whose K split takes a workspace), whatever the batch.
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                   const Q8Scale *scales, int64_t m, float *y, bool vector_only = false);
+// matvec.hip: resolves this GPU's address of the file-scope scratch array (dev's GPU must be current).
+int noalloc_scratch_init(candy_hip_device *dev);
 // matvec.hip: one activation row against up to three weights in one launch, optional residuals.
 int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *ws, float *const *ys,
                         const float *const *res, int n, const int8_t *qs, const Q8Scale *scales);

@@ -620,6 +620,20 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
     }
 }
 
+// Scratch of the allocation-free entry point: the quantized activations of one call (planar quants, then scales).
+// One copy per GPU for the life of the process; every call on a GPU shares it.
+constexpr size_t NOALLOC_SCRATCH_BYTES = size_t(1) << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+int noalloc_scratch_init(candy_hip_device *dev) {
+    // The array's name is only a handle on the host: the address kernels may use is this GPU's, asked for here.
+    void *p = nullptr;
+    CANDY_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    CANDY_REQUIRE(p && ((uintptr_t)p & 255) == 0, "scratch array is not where it was declared to be");
+    dev->noalloc_scratch = p;
+    return CANDY_HIP_OK;
+}
+
 int mmq_min_m(const candy_hip_device *dev) { return dev->opt.mmq_min_m < 16 ? 16 : dev->opt.mmq_min_m; }
 
 int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
@@ -662,6 +676,26 @@ int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const f
     if (int rc = act_workspace(dev, m, w->cols, true, &a)) return rc;
     if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, a.qs, a.scales, nullptr)) return rc;
     return contract(dev, w, a, m, dev_y);
+}
+
+int candy_hip_qmatmul_noalloc(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m,
+                              float *dev_y) {
+    if (int rc = qmatmul_check(dev, w, m, dev_y)) return rc;
+    if (m == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(dev_x, "lhs is nil");
+    CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "lhs must be 16-byte aligned");
+    CANDY_REQUIRE(m <= 15, "the allocation-free contraction takes 1 .. 15 activation rows, got %lld", (long long)m);
+    const size_t q_bytes = ((size_t)(m * w->cols) + 255) & ~(size_t)255;
+    const size_t s_bytes = ((size_t)(m * (w->cols >> 5)) * sizeof(Q8Scale) + 255) & ~(size_t)255;
+    CANDY_REQUIRE(q_bytes + s_bytes <= NOALLOC_SCRATCH_BYTES,
+                  "%lld x %lld activations need %zu bytes of scratch, the allocation-free contraction has %zu",
+                  (long long)m, (long long)w->cols, q_bytes + s_bytes, NOALLOC_SCRATCH_BYTES);
+    CANDY_REQUIRE(dev->noalloc_scratch, "device handle has no scratch address");
+    if (int rc = use_device(dev)) return rc;
+    int8_t *qs = (int8_t *)dev->noalloc_scratch;  // the address hipGetSymbolAddress gave for this GPU, never the array's name
+    Q8Scale *scales = (Q8Scale *)((uint8_t *)dev->noalloc_scratch + q_bytes);
+    if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, qs, scales, nullptr)) return rc;
+    return launch_matvec(dev, w, qs, scales, m, dev_y, /*vector_only=*/true);
 }
 
 int candy_hip_qmatmul_q8(candy_hip_device *dev, const candy_hip_qtensor *w, const void *dev_x_q8_0, int64_t m,

@@ -160,6 +160,10 @@ int candy_hip_open(int ordinal, candy_hip_device **out) {
         candy_hip_close(dev);
         return fail(CANDY_HIP_ERR_HIP, "creating stream/events failed: %s", hipGetErrorString(e));
     }
+    if (int rc = noalloc_scratch_init(dev)) {  // this GPU is current: its copy of the scratch array
+        candy_hip_close(dev);
+        return rc;
+    }
     *out = dev;
     return CANDY_HIP_OK;
 }

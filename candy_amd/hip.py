@@ -64,6 +64,7 @@ SIGNATURES = {
     "candy_hip_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "candy_hip_quantize": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p]),
     "candy_hip_qmatmul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "candy_hip_qmatmul_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "candy_hip_qmatmul_q8": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "candy_hip_qact_create": (c_int, [c_void_p, c_int64, c_int64, POINTER(c_void_p)]),
     "candy_hip_qact_free": (c_int, [c_void_p]),

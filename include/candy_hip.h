@@ -147,6 +147,16 @@ int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64
 int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x,
                       int64_t m, float *dev_y);
 
+/* candy_hip_qmatmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no counterpart in the reference.  Same result as candy_hip_qmatmul,
+ * 1 <= m <= 15 activation rows (the matvec family; the vector kernels answer every batch, so from 5 rows on the
+ * bits may differ from candy_hip_qmatmul's tile kernel by f32 summation order).  The quantized activations live
+ * in a 1 MiB array inside the library that every call on a GPU shares: a call whose m * cols * 1.25 bytes (plus
+ * rounding to 256) exceed it fails with CANDY_HIP_ERR_INVALID, and calls that overlap on one GPU (two handles,
+ * two threads) race on it.  Calls no hipMalloc / hipFree. */
+int candy_hip_qmatmul_noalloc(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m,
+                              float *dev_y);
+
 /* Same contraction, activations already in Q8_0 blocks on the device ([m, cols/32] blocks). */
 int candy_hip_qmatmul_q8(candy_hip_device *dev, const candy_hip_qtensor *w, const void *dev_x_q8_0,
                          int64_t m, float *dev_y);
