@@ -158,10 +158,12 @@ __global__ __launch_bounds__(256) void k_index_select(const float *__restrict__ 
 }
 
 // conv.go:251-267 / :373-389: c[b,i,j] = sum_l a[b,i,l] * B[b,l,j]; one output per thread,
-// l ascending, single f32 accumulator (the CPU loop's order).
+// l ascending, single f32 accumulator (the CPU loop's order), the product rounded before it is added (no fused
+// multiply-add: the Go compiler does not fuse on amd64), so the result is the CPU loop's bit for bit.
 __global__ __launch_bounds__(256) void k_matmul_f32(const float *__restrict__ a, const float *__restrict__ b,
                                                     float *__restrict__ c, int64_t m, int64_t n, int64_t k,
                                                     int rhs_transposed) {
+#pragma clang fp contract(off)
     const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t i = blockIdx.y, bb = blockIdx.z;
     if (j >= n) return;
@@ -183,6 +185,7 @@ __global__ __launch_bounds__(256) void k_matmul_f32(const float *__restrict__ a,
 __global__ __launch_bounds__(256) void k_matmul_f32_strided(const float *__restrict__ a, const float *__restrict__ b,
                                                             float *__restrict__ c, int64_t n, int64_t k, int64_t ars,
                                                             int64_t acs, int64_t brs, int64_t bcs) {
+#pragma clang fp contract(off)
     const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t i = blockIdx.y;
     if (j >= n) return;

@@ -93,12 +93,12 @@ def test_matmul_f32_matches_naive_loop_bitwise(dev):
     bm = rng.standard_normal((b, k, n)).astype(np.float32)
     got = dev.matmul_f32(a, bm, b, m, n, k)
     want = o.naive_batched_matmul_f32(b, m, n, k, a, bm)
-    # same accumulation order (l ascending, one f32 accumulator); only FMA contraction may differ
-    assert close(got, want, 1e-5, 1e-5)
+    # same accumulation order (l ascending, one f32 accumulator), products rounded before the add: the same bits
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     wt = rng.standard_normal((n, k)).astype(np.float32)  # Linear's transposed weight view
     got_t = dev.matmul_f32(a[0], wt, 1, m, n, k, rhs_transposed=True)
     want_t = o.naive_batched_matmul_strided_f32(1, m, n, k, a[0], wt, [0, k, 1], [0, 1, k], [0, n, 1], m * n)
-    assert close(got_t, want_t, 1e-5, 1e-5)
+    assert np.array_equal(got_t.view(np.uint32), want_t.view(np.uint32))
     with pytest.raises(hip.CandyHipError, match="invalid matrix dimensions"):
         dev.matmul_f32(a, bm, 1, 0, n, k)
 
