@@ -130,6 +130,24 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 
+// 1 / sqrt(v) as reduce.go:3083-3085 evaluates it for RMSNorm: 1 / float32(math.Sqrt(float64(v))).  The square root
+// of an f32 taken in f64 and rounded back is the correctly rounded f32 square root (53 bits >= 2 * 24 + 2), which is
+// what sqrtf is here (hipcc rounds f32 sqrt and division correctly by default), so no f64 instruction is needed.
+__device__ __forceinline__ float rms_inv_sqrt(float v) { return 1.0f / sqrtf(v); }
+
+// (int)roundf(x / d) with the IEEE division of quantize_q8_1 (quantized.cu:3546-3547), without dividing in the
+// common case: x * (1 / d) with the hardware reciprocal is within 2 ulp of the quotient, and the two can only round
+// to different integers when a half-integer lies between them, i.e. when the product is within a few ulp of one.
+// Only then (and for products outside the range of levels: d subnormal, x not finite) is the division carried out.
+__device__ __forceinline__ int q8_level(float x, float d) {
+    const float t = x * __builtin_amdgcn_rcpf(d);
+    const float a = fabsf(t);
+    const float frac = a - truncf(a);           // exact
+    const bool near_half = fabsf(frac - 0.5f) <= 6.1e-5f;  // 8 ulp of 127.5: the quotient never exceeds that here
+    if (__builtin_expect(near_half || !(a < 128.0f), 0)) return (int)roundf(x / d);
+    return (int)roundf(t);
+}
+
 // Q8_0 quantization of 4 consecutive values held by one lane; the 8 lanes that share a 32-value
 // block must be consecutive lanes of one wavefront (lane % 8 == position in the block) and all
 // active.  quantize_q8_1 (quantized.cu:3521-3558) without its `sum`: amax over the block,
@@ -144,10 +162,10 @@ __device__ __forceinline__ uint32_t quantize_q8_lane4(float4 v, __half &d_half, 
     const float d = amax / 127.0f;
     int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
     if (amax != 0.0f) {
-        q0 = (int)roundf(v.x / d);
-        q1 = (int)roundf(v.y / d);
-        q2 = (int)roundf(v.z / d);
-        q3 = (int)roundf(v.w / d);
+        q0 = q8_level(v.x, d);
+        q1 = q8_level(v.y, d);
+        q2 = q8_level(v.z, d);
+        q3 = q8_level(v.w, d);
     }
     int s = q0 + q1 + q2 + q3;
     s += dpp_move_i<0xB1>(s);
@@ -181,7 +199,7 @@ __device__ __forceinline__ int quantize_q8_lane1(float v, __half &d_half, int &b
     amax = fmaxf(amax, dpp_move<0x140>(amax));
     amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
     const float d = amax / 127.0f;
-    const int q = amax != 0.0f ? (int)roundf(v / d) : 0;
+    const int q = amax != 0.0f ? q8_level(v, d) : 0;
     int s = q;
     s += dpp_move_i<0xB1>(s);
     s += dpp_move_i<0x4E>(s);

@@ -137,7 +137,7 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) tot += s_red[i];
         const float mean = tot / (float)K;
-        const float scale = 1.0f / (float)sqrt((double)(mean + a.eps));
+        const float scale = rms_inv_sqrt(mean + a.eps);
 #pragma unroll
         for (int i = 0; i < XF; ++i) {
             const int c = tid + i * T;

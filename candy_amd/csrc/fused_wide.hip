@@ -1,0 +1,321 @@
+// Decode-step matvecs of the big Q4_K shapes as ONE workgroup per compute unit.
+//
+// The fused kernels of fused.hip give every workgroup 16 or 32 rows and let each of them repeat the prologue
+// (RMSNorm + Q8_0 quantization of the hidden state: 32 KB from L2, a reduction, a barrier).  On a 7B layer that is
+// 688 prologues for gate/up and 768 for q/k/v, 2 us of each launch, and row counts that do not divide by the CUs
+// leave some CUs a third more bytes than others.  Here the grid is a multiple of the CU count, every workgroup
+// takes an equal share of the rows (to within one row) wherever they fall, its 16 (or 8) wavefronts walk that
+// share round-robin with every weight load in flight before the first dot, and the prologue runs once per CU.
+//   prologue RMS:    RMSNorm (reduce.go:3071-3092) + Q8_0 quantization (quantized.cu:3521-3558) of the f32 input
+//   prologue QUANT:  Q8_0 quantization of the f32 input as it is (the whole f32-in -> f32-out QMatMul of one row
+//                    as one launch: the same quants and scales as the quantize kernel, hence the same result)
+//   epilogue PLAIN:  y = W.x (+ residual), up to three weights as one run of rows
+//   epilogue PAIR:   silu(gate.x) * (up.x) quantized to planar Q8_0 for the down projection; a 32-value block
+//                    whose rows belong to two workgroups is quantized by whichever of them finishes last
+// Contraction and units are those of the batch-1 kernel (matvec.hip, units.h): same integer dots, same order of
+// additions per row, so the results are the bits the narrower kernels give.
+#include <algorithm>
+
+#include "blocks.h"
+#include "internal.h"
+#include "units.h"
+
+namespace candy {
+
+enum { WPRO_RMS = 0, WPRO_QUANT = 1 };
+enum { WEPI_PLAIN = 0, WEPI_PAIR = 1 };
+
+struct WideArgs {
+    MatvecJobs jobs;         // PLAIN: up to 3 weights, wg_end = END ROW of each in the run; PAIR: j[0] gate, j[1] up
+    int total;               // rows of the run (PLAIN) or row pairs (PAIR)
+    int K;
+    // RMS prologue
+    const float *x, *alpha;
+    float eps;
+    // PAIR epilogue
+    int8_t *oq;
+    Q8Scale *os;
+    float *pair_act;         // total floats of scratch
+    unsigned *pair_tickets;  // total / 32 counters, zero before and after every launch
+};
+
+__device__ __forceinline__ float wide_silu(float x) { return x / (1.0f + expf(-x)); }
+
+// First item of workgroup g when `total` items are dealt to G workgroups as evenly as they go.
+__device__ __forceinline__ int wide_start(int g, int total, int G) { return (int)(((long long)g * total) / G); }
+// The workgroup that item p falls to under wide_start.
+__device__ __forceinline__ int wide_owner(int p, int total, int G) { return (int)((((long long)p + 1) * G - 1) / total); }
+
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec_wide(const WideArgs a) {
+    constexpr int T = WAVES * 64;
+    constexpr int CAP = ITER * 64 * U::ELEMS;   // activation values the LDS image is sized for
+    constexpr int XF = (CAP / 4 + T - 1) / T;   // float4 of prologue input per thread
+    constexpr int NW = EPI == WEPI_PAIR ? 2 : 1;
+    extern __shared__ __align__(16) uint8_t smem[];
+    int8_t *sq = (int8_t *)smem;
+    constexpr int QBYTES = XF * T * 4;
+    Q8Scale *ss = (Q8Scale *)(smem + QBYTES + ((QBYTES >> 8) << 4));
+    __shared__ float s_red[WAVES];
+    __shared__ float s_act[R * WAVES];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = a.K;
+    const int units = K / U::ELEMS;
+    const size_t rb = U::row_bytes(K);
+    const int G = gridDim.x;
+    const int start = wide_start(blockIdx.x, a.total, G), end = wide_start(blockIdx.x + 1, a.total, G);
+    const int n4 = K >> 2;
+
+    // ---- prologue inputs first (they return first)
+    float4 xv[XF], av[XF];
+#pragma unroll
+    for (int i = 0; i < XF; ++i) {
+        const int c = min(tid + i * T, n4 - 1);
+        xv[i] = ((const float4 *)a.x)[c];
+        if (PRO == WPRO_RMS) av[i] = ((const float4 *)a.alpha)[c];
+    }
+
+    // ---- every weight load of the wavefront: items start + wave + WAVES * r
+    typename U::W w[NW][R][ITER];
+    int job[R], jrow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int g = min(start + wave + WAVES * r, a.total - 1);  // clamped: a valid row, dropped at the store
+        if (EPI == WEPI_PAIR) {
+            job[r] = 0;
+            jrow[r] = g;
+        } else {
+            const int e0 = a.jobs.j[0].wg_end, e1 = a.jobs.j[1].wg_end;
+            const int ji = (int)(g >= e0) + (int)(g >= e1);
+            job[r] = ji;
+            jrow[r] = g - (ji == 0 ? 0 : ji == 1 ? e0 : e1);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < NW; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint8_t *row = a.jobs.j[EPI == WEPI_PAIR ? m : job[r]].W + (size_t)jrow[r] * rb;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
+        }
+
+    // ---- the activation row: normalised (or merged) and quantized into LDS, once per workgroup
+    float4 val[XF];
+    if (PRO == WPRO_QUANT) {
+#pragma unroll
+        for (int i = 0; i < XF; ++i) val[i] = xv[i];
+    } else if (PRO == WPRO_RMS) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < XF; ++i) {
+            const float4 v = xv[i];
+            const float t = v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            s += (tid + i * T < n4) ? t : 0.0f;
+        }
+        s = wave_sum(s);
+        if (lane == 0) s_red[wave] = s;
+        __syncthreads();
+        float tot = 0.0f;
+#pragma unroll
+        for (int i = 0; i < WAVES; ++i) tot += s_red[i];
+        const float mean = tot / (float)K;
+        const float scale = rms_inv_sqrt(mean + a.eps);
+#pragma unroll
+        for (int i = 0; i < XF; ++i) {
+            const float4 v = xv[i], al = av[i];
+            val[i] = make_float4(scale * v.x * al.x, scale * v.y * al.y, scale * v.z * al.z, scale * v.w * al.w);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < XF; ++i) {
+        const int c = tid + i * T;
+        __half hd;
+        int bsum;
+        const uint32_t packed = quantize_q8_lane4(val[i], hd, bsum);
+        *(uint32_t *)(sq + skewed(4 * c)) = packed;  // c past the row lands in the padding
+        if ((c & 7) == 0) {
+            Q8Scale sc;
+            sc.d = __half2float(hd);
+            sc.bsum = bsum;
+            ss[c >> 3] = sc;
+        }
+    }
+    __syncthreads();
+
+    // ---- contraction
+    float acc[NW][R];
+#pragma unroll
+    for (int m = 0; m < NW; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int u = it * 64 + lane;
+        const bool live = u < units;
+        const int uc = live ? u : units - 1;
+#pragma unroll
+        for (int m = 0; m < NW; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float v = U::dot(w[m][r][it], uc, sq, ss);
+                acc[m][r] += live ? v : 0.0f;
+            }
+    }
+
+    if (EPI == WEPI_PLAIN) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float v = wave_sum(acc[0][r]);
+            if (lane == 0 && start + wave + WAVES * r < end) {
+                float *y = a.jobs.j[job[r]].y;  // may alias res (h += W.x)
+                const float *res = a.jobs.j[job[r]].res;
+                y[jrow[r]] = res ? res[jrow[r]] + v : v;
+            }
+        }
+        return;
+    }
+
+    // ---- PAIR: silu(gate) * up of this workgroup's pairs, then the 32-value blocks they belong to
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float g = wave_sum(acc[0][r]), u = wave_sum(acc[1][r]);
+        if (lane == 0) s_act[wave + WAVES * r] = wide_silu(g) * u;  // slots past `end` hold a clamped row: never read
+    }
+    __syncthreads();
+    const int b0 = start >> 5, b1 = (end - 1) >> 5;
+    for (int blk = b0 + wave; blk <= b1; blk += WAVES) {  // wavefront-uniform: one block per wavefront
+        const int first = blk << 5;
+        const int lo = max(start, first), hi = min(end, first + 32);
+        const int l32 = lane & 31;
+        float mine;
+        if (hi - lo == 32) {
+            mine = s_act[first + l32 - start];
+        } else {
+            // Part of the block lies with a neighbouring workgroup.  This part goes to pair_act with agent-scope
+            // atomic stores, which on gfx950 write through to the memory side where every XCD sees them; the store
+            // counter reaching zero means they have arrived (no release fence: that would write the whole L2 back).
+            // Then a ticket of the block is drawn; whoever draws the last one reads all 32 values back with
+            // agent-scope atomic loads (which do not hit a stale cache line), quantizes them, and puts the counter
+            // back to zero.  This rests on those two hardware properties, not on the HIP memory model.
+            if (lane < 32 && first + lane >= lo && first + lane < hi)
+                __hip_atomic_store(a.pair_act + first + lane, s_act[first + lane - start], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            const unsigned expected = (unsigned)(wide_owner(first + 31, a.total, G) - wide_owner(first, a.total, G) + 1);
+            unsigned old = 0;
+            if (lane == 0) old = __hip_atomic_fetch_add(a.pair_tickets + blk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
+            if (old != expected - 1) continue;  // a later workgroup finishes the block
+            asm volatile("" ::: "memory");
+            mine = __hip_atomic_load(a.pair_act + first + l32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) __hip_atomic_store(a.pair_tickets + blk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __half hd;
+        int bsum;
+        const int q = quantize_q8_lane1(mine, hd, bsum);
+        if (lane < 32) a.oq[(size_t)first + lane] = (int8_t)q;
+        if (lane == 0) {
+            Q8Scale sc;
+            sc.d = __half2float(hd);
+            sc.bsum = bsum;
+            a.os[blk] = sc;
+        }
+    }
+}
+
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
+static int launch_wide_cfg(candy_hip_device *dev, const WideArgs &a, int grid) {
+    constexpr int T = WAVES * 64, CAP = ITER * 64 * U::ELEMS;
+    constexpr int XF = (CAP / 4 + T - 1) / T;
+    constexpr size_t QBYTES = (size_t)XF * T * 4;
+    constexpr size_t smem = QBYTES + ((QBYTES >> 8) << 4) + ((size_t)XF * T / 8 + 1) * 8;
+    static_assert(smem <= 48 * 1024, "LDS image too large");
+    hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+// The shapes these kernels exist for: Q4_K weights, rows up to 8192 values (two rounds of units), at least a
+// few rows per wavefront.  Anything else: CANDY_HIP_ERR_UNSUPPORTED without error text (the caller takes the
+// narrower kernels).
+int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
+    const int n = L.n;
+    if (n < 1 || n > 3 || !dev->opt.fused_wide) return CANDY_HIP_ERR_UNSUPPORTED;
+    const candy_hip_qtensor *w0 = L.w[0];
+    for (int i = 0; i < n; ++i) {
+        if (L.w[i]->fmt != CANDY_HIP_Q4_K || L.w[i]->cols != w0->cols || ((uintptr_t)L.w[i]->data & 15) != 0) return CANDY_HIP_ERR_UNSUPPORTED;
+        if (L.w[i]->rows > 0x3FFFFFFF) return CANDY_HIP_ERR_UNSUPPORTED;
+    }
+    const int64_t K = w0->cols;
+    if (K % 256 != 0 || K > 8192) return CANDY_HIP_ERR_UNSUPPORTED;
+    const int iter = (int)((K / 64 + 63) / 64);
+    const bool quant = L.alpha == nullptr;
+    if (!L.x || ((uintptr_t)L.x & 15) != 0) return CANDY_HIP_ERR_UNSUPPORTED;
+    if (quant && L.pair) return CANDY_HIP_ERR_UNSUPPORTED;
+    WideArgs a{};
+    a.jobs.n = n;
+    int rows = 0;
+    for (int i = 0; i < 3; ++i) {
+        if (i < n) {
+            a.jobs.j[i].W = (const uint8_t *)L.w[i]->data;
+            a.jobs.j[i].y = L.y[i];
+            a.jobs.j[i].res = L.res[i];
+            a.jobs.j[i].N = (int)L.w[i]->rows;
+            rows += (int)L.w[i]->rows;
+        }
+        a.jobs.j[i].wg_end = rows;
+    }
+    a.K = (int)K;
+    a.x = L.x; a.alpha = L.alpha; a.eps = L.eps;
+    a.oq = L.oq; a.os = L.os; a.pair_act = L.pair_act; a.pair_tickets = L.pair_tickets;
+    const int cus = dev->num_cus;
+    if (L.pair) {
+        if (n != 2 || L.w[0]->rows != L.w[1]->rows || w0->rows % 32 != 0 || !L.pair_act || !L.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
+        a.total = (int)w0->rows;
+        a.jobs.j[0].wg_end = a.jobs.j[1].wg_end = a.jobs.j[2].wg_end = a.total;
+        if (a.total < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
+        // one workgroup per CU; 16 wavefronts x 3 pairs while a CU's share fits, else 8 wavefronts x up to 8 pairs
+        // (the weights of a wavefront's pairs stay in registers: 24 per pair and round of units)
+        const int per = (a.total + cus - 1) / cus;
+        if (iter == 1 && dev->opt.wide_waves == 8) {  // two workgroups of eight wavefronts per CU
+            const int per2 = (a.total + 2 * cus - 1) / (2 * cus);
+            if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+            if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+        }
+        if (iter == 1) {
+            if (per <= 32) return launch_wide_cfg<UnitQ4K, 1, 2, 16, WPRO_RMS, WEPI_PAIR>(dev, a, cus);
+            if (per <= 48) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PAIR>(dev, a, cus);
+            if (per <= 64) return launch_wide_cfg<UnitQ4K, 1, 8, 8, WPRO_RMS, WEPI_PAIR>(dev, a, cus);
+            if (per <= 96) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+        }
+        return CANDY_HIP_ERR_UNSUPPORTED;
+    }
+    a.total = rows;
+    if (rows < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
+    const int per = (rows + cus - 1) / cus;
+    if (quant) {
+        // the whole f32-in -> f32-out contraction of one row as one launch: measured ahead of quantize + matvec only
+        // for short rows and one row per wavefront (4096 x 4096: 5.0 against 5.8 us; 11008 x 4096: 9.5 against 8.2;
+        // 4096 x 11008: 9.0 against 8.9), where the prologue's 16 KB do not hold the weight stream up
+        if (iter == 1 && per <= 16) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_QUANT, WEPI_PLAIN>(dev, a, cus);
+        return CANDY_HIP_ERR_UNSUPPORTED;
+    }
+    if (iter == 1) {
+        if (dev->opt.wide_waves == 8) {
+            const int per2 = (rows + 2 * cus - 1) / (2 * cus);
+            if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
+            if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
+            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
+        }
+        if (per <= 16) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
+        if (per <= 32) return launch_wide_cfg<UnitQ4K, 1, 2, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
+        if (per <= 48) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
+        if (per <= 64) return launch_wide_cfg<UnitQ4K, 1, 4, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
+        if (per <= 128) return launch_wide_cfg<UnitQ4K, 1, 4, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
+    }
+    return CANDY_HIP_ERR_UNSUPPORTED;
+}
+
+}  // namespace candy

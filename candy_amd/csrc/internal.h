@@ -60,6 +60,8 @@ struct Options {
     int rms_rows = 0;            // fused RMSNorm prologue: rows per workgroup, 16 / 24 (0: the most even split)
     int prefill_attention_valu = 0;  // prompt attention for head_dim 128 on the vector ALU instead of the matrix cores
     int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
+    int fused_wide = 1;          // decode step: one-workgroup-per-CU kernels for the big Q4_K shapes (0: the narrower ones)
+    int wide_waves = 8;          // wavefronts per workgroup of those kernels: 8 (two workgroups per CU) or 16 (one)
 };
 
 }  // namespace candy
@@ -202,6 +204,23 @@ struct FusedLaunch {
     unsigned *pair_tickets = nullptr;
 };
 int launch_matvec_fused(candy_hip_device *dev, const FusedLaunch &launch);
+// fused_wide.hip: the same contractions for the big Q4_K shapes as one workgroup per compute unit (an even share of
+// the rows each, the prologue once or twice per CU).  Prologue: RMSNorm + quantize of x (x, alpha, eps), or the
+// plain quantization of x (alpha null).  Returns CANDY_HIP_ERR_UNSUPPORTED (no error text) for shapes it does not cover.
+struct WideLaunch {
+    int n = 0;
+    const candy_hip_qtensor *w[3] = {nullptr, nullptr, nullptr};
+    float *y[3] = {nullptr, nullptr, nullptr};
+    const float *res[3] = {nullptr, nullptr, nullptr};
+    const float *x = nullptr, *alpha = nullptr;
+    float eps = 0.0f;
+    bool pair = false;
+    int8_t *oq = nullptr;
+    Q8Scale *os = nullptr;
+    float *pair_act = nullptr;
+    unsigned *pair_tickets = nullptr;
+};
+int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &launch);
 // attention.hip
 struct AttnLaunch {
     const float *q = nullptr;      // [n_heads, head_dim]; pre-Rope when k_new is set

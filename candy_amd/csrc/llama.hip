@@ -221,6 +221,7 @@ int candy_hip_llama_set_norm(candy_hip_llama *m, int which, int layer, const flo
 int candy_hip_llama_set_graph(candy_hip_llama *m, int enable) {
     CANDY_REQUIRE(m, "model is nil");
     m->use_graph = enable != 0;
+    m->graph_dirty = true;  // also the way to have a changed device option picked up: the step is captured again
     return CANDY_HIP_OK;
 }
 
@@ -268,11 +269,18 @@ static void *layer_cache(const candy_hip_llama *m, float *base, int l) {
 static int norm_linear(candy_hip_llama *m, const float *alpha, const candy_hip_qtensor *const *ws, float *const *ys,
                        int n) {
     const candy_hip_llama_config &c = m->cfg;
+    int rc;
+    WideLaunch Wd;
+    Wd.n = n;
+    for (int i = 0; i < n; ++i) { Wd.w[i] = ws[i]; Wd.y[i] = ys[i]; }
+    Wd.x = m->h; Wd.alpha = alpha; Wd.eps = c.rms_eps;
+    rc = launch_matvec_wide(m->dev, Wd);
+    if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     FusedLaunch F;
     F.n = n;
     for (int i = 0; i < n; ++i) { F.w[i] = ws[i]; F.y[i] = ys[i]; }
     F.x = m->h; F.alpha = alpha; F.eps = c.rms_eps;
-    int rc = launch_matvec_fused(m->dev, F);
+    rc = launch_matvec_fused(m->dev, F);
     if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     if ((rc = launch_rms_norm_quant(m->dev, m->h, alpha, c.rms_eps, 1, c.d_model, nullptr, m->xq, m->xs))) return rc;
     return launch_matvec_multi(m->dev, ws, ys, nullptr, n, m->xq, m->xs);
@@ -324,6 +332,16 @@ static int llama_enqueue_step(candy_hip_llama *m) {
         }
         if ((rc = linear_residual(m, L.wo))) return rc;  // h += Wo . att
         {   // RMSNorm + quantize + gate/up + SiLU*Mul + quantize
+            WideLaunch Wd;
+            Wd.n = 2; Wd.w[0] = L.gate; Wd.w[1] = L.up; Wd.pair = true;
+            Wd.x = m->h; Wd.alpha = L.ffn_norm; Wd.eps = c.rms_eps; Wd.oq = m->xq; Wd.os = m->xs;
+            Wd.pair_act = m->gate_o; Wd.pair_tickets = m->pair_tickets;
+            rc = launch_matvec_wide(dev, Wd);
+            if (rc == CANDY_HIP_OK) {
+                if ((rc = linear_residual(m, L.down))) return rc;  // h += Wdown . act
+                continue;
+            }
+            if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
             FusedLaunch F;
             F.n = 2; F.w[0] = L.gate; F.w[1] = L.up; F.pair = true;
             F.x = m->h; F.alpha = L.ffn_norm; F.eps = c.rms_eps; F.oq = m->xq; F.os = m->xs;
@@ -364,6 +382,9 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
             if (m->graph) CANDY_HIP_TRY(hipGraphDestroy(m->graph));
             m->graph_exec = nullptr;
             m->graph = nullptr;
+            // the gate/up kernels count on their per-block tickets being zero at launch and leave them so; a step
+            // that was cut short (an error, a device reset) may not have: start every new graph from zero
+            if ((rc = launch_zero(dev, m->pair_tickets, ((size_t)m->cfg.d_ffn / 32 + 1) * sizeof(unsigned)))) return rc;
             CANDY_HIP_TRY(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
             rc = llama_enqueue_step(m);
             hipError_t e = hipStreamEndCapture(dev->stream, &m->graph);
@@ -373,8 +394,9 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
             m->graph_dirty = false;
         }
         CANDY_HIP_TRY(hipGraphLaunch(m->graph_exec, dev->stream));
-    } else {
-        if ((rc = llama_enqueue_step(m))) return rc;
+    } else if ((rc = llama_enqueue_step(m))) {
+        (void)launch_zero(dev, m->pair_tickets, ((size_t)m->cfg.d_ffn / 32 + 1) * sizeof(unsigned));  // see above
+        return rc;
     }
     if (dev_logits) *dev_logits = m->logits;
     if (next_token) {

@@ -666,6 +666,20 @@ static int contract(candy_hip_device *dev, const candy_hip_qtensor *w, const Act
     return m < mmq_min_m(dev) ? launch_matvec(dev, w, a.qs, a.scales, m, y) : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws);
 }
 
+// f32 in -> f32 out.  One row against a big Q4_K weight is ONE launch (the row is quantized in the contraction's
+// prologue, once per compute unit); everything else quantizes into the workspace first.  Same quants either way.
+static int qmatmul_f32(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m, float *dev_y,
+                       const ActWorkspace &a) {
+    if (m == 1) {
+        WideLaunch Wd;
+        Wd.n = 1; Wd.w[0] = w; Wd.y[0] = dev_y; Wd.x = dev_x;
+        const int rc = launch_matvec_wide(dev, Wd);
+        if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+    }
+    if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, a.qs, a.scales, nullptr)) return rc;
+    return contract(dev, w, a, m, dev_y);
+}
+
 int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m, float *dev_y) {
     if (int rc = qmatmul_check(dev, w, m, dev_y)) return rc;
     if (m == 0) return CANDY_HIP_OK;
@@ -674,8 +688,7 @@ int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const f
     if (int rc = use_device(dev)) return rc;
     ActWorkspace a;
     if (int rc = act_workspace(dev, m, w->cols, true, &a)) return rc;
-    if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, a.qs, a.scales, nullptr)) return rc;
-    return contract(dev, w, a, m, dev_y);
+    return qmatmul_f32(dev, w, dev_x, m, dev_y, a);
 }
 
 int candy_hip_qmatmul_noalloc(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, int64_t m,
@@ -783,9 +796,9 @@ int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *cons
     if (int rc = launch_quantize_q8(dev, dev_x, m, K, a.qs, a.scales, nullptr)) return rc;
     CANDY_HIP_TRY(hipEventRecord(dev->ev_start, dev->stream));
     for (int i = 0; i < iters; ++i) {
-        if (quantize_each)
-            if (int rc = launch_quantize_q8(dev, dev_x, m, K, a.qs, a.scales, nullptr)) return rc;
-        if (int rc = contract(dev, ws[i % n_ws], a, m, dev_y)) return rc;
+        if (quantize_each) {
+            if (int rc = qmatmul_f32(dev, ws[i % n_ws], dev_x, m, dev_y, a)) return rc;
+        } else if (int rc = contract(dev, ws[i % n_ws], a, m, dev_y)) return rc;
     }
     CANDY_HIP_TRY(hipEventRecord(dev->ev_stop, dev->stream));
     CANDY_HIP_TRY(hipEventSynchronize(dev->ev_stop));

@@ -31,6 +31,8 @@ namespace candy {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ half2v bits_h2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
 
 constexpr int BIG_BK = 64;
 constexpr int BIG_PITCH = BIG_BK + 8;  // halves per LDS row (144 bytes)
@@ -49,20 +51,34 @@ struct BigQ4K {
 #pragma unroll
         for (int g = 0; g < 4; ++g) r.q[g] = *(const u32x2 *)(blk + 16 + g * 32 + c * 8);
     }
-    // group g holds sub-blocks 2g (low nibbles, k = 0..31 of the step) and 2g+1 (high nibbles, k = 32..63)
+    // group g holds sub-blocks 2g (low nibbles, k = 0..31 of the step) and 2g+1 (high nibbles, k = 32..63).
+    // A nibble n is placed in the mantissa of the half 1024 (bits 0x6400 | n = 1024 + n, exact), two nibbles per
+    // instruction, and each value is one mixed-precision multiply-add (f16 operand, f32 scale and offset, f32
+    // arithmetic, rounded once to fp16): (1024 + n) * (d*sc) + (-(dmin*m) - 1024 * (d*sc)) = (d*sc)*n - dmin*m.
+    // The offset's own f32 rounding (2^-24 of 1024 d*sc) is a thirtieth of the fp16 rounding that follows.
     __device__ static __forceinline__ void dequant(const Raw &r, int g, int c, half8 &o0, half8 &o1, int &k0, int &k1) {
         uint32_t sc2, m2;
         q4k_scale_min_pair(r.hdr.y, r.hdr.z, r.hdr.w, g, sc2, m2);
         const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFF));
         const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
         const float d_lo = d * (float)(sc2 & 0xFF), d_hi = d * (float)((sc2 >> 8) & 0xFF);
-        const float m_lo = dmin * (float)(m2 & 0xFF), m_hi = dmin * (float)((m2 >> 8) & 0xFF);
+        const float c_lo = fmaf(-1024.0f, d_lo, -(dmin * (float)(m2 & 0xFF)));
+        const float c_hi = fmaf(-1024.0f, d_hi, -(dmin * (float)((m2 >> 8) & 0xFF)));
         const u32x2 q = r.q[g];
 #pragma unroll
-        for (int l = 0; l < 8; ++l) {
-            const uint32_t byte = ((l < 4 ? q.x : q.y) >> (8 * (l & 3))) & 0xFF;
-            o0[l] = (_Float16)(d_lo * (float)(byte & 0xF) - m_lo);
-            o1[l] = (_Float16)(d_hi * (float)(byte >> 4) - m_hi);
+        for (int wi = 0; wi < 2; ++wi) {
+            const uint32_t w = wi ? q.y : q.x;
+            const uint32_t MAGIC = 0x64006400u, M = 0x000F000Fu;
+            const half2v l02 = bits_h2((w & M) | MAGIC), l13 = bits_h2(((w >> 8) & M) | MAGIC);
+            const half2v h02 = bits_h2(((w >> 4) & M) | MAGIC), h13 = bits_h2(((w >> 12) & M) | MAGIC);
+            o0[4 * wi + 0] = (_Float16)fmaf((float)l02[0], d_lo, c_lo);
+            o0[4 * wi + 1] = (_Float16)fmaf((float)l13[0], d_lo, c_lo);
+            o0[4 * wi + 2] = (_Float16)fmaf((float)l02[1], d_lo, c_lo);
+            o0[4 * wi + 3] = (_Float16)fmaf((float)l13[1], d_lo, c_lo);
+            o1[4 * wi + 0] = (_Float16)fmaf((float)h02[0], d_hi, c_hi);
+            o1[4 * wi + 1] = (_Float16)fmaf((float)h13[0], d_hi, c_hi);
+            o1[4 * wi + 2] = (_Float16)fmaf((float)h02[1], d_hi, c_hi);
+            o1[4 * wi + 3] = (_Float16)fmaf((float)h13[1], d_hi, c_hi);
         }
         k0 = c * 8;
         k1 = 32 + c * 8;

@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void k_rms_norm(const float *__restrict__ x, c
     for (int c = threadIdx.x; c < cols; c += blockDim.x) s += xr[c] * xr[c];
     s = block_reduce<false>(s, red);
     const float mean = s / (float)cols;
-    const float scale = 1.0f / (float)sqrt((double)(mean + eps));
+    const float scale = rms_inv_sqrt(mean + eps);
     for (int c = threadIdx.x; c < cols; c += blockDim.x)
         orow[c] = alpha ? scale * xr[c] * alpha[c] : scale * xr[c];
 }
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict_
     }
     s = block_reduce<false>(s, red);
     const float mean = s / (float)cols;
-    const float scale = 1.0f / (float)sqrt((double)(mean + eps));
+    const float scale = rms_inv_sqrt(mean + eps);
     const int n4_pad = (n4 + 255) & ~255;  // whole wavefronts take part in the cross-lane steps
     for (int c = threadIdx.x; c < n4_pad; c += 256) {
         const bool live = c < n4;

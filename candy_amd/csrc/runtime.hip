@@ -350,6 +350,8 @@ const OptionKey OPTION_KEYS[] = {
     {"fused.rms_rows", &candy::Options::rms_rows, 0, 24},
     {"prefill.attention_valu", &candy::Options::prefill_attention_valu, 0, 1},
     {"llama.graph", &candy::Options::llama_graph, 0, 1},
+    {"fused.wide", &candy::Options::fused_wide, 0, 1},
+    {"fused.wide_waves", &candy::Options::wide_waves, 8, 16},
 };
 const OptionKey *find_option(const char *key) {
     for (const OptionKey &k : OPTION_KEYS)

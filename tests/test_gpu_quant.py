@@ -77,6 +77,31 @@ def test_quantize_q8_0_edge_blocks(dev):
     assert list(blk["qs"][3 * 8][:8]) == [127, 1, -1, 2, -2, 3, -3, 127]
 
 
+def test_quantize_q8_0_quotients_next_to_half_integers(dev):
+    # The device forms x / d as x * (1 / d) and divides only where that product is within a few ulp of a
+    # half-integer (where the two could round to different levels).  Blocks built to sit on that edge: one element
+    # fixes the scale, the others are the f32 numbers around d * (k + 0.5) for every k, for many scales.
+    rng = np.random.default_rng(77)
+    rows = []
+    for trial in range(400):
+        amax = np.float32(rng.uniform(0.01, 100.0) * 10.0 ** rng.integers(-3, 3))
+        d = np.float32(amax / np.float32(127.0))
+        ks = rng.integers(0, 127, 31)
+        halves = (d.astype(np.float64) * (ks + 0.5)).astype(np.float32)
+        steps = rng.integers(-3, 4, 31)
+        xs = halves.copy()
+        for i, st in enumerate(steps):  # walk a few representable numbers to either side of the midpoint
+            for _ in range(abs(int(st))):
+                xs[i] = np.nextafter(xs[i], np.float32(np.inf if st > 0 else -np.inf))
+        xs *= rng.choice(np.array([-1.0, 1.0], np.float32), 31)
+        rows.append(np.concatenate([[amax if trial % 2 else -amax], xs]).astype(np.float32))
+    x = np.stack(rows)
+    got, want = dev.quantize_q8_0(x), o.quantize_q8_0(x)
+    assert np.array_equal(got, want)
+    levels = want.view(synth.BLOCK_DTYPES[synth.Q8_0])["qs"]
+    assert np.abs(levels).max() == 127 and len(np.unique(np.abs(levels))) > 100
+
+
 def test_quantize_q8_0_errors(dev):
     with pytest.raises(hip.CandyHipError, match="multiple of the block size"):
         dev.quantize_q8_0(np.zeros((2, 48), np.float32))
