@@ -468,11 +468,11 @@ def main():
 
     if not args.no_prefill:
         # batched prefill: Q4_K 14336x4096 x f32 [M, 4096], f32 in -> f32 out (activation quantization included).
-        # m < 256 runs on the int8 matrix cores (exact integer dots; peak 5.0 POP/s), m >= 256 on fp16 tiles
-        # (peak 2.5 PFLOP/s).  roofline_us = the larger of the bytes at 8 TB/s and the contraction at that peak.
+        # m < 96 runs on the int8 matrix cores (exact integer dots; peak 5.0 POP/s), m >= 96 on fp16 tiles
+        # (operands rounded to fp16, 3e-4 per matmul; peak 2.5 PFLOP/s).  roofline_us = the larger of the bytes at 8 TB/s and the contraction at that peak.
         pre = []
         r, k = 14336, 4096
-        big_min = dev.get_option("mmq.f16_big_min_m")
+        big_min = dev.get_option("mmq.f16_api_min_m")
         for m in (16, 128, 512):
             ms, _ = time_matvec(dev, synth.Q4_K, r, k, 200, 20, quantize_each=True, seed=m, m=m)
             flops = 2.0 * m * r * k
@@ -480,7 +480,7 @@ def main():
             int8 = m < big_min
             peak = MFMA_I8_PEAK_TOPS if int8 else MFMA_F16_PEAK_TFLOPS
             roof_us = max(byts / (HBM_PEAK_GBPS * 1e9), flops / (peak * 1e12)) * 1e6
-            pre.append({"m": m, "kernel": ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else "k_mmq_f16<BigQ4K,128,256,2,4> (fp16 MFMA)",
+            pre.append({"m": m, "kernel": ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else ("k_mmq_f16<BigQ4K,128,%d,2,4> (fp16 MFMA)" % (128 if m <= 128 else 256)),
                         "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
                         "mfma_peak_TFLOPs": peak, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / peak, 4),
                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),

@@ -53,7 +53,8 @@ struct Options {
     int small_batch_kernel = 1;  // 2..8 rows: the one-workgroup-per-CU kernel (0: the looping kernel only)
     int i8_min_m = 0;            // 5..15 rows: int8 tiles from this batch on (0: whichever the fitted times say)
     int mmq_min_m = 16;          // batch from which the tile kernels take over from the matvec family (>= 16)
-    int f16_big_min_m = 256;     // batch from which the fp16 big tiles take over from the int8 tiles
+    int f16_big_min_m = 256;     // decoder prompt pass: batch from which the fp16 big tiles take over from the int8 tiles
+    int f16_api_min_m = 96;      // candy_hip_qmatmul*: the same threshold for a single contraction (3e-4 per matmul)
     int mmq_fp16_only = 0;       // 1: every tile contraction on the single-buffered fp16 tiles
     int i8_grid_split = 1;       // int8 tiles: split K over workgroups on small grids
     int pair_rows = 0;           // fused gate/up: row pairs per workgroup, 32 / 16 / 8 (0: the most even split)
@@ -166,15 +167,16 @@ int64_t mmq_m_pad(int64_t m);
 bool mmq_fuses_residual(const candy_hip_qtensor *w, int64_t m);
 // xh_ready (optional): the activations already expanded to fp16 [>= mmq_m_pad(m) rows][cols] (rows past m
 // may hold anything); res (optional, may alias y): y = res + x . W^T.
+// f16_min_m: batch from which the fp16 big tiles may answer (0: the decoder's threshold, opt.f16_big_min_m)
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                const Q8Scale *scales, int64_t m, float *y, void *half_ws, const _Float16 *xh_ready = nullptr,
-               const float *res = nullptr);
+               const float *res = nullptr, int f16_min_m = 0);
 // mmq_i8.hip: Q4_K / Q6_K on v_mfma_i32_16x16x32_i8 with the batch-1 kernels' integer arithmetic.
 bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs);
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                   const Q8Scale *scales, int64_t m, float *y);
 // mmq_f16.hip: Q4_K with prompt-sized batches on big fp16 tiles. xh: fp16 activations [mmq_m_pad(m)][K].
-bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m);
+bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m = 0);
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                        const float *res = nullptr);
 // ops.hip: fused decode-step stages (all enqueue on dev->stream, no allocation, no sync).

@@ -663,7 +663,8 @@ static int qmatmul_check(candy_hip_device *dev, const candy_hip_qtensor *w, int6
 }
 
 static int contract(candy_hip_device *dev, const candy_hip_qtensor *w, const ActWorkspace &a, int64_t m, float *y) {
-    return m < mmq_min_m(dev) ? launch_matvec(dev, w, a.qs, a.scales, m, y) : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws);
+    return m < mmq_min_m(dev) ? launch_matvec(dev, w, a.qs, a.scales, m, y)
+                               : launch_mmq(dev, w, a.qs, a.scales, m, y, a.half_ws, nullptr, nullptr, dev->opt.f16_api_min_m);
 }
 
 // f32 in -> f32 out.  One row against a big Q4_K weight is ONE launch (the row is quantized in the contraction's

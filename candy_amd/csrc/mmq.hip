@@ -314,7 +314,8 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const _
 int64_t mmq_m_pad(int64_t m) { return (m + 255) / 256 * 256; }  // a multiple of every tile height
 
 static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                        int64_t m, float *y, void *half_ws, const _Float16 *xh_ready, const float *res, bool *res_done);
+                        int64_t m, float *y, void *half_ws, const _Float16 *xh_ready, const float *res, bool *res_done,
+                        int f16_min_m);
 
 static bool force_old_fp16(const candy_hip_device *dev) { return dev->opt.mmq_fp16_only != 0; }
 
@@ -323,16 +324,17 @@ bool mmq_fuses_residual(const candy_hip_qtensor *w, int64_t m) {
 }
 
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int64_t m,
-               float *y, void *half_ws, const _Float16 *xh_ready, const float *res) {
+               float *y, void *half_ws, const _Float16 *xh_ready, const float *res, int f16_min_m) {
     CANDY_REQUIRE(res != y || mmq_fuses_residual(w, m), "internal: in-place residual needs the fused epilogue");
     bool res_done = false;
-    if (int rc = mmq_dispatch(dev, w, qs, scales, m, y, half_ws, xh_ready, res, &res_done)) return rc;
+    if (int rc = mmq_dispatch(dev, w, qs, scales, m, y, half_ws, xh_ready, res, &res_done, f16_min_m)) return rc;
     if (res && !res_done) return candy_hip_add(dev, res, y, m * w->rows, y);  // kernels without a residual epilogue
     return CANDY_HIP_OK;
 }
 
 static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
-                        int64_t m, float *y, void *half_ws, const _Float16 *xh_ready, const float *res, bool *res_done) {
+                        int64_t m, float *y, void *half_ws, const _Float16 *xh_ready, const float *res, bool *res_done,
+                        int f16_min_m) {
     const int64_t K = w->cols;
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && K <= 0x7FFFFFFF && m <= 0x7FFFFFFF, "matrix too large");
     if (K % 64 != 0) return launch_matvec(dev, w, qs, scales, m, y);  // odd block counts: small-batch kernel in slices
@@ -340,7 +342,7 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     // prompt-sized batches of Q4_K: big fp16 tiles (the integer kernel is bound by its per-sub-block rescale there);
     // smaller batches of Q4_K and Q6_K: int8 matrix cores (exact); the fp16 tile kernel below serves the rest
     const bool force_fp16 = force_old_fp16(dev);
-    const bool big = !force_fp16 && mmq_f16_big_covers(w, m);
+    const bool big = !force_fp16 && mmq_f16_big_covers(w, m, f16_min_m);
     // the 32-value formats (Q8_0, Q4_0, Q4_1, Q5_0, Q5_1) on the int8 tiles as well, except where the 128 x 128 fp16 tiles below fill the chip (many weight rows and
     // a prompt-sized batch; measured: 11008x4096 m = 256 127 against 123 us, m = 512 228 against 134; 32000x4096
     // m = 128 165 against 129; but 4096x11008 m = 128 68 against 313, 4096x4096 m = 512 88 against 121)

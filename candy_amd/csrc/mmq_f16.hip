@@ -456,8 +456,10 @@ static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _
     return CANDY_HIP_OK;
 }
 
-bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m) {
-    const int min_m = w->dev->opt.f16_big_min_m;
+bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m) {
+    // a lower threshold (single contractions through the API) holds for Q4_K only: its tiles have the cheap
+    // dequantization and the 128 x 128 shape; the other formats' int8 tiles stay ahead up to the decoder's threshold
+    if (min_m <= 0 || w->fmt != CANDY_HIP_Q4_K) min_m = w->dev->opt.f16_big_min_m;
     if (m < min_m || w->cols % 256 != 0) return false;
     if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
     if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML)
@@ -473,6 +475,8 @@ int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const 
     if (w->fmt == CANDY_HIP_Q8_0) return launch_big<BigQ8_0, 128, 256, 2, 4>(dev, w, xh, m, y, res);
     if (w->fmt == CANDY_HIP_Q4_0) return launch_big<BigQ4_0<false>, 128, 256, 2, 4>(dev, w, xh, m, y, res);
     if (w->fmt == CANDY_HIP_Q4_0_GGML) return launch_big<BigQ4_0<true>, 128, 256, 2, 4>(dev, w, xh, m, y, res);
+    // up to 128 activation rows: 128 x 128 tiles (two workgroups per CU), K split over workgroups to fill the chip
+    if (m <= 128) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, w, xh, m, y, res);
     return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
 }
 

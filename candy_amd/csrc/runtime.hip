@@ -344,6 +344,7 @@ const OptionKey OPTION_KEYS[] = {
     {"mmq.i8_min_m", &candy::Options::i8_min_m, 0, 1 << 20},
     {"mmq.min_m", &candy::Options::mmq_min_m, 16, 1 << 20},
     {"mmq.f16_big_min_m", &candy::Options::f16_big_min_m, 16, 1 << 30},
+    {"mmq.f16_api_min_m", &candy::Options::f16_api_min_m, 16, 1 << 30},
     {"mmq.fp16_only", &candy::Options::mmq_fp16_only, 0, 1},
     {"mmq.i8_grid_split", &candy::Options::i8_grid_split, 0, 1},
     {"fused.pair_rows", &candy::Options::pair_rows, 0, 32},

@@ -48,11 +48,31 @@ def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
     # rows off every 4/16/64 boundary, block counts off every stage length, m off every tile height
     w = synth.random_weight(fmt, rows, cols, seed=rows + m)
     x = synth.random_activations(m, cols, seed=cols + m)
-    got = dev.qmatmul(dev.qtensor(fmt, rows, cols, w), x)
+    # single Q4_K contractions move to the fp16 tiles from 96 rows on; here the int8 tiles are asked for up to the
+    # decoder's threshold (what its prompt pass uses)
+    dev.set_option("mmq.f16_api_min_m", 256)
+    try:
+        got = dev.qmatmul(dev.qtensor(fmt, rows, cols, w), x)
+    finally:
+        dev.set_option("mmq.f16_api_min_m", 96)
     want = o.qmatmul(fmt, w, rows, cols, x)
     assert got.shape == (m, rows)
     # 256 activation rows or more run on the fp16 tiles (operands rounded to fp16)
     assert rel_err(got, want) <= (5e-4 if m >= 256 and fmt in (synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML) else 2e-5)
+
+
+@pytest.mark.parametrize("m", [96, 97, 100, 128, 129, 200, 255])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (127, 512), (129, 1024), (300, 2304), (1030, 768), (130, 4352)])
+def test_q4k_fp16_tiles_from_96_rows(dev, m, rows, cols):
+    # a single Q4_K contraction of 96 .. 255 rows: 128 x 128 tiles up to 128 rows, 128 x 256 above, K split over
+    # workgroups on small grids; fp16 operands (the bar of the big tiles), the same bits from call to call
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=7 * rows + m)
+    x = synth.random_activations(m, cols, seed=cols + 3 * m)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    err = rel_err(got, o.qmatmul(synth.Q4_K, w, rows, cols, x))
+    assert err <= 5e-4, err
+    assert np.array_equal(got, dev.qmatmul(q, x))
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K])
