@@ -468,7 +468,8 @@ def main():
 
     if not args.no_prefill:
         # batched prefill: Q4_K 14336x4096 x f32 [M, 4096], f32 in -> f32 out (activation quantization included).
-        # m < 96 runs on the int8 matrix cores (exact integer dots; peak 5.0 POP/s), m >= 96 on fp16 tiles
+        # m <= 16 is one pass over the weights on the int8 matrix cores (k_mmv_q4k), 16 < m < 96 the int8 tile kernel
+        # (both exact integer dots; peak 5.0 POP/s), m >= 96 fp16 tiles
         # (operands rounded to fp16, 3e-4 per matmul; peak 2.5 PFLOP/s).  roofline_us = the larger of the bytes at 8 TB/s and the contraction at that peak.
         pre = []
         r, k = 14336, 4096
@@ -480,7 +481,8 @@ def main():
             int8 = m < big_min
             peak = MFMA_I8_PEAK_TOPS if int8 else MFMA_F16_PEAK_TFLOPS
             roof_us = max(byts / (HBM_PEAK_GBPS * 1e9), flops / (peak * 1e12)) * 1e6
-            pre.append({"m": m, "kernel": ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else ("k_mmq_f16<BigQ4K,128,%d,2,4> (fp16 MFMA)" % (128 if m <= 128 else 256)),
+            pre.append({"m": m, "kernel": "k_mmv_q4k<2,2,8> (int8 MFMA, one pass)" if m <= dev.get_option("mmv.max_m") else
+                        ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else ("k_mmq_f16<BigQ4K,128,%d,2,4> (fp16 MFMA)" % (128 if m <= 128 else 256)),
                         "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
                         "mfma_peak_TFLOPs": peak, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / peak, 4),
                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),

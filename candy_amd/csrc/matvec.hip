@@ -572,11 +572,13 @@ int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quan
     const size_t q_bytes = need_quants ? (((size_t)(m * cols) + 255) & ~(size_t)255) : 0;
     const size_t s_bytes = need_quants ? (((size_t)(m * (cols >> 5)) * sizeof(Q8Scale) + 255) & ~(size_t)255) : 0;
     const size_t h_bytes = m >= 16 ? (size_t)(mmq_m_pad(m) * cols) * 2 : 0;
+    const size_t v_bytes = need_quants && m >= 2 && m <= 16 && cols % 256 == 0 ? mmv_workspace_bytes(cols) : 0;
     void *ws = nullptr;
-    if (int rc = workspace(dev, q_bytes + s_bytes + h_bytes + 256, &ws)) return rc;
+    if (int rc = workspace(dev, q_bytes + s_bytes + h_bytes + v_bytes + 256, &ws)) return rc;
     out->qs = (int8_t *)ws;
     out->scales = (Q8Scale *)((uint8_t *)ws + q_bytes);
     out->half_ws = h_bytes ? (uint8_t *)ws + q_bytes + s_bytes : nullptr;
+    out->mmv_ws = v_bytes ? (uint8_t *)ws + q_bytes + s_bytes + h_bytes : nullptr;
     return CANDY_HIP_OK;
 }
 
@@ -677,6 +679,7 @@ static int qmatmul_f32(candy_hip_device *dev, const candy_hip_qtensor *w, const 
         const int rc = launch_matvec_wide(dev, Wd);
         if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     }
+    if (a.mmv_ws && mmv_covers(w, m)) return launch_mmv(dev, w, dev_x, nullptr, m, dev_y, a.mmv_ws);
     if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, a.qs, a.scales, nullptr)) return rc;
     return contract(dev, w, a, m, dev_y);
 }
@@ -721,6 +724,7 @@ int candy_hip_qmatmul_q8(candy_hip_device *dev, const candy_hip_qtensor *w, cons
     if (int rc = use_device(dev)) return rc;
     ActWorkspace a;
     if (int rc = act_workspace(dev, m, w->cols, true, &a)) return rc;
+    if (a.mmv_ws && mmv_covers(w, m)) return launch_mmv(dev, w, nullptr, dev_x_q8_0, m, dev_y, a.mmv_ws);
     if (int rc = launch_q8_blocks_to_planar(dev, dev_x_q8_0, m * (w->cols >> 5), a.qs, a.scales)) return rc;
     return contract(dev, w, a, m, dev_y);
 }

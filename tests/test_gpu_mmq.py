@@ -83,18 +83,22 @@ def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, 
     # fixed order: the answer moves by f32 summation order only, and is the same from call to call
     w = synth.random_weight(fmt, rows, cols, seed=rows + cols + fmt)
     q = dev.qtensor(fmt, rows, cols, w)
-    for m in (16, 24, 33, 64, 130):
-        x = synth.random_activations(m, cols, seed=m * 7 + fmt)
-        got = dev.qmatmul(q, x)
-        assert np.array_equal(got.view(np.uint32), dev.qmatmul(q, x).view(np.uint32))
-        if m in (16, 33):
-            assert rel_err(got, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5, m
-        dev.set_option("mmq.i8_grid_split", 0)
-        try:
-            whole = dev.qmatmul(q, x)
-        finally:
-            dev.set_option("mmq.i8_grid_split", 1)
-        assert rel_err(got, whole) <= 2e-6, m
+    dev.set_option("mmv.max_m", 0)  # 16 rows of Q4_K on the tile kernel here, not on the one-pass kernel
+    try:
+        for m in (16, 24, 33, 64, 130):
+            x = synth.random_activations(m, cols, seed=m * 7 + fmt)
+            got = dev.qmatmul(q, x)
+            assert np.array_equal(got.view(np.uint32), dev.qmatmul(q, x).view(np.uint32))
+            if m in (16, 33):
+                assert rel_err(got, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5, m
+            dev.set_option("mmq.i8_grid_split", 0)
+            try:
+                whole = dev.qmatmul(q, x)
+            finally:
+                dev.set_option("mmq.i8_grid_split", 1)
+            assert rel_err(got, whole) <= 2e-6, m
+    finally:
+        dev.set_option("mmv.max_m", 16)
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML])

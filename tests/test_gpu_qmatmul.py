@@ -100,6 +100,57 @@ def test_config_q4_0_4096x4096(dev):
     assert rel_err(got[:, sub], lit) <= 1e-4
 
 
+@pytest.mark.parametrize("rows,cols,variant", [(64, 1024, 0), (48, 2048, 0),          # up to 8 super-blocks a row
+                                               (4096, 4096, 1), (4096, 4096, 2),      # 16: one / two strips a wavefront
+                                               (160, 6144, 0),                        # 24: three super-blocks a slice
+                                               (96, 8192, 1), (96, 8192, 2),          # 32
+                                               (128, 11008, 0),                       # 43: slices past the end of K
+                                               (64, 12288, 0)])                       # 48: the longest row it takes
+@pytest.mark.parametrize("m", [2, 3, 7, 16])
+def test_small_batch_int8_one_pass(dev, rows, cols, variant, m):
+    # 2 .. 16 activation rows against Q4_K on the int8 matrix cores, one pass over the weights (the role of
+    # mul_mat_vec_q<ncols_y>, quantized.cu:2787-2871): integer sub-block dots, scales applied as
+    # vec_dot_q4_K_q8_1 does (quantized.cu:2239-2263); only the f32 summation order differs from the CPU loop
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=rows + cols + m)
+    x = synth.random_activations(m, cols, seed=cols + 5 * m)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    try:
+        dev.set_option("mmv.min_m", 2)
+        dev.set_option("mmv.variant", variant)
+        got = dev.qmatmul(q, x)
+        dev.set_option("mmv.max_m", 0)
+        other = dev.qmatmul(q, x)  # the vector / tile kernels on the same quantized activations
+    finally:
+        dev.set_option("mmv.min_m", 3), dev.set_option("mmv.max_m", 16), dev.set_option("mmv.variant", 0)
+    assert got.shape == (m, rows)
+    if rows * cols <= 1 << 21:
+        want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
+    else:
+        sub = np.arange(0, rows, rows // 128)
+        want = o.qmatmul(synth.Q4_K, w.reshape(rows, -1)[sub].reshape(-1), len(sub), cols, x)
+        got, other = got[:, sub], other[:, sub]
+    assert rel_err(got, want) <= 2e-5
+    assert rel_err(got, other) <= 2e-5
+    q.free()
+
+
+def test_small_batch_int8_one_pass_leaves_other_shapes_alone(dev):
+    # rows off the 16-row strips, rows longer than 48 super-blocks and other formats keep their kernels: same bits
+    # whether the option is on or off
+    for fmt, rows, cols in ((synth.Q4_K, 100, 4096), (synth.Q4_K, 64, 14336), (synth.Q6_K, 64, 4096), (synth.Q8_0, 64, 4096)):
+        w = synth.random_weight(fmt, rows, cols, seed=rows + fmt)
+        x = synth.random_activations(5, cols, seed=9)
+        q = dev.qtensor(fmt, rows, cols, w)
+        a = dev.qmatmul(q, x)
+        dev.set_option("mmv.max_m", 0)
+        try:
+            b = dev.qmatmul(q, x)
+        finally:
+            dev.set_option("mmv.max_m", 16)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (fmt, rows, cols)
+        assert rel_err(a, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5
+
+
 @pytest.mark.parametrize("fmt", [synth.Q8_0, synth.Q4_K])
 @pytest.mark.parametrize("rows,cols", [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)])
 def test_config_sweep_full_shapes(dev, fmt, rows, cols):
