@@ -481,7 +481,7 @@ def main():
             int8 = m < big_min
             peak = MFMA_I8_PEAK_TOPS if int8 else MFMA_F16_PEAK_TFLOPS
             roof_us = max(byts / (HBM_PEAK_GBPS * 1e9), flops / (peak * 1e12)) * 1e6
-            pre.append({"m": m, "kernel": "k_mmv_q4k<2,2,8> (int8 MFMA, one pass)" if m <= dev.get_option("mmv.max_m") else
+            pre.append({"m": m, "kernel": "k_mmv_q4k<1,2,2,8> (int8 MFMA, one pass)" if m <= 16 else
                         ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else ("k_mmq_f16<BigQ4K,128,%d,2,4> (fp16 MFMA)" % (128 if m <= 128 else 256)),
                         "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
                         "mfma_peak_TFLOPs": peak, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / peak, 4),

@@ -58,7 +58,7 @@ struct Options {
     int mmq_fp16_only = 0;       // 1: every tile contraction on the single-buffered fp16 tiles
     int i8_grid_split = 1;       // int8 tiles: split K over workgroups on small grids
     int mmv_min_m = 3;           // f32 x Q4_K with this many .. mmv_max_m rows: the one-pass int8 kernel
-    int mmv_max_m = 16;          //   (0: never)
+    int mmv_max_m = 32;          //   (0: never; more than 16 rows only for rows of up to 4096 values)
     int mmv_variant = 0;         // comparison runs: 1 = one 16-row strip per wavefront, 2 = two
     int pair_rows = 0;           // fused gate/up: row pairs per workgroup, 32 / 16 / 8 (0: the most even split)
     int rms_rows = 0;            // fused RMSNorm prologue: rows per workgroup, 16 / 24 (0: the most even split)
@@ -176,7 +176,7 @@ int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *
                const float *res = nullptr, int f16_min_m = 0);
 // mmq_i8.hip: Q4_K / Q6_K on v_mfma_i32_16x16x32_i8 with the batch-1 kernels' integer arithmetic.
 bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs);
-// mmv_i8.hip: 2 .. 16 f32 activation rows against a Q4_K weight, one pass over the weights on the int8 matrix cores
+// mmv_i8.hip: 2 .. 32 activation rows against a Q4_K weight, one pass over the weights on the int8 matrix cores
 size_t mmv_workspace_bytes(int64_t K);
 bool mmv_covers(const candy_hip_qtensor *w, int64_t m);
 int launch_mmv(candy_hip_device *dev, const candy_hip_qtensor *w, const float *x, const void *q8_blocks, int64_t m,
@@ -261,7 +261,7 @@ struct ActWorkspace {
     int8_t *qs;
     Q8Scale *scales;
     void *half_ws;
-    void *mmv_ws = nullptr;  // operand-order activations for the small-batch int8 kernel (2 .. 16 rows)
+    void *mmv_ws = nullptr;  // operand-order activations for the small-batch int8 kernel (2 .. 32 rows)
 };
 int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quants, ActWorkspace *out);
 // matvec.hip: y[m, rows] = x . W^T for any m from planar activations that live OUTSIDE the device

@@ -572,7 +572,7 @@ int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quan
     const size_t q_bytes = need_quants ? (((size_t)(m * cols) + 255) & ~(size_t)255) : 0;
     const size_t s_bytes = need_quants ? (((size_t)(m * (cols >> 5)) * sizeof(Q8Scale) + 255) & ~(size_t)255) : 0;
     const size_t h_bytes = m >= 16 ? (size_t)(mmq_m_pad(m) * cols) * 2 : 0;
-    const size_t v_bytes = need_quants && m >= 2 && m <= 16 && cols % 256 == 0 ? mmv_workspace_bytes(cols) : 0;
+    const size_t v_bytes = need_quants && m >= 2 && m <= 32 && cols % 256 == 0 ? mmv_workspace_bytes(cols) : 0;
     void *ws = nullptr;
     if (int rc = workspace(dev, q_bytes + s_bytes + h_bytes + v_bytes + 256, &ws)) return rc;
     out->qs = (int8_t *)ws;

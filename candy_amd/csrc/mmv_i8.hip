@@ -1,4 +1,4 @@
-// Small batches (2 .. 16 activation rows) of Q4_K on the int8 matrix cores, shaped like the batch-1 matvec:
+// Small batches (2 .. 32 activation rows) of Q4_K on the int8 matrix cores, shaped like the batch-1 matvec:
 // y[m, N] = x[m, K] . W^T, weights read once, every load of a wavefront in flight before its first dot, no loop.
 //
 // mul_mat_vec_q<ncols_y> (tensor/internal/cuda/kernels/quantized.cu:2787-2871) serves 1 .. 8 activation rows from
@@ -33,9 +33,15 @@ __device__ __forceinline__ void mmv_wave_lds_fence() {
 }
 
 // ------------------------------------------------------------------ activations in operand order
+// Activation rows come in tiles of 16 (one or two tiles).  Per tile:
 // xfrag: [K/256][4][64 lanes][16 bytes]: lane (row r = lane & 15, chunk c = lane >> 4) of pair tp holds values
-//        8c .. 8c+7 of sub-blocks 2tp and 2tp+1 of row r.  Rows m .. 15 are zero.
+//        8c .. 8c+7 of sub-blocks 2tp and 2tp+1 of row r.  Rows from m on are zero.
 // xd:    [K/256 + 1][16 rows][8 sub-blocks] d;  xm: the same shape, d * sum(q8).  The last block of both is zero.
+struct MmvOperands {
+    uint8_t *xfrag;
+    float *xd, *xm;
+    size_t frag_stride, scale_stride;  // bytes / floats from one tile to the next
+};
 __device__ __forceinline__ size_t mmv_frag_offset(int r, int k) {
     const int sb = k >> 8, t = (k >> 5) & 7, c = (k >> 3) & 3;
     return ((size_t)((sb * 4 + (t >> 1)) * 64 + c * 16 + r)) * 16 + (t & 1) * 8 + (k & 7);
@@ -43,38 +49,39 @@ __device__ __forceinline__ size_t mmv_frag_offset(int r, int k) {
 
 // f32 [m, K] -> Q8_0 (quantize_q8_1 without its sum, quantized.cu:3521-3558; the same lane code as the quantize
 // kernel, hence the same quants and scales) written in operand order for 16 rows.
-__global__ __launch_bounds__(256) void k_mmv_quantize_pack(const float4 *__restrict__ x, int m, int K,
-                                                          uint8_t *__restrict__ xfrag, float *__restrict__ xd,
-                                                          float *__restrict__ xm) {
+__global__ __launch_bounds__(256) void k_mmv_quantize_pack(const float4 *__restrict__ x, int m, int K, MmvOperands o) {
     const int per_row = K >> 2;
-    const int i = blockIdx.x * 256 + threadIdx.x;  // 16 * per_row lanes in all (a multiple of 256)
-    const int r = i / per_row, k = (i - r * per_row) * 4;
-    const float4 v = r < m ? x[(size_t)r * per_row + (k >> 2)] : make_float4(0.f, 0.f, 0.f, 0.f);
+    const int i = blockIdx.x * 256 + threadIdx.x;  // 16 * tiles * per_row lanes in all (a multiple of 256)
+    const int row = i / per_row, k = (i - row * per_row) * 4;
+    const int tile = row >> 4, r = row & 15;
+    const float4 v = row < m ? x[(size_t)row * per_row + (k >> 2)] : make_float4(0.f, 0.f, 0.f, 0.f);
     __half h;
     int bsum;
     const uint32_t packed = quantize_q8_lane4(v, h, bsum);
-    *(uint32_t *)(xfrag + mmv_frag_offset(r, k)) = packed;
+    *(uint32_t *)(o.xfrag + tile * o.frag_stride + mmv_frag_offset(r, k)) = packed;
     if ((k & 31) == 0) {
         const float d = __half2float(h);
-        const size_t at = ((size_t)(k >> 8) * 16 + r) * 8 + ((k >> 5) & 7);
-        xd[at] = d;
-        xm[at] = d * (float)bsum;
-        if (k < 256) xd[at + (size_t)(K >> 8) * 128] = xm[at + (size_t)(K >> 8) * 128] = 0.0f;
+        const size_t at = tile * o.scale_stride + ((size_t)(k >> 8) * 16 + r) * 8 + ((k >> 5) & 7);
+        o.xd[at] = d;
+        o.xm[at] = d * (float)bsum;
+        if (k < 256) o.xd[at + (size_t)(K >> 8) * 128] = o.xm[at + (size_t)(K >> 8) * 128] = 0.0f;
     }
 }
 
 // Q8_0 blocks [m, K / 32] (34 bytes each) -> the same operand order; one lane per block of each of the 16 rows.
-__global__ __launch_bounds__(256) void k_mmv_pack_blocks(const BlockQ8_0 *__restrict__ blocks, int m, int K,
-                                                        uint8_t *__restrict__ xfrag, float *__restrict__ xd,
-                                                        float *__restrict__ xm) {
+__global__ __launch_bounds__(256) void k_mmv_pack_blocks(const BlockQ8_0 *__restrict__ blocks, int m, int tiles, int K,
+                                                        MmvOperands o) {
     const int bpr = K >> 5;
-    const int i = blockIdx.x * 256 + threadIdx.x;  // 16 * bpr lanes in all (a multiple of 128)
-    if (i >= 16 * bpr) return;
-    const int r = i / bpr, blk = i - r * bpr, k = blk * 32;
+    const int i = blockIdx.x * 256 + threadIdx.x;  // 16 * tiles * bpr lanes in all (a multiple of 128)
+    if (i >= 16 * tiles * bpr) return;
+    const int row = i / bpr, blk = i - row * bpr, k = blk * 32;
+    const int tile = row >> 4, r = row & 15;
+    uint8_t *xfrag = o.xfrag + tile * o.frag_stride;
+    float *xd = o.xd + tile * o.scale_stride, *xm = o.xm + tile * o.scale_stride;
     u32x4 a = {0u, 0u, 0u, 0u}, c = {0u, 0u, 0u, 0u};
     float d = 0.0f;
-    if (r < m) {
-        const BlockQ8_0 *src = blocks + (size_t)r * bpr + blk;
+    if (row < m) {
+        const BlockQ8_0 *src = blocks + (size_t)row * bpr + blk;
         a = *(const u32x4_a2 *)(src->qs);
         c = *(const u32x4_a2 *)(src->qs + 16);
         d = half_bits_to_float(src->d);
@@ -95,7 +102,7 @@ __global__ __launch_bounds__(256) void k_mmv_pack_blocks(const BlockQ8_0 *__rest
 }
 
 // ------------------------------------------------------------------ contraction
-template <int STRIPS, int SBW, int WAVES>
+template <int MT, int STRIPS, int SBW, int WAVES>
 struct MmvShape {
     static constexpr int CHUNKS_ROW = 9 * SBW;                 // 16-byte pieces of one row's slice
     static constexpr int ROWS_LD = 64 / CHUNKS_ROW;            // whole rows one load instruction covers
@@ -104,19 +111,18 @@ struct MmvShape {
     static constexpr int STAGE_BYTES = 16 * PITCH;
     static constexpr int EX_BYTES = 8 * 16 * 4;                // d * scale [sub-block][row]
     static constexpr int WAVE_LDS = STAGE_BYTES + EX_BYTES;
-    static constexpr int OUT = STRIPS * 4;                     // output registers of a lane
+    static constexpr int OUT = MT * STRIPS * 4;                // output registers of a lane
     static constexpr size_t SMEM = (size_t)WAVES * WAVE_LDS + (size_t)WAVES * OUT * 64 * sizeof(float);
 };
 
 // A workgroup owns 16 * STRIPS weight rows.  Each wavefront issues the loads of its K slice for every strip at once,
 // then takes the strips in the order their bytes return (loads complete in order): strip s is parked in LDS and
 // contracted while strip s+1 is still arriving, and the B operands and activation scales, which depend on the slice
-// only, stay in registers for all strips.
-template <int STRIPS, int SBW, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xfrag,
-                                                        const float *__restrict__ xd, const float *__restrict__ xm,
+// only, stay in registers for all strips.  MT tiles of 16 activation rows share every A operand.
+template <int MT, int STRIPS, int SBW, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restrict__ W, MmvOperands o,
                                                         float *__restrict__ y, int N, int M, int K) {
-    using S = MmvShape<STRIPS, SBW, WAVES>;
+    using S = MmvShape<MT, STRIPS, SBW, WAVES>;
     static_assert(S::ROWS_LD >= 1, "a row's slice must fit one load instruction");
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -135,10 +141,13 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
 
     // ---- activation scales and operands of this K slice first (they come from L2 and return first).
     // Wavefront-uniform bases, 32-bit lane offsets: the address arithmetic stays on the scalar unit.
-    float4 d8[SBW][2];
-    float2 xmv[SBW];
-    u32x4 bf[SBW][4];
-    {
+    float4 d8[MT][SBW][2];
+    float2 xmv[MT][SBW];
+    u32x4 bf[MT][SBW][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const uint8_t *xfrag = o.xfrag + mt * o.frag_stride;
+        const float *xd = o.xd + mt * o.scale_stride, *xm = o.xm + mt * o.scale_stride;
         const uint32_t at_d = (uint32_t)j * 32u, at_m = (uint32_t)j * 32u + (uint32_t)c * 8u, at_f = (uint32_t)lane * 16u;
 #pragma unroll
         for (int b = 0; b < SBW; ++b) {
@@ -148,11 +157,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
             const int sb = min(sb0 + b, nsb - 1), sbz = min(sb0 + b, nsb);
             const uint8_t *pd = (const uint8_t *)xd + (size_t)sbz * 512, *pm = (const uint8_t *)xm + (size_t)sbz * 512;
             const uint8_t *pf = xfrag + (size_t)sb * 4096;
-            d8[b][0] = *(const float4 *)(pd + at_d);
-            d8[b][1] = *(const float4 *)(pd + at_d + 16);
-            xmv[b] = *(const float2 *)(pm + at_m);
+            d8[mt][b][0] = *(const float4 *)(pd + at_d);
+            d8[mt][b][1] = *(const float4 *)(pd + at_d + 16);
+            xmv[mt][b] = *(const float2 *)(pm + at_m);
 #pragma unroll
-            for (int tp = 0; tp < 4; ++tp) bf[b][tp] = *(const u32x4 *)(pf + tp * 1024 + at_f);
+            for (int tp = 0; tp < 4; ++tp) bf[mt][b][tp] = *(const u32x4 *)(pf + tp * 1024 + at_f);
         }
     }
 
@@ -178,15 +187,18 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
     }
     __builtin_amdgcn_sched_barrier(0);  // every load above is issued before anything below waits
 
-    float acc[STRIPS][4];
-    float4v accm[STRIPS];
+    float acc[MT][STRIPS][4];
+    float4v accm[MT][STRIPS];
     const uint8_t *mine = stage + j * S::PITCH;
 
 #pragma unroll
     for (int s = 0; s < STRIPS; ++s) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[s][i] = 0.0f;
-        accm[s] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[mt][s][i] = 0.0f;
+            accm[mt][s] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+        }
         // park strip s (the previous strip's operand reads are done: fence at the end of its last super-block)
 #pragma unroll
         for (int n = 0; n < S::NLD; ++n)
@@ -204,27 +216,35 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
                 s_dsc[(2 * c) * 16 + j] = d * (float)(sc2 & 0xFF);
                 s_dsc[(2 * c + 1) * 16 + j] = d * (float)(sc2 >> 8);
                 // sum over the 8 sub-blocks of (dmin * m)[weight row] * (d8 * bsum)[activation row]: k = pair c, two halves
-                accm[s] = __builtin_amdgcn_mfma_f32_16x16x4f32(dmin * (float)(m2 & 0xFF), xmv[b].x, accm[s], 0, 0, 0);
-                accm[s] = __builtin_amdgcn_mfma_f32_16x16x4f32(dmin * (float)(m2 >> 8), xmv[b].y, accm[s], 0, 0, 0);
+                const float m_lo = dmin * (float)(m2 & 0xFF), m_hi = dmin * (float)(m2 >> 8);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    accm[mt][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(m_lo, xmv[mt][b].x, accm[mt][s], 0, 0, 0);
+                    accm[mt][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(m_hi, xmv[mt][b].y, accm[mt][s], 0, 0, 0);
+                }
             }
             mmv_wave_lds_fence();
-            const float d8a[8] = {d8[b][0].x, d8[b][0].y, d8[b][0].z, d8[b][0].w, d8[b][1].x, d8[b][1].y, d8[b][1].z, d8[b][1].w};
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 const u32x2 qa = *(const u32x2 *)(blk + 16 + 32 * p + 8 * c);
-                const u32x4 bb = bf[b][p];
                 const long a_lo = (long)(((uint64_t)(qa.y & 0x0F0F0F0Fu) << 32) | (qa.x & 0x0F0F0F0Fu));
                 const long a_hi = (long)(((uint64_t)((qa.y >> 4) & 0x0F0F0F0Fu) << 32) | ((qa.x >> 4) & 0x0F0F0F0Fu));
-                const long b_lo = (long)(((uint64_t)bb.y << 32) | bb.x), b_hi = (long)(((uint64_t)bb.w << 32) | bb.z);
-                const int4v d_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, b_lo, int4v{0, 0, 0, 0}, 0, 0, 0);
-                const int4v d_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, b_hi, int4v{0, 0, 0, 0}, 0, 0, 0);
                 // C layout: lane (activation row j, weight rows 4c .. 4c+3)
                 const float4 sc_lo = *(const float4 *)&s_dsc[(2 * p) * 16 + 4 * c], sc_hi = *(const float4 *)&s_dsc[(2 * p + 1) * 16 + 4 * c];
                 const float dl[4] = {sc_lo.x, sc_lo.y, sc_lo.z, sc_lo.w}, dh[4] = {sc_hi.x, sc_hi.y, sc_hi.z, sc_hi.w};
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc[s][i] += d8a[2 * p] * ((float)d_lo[i] * dl[i]);  // d8 * (d * sc) * dot
-                    acc[s][i] += d8a[2 * p + 1] * ((float)d_hi[i] * dh[i]);
+                for (int mt = 0; mt < MT; ++mt) {
+                    const u32x4 bb = bf[mt][b][p];
+                    const long b_lo = (long)(((uint64_t)bb.y << 32) | bb.x), b_hi = (long)(((uint64_t)bb.w << 32) | bb.z);
+                    const int4v d_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, b_lo, int4v{0, 0, 0, 0}, 0, 0, 0);
+                    const int4v d_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, b_hi, int4v{0, 0, 0, 0}, 0, 0, 0);
+                    const float4 dq = d8[mt][b][p >> 1];
+                    const float d8_lo = (p & 1) ? dq.z : dq.x, d8_hi = (p & 1) ? dq.w : dq.y;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[mt][s][i] += d8_lo * ((float)d_lo[i] * dl[i]);  // d8 * (d * sc) * dot
+                        acc[mt][s][i] += d8_hi * ((float)d_hi[i] * dh[i]);
+                    }
                 }
             }
             mmv_wave_lds_fence();  // the slots are rewritten by the next super-block / strip
@@ -233,59 +253,67 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
 
     // ---- the K slices meet: each output register is summed by one wavefront, slices in order
 #pragma unroll
-    for (int s = 0; s < STRIPS; ++s)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_red[(wave * S::OUT + s * 4 + i) * 64 + lane] = acc[s][i] - accm[s][i];
+        for (int s = 0; s < STRIPS; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                s_red[(wave * S::OUT + (mt * STRIPS + s) * 4 + i) * 64 + lane] = acc[mt][s][i] - accm[mt][s][i];
     __syncthreads();
-    for (int o = wave; o < S::OUT; o += WAVES) {
+    for (int r = wave; r < S::OUT; r += WAVES) {
         float sum = 0.0f;
 #pragma unroll
-        for (int w2 = 0; w2 < WAVES; ++w2) sum += s_red[(w2 * S::OUT + o) * 64 + lane];
-        const int n = n0 + 16 * (o >> 2) + 4 * c + (o & 3);
-        if (j < M) y[(size_t)j * N + n] = sum;
+        for (int w2 = 0; w2 < WAVES; ++w2) sum += s_red[(w2 * S::OUT + r) * 64 + lane];
+        const int mt = r / (STRIPS * 4), s = (r >> 2) % STRIPS;
+        const int n = n0 + 16 * s + 4 * c + (r & 3), row = 16 * mt + j;
+        if (row < M) y[(size_t)row * N + n] = sum;
     }
 }
 
-template <int STRIPS, int SBW, int WAVES>
-static int launch_mmv_cfg(candy_hip_device *dev, const candy_hip_qtensor *w, const uint8_t *xfrag, const float *xd,
-                          const float *xm, int M, float *y) {
-    using S = MmvShape<STRIPS, SBW, WAVES>;
+template <int MT, int STRIPS, int SBW, int WAVES>
+static int launch_mmv_cfg(candy_hip_device *dev, const candy_hip_qtensor *w, const MmvOperands &o, int M, float *y) {
+    using S = MmvShape<MT, STRIPS, SBW, WAVES>;
     static_assert(S::SMEM <= 150 * 1024, "LDS");
-    auto kern = k_mmv_q4k<STRIPS, SBW, WAVES>;
+    auto kern = k_mmv_q4k<MT, STRIPS, SBW, WAVES>;
     if (S::SMEM > 48 * 1024)
         CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::SMEM));
     const int N = (int)w->rows, K = (int)w->cols;
     hipLaunchKernelGGL(kern, dim3((unsigned)(N / (16 * STRIPS))), dim3(WAVES * 64), S::SMEM, dev->stream,
-                       (const uint8_t *)w->data, xfrag, xd, xm, y, N, M, K);
+                       (const uint8_t *)w->data, o, y, N, M, K);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
 
 static size_t mmv_scales_bytes(int64_t K) { return (((size_t)((K >> 8) + 1) * 16 * 8 * sizeof(float)) + 255) & ~(size_t)255; }
 static size_t mmv_frag_bytes(int64_t K) { return ((size_t)16 * (size_t)K + 255) & ~(size_t)255; }
-size_t mmv_workspace_bytes(int64_t K) { return mmv_frag_bytes(K) + 2 * mmv_scales_bytes(K) + 256; }
+size_t mmv_workspace_bytes(int64_t K) { return 2 * (mmv_frag_bytes(K) + 2 * mmv_scales_bytes(K)) + 256; }
 
 bool mmv_covers(const candy_hip_qtensor *w, int64_t m) {
-    if (w->fmt != CANDY_HIP_Q4_K || m < 2 || m > 16 || ((uintptr_t)w->data & 15) != 0) return false;
+    if (w->fmt != CANDY_HIP_Q4_K || m < 2 || m > 32 || ((uintptr_t)w->data & 15) != 0) return false;
     if (m < w->dev->opt.mmv_min_m || m > w->dev->opt.mmv_max_m) return false;
     const int64_t nsb = w->cols >> 8;
-    return w->cols % 256 == 0 && nsb >= 1 && nsb <= 48 && w->rows >= 16 && w->rows % 16 == 0 && w->rows <= 0x7FFFFFFF;
+    // two tiles of activation rows keep twice the operands in registers: rows of up to 16 super-blocks only
+    return w->cols % 256 == 0 && nsb >= 1 && nsb <= (m > 16 ? 16 : 48) && w->rows >= 16 && w->rows % 16 == 0 &&
+           w->rows <= 0x7FFFFFFF;
 }
 
-// Activations [m, K] (2 <= m <= 16), f32 (x) or Q8_0 blocks (x null), against a Q4_K weight: into operand order
+// Activations [m, K] (2 <= m <= 32), f32 (x) or Q8_0 blocks (x null), against a Q4_K weight: into operand order
 // (quantizing the f32), then one pass over the weights.  ws: mmv_workspace_bytes(K) of device memory.
 int launch_mmv(candy_hip_device *dev, const candy_hip_qtensor *w, const float *x, const void *q8_blocks, int64_t m,
                float *y, void *ws) {
-    const int K = (int)w->cols, nsb = K >> 8;
-    uint8_t *xfrag = (uint8_t *)ws;
-    float *xd = (float *)((uint8_t *)ws + mmv_frag_bytes(K));
-    float *xm = (float *)((uint8_t *)xd + mmv_scales_bytes(K));
+    const int K = (int)w->cols, nsb = K >> 8, tiles = m > 16 ? 2 : 1;
+    MmvOperands o;
+    o.frag_stride = mmv_frag_bytes(K);
+    o.scale_stride = mmv_scales_bytes(K) / sizeof(float);
+    o.xfrag = (uint8_t *)ws;
+    o.xd = (float *)((uint8_t *)ws + 2 * o.frag_stride);
+    o.xm = o.xd + 2 * o.scale_stride;
     if (x)
-        hipLaunchKernelGGL(k_mmv_quantize_pack, dim3((unsigned)(16 * (K >> 2) / 256)), dim3(256), 0, dev->stream,
-                           (const float4 *)x, (int)m, K, xfrag, xd, xm);
+        hipLaunchKernelGGL(k_mmv_quantize_pack, dim3((unsigned)(16 * tiles * (K >> 2) / 256)), dim3(256), 0, dev->stream,
+                           (const float4 *)x, (int)m, K, o);
     else
-        hipLaunchKernelGGL(k_mmv_pack_blocks, dim3((unsigned)((16 * (K >> 5) + 255) / 256)), dim3(256), 0, dev->stream,
-                           (const BlockQ8_0 *)q8_blocks, (int)m, K, xfrag, xd, xm);
+        hipLaunchKernelGGL(k_mmv_pack_blocks, dim3((unsigned)((16 * tiles * (K >> 5) + 255) / 256)), dim3(256), 0,
+                           dev->stream, (const BlockQ8_0 *)q8_blocks, (int)m, tiles, K, o);
     CANDY_LAUNCH_CHECK();
     const int M = (int)m;
     const int variant = dev->opt.mmv_variant;  // comparison runs: 1 one strip per wavefront, 2 two
@@ -293,17 +321,22 @@ int launch_mmv(candy_hip_device *dev, const candy_hip_qtensor *w, const float *x
     // wavefront has work anyway, 14336 x 4096 14.5 against 15.9, 32000 x 4096 25.5 against 28.1; below that the
     // extra wavefronts of the one-strip shape win, 11008 x 4096 13.1 against 13.8, 4096 x 4096 7.7 against 9.6.
     const bool two = w->rows % 32 == 0 && (variant ? variant == 2 : w->rows >= 48 * (int64_t)dev->num_cus);
-    if (nsb <= 8) return launch_mmv_cfg<1, 1, 8>(dev, w, xfrag, xd, xm, M, y);
+    if (tiles == 2) {
+        if (nsb <= 8) return launch_mmv_cfg<2, 1, 1, 8>(dev, w, o, M, y);
+        if (two) return launch_mmv_cfg<2, 2, 1, 16>(dev, w, o, M, y);
+        return launch_mmv_cfg<2, 1, 1, 16>(dev, w, o, M, y);
+    }
+    if (nsb <= 8) return launch_mmv_cfg<1, 1, 1, 8>(dev, w, o, M, y);
     if (nsb <= 16) {
-        if (two) return launch_mmv_cfg<2, 2, 8>(dev, w, xfrag, xd, xm, M, y);
-        return launch_mmv_cfg<1, 1, 16>(dev, w, xfrag, xd, xm, M, y);
+        if (two) return launch_mmv_cfg<1, 2, 2, 8>(dev, w, o, M, y);
+        return launch_mmv_cfg<1, 1, 1, 16>(dev, w, o, M, y);
     }
-    if (nsb <= 24) return launch_mmv_cfg<1, 3, 8>(dev, w, xfrag, xd, xm, M, y);
+    if (nsb <= 24) return launch_mmv_cfg<1, 1, 3, 8>(dev, w, o, M, y);
     if (nsb <= 32) {
-        if (two) return launch_mmv_cfg<2, 2, 16>(dev, w, xfrag, xd, xm, M, y);
-        return launch_mmv_cfg<1, 2, 16>(dev, w, xfrag, xd, xm, M, y);
+        if (two) return launch_mmv_cfg<1, 2, 2, 16>(dev, w, o, M, y);
+        return launch_mmv_cfg<1, 1, 2, 16>(dev, w, o, M, y);
     }
-    return launch_mmv_cfg<1, 3, 16>(dev, w, xfrag, xd, xm, M, y);
+    return launch_mmv_cfg<1, 1, 3, 16>(dev, w, o, M, y);
 }
 
 }  // namespace candy

@@ -347,8 +347,8 @@ const OptionKey OPTION_KEYS[] = {
     {"mmq.f16_api_min_m", &candy::Options::f16_api_min_m, 16, 1 << 30},
     {"mmq.fp16_only", &candy::Options::mmq_fp16_only, 0, 1},
     {"mmq.i8_grid_split", &candy::Options::i8_grid_split, 0, 1},
-    {"mmv.min_m", &candy::Options::mmv_min_m, 2, 16},
-    {"mmv.max_m", &candy::Options::mmv_max_m, 0, 16},
+    {"mmv.min_m", &candy::Options::mmv_min_m, 2, 32},
+    {"mmv.max_m", &candy::Options::mmv_max_m, 0, 32},
     {"mmv.variant", &candy::Options::mmv_variant, 0, 2},
     {"fused.pair_rows", &candy::Options::pair_rows, 0, 32},
     {"fused.rms_rows", &candy::Options::rms_rows, 0, 24},

@@ -91,7 +91,7 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   "mmq.fp16_only"              0        every tile contraction on the single-buffered fp16 tiles
  *   "mmq.i8_grid_split"          1        int8 tiles split K over workgroups on small grids
  *   "mmv.min_m"                  3        candy_hip_qmatmul on Q4_K: batches of this many .. "mmv.max_m" rows take the
- *   "mmv.max_m"                  16         one-pass int8 matrix-core kernel (max 0: never)
+ *   "mmv.max_m"                  32         one-pass int8 matrix-core kernel (max 0: never)
  *   "mmv.variant"                0        that kernel with one (1) or two (2) 16-row strips per wavefront (0: by shape)
  *   "fused.pair_rows"            0        fused gate/up: row pairs per workgroup 32 / 16 / 8 (0: most even split)
  *   "fused.rms_rows"             0        fused RMSNorm prologue: rows per workgroup 16 / 24 (0: most even split)
@@ -150,8 +150,9 @@ int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64
 /* y[m, rows] = x[m, cols] . W^T, activations quantized to Q8_0 on the device first.
  * m < 16 runs the bandwidth-bound matvec family (QCU:2787-2871 mul_mat_vec_q and its entry
  * points :2874, :2906, :2930, :2946); m >= 16 the MFMA tile kernel (QCU:455-578 mul_mat_q).
- * Q4_K with 3 <= m <= 16, rows % 16 == 0 and cols <= 12288: one pass over the weights with the
- * batch on the 16-wide side of the int8 matrix instruction (same integer dots, same scales).
+ * Q4_K with 3 <= m <= 16, rows % 16 == 0 and cols <= 12288 (m <= 32 for cols <= 4096): one pass over
+ * the weights with the batch on the 16-wide side of the int8 matrix instruction (same integer dots,
+ * same scales).
  * y is row-major [m, rows] (candy's result layout, tensor/ops.go:1264). */
 int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x,
                       int64_t m, float *dev_y);

@@ -83,7 +83,7 @@ def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, 
     # fixed order: the answer moves by f32 summation order only, and is the same from call to call
     w = synth.random_weight(fmt, rows, cols, seed=rows + cols + fmt)
     q = dev.qtensor(fmt, rows, cols, w)
-    dev.set_option("mmv.max_m", 0)  # 16 rows of Q4_K on the tile kernel here, not on the one-pass kernel
+    dev.set_option("mmv.max_m", 0)  # 16 .. 32 rows of Q4_K on the tile kernel here, not on the one-pass kernel
     try:
         for m in (16, 24, 33, 64, 130):
             x = synth.random_activations(m, cols, seed=m * 7 + fmt)
@@ -98,7 +98,7 @@ def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, 
                 dev.set_option("mmq.i8_grid_split", 1)
             assert rel_err(got, whole) <= 2e-6, m
     finally:
-        dev.set_option("mmv.max_m", 16)
+        dev.set_option("mmv.max_m", 32)
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML])

@@ -106,9 +106,10 @@ def test_config_q4_0_4096x4096(dev):
                                                (96, 8192, 1), (96, 8192, 2),          # 32
                                                (128, 11008, 0),                       # 43: slices past the end of K
                                                (64, 12288, 0)])                       # 48: the longest row it takes
-@pytest.mark.parametrize("m", [2, 3, 7, 16])
+@pytest.mark.parametrize("m", [2, 3, 7, 16, 17, 25, 32])
 def test_small_batch_int8_one_pass(dev, rows, cols, variant, m):
-    # 2 .. 16 activation rows against Q4_K on the int8 matrix cores, one pass over the weights (the role of
+    # 2 .. 16 activation rows (up to 32, as two tiles of 16, for rows of up to 4096 values) against Q4_K on the
+    # int8 matrix cores, one pass over the weights (the role of
     # mul_mat_vec_q<ncols_y>, quantized.cu:2787-2871): integer sub-block dots, scales applied as
     # vec_dot_q4_K_q8_1 does (quantized.cu:2239-2263); only the f32 summation order differs from the CPU loop
     w = synth.random_weight(synth.Q4_K, rows, cols, seed=rows + cols + m)
@@ -121,7 +122,7 @@ def test_small_batch_int8_one_pass(dev, rows, cols, variant, m):
         dev.set_option("mmv.max_m", 0)
         other = dev.qmatmul(q, x)  # the vector / tile kernels on the same quantized activations
     finally:
-        dev.set_option("mmv.min_m", 3), dev.set_option("mmv.max_m", 16), dev.set_option("mmv.variant", 0)
+        dev.set_option("mmv.min_m", 3), dev.set_option("mmv.max_m", 32), dev.set_option("mmv.variant", 0)
     assert got.shape == (m, rows)
     if rows * cols <= 1 << 21:
         want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
@@ -146,7 +147,7 @@ def test_small_batch_int8_one_pass_leaves_other_shapes_alone(dev):
         try:
             b = dev.qmatmul(q, x)
         finally:
-            dev.set_option("mmv.max_m", 16)
+            dev.set_option("mmv.max_m", 32)
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (fmt, rows, cols)
         assert rel_err(a, o.qmatmul(fmt, w, rows, cols, x)) <= 2e-5
 
