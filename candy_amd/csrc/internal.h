@@ -37,6 +37,7 @@ struct FormatInfo {
     int bytes;
 };
 FormatInfo format_info(int fmt);  // {0,0} if unknown
+int block_alignment(int fmt);      // alignment the block array of a format needs (its widest aligned load)
 
 // Planar Q8_0 activations: the matvec / MFMA kernels read the int8 quants and the
 // per-32 scale separately so every load is naturally aligned.

@@ -233,7 +233,7 @@ static int launch_dequant_more(candy_hip_device *dev, const void *blocks, int64_
 }
 
 // Alignment the block array of a format needs (its widest aligned load).
-static int block_alignment(int fmt) {
+int block_alignment(int fmt) {
     switch (fmt) {
     case CANDY_HIP_Q4_K:
     case CANDY_HIP_Q5_K: return 16;

@@ -61,6 +61,10 @@ SIGNATURES = {
                                        POINTER(c_size_t), POINTER(c_void_p)]),
     "candy_hip_dequantize_blocks": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "candy_hip_dequantize": (c_int, [c_void_p, c_void_p, c_void_p]),
+    "candy_hip_dequantize_blocks_f16": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
+    "candy_hip_dequantize_f16": (c_int, [c_void_p, c_void_p, c_void_p]),
+    "candy_hip_dequantize_blocks_f64": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
+    "candy_hip_dmmv": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "candy_hip_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "candy_hip_quantize": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_int64, c_void_p]),
     "candy_hip_qmatmul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
@@ -267,6 +271,35 @@ class Device:
         dst = self.alloc(q.rows * q.cols * 4)
         _check(lib().candy_hip_dequantize(self.handle, q.handle, dst.ptr))
         return dst.download(np.float32, q.rows * q.cols).reshape(q.rows, q.cols)
+
+    def dequantize_blocks_as(self, fmt: int, blocks: np.ndarray, dtype) -> np.ndarray:
+        """Blocks -> float16 or float64 values (the reference's other dequantize outputs)."""
+        dtype = np.dtype(dtype)
+        entry = {np.dtype(np.float16): lib().candy_hip_dequantize_blocks_f16,
+                 np.dtype(np.float64): lib().candy_hip_dequantize_blocks_f64}[dtype]
+        b = np.ascontiguousarray(blocks).view(np.uint8).reshape(-1)
+        bs, qk = lib().candy_hip_block_bytes(fmt), lib().candy_hip_block_elems(fmt)
+        if bs == 0:
+            _check(entry(self.handle, fmt, None, 0, None))
+        nb = b.size // bs
+        src = self.from_numpy(b)
+        dst = self.alloc(max(nb * qk * dtype.itemsize, 16))
+        _check(entry(self.handle, fmt, src.ptr, nb, dst.ptr))
+        return dst.download(dtype, nb * qk)
+
+    def dequantize_f16(self, q: QTensor) -> np.ndarray:
+        dst = self.alloc(q.rows * q.cols * 2)
+        _check(lib().candy_hip_dequantize_f16(self.handle, q.handle, dst.ptr))
+        return dst.download(np.float16, q.rows * q.cols).reshape(q.rows, q.cols)
+
+    def dmmv(self, q: QTensor, x: np.ndarray) -> np.ndarray:
+        """y[rows] = dequantize(W) . x with f32 activations (no activation quantizer)."""
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        assert x.size == q.cols
+        src = self.from_numpy(x)
+        dst = self.alloc(max(q.rows * 4, 16))
+        _check(lib().candy_hip_dmmv(self.handle, q.handle, src.ptr, dst.ptr))
+        return dst.download(np.float32, q.rows)
 
     def quantize_q8_0(self, x: np.ndarray) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32)

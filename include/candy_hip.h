@@ -134,6 +134,19 @@ int candy_hip_dequantize_blocks(candy_hip_device *dev, int fmt, const void *dev_
                                 int64_t n_blocks, float *dev_out);
 int candy_hip_dequantize(candy_hip_device *dev, const candy_hip_qtensor *q, float *dev_out);
 
+/* The same values as fp16: dequantize_block_*_f16 (tensor/internal/cuda/kernels/kernels.go:486-505; template
+ * QCU:1229-1249 and the K-quant kernels with dst_t = half).  Each value is computed in f32 as above and rounded to
+ * nearest even on the store: bit-exact against the f32 output rounded to fp16.  dev_out: 8-byte aligned. */
+int candy_hip_dequantize_blocks_f16(candy_hip_device *dev, int fmt, const void *dev_blocks,
+                                    int64_t n_blocks, void *dev_out_f16);
+int candy_hip_dequantize_f16(candy_hip_device *dev, const candy_hip_qtensor *q, void *dev_out_f16);
+
+/* float64 output for the formats whose CPU kernels have float64 twins: QGO:96-104 DequantizeBlockQ4_0F64,
+ * QGO:119-128 DequantizeBlockQ4_1F64, QGO:139-144 DequantizeBlockQ8_0F64 (the f32-widened scale times the level,
+ * in float64).  Other formats: CANDY_HIP_ERR_UNSUPPORTED.  Bit-exact. */
+int candy_hip_dequantize_blocks_f64(candy_hip_device *dev, int fmt, const void *dev_blocks,
+                                    int64_t n_blocks, double *dev_out);
+
 /* f32 [rows, cols] -> Q8_0 blocks (34 B each, rows*cols/32 of them), cols % 32 == 0.
  * QCU:3521-3558 quantize_q8_1 without its `sum` half.  Bit-exact. */
 int candy_hip_quantize_q8_0(candy_hip_device *dev, const float *dev_x, int64_t rows, int64_t cols,
@@ -156,6 +169,13 @@ int candy_hip_quantize(candy_hip_device *dev, int fmt, const float *dev_x, int64
  * y is row-major [m, rows] (candy's result layout, tensor/ops.go:1264). */
 int candy_hip_qmatmul(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x,
                       int64_t m, float *dev_y);
+
+/* y[rows] = dequantize(W)[rows, cols] . x[cols] with f32 activations and no activation quantizer: the reference's
+ * other matvec, dequantize_mul_mat_vec (QCU:1251-1345 for the 32-value formats, :1550-1693 q4_K, :1810-1911 q6_K
+ * and the other K-quants beside them).  It equals what candy's CPU backend computes (Dequantize, then the naive f32
+ * MatMul) up to f32 summation order, and does not carry the Q8_0 rounding of the activations that
+ * candy_hip_qmatmul does.  Batch 1.  dev_x: 16-byte aligned. */
+int candy_hip_dmmv(candy_hip_device *dev, const candy_hip_qtensor *w, const float *dev_x, float *dev_y);
 
 /* candy_hip_qmatmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): no counterpart in the reference.  Same result as candy_hip_qmatmul,

@@ -131,6 +131,41 @@ def dequantize(fmt: int, blocks) -> np.ndarray:
     return y
 
 
+def dequantize_f16(fmt: int, blocks) -> np.ndarray:
+    """dequantize_block_*_f16 (tensor/internal/cuda/kernels/kernels.go:486-505): the kernels of the f32 output with
+    dst_t = half (template quantized.cu:1229-1249 `y[...] = v.x`, and the K-quant kernels' `y[l] = d * q - m`), i.e.
+    each f32 value converted on the store, which is round to nearest even."""
+    return dequantize(fmt, blocks).astype(np.float16)
+
+
+def dequantize_f64(fmt: int, blocks) -> np.ndarray:
+    """DequantizeBlockQ4_0F64 / Q4_1F64 / Q8_0F64 (tensor/internal/cpu/kernels/quantized.go:96-104, 119-128, 139-144):
+    d (and m) are the fp16 fields widened to f32 and then to f64, the arithmetic is float64."""
+    b = _u8(blocks)
+    if fmt == Q4_0:
+        blk = b.reshape(-1, 18)
+        d = blk[:, :2].copy().view(np.float16).astype(np.float32).astype(np.float64)
+        qs = blk[:, 2:]
+        y = np.empty((blk.shape[0], 32), np.float64)
+        y[:, 0::2] = d * ((qs & 0xF).astype(np.float64) - 8)
+        y[:, 1::2] = d * ((qs >> 4).astype(np.float64) - 8)
+    elif fmt == 3:  # Q4_1
+        blk = b.reshape(-1, 20)
+        d = blk[:, :2].copy().view(np.float16).astype(np.float32).astype(np.float64)
+        m = blk[:, 2:4].copy().view(np.float16).astype(np.float32).astype(np.float64)
+        qs = blk[:, 4:]
+        y = np.empty((blk.shape[0], 32), np.float64)
+        y[:, 0::2] = d * (qs & 0xF).astype(np.float64) + m
+        y[:, 1::2] = d * (qs >> 4).astype(np.float64) + m
+    elif fmt == Q8_0:
+        blk = b.reshape(-1, 34)
+        d = blk[:, :2].copy().view(np.float16).astype(np.float32).astype(np.float64)
+        y = d * blk[:, 2:].copy().view(np.int8).astype(np.float64)
+    else:
+        raise ValueError(f"no float64 dequantize for format {fmt}")
+    return y.reshape(-1)
+
+
 def quantize_q8_0(x, rows: int | None = None, cols: int | None = None) -> np.ndarray:
     x = _f32(x)
     if rows is None:

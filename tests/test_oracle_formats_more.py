@@ -161,3 +161,52 @@ def test_q8_k_has_no_weight_vec_dot():
     w = synth.random_weight(Q8_K, 1, 256, seed=1)
     xq = o.quantize_q8_0(synth.random_activations(1, 256, seed=2))
     assert np.isnan(o.vec_dot_q8_0(Q8_K, w, xq, 256))
+
+
+# ---------------------------------------------------------------------- the other dequantize outputs
+def test_f64_twins_are_the_exact_values_rounded_once():
+    # quantized.go:96-104, 119-128, 139-144.  Exact rational value of each element -> nearest double must be what the
+    # oracle returns; a dropped "- 8", a swapped nibble or the min taken from the wrong half fails.  For Q4_0 and Q8_0
+    # the product fits 24 bits, so the float64 twin is also the f32 output widened.
+    rng = np.random.default_rng(5)
+    for fmt, width in ((synth.Q4_0, 18), (Q4_1, 20), (Q8_0, 34)):
+        blocks = rng.integers(0, 256, (40, width), dtype=np.uint8)
+        for i, h in enumerate(SPECIAL):           # special scale values, and a finite min for Q4_1
+            blocks[i, 0], blocks[i, 1] = h & 0xFF, h >> 8
+        blocks[:, 1] &= 0x7B                       # keep d finite
+        if fmt == Q4_1:
+            blocks[:, 3] &= 0x7B
+        got = o.dequantize_f64(fmt, blocks)
+        for b in range(blocks.shape[0]):
+            d = half_fraction(int(blocks[b, 0]) | int(blocks[b, 1]) << 8)
+            for e in range(32):
+                if fmt == synth.Q4_0:
+                    q = (int(blocks[b, 2 + e // 2]) >> (4 * (e & 1))) & 15
+                    exact = d * (q - 8)
+                elif fmt == Q4_1:
+                    q = (int(blocks[b, 4 + e // 2]) >> (4 * (e & 1))) & 15
+                    exact = d * q + half_fraction(int(blocks[b, 2]) | int(blocks[b, 3]) << 8)
+                else:
+                    exact = d * int(np.int8(blocks[b, 2 + e]))
+                assert got[b * 32 + e] == float(exact), (fmt, b, e)   # float(Fraction) rounds to nearest even
+        if fmt != Q4_1:
+            assert np.array_equal(got, o.dequantize(fmt, blocks).astype(np.float64))
+
+
+def test_f16_output_is_the_f32_output_rounded_to_nearest_even():
+    # kernels.go:486-505: same kernels with dst_t = half.  Checked against the exact value rounded by hand for the
+    # 32-value formats (one rounding when the f32 value is exact, which it is for Q4_0 / Q8_0: at most 19 bits)
+    rng = np.random.default_rng(6)
+    for fmt, width in ((synth.Q4_0, 18), (Q8_0, 34)):
+        blocks = rng.integers(0, 256, (64, width), dtype=np.uint8)
+        blocks[:, 1] &= 0x3F                       # |d| < 2: products stay inside fp16's range
+        got = o.dequantize_f16(fmt, blocks)
+        assert got.dtype == np.float16
+        for b in range(0, 64, 7):
+            d = half_fraction(int(blocks[b, 0]) | int(blocks[b, 1]) << 8)
+            for e in range(32):
+                q = ((int(blocks[b, 2 + e // 2]) >> (4 * (e & 1))) & 15) - 8 if fmt == synth.Q4_0 else int(np.int8(blocks[b, 2 + e]))
+                exact = d * q
+                lo, hi = np.float16(float(exact)), got[b * 32 + e]
+                # float(exact) is exact here (19 bits), and numpy's float64 -> float16 is round to nearest even
+                assert lo == hi or (np.isnan(lo) and np.isnan(hi)), (fmt, b, e)
