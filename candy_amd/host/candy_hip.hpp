@@ -337,6 +337,36 @@ public:
         return out;
     }
 
+    // The float64 twin of Dequantize (kernels/quantized.go:96-104, 119-128, 139-144: Q4_0, Q4_1, Q8_0 only)
+    Result<HipStorage<double>::Ptr> DequantizeF64() const {
+        auto out = HipStorage<double>::Alloc(dev_, (size_t)rows_ * cols_);
+        if (!out.ok()) return out;
+        void *blocks = nullptr;
+        if (Error e = last_error(candy_hip_qtensor_info(h_, nullptr, nullptr, nullptr, nullptr, &blocks), "dequantize")) return {nullptr, e};
+        const int64_t nb = (int64_t)rows_ * cols_ / candy_hip_block_elems((int)f_);
+        if (Error e = last_error(candy_hip_dequantize_blocks_f64(dev_->handle(), (int)f_, blocks, nb, (double *)out.value->ptr()), "dequantize"))
+            return {nullptr, e};
+        return out;
+    }
+    // fp16 output (kernels.go:486-505 dequantize_block_*_f16); the storage holds the IEEE half bits
+    Result<HipStorage<uint16_t>::Ptr> DequantizeF16() const {
+        auto out = HipStorage<uint16_t>::Alloc(dev_, (size_t)rows_ * cols_);
+        if (!out.ok()) return out;
+        if (Error e = last_error(candy_hip_dequantize_f16(dev_->handle(), h_, out.value->ptr()), "dequantize")) return {nullptr, e};
+        return out;
+    }
+    // y[Rows] = dequantize(W) . x with f32 activations (quantized.cu:1251-1345, :1550-1693, :1810-1911): what the CPU
+    // backend's Dequantize + MatMul gives, without the Q8_0 rounding of x that QMatMul carries
+    Result<HipStorage<float>::Ptr> DequantizeMulMatVec(const HipStorage<float>::Ptr &x) const {
+        if (!x) return {nullptr, Errorf("dmmv: lhs must live on the HIP device")};
+        if ((int64_t)x->Len() != cols_) return {nullptr, Errorf("dmmv: shape mismatch, lhs has " + std::to_string(x->Len()) + " values, weight [" +
+                                                               std::to_string(rows_) + " " + std::to_string(cols_) + "]")};
+        auto out = HipStorage<float>::Alloc(dev_, (size_t)rows_);
+        if (!out.ok()) return out;
+        if (Error e = last_error(candy_hip_dmmv(dev_->handle(), h_, (const float *)x->ptr(), (float *)out.value->ptr()), "dmmv")) return {nullptr, e};
+        return out;
+    }
+
     // y[m, Rows] = x[m, Cols] . W^T; x contiguous f32 on the same device
     Result<HipStorage<float>::Ptr> QMatMul(const HipStorage<float>::Ptr &x, const Layout *xLayout) const {
         if (!x) return {nullptr, Errorf("qmatmul: lhs must live on the HIP device")};

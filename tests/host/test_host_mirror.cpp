@@ -178,6 +178,27 @@ int main() {
             co_dequantize(fm.id, blocks.data(), rows * cols / co_block_elems(fm.id), want_dq.data());
             auto dq = q.value->Dequantize().value->Data();
             CHECK(std::memcmp(dq.data(), want_dq.data(), dq.size() * 4) == 0, "Dequantize bit-exact fmt %d", fm.id);
+            {   // the other outputs: float64 where the CPU kernels have a twin (for these formats it is the f32 value
+                // widened: an fp16 scale times at most 8 bits is exact in both), fp16 = the f32 value rounded once
+                auto d64 = q.value->DequantizeF64();
+                if (fm.id == CO_Q8_0 || fm.id == CO_Q4_0) {
+                    bool same = d64.ok();
+                    if (same) { auto v = d64.value->Data(); for (size_t i = 0; i < v.size() && same; ++i) same = v[i] == (double)want_dq[i]; }
+                    CHECK(same, "DequantizeF64 fmt %d", fm.id);
+                } else {
+                    CHECK(!d64.ok(), "DequantizeF64 refuses fmt %d", fm.id);
+                }
+                auto h16 = q.value->DequantizeF16();
+                bool same = h16.ok();
+                if (same) { auto v = h16.value->Data(); for (size_t i = 0; i < v.size() && same; ++i) same = v[i] == co_f32_to_fp16(want_dq[i]); }
+                CHECK(same, "DequantizeF16 fmt %d", fm.id);
+                // f32-activation matvec against Dequantize + the naive loop
+                std::vector<float> x1(cols), want1(rows);
+                for (auto &v : x1) v = nd(rng);
+                for (int r = 0; r < rows; ++r) { float a = 0; for (int k = 0; k < cols; ++k) a += want_dq[(size_t)r * cols + k] * x1[k]; want1[r] = a; }
+                auto y1 = q.value->DequantizeMulMatVec(F::FromSlice(dev, x1).value);
+                CHECK(y1.ok() && rel_err(y1.value->Data(), want1) <= 2e-5, "DequantizeMulMatVec fmt %d", fm.id);
+            }
             for (int m : {1, 5, 32}) {
                 std::vector<float> x((size_t)m * cols), want((size_t)m * rows);
                 for (auto &v : x) v = nd(rng);
