@@ -680,6 +680,12 @@ static int qmatmul_f32(candy_hip_device *dev, const candy_hip_qtensor *w, const 
         if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     }
     if (a.mmv_ws && mmv_covers(w, m)) return launch_mmv(dev, w, dev_x, nullptr, m, dev_y, a.mmv_ws);
+    if (a.half_ws && m >= mmq_min_m(dev) && !dev->opt.mmq_fp16_only && mmq_f16_big_covers(w, m, dev->opt.f16_api_min_m)) {
+        // the fp16 tiles read d * q as fp16: the quantizer writes that image directly (one launch, no int8 copy)
+        if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, nullptr, nullptr, nullptr, (_Float16 *)a.half_ws)) return rc;
+        return launch_mmq(dev, w, nullptr, nullptr, m, dev_y, a.half_ws, (const _Float16 *)a.half_ws, nullptr,
+                          dev->opt.f16_api_min_m);
+    }
     if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, a.qs, a.scales, nullptr)) return rc;
     return contract(dev, w, a, m, dev_y);
 }

@@ -347,6 +347,8 @@ const OptionKey OPTION_KEYS[] = {
     {"mmq.f16_api_min_m", &candy::Options::f16_api_min_m, 16, 1 << 30},
     {"mmq.fp16_only", &candy::Options::mmq_fp16_only, 0, 1},
     {"mmq.i8_grid_split", &candy::Options::i8_grid_split, 0, 1},
+    {"mmq.f16_shape", &candy::Options::f16_shape, 0, 3},
+    {"mmq.f16_split", &candy::Options::f16_split, 0, 16},
     {"mmv.min_m", &candy::Options::mmv_min_m, 2, 32},
     {"mmv.max_m", &candy::Options::mmv_max_m, 0, 32},
     {"mmv.variant", &candy::Options::mmv_variant, 0, 2},
