@@ -324,6 +324,9 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the batched-prefill (MFMA) leg")
     ap.add_argument("--no-llama3", action="store_true", help="skip the Llama-3-8B-shaped prefill + decode leg")
     ap.add_argument("--decode-steps", type=int, default=32)
+    ap.add_argument("--eager", action="store_true",
+                    help="decoders launch their kernels one by one instead of replaying a captured HIP graph (for "
+                         "profiler runs: each launch is then a dispatch the tool sees on its own)")
     ap.add_argument("--no-fp16-kv", action="store_true", help="skip the decode leg's second figure (fp16 KV cache)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for counter runs)")
@@ -339,6 +342,8 @@ def main():
     from candy_amd import hip, synth
     dev = hip.Device(0)
     log("device:", dev.name)
+    if args.eager:
+        dev.set_option("llama.graph", 0)
     fmt, rows, cols = synth.Q4_K, 4096, 11008
     alg = algorithmic_bytes(fmt, rows, cols)
     if args.calibrate_copy:
@@ -410,12 +415,30 @@ def main():
         # small batches (mul_mat_vec_q serves 1..8 rows in the reference): f32 in -> f32 out, quantization included
         small = []
         for f, r, k in ((synth.Q4_K, 4096, 11008), (synth.Q4_K, 11008, 4096), (synth.Q6_K, 32000, 4096)):
-            for m in (2, 4, 8, 15):
+            for m in (2, 4, 8, 15, 16, 32):
                 ms, _ = time_matvec(dev, f, r, k, s_steps, s_warm, quantize_each=True, seed=r + k + f + m, m=m)
                 small.append({"fmt": synth.FORMAT_NAMES[f], "rows": r, "cols": k, "m": m, "us": round(ms * 1e3, 2),
                               "GBps": round(algorithmic_bytes(f, r, k, m) / (ms * 1e-3) / 1e9, 1)})
                 log(f"  {synth.FORMAT_NAMES[f]} {r}x{k} m={m}: {ms * 1e3:.2f} us")
         out["small_batch"] = small
+        # the reference's other matvec: f32 activations, no activation quantizer (dequantize_mul_mat_vec)
+        dm = []
+        for f, r, k in ((synth.Q4_K, 4096, 11008), (synth.Q4_K, 11008, 4096), (synth.Q6_K, 32000, 4096)):
+            ws, nbytes = make_rotation(dev, f, r, k, seed=r + k + 3)
+            x = dev.from_numpy(synth.random_activations(1, k, seed=5))
+            y = dev.alloc(4 * r)
+            for timed in (False, True):
+                dev.synchronize()
+                dev.timer_start()
+                for i in range(s_steps):
+                    hip._check(hip.lib().candy_hip_dmmv(dev.handle, ws[i % len(ws)].handle, x.ptr, y.ptr))
+                ms = dev.timer_stop() / s_steps
+            for w in ws:
+                w.free()
+            dm.append({"fmt": synth.FORMAT_NAMES[f], "rows": r, "cols": k, "us": round(ms * 1e3, 2),
+                       "GBps": round(algorithmic_bytes(f, r, k) / (ms * 1e-3) / 1e9, 1)})
+            log(f"  dmmv {synth.FORMAT_NAMES[f]} {r}x{k}: {ms * 1e3:.2f} us")
+        out["dmmv"] = dm
 
     if not args.no_sweep:
         # weight quantizers from f32 (load-time): 4096x11008, one launch each
