@@ -171,3 +171,23 @@ def test_mixed_format_prefill_q6k_down_proj(dev, m):
     assert rel_err(got[:, sub], want) <= TOL
     # split-K partial sums are added in a fixed order: the same call gives the same bits
     assert np.array_equal(got, dev.qmatmul(q, x))
+
+
+def test_batch_size_boundaries_agree_within_their_bars(dev):
+    # Which kernel contracts depends on the number of activation rows.  Rows computed in a batch of one size and
+    # again in a batch across the next boundary agree to f32 summation order where both kernels are integer-exact
+    # (2 | 3: vector | one-pass; 16 | 17: one tile | two tiles; 32 | 33: one-pass | int8 tiles) and to the
+    # fp16-operand bar across the fp16 threshold (95 | 96 for a single Q4_K contraction).
+    rows, cols = 512, 2048
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=41)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    x = synth.random_activations(96, cols, seed=42)
+    want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
+    for lo, hi, bar in ((2, 3, 2e-6), (16, 17, 2e-6), (32, 33, 2e-6), (95, 96, 1e-3)):
+        a, b = dev.qmatmul(q, x[:lo]), dev.qmatmul(q, x[:hi])
+        d = rel_err(b[:lo], a.astype(np.float64))
+        assert d <= bar, (lo, hi, d)
+        assert rel_err(a, want[:lo]) <= 2e-5                      # below the threshold: exact kernels
+        assert rel_err(b, want[:hi]) <= (5e-4 if hi >= 96 else 2e-5)
+    a, b = dev.qmatmul(q, x[:95]), dev.qmatmul(q, x[:96])
+    assert rel_err(b[:95], a.astype(np.float64)) > 1e-6           # and it IS another kernel: not the same bits

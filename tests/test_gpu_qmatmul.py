@@ -196,6 +196,27 @@ def test_q6_k_llama3_head_shape(dev):
     q.free()
 
 
+def test_rows_past_the_small_batch_limit_are_an_error_not_a_fault(dev):
+    # with fewer than 16 activation rows the quantized image of a row must fit LDS (about 49 900 values) unless the
+    # batch-1 kernel takes it (Q4_K: up to 8 x 64 units = 32768 values... its image has the same limit): longer rows
+    # are refused with a message, from 16 rows on the tile kernels have no such limit
+    rows, cols = 16, 65536
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=3)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    for m in (1, 3, 15):
+        x = synth.random_activations(m, cols, seed=m)
+        try:
+            got = dev.qmatmul(q, x)
+        except hip.CandyHipError as e:
+            assert "too large for the matvec kernel" in str(e), str(e)
+        else:
+            assert rel_err(got, o.qmatmul(synth.Q4_K, w, rows, cols, x)) <= 2e-5
+    x = synth.random_activations(16, cols, seed=16)
+    assert rel_err(dev.qmatmul(q, x), o.qmatmul(synth.Q4_K, w, rows, cols, x)) <= 2e-5
+    dev.synchronize()  # the handle is still good
+    q.free()
+
+
 def test_qmatmul_from_prequantized_blocks(dev):
     rows, cols, m = 64, 1024, 3
     w = synth.random_weight(synth.Q4_K, rows, cols, seed=1)
