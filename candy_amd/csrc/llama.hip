@@ -378,6 +378,8 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
     }
     if (m->use_graph) {
         if (m->graph_dirty) {
+            // a replay of the old graph may still be in flight (a caller that did not ask for the token): drain first
+            if (m->graph_exec) CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
             if (m->graph_exec) CANDY_HIP_TRY(hipGraphExecDestroy(m->graph_exec));
             if (m->graph) CANDY_HIP_TRY(hipGraphDestroy(m->graph));
             m->graph_exec = nullptr;
