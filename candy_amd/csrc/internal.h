@@ -100,6 +100,7 @@ struct candy_hip_qtensor {
     size_t nbytes = 0;
     void *data = nullptr;
     bool owned = false;
+    bool padded = false;  // at least 16 readable bytes follow the last block
 };
 
 namespace candy {

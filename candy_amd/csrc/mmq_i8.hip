@@ -707,9 +707,9 @@ static int launch_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const in
 bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs) {
     if (((uintptr_t)qs & 15) != 0 || w->cols % 256 != 0) return false;
     if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
-    // the last chunk of a Q6_K row runs 14 bytes past the block: only buffers allocated by the library
-    // (which pads them) are known to have that room after the last row
-    if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q2_K || w->fmt == CANDY_HIP_Q3_K) return w->owned && ((uintptr_t)w->data & 1) == 0;
+    // the last chunk of a Q6_K row runs 14 bytes past the block: only buffers known to have that room after the
+    // last row (allocated by the library, which pads them, or wrapped with a size that says so)
+    if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q2_K || w->fmt == CANDY_HIP_Q3_K) return w->padded && ((uintptr_t)w->data & 1) == 0;
     switch (w->fmt) {
     case CANDY_HIP_Q8_0: case CANDY_HIP_Q4_0: case CANDY_HIP_Q4_0_GGML: case CANDY_HIP_Q4_1: case CANDY_HIP_Q4_1_GGML:
     case CANDY_HIP_Q5_0: case CANDY_HIP_Q5_1:

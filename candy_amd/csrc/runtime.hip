@@ -268,15 +268,15 @@ size_t candy_hip_qweight_bytes(int fmt, int64_t rows, int64_t cols) {
     return (size_t)rows * (size_t)(cols / fi.elems) * (size_t)fi.bytes;
 }
 
-static int qtensor_check(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols, size_t nbytes) {
+static int qtensor_check(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols, size_t nbytes, bool exact = true) {
     FormatInfo fi = format_info(fmt);
     CANDY_REQUIRE(dev, "device handle is nil");
     CANDY_REQUIRE(fi.elems != 0, "unknown quantized format %d", fmt);
     CANDY_REQUIRE(rows > 0 && cols > 0, "invalid matrix dimensions %lld x %lld", (long long)rows, (long long)cols);
     CANDY_REQUIRE(cols % fi.elems == 0, "cols %lld is not a multiple of the block size %d", (long long)cols, fi.elems);
     size_t want = candy_hip_qweight_bytes(fmt, rows, cols);
-    CANDY_REQUIRE(nbytes == want, "weight has %zu bytes, %lld x %lld blocks of format %d need %zu", nbytes,
-                  (long long)rows, (long long)cols, fmt, want);
+    CANDY_REQUIRE(exact ? nbytes == want : nbytes >= want, "weight has %zu bytes, %lld x %lld blocks of format %d need %zu",
+                  nbytes, (long long)rows, (long long)cols, fmt, want);
     return CANDY_HIP_OK;
 }
 
@@ -295,6 +295,7 @@ int candy_hip_qtensor_upload(candy_hip_device *dev, int fmt, int64_t rows, int64
     }
     candy_hip_qtensor *q = new candy_hip_qtensor();
     q->dev = dev; q->fmt = fmt; q->rows = rows; q->cols = cols; q->nbytes = nbytes; q->data = d; q->owned = true;
+    q->padded = true;
     *out = q;
     return CANDY_HIP_OK;
 }
@@ -303,11 +304,13 @@ int candy_hip_qtensor_wrap(candy_hip_device *dev, int fmt, int64_t rows, int64_t
                            size_t nbytes, candy_hip_qtensor **out) {
     CANDY_REQUIRE(out, "out is nil");
     *out = nullptr;
-    if (int rc = qtensor_check(dev, fmt, rows, cols, nbytes)) return rc;
+    if (int rc = qtensor_check(dev, fmt, rows, cols, nbytes, /*exact=*/false)) return rc;
     CANDY_REQUIRE(dev_blocks, "dev_blocks is nil");
     CANDY_REQUIRE(((uintptr_t)dev_blocks & 15) == 0, "device blocks must be 16-byte aligned");
     candy_hip_qtensor *q = new candy_hip_qtensor();
-    q->dev = dev; q->fmt = fmt; q->rows = rows; q->cols = cols; q->nbytes = nbytes; q->data = dev_blocks; q->owned = false;
+    const size_t want = candy_hip_qweight_bytes(fmt, rows, cols);
+    q->dev = dev; q->fmt = fmt; q->rows = rows; q->cols = cols; q->nbytes = want; q->data = dev_blocks; q->owned = false;
+    q->padded = nbytes >= want + 16;  // room for the widest load that starts inside the last block
     *out = q;
     return CANDY_HIP_OK;
 }

@@ -195,11 +195,11 @@ class QTensor:
         rows, cols = x.reshape(-1, x.shape[-1]).shape
         nbytes = lib().candy_hip_qweight_bytes(fmt, rows, cols)
         src = dev.from_numpy(x)
-        dst = dev.alloc(max(nbytes, 2))
+        dst = dev.alloc(nbytes + 64)  # spare bytes after the blocks: every tile kernel may take the weight
         _check(lib().candy_hip_quantize(dev.handle, fmt, src.ptr, rows, cols, dst.ptr))
         q = cls.__new__(cls)
         h = c_void_p()
-        _check(lib().candy_hip_qtensor_wrap(dev.handle, fmt, rows, cols, dst.ptr, nbytes, byref(h)))
+        _check(lib().candy_hip_qtensor_wrap(dev.handle, fmt, rows, cols, dst.ptr, nbytes + 64, byref(h)))
         q.dev, q.fmt, q.rows, q.cols, q.nbytes, q.handle = dev, fmt, rows, cols, nbytes, h.value
         q._blocks = dst  # the wrapped device memory stays owned here
         return q

@@ -308,11 +308,12 @@ public:
         const size_t nbytes = candy_hip_qweight_bytes((int)f, rows, cols);
         if (nbytes == 0) return {nullptr, Errorf("quantize: cols is not a multiple of the block size")};
         void *blocks = nullptr;
-        if (Error e = last_error(candy_hip_alloc(dev->handle(), nbytes, &blocks), "quantize")) return {nullptr, e};
+        const size_t room = nbytes + 64;  // spare bytes after the blocks: every tile kernel may take the weight
+        if (Error e = last_error(candy_hip_alloc(dev->handle(), room, &blocks), "quantize")) return {nullptr, e};
         int rc = (int)f == CANDY_HIP_Q8_0 ? candy_hip_quantize_q8_0(dev->handle(), (const float *)x->ptr(), rows, cols, blocks)
                                           : candy_hip_quantize(dev->handle(), (int)f, (const float *)x->ptr(), rows, cols, blocks);
         candy_hip_qtensor *h = nullptr;
-        if (!rc) rc = candy_hip_qtensor_wrap(dev->handle(), (int)f, rows, cols, blocks, nbytes, &h);
+        if (!rc) rc = candy_hip_qtensor_wrap(dev->handle(), (int)f, rows, cols, blocks, room, &h);
         if (Error e = last_error(rc, "quantize")) {
             candy_hip_free(dev->handle(), blocks);
             return {nullptr, e};

@@ -119,7 +119,10 @@ size_t candy_hip_qweight_bytes(int fmt, int64_t rows, int64_t cols);
 
 /* Quantized weight [rows, cols] (cols = contraction dim) kept on the device in the ORIGINAL
  * block layout, row-major blocks, as QCU:2827 indexes them (`x[kbx + row*blocks_per_row]`).
- * upload copies host blocks; wrap adopts device memory the caller keeps owning. */
+ * upload copies host blocks; wrap adopts device memory the caller keeps owning: nbytes is the size of
+ * that buffer, at least candy_hip_qweight_bytes(); a buffer with 16 or more spare bytes after the blocks
+ * lets Q6_K / Q2_K / Q3_K weights take the int8 tile kernel (its last load of a row starts inside the
+ * last block and runs past it), otherwise they take the fp16 tiles. */
 int candy_hip_qtensor_upload(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols,
                              const void *host_blocks, size_t nbytes, candy_hip_qtensor **out);
 int candy_hip_qtensor_wrap(candy_hip_device *dev, int fmt, int64_t rows, int64_t cols,

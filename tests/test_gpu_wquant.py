@@ -74,6 +74,35 @@ def test_quantized_weight_feeds_the_matmul(dev, fmt):
     q.free()
 
 
+def test_weight_quantized_on_the_device_takes_the_same_kernels_as_an_uploaded_one(dev):
+    # a Q6_K row's last 16-byte load in the int8 tile kernel starts inside the last block and runs past it, so the
+    # kernel takes only buffers known to have room there: uploads (padded by the library) and wrapped buffers whose
+    # stated size says so, which is how QTensor.quantize wraps its blocks.  Same kernel, same bits at 8 and 40 rows.
+    rng = np.random.default_rng(18)
+    rows, cols = 256, 2048
+    w = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)
+    q_dev = hip.QTensor.quantize(dev, synth.Q6_K, w)
+    q_up = dev.qtensor(synth.Q6_K, rows, cols, dev.quantize(synth.Q6_K, w))
+    for m in (8, 40):
+        x = synth.random_activations(m, cols, seed=m)
+        a, b = dev.qmatmul(q_dev, x), dev.qmatmul(q_up, x)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), m
+    # a wrapped buffer without spare bytes still works (other tiles, fp16 operands from 16 rows on)
+    blocks = dev.from_numpy(dev.quantize(synth.Q6_K, w))
+    h = hip.c_void_p()
+    hip._check(hip.lib().candy_hip_qtensor_wrap(dev.handle, synth.Q6_K, rows, cols, blocks.ptr, blocks.nbytes, hip.byref(h)))
+    tight = hip.QTensor.__new__(hip.QTensor)
+    tight.dev, tight.fmt, tight.rows, tight.cols, tight.nbytes, tight.handle, tight._blocks = dev, synth.Q6_K, rows, cols, blocks.nbytes, h.value, blocks
+    x = synth.random_activations(40, cols, seed=40)
+    want = dev.qmatmul(q_up, x)
+    got = dev.qmatmul(tight, x)
+    assert np.max(np.abs(got - want)) <= 1e-3 * np.max(np.abs(want))
+    with pytest.raises(hip.CandyHipError, match="need"):   # a buffer smaller than the blocks is refused
+        hip._check(hip.lib().candy_hip_qtensor_wrap(dev.handle, synth.Q6_K, rows, cols, blocks.ptr, blocks.nbytes - 1, hip.byref(h)))
+    for t in (q_dev, q_up, tight):
+        t.free()
+
+
 def test_quantize_errors_and_empty(dev):
     assert dev.quantize(synth.Q4_K, np.zeros((0, 256), np.float32)).size == 0
     with pytest.raises(hip.CandyHipError, match="multiple of the block"):
