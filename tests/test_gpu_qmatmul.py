@@ -135,6 +135,31 @@ def test_small_batch_int8_one_pass(dev, rows, cols, variant, m):
     q.free()
 
 
+def test_small_batch_int8_one_pass_random_shapes(dev):
+    # seeded random shapes over everything the kernel takes: 16 .. 640 weight rows in steps of 16, 1 .. 48
+    # super-blocks per row, 2 .. 32 activation rows (more than 16 only up to 16 super-blocks), both strip variants
+    rng = np.random.default_rng(2024)
+    dev.set_option("mmv.min_m", 2)
+    try:
+        for case in range(48):
+            nsb = int(rng.integers(1, 49))
+            rows = 16 * int(rng.integers(1, 41))
+            m = int(rng.integers(2, 33 if nsb <= 16 else 17))
+            cols = 256 * nsb
+            w = synth.random_weight(synth.Q4_K, rows, cols, seed=1000 + case)
+            x = synth.random_activations(m, cols, seed=2000 + case)
+            q = dev.qtensor(synth.Q4_K, rows, cols, w)
+            dev.set_option("mmv.variant", int(rng.integers(0, 3)))
+            got = dev.qmatmul(q, x)
+            want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
+            assert got.shape == (m, rows) and rel_err(got, want) <= 2e-5, (case, rows, cols, m)
+            xb = o.quantize_q8_0(x)     # and from Q8_0 blocks: the same quants, the same kernel, the same bits
+            assert np.array_equal(dev.qmatmul_q8(q, xb, m).view(np.uint32), got.view(np.uint32)), (case, rows, cols, m)
+            q.free()
+    finally:
+        dev.set_option("mmv.min_m", 3), dev.set_option("mmv.variant", 0)
+
+
 def test_small_batch_int8_one_pass_leaves_other_shapes_alone(dev):
     # rows off the 16-row strips, rows longer than 48 super-blocks and other formats keep their kernels: same bits
     # whether the option is on or off
