@@ -109,7 +109,7 @@ struct MmvShape {
     static constexpr int NLD = (16 + ROWS_LD - 1) / ROWS_LD;   // load instructions per 16-row strip
     static constexpr int PITCH = SBW * 144 + 16;               // LDS pitch of a row's slice (bank spread, 16-byte aligned)
     static constexpr int STAGE_BYTES = 16 * PITCH;
-    static constexpr int EX_BYTES = 8 * 16 * 4;                // d * scale [sub-block][row]
+    static constexpr int EX_BYTES = SBW * 8 * 16 * 4;          // d * scale [super-block of the slice][sub-block][row]
     static constexpr int WAVE_LDS = STAGE_BYTES + EX_BYTES;
     static constexpr int OUT = MT * STRIPS * 4;                // output registers of a lane
     static constexpr size_t SMEM = (size_t)WAVES * WAVE_LDS + (size_t)WAVES * OUT * 64 * sizeof(float);
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, c = lane >> 4;
     uint8_t *stage = smem + wave * S::WAVE_LDS;                 // [16 rows][PITCH]
-    float *s_dsc = (float *)(stage + S::STAGE_BYTES);           // [8][16]
+    float *s_dsc = (float *)(stage + S::STAGE_BYTES);           // [SBW][8][16]
     float *s_red = (float *)(smem + WAVES * S::WAVE_LDS);       // [WAVES][OUT][64]
 
     const int nsb = K >> 8;
@@ -204,33 +204,39 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
         for (int n = 0; n < S::NLD; ++n)
             *(u32x4 *)(stage + n * S::ROWS_LD * S::PITCH + (n == S::NLD - 1 ? park_last : park_at)) = wq[s][n];
         mmv_wave_lds_fence();
+        // (a) every super-block's scales: lane (row j, pair c) unpacks the pair's two scales and mins, folds the row's
+        // d and dmin in, parks d * scale for the lanes that own the row in the C layout and feeds dmin * min to the
+        // f32 matrix instruction; (b) one fence; (c) the sub-block dots.  Two fences per strip, not per super-block.
 #pragma unroll
         for (int b = 0; b < SBW; ++b) {
             // a slice past the end of K contracts the last block it has again (finite numbers) against zero scales
             const uint8_t *blk = mine + min(b, max(nvalid, 1) - 1) * 144;
-            {   // lane (row j, pair c): the pair's two scales and mins times the row's d and dmin
-                const u32x4 h = *(const u32x4 *)blk;
-                uint32_t sc2, m2;
-                q4k_scale_min_pair(h.y, h.z, h.w, c, sc2, m2);
-                const float d = half_bits_to_float((uint16_t)(h.x & 0xFFFF)), dmin = half_bits_to_float((uint16_t)(h.x >> 16));
-                s_dsc[(2 * c) * 16 + j] = d * (float)(sc2 & 0xFF);
-                s_dsc[(2 * c + 1) * 16 + j] = d * (float)(sc2 >> 8);
-                // sum over the 8 sub-blocks of (dmin * m)[weight row] * (d8 * bsum)[activation row]: k = pair c, two halves
-                const float m_lo = dmin * (float)(m2 & 0xFF), m_hi = dmin * (float)(m2 >> 8);
+            const u32x4 h = *(const u32x4 *)blk;
+            uint32_t sc2, m2;
+            q4k_scale_min_pair(h.y, h.z, h.w, c, sc2, m2);
+            const float d = half_bits_to_float((uint16_t)(h.x & 0xFFFF)), dmin = half_bits_to_float((uint16_t)(h.x >> 16));
+            s_dsc[b * 128 + (2 * c) * 16 + j] = d * (float)(sc2 & 0xFF);
+            s_dsc[b * 128 + (2 * c + 1) * 16 + j] = d * (float)(sc2 >> 8);
+            // sum over the 8 sub-blocks of (dmin * m)[weight row] * (d8 * bsum)[activation row]: k = pair c, two halves
+            const float m_lo = dmin * (float)(m2 & 0xFF), m_hi = dmin * (float)(m2 >> 8);
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    accm[mt][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(m_lo, xmv[mt][b].x, accm[mt][s], 0, 0, 0);
-                    accm[mt][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(m_hi, xmv[mt][b].y, accm[mt][s], 0, 0, 0);
-                }
+            for (int mt = 0; mt < MT; ++mt) {
+                accm[mt][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(m_lo, xmv[mt][b].x, accm[mt][s], 0, 0, 0);
+                accm[mt][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(m_hi, xmv[mt][b].y, accm[mt][s], 0, 0, 0);
             }
-            mmv_wave_lds_fence();
+        }
+        mmv_wave_lds_fence();
+#pragma unroll
+        for (int b = 0; b < SBW; ++b) {
+            const uint8_t *blk = mine + min(b, max(nvalid, 1) - 1) * 144;
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 const u32x2 qa = *(const u32x2 *)(blk + 16 + 32 * p + 8 * c);
                 const long a_lo = (long)(((uint64_t)(qa.y & 0x0F0F0F0Fu) << 32) | (qa.x & 0x0F0F0F0Fu));
                 const long a_hi = (long)(((uint64_t)((qa.y >> 4) & 0x0F0F0F0Fu) << 32) | ((qa.x >> 4) & 0x0F0F0F0Fu));
                 // C layout: lane (activation row j, weight rows 4c .. 4c+3)
-                const float4 sc_lo = *(const float4 *)&s_dsc[(2 * p) * 16 + 4 * c], sc_hi = *(const float4 *)&s_dsc[(2 * p + 1) * 16 + 4 * c];
+                const float4 sc_lo = *(const float4 *)&s_dsc[b * 128 + (2 * p) * 16 + 4 * c];
+                const float4 sc_hi = *(const float4 *)&s_dsc[b * 128 + (2 * p + 1) * 16 + 4 * c];
                 const float dl[4] = {sc_lo.x, sc_lo.y, sc_lo.z, sc_lo.w}, dh[4] = {sc_hi.x, sc_hi.y, sc_hi.z, sc_hi.w};
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
@@ -247,8 +253,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
                     }
                 }
             }
-            mmv_wave_lds_fence();  // the slots are rewritten by the next super-block / strip
         }
+        mmv_wave_lds_fence();  // the stage and the scale slots are rewritten by the next strip
     }
 
     // ---- the K slices meet: each output register is summed by one wavefront, slices in order
@@ -273,7 +279,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restric
 template <int MT, int STRIPS, int SBW, int WAVES>
 static int launch_mmv_cfg(candy_hip_device *dev, const candy_hip_qtensor *w, const MmvOperands &o, int M, float *y) {
     using S = MmvShape<MT, STRIPS, SBW, WAVES>;
-    static_assert(S::SMEM <= 150 * 1024, "LDS");
+    static_assert(S::SMEM <= 160 * 1024, "LDS");
     auto kern = k_mmv_q4k<MT, STRIPS, SBW, WAVES>;
     if (S::SMEM > 48 * 1024)
         CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::SMEM));
