@@ -58,7 +58,7 @@ struct Options {
     int f16_api_min_m = 96;      // candy_hip_qmatmul*: the same threshold for a single contraction (3e-4 per matmul)
     int mmq_fp16_only = 0;       // 1: every tile contraction on the single-buffered fp16 tiles
     int i8_grid_split = 1;       // int8 tiles: split K over workgroups on small grids
-    int f16_shape = 0;           // comparison runs: Q4_K fp16 tiles 128 x 128 (2), 128 x 256 (3)
+    int f16_shape = 0;           // comparison runs: Q4_K fp16 tiles 128 x 128 (2); single-role 128 x 256 kernel (3)
     int f16_split = 0;           // comparison runs: workgroups that share one fp16 tile's K (0: by grid size)
     int mmv_min_m = 3;           // f32 x Q4_K with this many .. mmv_max_m rows: the one-pass int8 kernel
     int mmv_max_m = 32;          //   (0: never; more than 16 rows only for rows of up to 4096 values)

@@ -35,7 +35,17 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ half2v bits_h2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
 
 constexpr int BIG_BK = 64;
-constexpr int BIG_PITCH = BIG_BK + 8;  // halves per LDS row (144 bytes)
+// LDS tiles are stored as the matrix instruction reads them: a fragment of 16 rows x 32 values of K is 1 KB, its
+// 16-byte pieces (8 values of K of one row) in the order lane = 16 * (piece of K) + row, so that a wavefront's
+// operand read is 64 consecutive pieces.  (With rows laid end to end, padded or not, the 8 lanes of a group
+// straddle both halves of the 64 banks and every 128-bit read takes close to twice the cycles; measured with a
+// read-only probe: 2.8 against 4.7 ticks per instruction at 16 wavefronts.)  Offset in halves of piece (row, k):
+__device__ __forceinline__ int frag_off(int row, int k) {
+    const int piece = (k >> 3) & 3;
+    return (((row >> 4) * 2 + (k >> 5)) << 9) + (((piece << 4) + ((row & 15) ^ piece)) << 3);
+}
+// ... and of the piece lane `lane` of a wavefront reads from a fragment
+__device__ __forceinline__ int frag_lane_off(int lane) { return (((lane >> 4) << 4) + ((lane & 15) ^ (lane >> 4))) << 3; }
 
 // ------------------------------------------------------------------ per-format policies
 // A task is (row, quarter c in 0..3) of one 64-wide step g in 0..3 of a super-block: 16 weights.
@@ -247,11 +257,16 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
     constexpr int BCH = BM * 8 / T;   // 16-byte activation chunks per thread per step
     static_assert(BN * 4 % T == 0 && BM * 8 % T == 0 && TN >= 1 && TM >= 1, "tile shape");
     extern __shared__ __align__(16) uint8_t smem_raw[];
-    _Float16 *sA = (_Float16 *)smem_raw;               // [2][BN][PITCH]
-    _Float16 *sB = sA + 2 * BN * BIG_PITCH;            // [2][BM][PITCH]
+    _Float16 *sA = (_Float16 *)smem_raw;               // [2][BN / 16][2] fragments
+    _Float16 *sB = sA + 2 * BN * BIG_BK;               // [2][BM / 16][2] fragments
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wn = wave % WN, wm = wave / WN;
+    // Staging lane maps: neighbouring lanes take neighbouring pieces of a row (global loads of whole 64- and 128-byte
+    // runs); the 32 lanes of a half-wavefront take rows {x, x+4, x+8, x+12}, which the row ^ piece term of the
+    // layout spreads over all 16 bank windows.
+    const int a_c = lane & 3, a_r = 4 * ((lane >> 2) & 3) + (lane >> 4);
+    const int b_kc = lane & 7, b_r = 4 * ((lane >> 3) & 3) + (lane >> 5);  // + 2 (i & 1)
 
     // tile numbering: the hardware deals workgroups round-robin to the 8 XCDs; give each XCD a
     // contiguous run of weight tiles inside one activation tile
@@ -275,33 +290,33 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
     auto gload_a = [&](int sb, int slot) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < ATK; ++i) {
-            const int task = tid + i * T, row = task >> 2, c = task & 3;
-            F::load(W + (size_t)min(n0 + row, N - 1) * rb + (size_t)sb * F::BLOCK, c, raw[slot][i]);
+            const int row = ((tid + i * T) >> 6) * 16 + a_r;
+            F::load(W + (size_t)min(n0 + row, N - 1) * rb + (size_t)sb * F::BLOCK, a_c, raw[slot][i]);
         }
     };
     auto gload_b = [&](int ks, int slot) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < BCH; ++i) {
-            const int ch = tid + i * T, r = ch >> 3, kc = ch & 7;
-            xr[slot][i] = *(const u32x4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BIG_BK + kc * 8);
+            const int r = (wave + (T / 64) * (i >> 1)) * 16 + 2 * (i & 1) + b_r;
+            xr[slot][i] = *(const u32x4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BIG_BK + b_kc * 8);
         }
     };
     auto stage = [&](int g, int aslot, int bslot, int buf) __attribute__((always_inline)) {
-        _Float16 *a = sA + buf * BN * BIG_PITCH;
-        _Float16 *b = sB + buf * BM * BIG_PITCH;
+        _Float16 *a = sA + buf * BN * BIG_BK;
+        _Float16 *b = sB + buf * BM * BIG_BK;
 #pragma unroll
         for (int i = 0; i < ATK; ++i) {
-            const int task = tid + i * T, row = task >> 2, c = task & 3;
+            const int row = ((tid + i * T) >> 6) * 16 + a_r;
             half8 o0, o1;
             int k0, k1;
-            F::dequant(raw[aslot][i], g, c, o0, o1, k0, k1);
-            *(half8 *)&a[row * BIG_PITCH + k0] = o0;
-            *(half8 *)&a[row * BIG_PITCH + k1] = o1;
+            F::dequant(raw[aslot][i], g, a_c, o0, o1, k0, k1);
+            *(half8 *)&a[frag_off(row, k0)] = o0;
+            *(half8 *)&a[frag_off(row, k1)] = o1;
         }
 #pragma unroll
         for (int i = 0; i < BCH; ++i) {
-            const int ch = tid + i * T, r = ch >> 3, kc = ch & 7;
-            *(u32x4 *)&b[r * BIG_PITCH + kc * 8] = xr[bslot][i];
+            const int r = (wave + (T / 64) * (i >> 1)) * 16 + 2 * (i & 1) + b_r;
+            *(u32x4 *)&b[frag_off(r, b_kc * 8)] = xr[bslot][i];
         }
     };
 
@@ -312,15 +327,15 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
         for (int b = 0; b < TM; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
 
     auto compute = [&](int buf) __attribute__((always_inline)) {
-        const _Float16 *a = sA + buf * BN * BIG_PITCH + (wn * (BN / WN) + (lane & 15)) * BIG_PITCH + (lane >> 4) * 8;
-        const _Float16 *b = sB + buf * BM * BIG_PITCH + (wm * (BM / WM) + (lane & 15)) * BIG_PITCH + (lane >> 4) * 8;
+        const _Float16 *a = sA + buf * BN * BIG_BK + wn * (BN / WN) * BIG_BK + frag_lane_off(lane);
+        const _Float16 *b = sB + buf * BM * BIG_BK + wm * (BM / WM) * BIG_BK + frag_lane_off(lane);
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
             half8 af[TN], bf[TM];
 #pragma unroll
-            for (int tn = 0; tn < TN; ++tn) af[tn] = *(const half8 *)&a[tn * 16 * BIG_PITCH + kk * 32];
+            for (int tn = 0; tn < TN; ++tn) af[tn] = *(const half8 *)&a[(tn * 2 + kk) * 512];
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) bf[tm] = *(const half8 *)&b[tm * 16 * BIG_PITCH + kk * 32];
+            for (int tm = 0; tm < TM; ++tm) bf[tm] = *(const half8 *)&b[(tm * 2 + kk) * 512];
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -386,6 +401,178 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
         }
 }
 
+// ------------------------------------------------------------------ the same tile with the work split by role
+// 128 weight rows x 256 activation rows, 8 wavefronts: wavefronts 0-3 (one per SIMD) are producers, 4-7 consumers.
+// Producers request weights and activations, dequantize and fill the LDS buffers of step s + 1 while the
+// consumers read the operands of step s (each a 64 x 128 sub-tile: 24 KB of LDS reads per step instead of the
+// 4 x 8 KB that two 64 x 64 wavefronts of a SIMD read for the same matrix work) and issue its matrix
+// instructions; one workgroup barrier per step hands a buffer over.  In the single-role kernel every wavefront
+// walks the same phases in step (operand reads, matrix instructions, dequantization, LDS writes), so the LDS port,
+// the matrix cores and the vector ALU take turns; here a SIMD's two wavefronts are in different phases by
+// construction.  The two roles are separate loops with the same number of barriers, so that their registers
+// (accumulators and operand fragments here, raw blocks and activation chunks there) share one allocation.
+template <class F, bool RES>
+__global__ __launch_bounds__(512) void k_mmq_f16_pc(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xh,
+                                                    float *out, const float *res, int N, int M, int K, int n_tiles,
+                                                    int m_tiles, int sb_per) {
+    constexpr int BN = 128, BM = 256, PT = 256;
+    constexpr int ATK = BN * 4 / PT;  // dequantization tasks per producer thread per step
+    constexpr int BCH = BM * 8 / PT;  // 16-byte activation chunks per producer thread per step
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    _Float16 *sA = (_Float16 *)smem_raw;               // [2][BN / 16][2] fragments
+    _Float16 *sB = sA + 2 * BN * BIG_BK;               // [2][BM / 16][2] fragments
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    const int total = n_tiles * m_tiles;
+    const int split = blockIdx.x / total;
+    int v = blockIdx.x - split * total;
+    if ((total & 7) == 0) v = (v & 7) * (total >> 3) + (v >> 3);
+    const int mt = v / n_tiles, nt = v - mt * n_tiles;
+    const int n0 = nt * BN, m0 = mt * BM;
+
+    const size_t rb = (size_t)(K >> 8) * F::BLOCK;
+    const int sb0 = split * sb_per;
+    const int n_sb = min(K >> 8, sb0 + sb_per) - sb0;  // >= 1 by construction of the grid
+    const int steps = n_sb * 4;
+    W += (size_t)sb0 * F::BLOCK;
+    xh += (size_t)sb0 * 256;
+    out += (size_t)split * M * N;
+
+    if (wave < 4) {
+        // ---------------- producers
+        typename F::Raw raw[2][ATK];
+        u32x4 xr[2][BCH];
+        // neighbouring lanes take neighbouring pieces of a row; a half-wavefront takes rows {x, x+4, x+8, x+12}
+        const int a_c = lane & 3, a_row = 16 * wave + 4 * ((lane >> 2) & 3) + (lane >> 4);   // + 64 i
+        const int b_kc = lane & 7, b_row = 4 * ((lane >> 3) & 3) + (lane >> 5);              // + 16 block + 2 half
+        auto gload_a = [&](int sb, int slot) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < ATK; ++i)
+                F::load(W + (size_t)min(n0 + a_row + 64 * i, N - 1) * rb + (size_t)sb * F::BLOCK, a_c, raw[slot][i]);
+        };
+        auto gload_b = [&](int ks, int slot) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < BCH; ++i) {
+                const int r = 16 * (wave * 4 + (i >> 1)) + 2 * (i & 1) + b_row;
+                xr[slot][i] = *(const u32x4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BIG_BK + b_kc * 8);
+            }
+        };
+        auto stage = [&](int g, int aslot, int bslot, int buf) __attribute__((always_inline)) {
+            _Float16 *a = sA + buf * BN * BIG_BK;
+            _Float16 *b = sB + buf * BM * BIG_BK;
+#pragma unroll
+            for (int i = 0; i < ATK; ++i) {
+                half8 o0, o1;
+                int k0, k1;
+                F::dequant(raw[aslot][i], g, a_c, o0, o1, k0, k1);
+                *(half8 *)&a[frag_off(a_row + 64 * i, k0)] = o0;
+                *(half8 *)&a[frag_off(a_row + 64 * i, k1)] = o1;
+            }
+#pragma unroll
+            for (int i = 0; i < BCH; ++i) {
+                const int r = 16 * (wave * 4 + (i >> 1)) + 2 * (i & 1) + b_row;
+                *(u32x4 *)&b[frag_off(r, b_kc * 8)] = xr[bslot][i];
+            }
+        };
+        gload_a(0, 0);
+        gload_b(0, 0);
+        gload_b(1, 1);
+        gload_a(min(1, n_sb - 1), 1);
+        stage(0, 0, 0, 0);
+        gload_b(2, 0);
+        __syncthreads();
+        for (int sb2 = 0; sb2 < n_sb; sb2 += 2) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int sb = sb2 + half;
+                if (sb >= n_sb) break;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int ks = sb * 4 + g;
+                    // while the consumers contract step ks from buffer g & 1: fill the other buffer with step ks + 1
+                    if (g < 3) stage(g + 1, half, (g + 1) & 1, (g + 1) & 1);
+                    else stage(0, half ^ 1, 0, 0);
+                    gload_b(min(ks + 3, steps - 1), (g + 1) & 1);
+                    if (g == 3) gload_a(min(sb + 2, n_sb - 1), half);
+                    __syncthreads();
+                }
+            }
+        }
+        return;
+    }
+
+    // ---------------- consumers: 2 x 2 wavefronts of 64 weight rows x 128 activation rows
+    const int cw = wave - 4, cn = cw & 1, cm = cw >> 1;
+    float4v acc[4][8];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 8; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](int buf) __attribute__((always_inline)) {
+        const _Float16 *a = sA + buf * BN * BIG_BK + cn * 64 * BIG_BK + frag_lane_off(lane);
+        const _Float16 *b = sB + buf * BM * BIG_BK + cm * 128 * BIG_BK + frag_lane_off(lane);
+        half8 af[2][4], bf[2][8];
+        auto fetch = [&](int kk) __attribute__((always_inline)) {
+#pragma unroll
+            for (int tn = 0; tn < 4; ++tn) af[kk][tn] = *(const half8 *)&a[(tn * 2 + kk) * 512];
+#pragma unroll
+            for (int tm = 0; tm < 8; ++tm) bf[kk][tm] = *(const half8 *)&b[(tm * 2 + kk) * 512];
+        };
+        auto mma = [&](int kk) __attribute__((always_inline)) {
+#pragma unroll
+            for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+                for (int tm = 0; tm < 8; ++tm)
+                    acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[kk][tn], bf[kk][tm], acc[tn][tm], 0, 0, 0);
+        };
+        // the second half's operands are read while the first half's matrix instructions run
+        fetch(0);
+        fetch(1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(0);
+        mma(1);
+    };
+    __syncthreads();
+    for (int sb2 = 0; sb2 < n_sb; sb2 += 2) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int sb = sb2 + half;
+            if (sb >= n_sb) break;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                compute(g & 1);
+                __syncthreads();
+            }
+        }
+    }
+
+    // C layout of a 16x16 tile: lane holds activation row (lane & 15) and weight rows 4*(lane>>4)..+3
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < 8; ++tm) {
+            const int m = m0 + cm * 128 + tm * 16 + (lane & 15);
+            const int n = n0 + cn * 64 + tn * 16 + 4 * (lane >> 4);
+            if (m >= M) continue;
+            float *dst = out + (size_t)m * N + n;
+            const float *r = RES ? res + (size_t)m * N + n : nullptr;  // may alias dst: read before the store
+            if (n + 3 < N && (N & 3) == 0) {
+                float4 o = make_float4(acc[tn][tm][0], acc[tn][tm][1], acc[tn][tm][2], acc[tn][tm][3]);
+                if (r) {
+                    const float4 rv = *(const float4 *)r;
+                    o = make_float4(rv.x + o.x, rv.y + o.y, rv.z + o.z, rv.w + o.w);
+                }
+                *(float4 *)dst = o;
+            } else {
+#pragma unroll
+                for (int l = 0; l < 4; ++l)
+                    if (n + l < N) dst[l] = r ? r[l] + acc[tn][tm][l] : acc[tn][tm][l];
+            }
+        }
+}
+
 // y[i] = (res[i] +) part[0][i] + part[1][i] + ... in that order; res may alias y
 __global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ part, float *y, const float *res, size_t count,
                                                     int n_split) {
@@ -418,9 +605,10 @@ int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const 
     return CANDY_HIP_OK;
 }
 
-template <class F, int BN, int BM, int WN, int WM>
+template <class F, int BN, int BM, int WN, int WM, bool PC = false>
 static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                       const float *res) {
+    static_assert(!PC || (BN == 128 && BM == 256 && WN * WM == 8), "the role-split kernel is the 128 x 256 tile");
     const int N = (int)w->rows, K = (int)w->cols;
     const int n_tiles = (N + BN - 1) / BN, m_tiles = (int)((m + BM - 1) / BM);
     const int tiles = n_tiles * m_tiles, n_sb = K >> 8;
@@ -444,9 +632,11 @@ static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _
         if (int rc = splitk_workspace(dev, (size_t)n_split * (size_t)m * N * sizeof(float), &p)) return rc;
         out = (float *)p;
     }
-    constexpr size_t smem = (size_t)2 * (BN + BM) * BIG_PITCH * sizeof(_Float16);
+    constexpr size_t smem = (size_t)2 * (BN + BM) * BIG_BK * sizeof(_Float16);
     const bool epi_res = res && n_split == 1;  // otherwise the split sum adds it
-    auto kern = epi_res ? k_mmq_f16<F, BN, BM, WN, WM, true> : k_mmq_f16<F, BN, BM, WN, WM, false>;
+    void (*kern)(const uint8_t *, const _Float16 *, float *, const float *, int, int, int, int, int, int);
+    if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, true> : k_mmq_f16_pc<F, false>;
+    else kern = epi_res ? k_mmq_f16<F, BN, BM, WN, WM, true> : k_mmq_f16<F, BN, BM, WN, WM, false>;
     CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream,
                        (const uint8_t *)w->data, xh, out, epi_res ? res : nullptr, N, (int)m, K, n_tiles, m_tiles, sb_per);
@@ -474,11 +664,12 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m) {
 // xh: fp16 activations [mmq_m_pad(m)][K], rows past m zero.
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                        const float *res) {
-    if (w->fmt == CANDY_HIP_Q6_K) return launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q5_K) return launch_big<BigQ5K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q8_0) return launch_big<BigQ8_0, 128, 256, 2, 4>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q4_0) return launch_big<BigQ4_0<false>, 128, 256, 2, 4>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q4_0_GGML) return launch_big<BigQ4_0<true>, 128, 256, 2, 4>(dev, w, xh, m, y, res);
+    const bool single = dev->opt.f16_shape == 3;  // comparison runs: every wavefront in both roles
+    if (w->fmt == CANDY_HIP_Q6_K) return single ? launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ6K, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
+    if (w->fmt == CANDY_HIP_Q5_K) return single ? launch_big<BigQ5K, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ5K, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
+    if (w->fmt == CANDY_HIP_Q8_0) return single ? launch_big<BigQ8_0, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ8_0, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
+    if (w->fmt == CANDY_HIP_Q4_0) return single ? launch_big<BigQ4_0<false>, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ4_0<false>, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
+    if (w->fmt == CANDY_HIP_Q4_0_GGML) return single ? launch_big<BigQ4_0<true>, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ4_0<true>, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
     // up to 128 activation rows: 128 x 128 tiles (two workgroups per CU), K split over workgroups to fill the chip
     const int shape = dev->opt.f16_shape;  // comparison runs
     if (shape == 2) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, w, xh, m, y, res);
@@ -489,7 +680,7 @@ int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const 
     const int64_t n128 = (w->rows + 127) / 128, fill = (3 * (int64_t)dev->num_cus) / 4;
     if (m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill)
         return launch_big<BigQ4K, 128, 128, 2, 4>(dev, w, xh, m, y, res);
-    return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
+    return launch_big<BigQ4K, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
 }
 
 }  // namespace candy

@@ -90,7 +90,11 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   "mmq.i8_min_m"               0        5..15 rows: int8 tiles from this batch on (0: by measured cost model)
  *   "mmq.fp16_only"              0        every tile contraction on the single-buffered fp16 tiles
  *   "mmq.i8_grid_split"          1        int8 tiles split K over workgroups on small grids
- *   "mmq.f16_shape"              0        Q4_K fp16 tiles of 128 x 128 (2) or 128 x 256 (3) at every batch (0: by shape)
+ *   "mmq.f16_shape"              0        comparison runs: Q4_K fp16 tiles of 128 x 128 at every batch (2); 128 x 256 tiles
+ *                                         computed by the kernel whose wavefronts each dequantize and multiply (3)
+ *                                         instead of the one that splits the two roles over wavefronts (0: by shape)
+ *   "mmq.f16_split"              0        comparison runs: K split of the fp16 tile kernels over this many workgroups per
+ *                                         tile, 1..16 (0: as many as fill the chip)
  *   "mmv.min_m"                  3        candy_hip_qmatmul on Q4_K: batches of this many .. "mmv.max_m" rows take the
  *   "mmv.max_m"                  32         one-pass int8 matrix-core kernel (max 0: never)
  *   "mmv.variant"                0        that kernel with one (1) or two (2) 16-row strips per wavefront (0: by shape)

@@ -118,6 +118,24 @@ def test_big_fp16_tiles(dev, fmt, m, rows, cols):
         assert np.max(per_row) <= 2 * TOL
 
 
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML])
+@pytest.mark.parametrize("m,rows,cols", [(256, 128, 256), (300, 129, 1024), (513, 1030, 768), (700, 130, 4352),
+                                         (260, 2100, 512)])
+def test_role_split_tiles_equal_the_single_role_tiles(dev, fmt, m, rows, cols):
+    # 128 x 256 tiles: producer / consumer wavefronts (the default) and the kernel whose wavefronts do both run
+    # the same multiply-adds in the same order on the same fp16 operands, with and without a K split
+    w = synth.random_weight(fmt, rows, cols, seed=rows + 3 * m)
+    x = synth.random_activations(m, cols, seed=cols + m)
+    q = dev.qtensor(fmt, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    dev.set_option("mmq.f16_shape", 3)
+    try:
+        single = dev.qmatmul(q, x)
+    finally:
+        dev.set_option("mmq.f16_shape", 0)
+    assert np.array_equal(got.view(np.uint32), single.view(np.uint32))
+
+
 def test_q8_0_wide_prompt_grid_takes_the_fp16_tiles(dev):
     # many weight rows and a prompt-sized batch: Q8_0 leaves the int8 tiles for the 128 x 128 fp16 tiles
     rows, cols, m = 8192, 256, 352
