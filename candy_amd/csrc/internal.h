@@ -65,6 +65,7 @@ struct Options {
     int mmv_variant = 0;         // comparison runs: 1 = one 16-row strip per wavefront, 2 = two
     int pair_rows = 0;           // fused gate/up: row pairs per workgroup, 32 / 16 / 8 (0: the most even split)
     int rms_rows = 0;            // fused RMSNorm prologue: rows per workgroup, 16 / 24 (0: the most even split)
+    int prefill_qkv_group = 1;       // prompt pass: q / k / v projections on one grid where they share the fp16 tiles
     int prefill_attention_valu = 0;  // prompt attention for head_dim 128 on the vector ALU instead of the matrix cores
     int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
     int fused_wide = 1;          // decode step: one-workgroup-per-CU kernels for the big Q4_K shapes (0: the narrower ones)
@@ -191,6 +192,10 @@ int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m = 0);
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                        const float *res = nullptr);
+// Two or three projections of the same activations on one grid (every tensor but the last: a multiple of 128 rows).
+bool mmq_f16_group_covers(const candy_hip_qtensor *const *ws, int count, int64_t m);
+int launch_mmq_f16_group(candy_hip_device *dev, const candy_hip_qtensor *const *ws, float *const *ys, int count,
+                         const _Float16 *xh, int64_t m);
 // ops.hip: fused decode-step stages (all enqueue on dev->stream, no allocation, no sync).
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
                           int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales, _Float16 *xh = nullptr);

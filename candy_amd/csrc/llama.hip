@@ -422,9 +422,11 @@ static int prompt_reserve(candy_hip_llama *m, int n) {
     int rc = CANDY_HIP_OK;
     if (!rc) rc = prompt_alloc(m, &P.ids, N);
     if (!rc) rc = prompt_alloc(m, &P.h, N * c.d_model);
-    if (!rc) rc = prompt_alloc(m, &P.q, N * qd);
-    if (!rc) rc = prompt_alloc(m, &P.k, N * kvd);
-    if (!rc) rc = prompt_alloc(m, &P.v, N * kvd);
+    if (!rc) rc = prompt_alloc(m, &P.q, N * (qd + 2 * kvd));  // q, k, v end to end: one split-K sum serves the three
+    if (!rc) {
+        P.k = P.q + N * qd;
+        P.v = P.k + N * kvd;
+    }
     if (!rc) rc = prompt_alloc(m, &P.att, N * qd);
     if (!rc) rc = prompt_alloc(m, &P.tmp, N * c.d_model);
     if (!rc) rc = prompt_alloc(m, &P.gate, N * c.d_ffn);
@@ -463,9 +465,15 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
         };
         _Float16 *xh = (xh_for(L.wq) || xh_for(L.wk) || xh_for(L.wv)) ? P.xh : nullptr;
         if ((rc = launch_rms_norm_quant(dev, P.h, L.attn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs, xh))) return rc;
-        if ((rc = launch_contract(dev, L.wq, P.xq, P.xs, n, P.q, xh_for(L.wq)))) return rc;
-        if ((rc = launch_contract(dev, L.wk, P.xq, P.xs, n, P.k, xh_for(L.wk)))) return rc;
-        if ((rc = launch_contract(dev, L.wv, P.xq, P.xs, n, P.v, xh_for(L.wv)))) return rc;
+        const candy_hip_qtensor *qkv_w[3] = {L.wq, L.wk, L.wv};
+        float *qkv_y[3] = {P.q, P.k, P.v};
+        if (xh && mmq_f16_group_covers(qkv_w, 3, n)) {  // one grid for the three projections
+            if ((rc = launch_mmq_f16_group(dev, qkv_w, qkv_y, 3, xh, n))) return rc;
+        } else {
+            if ((rc = launch_contract(dev, L.wq, P.xq, P.xs, n, P.q, xh_for(L.wq)))) return rc;
+            if ((rc = launch_contract(dev, L.wk, P.xq, P.xs, n, P.k, xh_for(L.wk)))) return rc;
+            if ((rc = launch_contract(dev, L.wv, P.xq, P.xs, n, P.v, xh_for(L.wv)))) return rc;
+        }
         if ((rc = launch_prefill_rope_kv(dev, P.q, P.k, P.v, m->cos_t, m->sin_t, kc, vc, m->kv_f16, n, pos0, c.n_heads,
                                          c.n_kv_heads, c.head_dim, cache_stride)))
             return rc;

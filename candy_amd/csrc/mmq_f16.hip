@@ -245,12 +245,30 @@ struct BigQ6K {
 };
 
 // ------------------------------------------------------------------ tile kernel
+// One launch may serve up to three weight tensors that share the activations (q / k / v of a prompt pass): weight
+// tiles [tile0, next tile0) belong to segment s, which has its own weights, row count, output and residual.
+struct F16Seg {
+    const uint8_t *W;
+    float *out;
+    const float *res;
+    int N, tile0;
+};
+struct F16Group {
+    F16Seg seg[3];
+    int count;
+    __device__ __forceinline__ F16Seg pick(int nt) const {
+        F16Seg s = seg[0];
+        if (count > 1 && nt >= seg[1].tile0) s = seg[1];
+        if (count > 2 && nt >= seg[2].tile0) s = seg[2];
+        return s;
+    }
+};
+
 // grid = tiles * n_split; workgroup (tile, split) contracts super-blocks [split*sb_per, ...) and writes
-// its tile to out + split * M * N (out = y when n_split == 1).
+// its tile to out + split * split_stride (out = y when n_split == 1).
 template <class F, int BN, int BM, int WN, int WM, bool RES>
-__global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xh,
-                                                          float *out, const float *res, int N, int M, int K,
-                                                          int n_tiles, int m_tiles, int sb_per) {
+__global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, const _Float16 *__restrict__ xh, int M, int K,
+                                                          int n_tiles, int m_tiles, int sb_per, size_t split_stride) {
     constexpr int T = WN * WM * 64;
     constexpr int TN = BN / WN / 16, TM = BM / WM / 16;
     constexpr int ATK = BN * 4 / T;   // dequantization tasks per thread per step
@@ -275,15 +293,18 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
     int v = blockIdx.x - split * total;
     if ((total & 7) == 0) v = (v & 7) * (total >> 3) + (v >> 3);
     const int mt = v / n_tiles, nt = v - mt * n_tiles;
-    const int n0 = nt * BN, m0 = mt * BM;
+    const F16Seg seg = grp.pick(nt);
+    const int N = seg.N;
+    const int n0 = (nt - seg.tile0) * BN, m0 = mt * BM;
 
     const size_t rb = (size_t)(K >> 8) * F::BLOCK;
     const int sb0 = split * sb_per;
     const int n_sb = min(K >> 8, sb0 + sb_per) - sb0;  // >= 1 by construction of the grid
     const int steps = n_sb * 4;
-    W += (size_t)sb0 * F::BLOCK;
+    const uint8_t *__restrict__ W = seg.W + (size_t)sb0 * F::BLOCK;
     xh += (size_t)sb0 * 256;
-    out += (size_t)split * M * N;
+    float *out = seg.out + (size_t)split * split_stride;
+    const float *res = seg.res;
 
     typename F::Raw raw[2][ATK];
     u32x4 xr[2][BCH];
@@ -385,7 +406,7 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
             const int n = n0 + wn * (BN / WN) + tn * 16 + 4 * (lane >> 4);
             if (m >= M) continue;
             float *dst = out + (size_t)m * N + n;
-            const float *r = RES ? res + (size_t)m * N + n : nullptr;  // may alias dst: read before the store
+            const float *r = RES && res ? res + (size_t)m * N + n : nullptr;  // may alias dst: read before the store
             if (n + 3 < N && (N & 3) == 0) {
                 float4 o = make_float4(acc[tn][tm][0], acc[tn][tm][1], acc[tn][tm][2], acc[tn][tm][3]);
                 if (r) {
@@ -412,9 +433,8 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const uint8_t *__restr
 // construction.  The two roles are separate loops with the same number of barriers, so that their registers
 // (accumulators and operand fragments here, raw blocks and activation chunks there) share one allocation.
 template <class F, bool RES>
-__global__ __launch_bounds__(512) void k_mmq_f16_pc(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xh,
-                                                    float *out, const float *res, int N, int M, int K, int n_tiles,
-                                                    int m_tiles, int sb_per) {
+__global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _Float16 *__restrict__ xh, int M, int K,
+                                                    int n_tiles, int m_tiles, int sb_per, size_t split_stride) {
     constexpr int BN = 128, BM = 256, PT = 256;
     constexpr int ATK = BN * 4 / PT;  // dequantization tasks per producer thread per step
     constexpr int BCH = BM * 8 / PT;  // 16-byte activation chunks per producer thread per step
@@ -430,15 +450,18 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const uint8_t *__restrict__ 
     int v = blockIdx.x - split * total;
     if ((total & 7) == 0) v = (v & 7) * (total >> 3) + (v >> 3);
     const int mt = v / n_tiles, nt = v - mt * n_tiles;
-    const int n0 = nt * BN, m0 = mt * BM;
+    const F16Seg seg = grp.pick(nt);
+    const int N = seg.N;
+    const int n0 = (nt - seg.tile0) * BN, m0 = mt * BM;
 
     const size_t rb = (size_t)(K >> 8) * F::BLOCK;
     const int sb0 = split * sb_per;
     const int n_sb = min(K >> 8, sb0 + sb_per) - sb0;  // >= 1 by construction of the grid
     const int steps = n_sb * 4;
-    W += (size_t)sb0 * F::BLOCK;
+    const uint8_t *__restrict__ W = seg.W + (size_t)sb0 * F::BLOCK;
     xh += (size_t)sb0 * 256;
-    out += (size_t)split * M * N;
+    float *out = seg.out + (size_t)split * split_stride;
+    const float *res = seg.res;
 
     if (wave < 4) {
         // ---------------- producers
@@ -557,7 +580,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const uint8_t *__restrict__ 
             const int n = n0 + cn * 64 + tn * 16 + 4 * (lane >> 4);
             if (m >= M) continue;
             float *dst = out + (size_t)m * N + n;
-            const float *r = RES ? res + (size_t)m * N + n : nullptr;  // may alias dst: read before the store
+            const float *r = RES && res ? res + (size_t)m * N + n : nullptr;  // may alias dst: read before the store
             if (n + 3 < N && (N & 3) == 0) {
                 float4 o = make_float4(acc[tn][tm][0], acc[tn][tm][1], acc[tn][tm][2], acc[tn][tm][3]);
                 if (r) {
@@ -573,15 +596,15 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const uint8_t *__restrict__ 
         }
 }
 
-// y[i] = (res[i] +) part[0][i] + part[1][i] + ... in that order; res may alias y
+// y[i] = (res[i] +) part[0][i] + part[1][i] + ... in that order (copies `stride` floats apart); res may alias y
 __global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ part, float *y, const float *res, size_t count,
-                                                    int n_split) {
+                                                    int n_split, size_t stride) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= count) return;
-    if (i + 4 <= count && ((uintptr_t)y & 15) == 0 && (count & 3) == 0) {
+    if (i + 4 <= count && (((uintptr_t)y | (uintptr_t)part | (uintptr_t)res) & 15) == 0 && ((count | stride) & 3) == 0) {
         float4 s = *(const float4 *)(part + i);
         for (int k = 1; k < n_split; ++k) {
-            const float4 v = *(const float4 *)(part + (size_t)k * count + i);
+            const float4 v = *(const float4 *)(part + (size_t)k * stride + i);
             s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
         }
         if (res) {
@@ -592,7 +615,7 @@ __global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ pa
     } else {
         for (size_t j = i; j < i + 4 && j < count; ++j) {
             float s = part[j];
-            for (int k = 1; k < n_split; ++k) s += part[(size_t)k * count + j];
+            for (int k = 1; k < n_split; ++k) s += part[(size_t)k * stride + j];
             y[j] = res ? res[j] + s : s;
         }
     }
@@ -600,17 +623,35 @@ __global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ pa
 
 int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split) {
     hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((count / 4 + 256) / 256)), dim3(256), 0, dev->stream, part, y, res,
-                       count, n_split);
+                       count, n_split, count);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
 
+// Up to three contractions that share the activations, in one launch (a single one: count = 1).  Every tensor but the
+// last has a multiple of BN rows (a tile belongs to one tensor).
+struct F16Job {
+    const candy_hip_qtensor *w;
+    float *y;
+    const float *res;
+};
+
 template <class F, int BN, int BM, int WN, int WM, bool PC = false>
-static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
-                      const float *res) {
+static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, const _Float16 *xh, int64_t m) {
     static_assert(!PC || (BN == 128 && BM == 256 && WN * WM == 8), "the role-split kernel is the 128 x 256 tile");
-    const int N = (int)w->rows, K = (int)w->cols;
-    const int n_tiles = (N + BN - 1) / BN, m_tiles = (int)((m + BM - 1) / BM);
+    const int K = (int)jobs[0].w->cols;
+    F16Group grp{};
+    grp.count = count;
+    int n_tiles = 0;
+    int64_t n_total = 0;
+    bool any_res = false;
+    for (int s = 0; s < count; ++s) {
+        grp.seg[s] = F16Seg{(const uint8_t *)jobs[s].w->data, jobs[s].y, jobs[s].res, (int)jobs[s].w->rows, n_tiles};
+        n_tiles += (int)((jobs[s].w->rows + BN - 1) / BN);
+        n_total += jobs[s].w->rows;
+        any_res = any_res || jobs[s].res;
+    }
+    const int m_tiles = (int)((m + BM - 1) / BM);
     const int tiles = n_tiles * m_tiles, n_sb = K >> 8;
     // split K until the grid covers the chip, keeping at least two super-blocks (8 steps) per workgroup: as many
     // workgroups per tile as leave every workgroup a CU of its own (measured against rounding up: 14336 x 4096 at
@@ -626,28 +667,54 @@ static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _
     if (dev->opt.f16_split > 0) n_split = std::min(dev->opt.f16_split, n_sb);  // comparison runs
     const int sb_per = (n_sb + n_split - 1) / n_split;
     n_split = (n_sb + sb_per - 1) / sb_per;  // no empty splits
-    float *out = y;
+    const size_t split_stride = (size_t)m * (size_t)n_total;
+    float *part = nullptr;
     if (n_split > 1) {
+        // each workgroup writes its partial tile to copy `split` of a workspace laid out [split][tensor][m][rows]
         void *p = nullptr;
-        if (int rc = splitk_workspace(dev, (size_t)n_split * (size_t)m * N * sizeof(float), &p)) return rc;
-        out = (float *)p;
+        if (int rc = splitk_workspace(dev, (size_t)n_split * split_stride * sizeof(float), &p)) return rc;
+        part = (float *)p;
+        size_t off = 0;
+        for (int s = 0; s < count; ++s) {
+            grp.seg[s].out = part + off;
+            grp.seg[s].res = nullptr;  // the split sum adds it
+            off += (size_t)m * (size_t)jobs[s].w->rows;
+        }
     }
     constexpr size_t smem = (size_t)2 * (BN + BM) * BIG_BK * sizeof(_Float16);
-    const bool epi_res = res && n_split == 1;  // otherwise the split sum adds it
-    void (*kern)(const uint8_t *, const _Float16 *, float *, const float *, int, int, int, int, int, int);
+    const bool epi_res = any_res && n_split == 1;
+    void (*kern)(const F16Group, const _Float16 *, int, int, int, int, int, size_t);
     if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, true> : k_mmq_f16_pc<F, false>;
     else kern = epi_res ? k_mmq_f16<F, BN, BM, WN, WM, true> : k_mmq_f16<F, BN, BM, WN, WM, false>;
     CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream,
-                       (const uint8_t *)w->data, xh, out, epi_res ? res : nullptr, N, (int)m, K, n_tiles, m_tiles, sb_per);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream, grp, xh, (int)m, K,
+                       n_tiles, m_tiles, sb_per, split_stride);
     CANDY_LAUNCH_CHECK();
     if (n_split > 1) {
-        const size_t count = (size_t)m * N;
-        hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((count / 4 + 256) / 256)), dim3(256), 0, dev->stream, out, y, res,
-                           count, n_split);
-        CANDY_LAUNCH_CHECK();
+        // one sum per run of outputs that lie end to end (the prompt pass allocates q, k and v that way)
+        size_t off = 0;
+        for (int s = 0; s < count;) {
+            size_t run = (size_t)m * (size_t)jobs[s].w->rows;
+            int e = s + 1;
+            while (e < count && !jobs[s].res && !jobs[e].res && jobs[e].y == jobs[s].y + run) {
+                run += (size_t)m * (size_t)jobs[e].w->rows;
+                ++e;
+            }
+            hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((run / 4 + 256) / 256)), dim3(256), 0, dev->stream, part + off,
+                               jobs[s].y, jobs[s].res, run, n_split, split_stride);
+            CANDY_LAUNCH_CHECK();
+            off += run;
+            s = e;
+        }
     }
     return CANDY_HIP_OK;
+}
+
+template <class F, int BN, int BM, int WN, int WM, bool PC = false>
+static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
+                      const float *res) {
+    const F16Job job{w, y, res};
+    return launch_big<F, BN, BM, WN, WM, PC>(dev, &job, 1, xh, m);
 }
 
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m) {
@@ -661,26 +728,55 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m) {
     return false;
 }
 
+static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, const _Float16 *xh, int64_t m) {
+    const int fmt = jobs[0].w->fmt;
+    const bool single = dev->opt.f16_shape == 3;  // comparison runs: every wavefront in both roles
+#define CANDY_BIG_256(F)                                                                      \
+    return single ? launch_big<F, 128, 256, 2, 4>(dev, jobs, count, xh, m)                  \
+                  : launch_big<F, 128, 256, 2, 4, true>(dev, jobs, count, xh, m)
+    if (fmt == CANDY_HIP_Q6_K) CANDY_BIG_256(BigQ6K);
+    if (fmt == CANDY_HIP_Q5_K) CANDY_BIG_256(BigQ5K);
+    if (fmt == CANDY_HIP_Q8_0) CANDY_BIG_256(BigQ8_0);
+    if (fmt == CANDY_HIP_Q4_0) CANDY_BIG_256(BigQ4_0<false>);
+    if (fmt == CANDY_HIP_Q4_0_GGML) CANDY_BIG_256(BigQ4_0<true>);
+    // Q4_K. Up to 128 activation rows: 128 x 128 tiles (two workgroups per CU), K split over workgroups to fill the chip
+    const int shape = dev->opt.f16_shape;  // comparison runs
+    if (shape == 2 || m <= 128) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m);
+    // up to 256 rows where the 128 x 128 tiles fill the chip and the 128 x 256 tiles would have to split K
+    // (14336 x 4096 at 256 rows: 70.7 us against 80.3)
+    int64_t n128 = 0;
+    for (int s = 0; s < count; ++s) n128 += (jobs[s].w->rows + 127) / 128;
+    const int64_t fill = (3 * (int64_t)dev->num_cus) / 4;
+    if (shape != 3 && m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill)
+        return launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m);
+    CANDY_BIG_256(BigQ4K);
+#undef CANDY_BIG_256
+}
+
 // xh: fp16 activations [mmq_m_pad(m)][K], rows past m zero.
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                        const float *res) {
-    const bool single = dev->opt.f16_shape == 3;  // comparison runs: every wavefront in both roles
-    if (w->fmt == CANDY_HIP_Q6_K) return single ? launch_big<BigQ6K, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ6K, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q5_K) return single ? launch_big<BigQ5K, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ5K, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q8_0) return single ? launch_big<BigQ8_0, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ8_0, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q4_0) return single ? launch_big<BigQ4_0<false>, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ4_0<false>, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
-    if (w->fmt == CANDY_HIP_Q4_0_GGML) return single ? launch_big<BigQ4_0<true>, 128, 256, 2, 4>(dev, w, xh, m, y, res) : launch_big<BigQ4_0<true>, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
-    // up to 128 activation rows: 128 x 128 tiles (two workgroups per CU), K split over workgroups to fill the chip
-    const int shape = dev->opt.f16_shape;  // comparison runs
-    if (shape == 2) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, w, xh, m, y, res);
-    if (shape == 3) return launch_big<BigQ4K, 128, 256, 2, 4>(dev, w, xh, m, y, res);
-    if (m <= 128) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, w, xh, m, y, res);
-    // up to 256 rows where the 128 x 128 tiles fill the chip and the 128 x 256 tiles would have to split K
-    // (14336 x 4096 at 256 rows: 70.7 us against 80.3)
-    const int64_t n128 = (w->rows + 127) / 128, fill = (3 * (int64_t)dev->num_cus) / 4;
-    if (m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill)
-        return launch_big<BigQ4K, 128, 128, 2, 4>(dev, w, xh, m, y, res);
-    return launch_big<BigQ4K, 128, 256, 2, 4, true>(dev, w, xh, m, y, res);
+    const F16Job job{w, y, res};
+    return launch_jobs(dev, &job, 1, xh, m);
+}
+
+// Two or three projections of the same activations (q / k / v) as one grid: their tiles fill the chip together where
+// each alone would split K many ways (Llama-3-8B shape, 512 rows: 1024 x 4096 alone is 16 tiles).
+bool mmq_f16_group_covers(const candy_hip_qtensor *const *ws, int count, int64_t m) {
+    if (count < 2 || count > 3 || !ws[0]->dev->opt.prefill_qkv_group || ws[0]->dev->opt.mmq_fp16_only) return false;
+    for (int s = 0; s < count; ++s) {
+        if (!mmq_f16_big_covers(ws[s], m) || ws[s]->fmt != ws[0]->fmt || ws[s]->cols != ws[0]->cols) return false;
+        if (s + 1 < count && ws[s]->rows % 128 != 0) return false;  // a tile belongs to one tensor
+    }
+    return true;
+}
+
+int launch_mmq_f16_group(candy_hip_device *dev, const candy_hip_qtensor *const *ws, float *const *ys, int count,
+                         const _Float16 *xh, int64_t m) {
+    CANDY_REQUIRE(mmq_f16_group_covers(ws, count, m), "internal: projections cannot share a grid");
+    F16Job jobs[3];
+    for (int s = 0; s < count; ++s) jobs[s] = F16Job{ws[s], ys[s], nullptr};
+    return launch_jobs(dev, jobs, count, xh, m);
 }
 
 }  // namespace candy

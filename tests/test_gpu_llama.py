@@ -384,6 +384,31 @@ def test_prompt_pass_of_256_rows_and_more_matches_cpu(dev, n):
         tok = rt
 
 
+@pytest.mark.parametrize("n", [256, 300, 512])
+def test_grouped_qkv_projection_agrees_with_separate_launches(dev, n):
+    # From 256 rows on the q / k / v projections share one grid of fp16 tiles (their outputs lie end to end, one sum
+    # over the K splits serves the three).  The same tiles one projection per launch split K differently, so the two
+    # agree to f32 summation order, not bit for bit: first-layer k / v within 1e-5, logits within 1e-4.
+    cfg, fmts = BIG_PROMPT_CFG, BIG_PROMPT_FMTS
+    _, a = build(dev, cfg, fmts, seed=71)
+    _, b = build(dev, cfg, fmts, seed=71)
+    tokens = [int(t) for t in np.random.default_rng(90 + n).integers(0, cfg["vocab"], n)]
+    ta, la = a.prefill(tokens, 0)
+    dev.set_option("prefill.qkv_group", 0)
+    try:
+        tb, lb = b.prefill(tokens, 0)
+    finally:
+        dev.set_option("prefill.qkv_group", 1)
+    shape = (cfg["n_layers"], cfg["n_kv_heads"], cfg["max_pos"], cfg["head_dim"])
+    ka, va = read_cache(dev, a, shape)
+    kb, vb = read_cache(dev, b, shape)
+    assert rel(ka[0, :, :n], kb[0, :, :n].astype(np.float64)) <= 1e-5
+    assert rel(va[0, :, :n], vb[0, :, :n].astype(np.float64)) <= 1e-5
+    assert not ka[:, :, n:].any() and not va[:, :, n:].any()
+    assert rel(la, lb.astype(np.float64)) <= 1e-4
+    assert ta == tb
+
+
 def test_full_width_prompt_pass_of_256_rows(dev):
     # One layer at the Llama-3-8B width (d_model 4096, 32 query / 8 kv heads x 128, d_ffn 14336, Q4_K with a Q6_K
     # down projection), 256 tokens: the shapes and kernels of the benchmark's prompt pass (fp16 big tiles, K split
