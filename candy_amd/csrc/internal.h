@@ -65,7 +65,7 @@ struct Options {
     int mmv_variant = 0;         // comparison runs: 1 = one 16-row strip per wavefront, 2 = two
     int pair_rows = 0;           // fused gate/up: row pairs per workgroup, 32 / 16 / 8 (0: the most even split)
     int rms_rows = 0;            // fused RMSNorm prologue: rows per workgroup, 16 / 24 (0: the most even split)
-    int prefill_qkv_group = 1;       // prompt pass: q / k / v projections on one grid where they share the fp16 tiles
+    int prefill_qkv_group = 1;       // prompt pass: q / k / v (and gate / up) on one grid each where they run on the fp16 tiles
     int prefill_attention_valu = 0;  // prompt attention for head_dim 128 on the vector ALU instead of the matrix cores
     int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
     int fused_wide = 1;          // decode step: one-workgroup-per-CU kernels for the big Q4_K shapes (0: the narrower ones)

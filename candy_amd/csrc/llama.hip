@@ -484,8 +484,14 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
         if ((rc = add_linear(L.wo))) return rc;  // h += Wo . att
         xh = (xh_for(L.gate) || xh_for(L.up)) ? P.xh : nullptr;
         if ((rc = launch_rms_norm_quant(dev, P.h, L.ffn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs, xh))) return rc;
-        if ((rc = launch_contract(dev, L.gate, P.xq, P.xs, n, P.gate, xh_for(L.gate)))) return rc;
-        if ((rc = launch_contract(dev, L.up, P.xq, P.xs, n, P.up, xh_for(L.up)))) return rc;
+        const candy_hip_qtensor *gu_w[2] = {L.gate, L.up};
+        float *gu_y[2] = {P.gate, P.up};
+        if (xh && mmq_f16_group_covers(gu_w, 2, n)) {  // the second projection's tiles fill the first one's last round
+            if ((rc = launch_mmq_f16_group(dev, gu_w, gu_y, 2, xh, n))) return rc;
+        } else {
+            if ((rc = launch_contract(dev, L.gate, P.xq, P.xs, n, P.gate, xh_for(L.gate)))) return rc;
+            if ((rc = launch_contract(dev, L.up, P.xq, P.xs, n, P.up, xh_for(L.up)))) return rc;
+        }
         if ((rc = launch_silu_mul_quant(dev, P.gate, P.up, (int64_t)n * c.d_ffn, nullptr, P.xq, P.xs, xh_for(L.down))))
             return rc;
         if ((rc = add_linear(L.down))) return rc;  // h += Wdown . act

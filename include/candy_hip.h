@@ -102,8 +102,8 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   "fused.rms_rows"             0        fused RMSNorm prologue: rows per workgroup 16 / 24 (0: most even split)
  *   "fused.wide"                 1        decode step: kernels that deal the rows of the big Q4_K shapes evenly over the CUs
  *   "fused.wide_waves"           8        wavefronts per workgroup of those kernels: 8 (two workgroups per CU) or 16 (one)
- *   "prefill.qkv_group"          1        prompt pass: the q / k / v projections as one grid where all three run on the
- *                                         fp16 tiles (0: one launch each)
+ *   "prefill.qkv_group"          1        prompt pass: projections that share their input (q / k / v; gate / up) as one
+ *                                         grid each where all of them run on the fp16 tiles (0: one launch each)
  *   "prefill.attention_valu"     0        prompt attention for head_dim 128 on the vector ALU */
 int candy_hip_set_option(candy_hip_device *dev, const char *key, int64_t value);
 int candy_hip_get_option(const candy_hip_device *dev, const char *key, int64_t *value);
