@@ -423,21 +423,24 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
 }
 
 // ------------------------------------------------------------------ the same tile with the work split by role
-// 128 weight rows x 256 activation rows, 8 wavefronts: wavefronts 0-3 (one per SIMD) are producers, 4-7 consumers.
+// 128 weight rows x BM (256 or 128) activation rows, 8 wavefronts: wavefronts 0-3 (one per SIMD) are producers, 4-7
+// consumers.
 // Producers request weights and activations, dequantize and fill the LDS buffers of step s + 1 while the
-// consumers read the operands of step s (each a 64 x 128 sub-tile: 24 KB of LDS reads per step instead of the
-// 4 x 8 KB that two 64 x 64 wavefronts of a SIMD read for the same matrix work) and issue its matrix
+// consumers read the operands of step s (each a 64 x BM / 2 sub-tile; at BM = 256 that is 24 KB of LDS reads per step
+// instead of the 4 x 8 KB that two 64 x 64 wavefronts of a SIMD read for the same matrix work) and issue its matrix
 // instructions; one workgroup barrier per step hands a buffer over.  In the single-role kernel every wavefront
 // walks the same phases in step (operand reads, matrix instructions, dequantization, LDS writes), so the LDS port,
 // the matrix cores and the vector ALU take turns; here a SIMD's two wavefronts are in different phases by
 // construction.  The two roles are separate loops with the same number of barriers, so that their registers
 // (accumulators and operand fragments here, raw blocks and activation chunks there) share one allocation.
-template <class F, bool RES>
+template <class F, int BM, bool RES>
 __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _Float16 *__restrict__ xh, int M, int K,
                                                     int n_tiles, int m_tiles, int sb_per, size_t split_stride) {
-    constexpr int BN = 128, BM = 256, PT = 256;
+    constexpr int BN = 128, PT = 256;
     constexpr int ATK = BN * 4 / PT;  // dequantization tasks per producer thread per step
     constexpr int BCH = BM * 8 / PT;  // 16-byte activation chunks per producer thread per step
+    constexpr int TM = BM / 32;       // 16-row activation fragments of a consumer's sub-tile
+    static_assert(BM == 256 || BM == 128, "activation rows per tile");
     extern __shared__ __align__(16) uint8_t smem_raw[];
     _Float16 *sA = (_Float16 *)smem_raw;               // [2][BN / 16][2] fragments
     _Float16 *sB = sA + 2 * BN * BIG_BK;               // [2][BM / 16][2] fragments
@@ -478,7 +481,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
         auto gload_b = [&](int ks, int slot) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < BCH; ++i) {
-                const int r = 16 * (wave * 4 + (i >> 1)) + 2 * (i & 1) + b_row;
+                const int r = 16 * (wave * (BCH / 2) + (i >> 1)) + 2 * (i & 1) + b_row;
                 xr[slot][i] = *(const u32x4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BIG_BK + b_kc * 8);
             }
         };
@@ -495,7 +498,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             }
 #pragma unroll
             for (int i = 0; i < BCH; ++i) {
-                const int r = 16 * (wave * 4 + (i >> 1)) + 2 * (i & 1) + b_row;
+                const int r = 16 * (wave * (BCH / 2) + (i >> 1)) + 2 * (i & 1) + b_row;
                 *(u32x4 *)&b[frag_off(r, b_kc * 8)] = xr[bslot][i];
             }
         };
@@ -526,28 +529,28 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
         return;
     }
 
-    // ---------------- consumers: 2 x 2 wavefronts of 64 weight rows x 128 activation rows
+    // ---------------- consumers: 2 x 2 wavefronts of 64 weight rows x BM / 2 activation rows
     const int cw = wave - 4, cn = cw & 1, cm = cw >> 1;
-    float4v acc[4][8];
+    float4v acc[4][TM];
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int b = 0; b < 8; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < TM; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
     auto compute = [&](int buf) __attribute__((always_inline)) {
         const _Float16 *a = sA + buf * BN * BIG_BK + cn * 64 * BIG_BK + frag_lane_off(lane);
-        const _Float16 *b = sB + buf * BM * BIG_BK + cm * 128 * BIG_BK + frag_lane_off(lane);
-        half8 af[2][4], bf[2][8];
+        const _Float16 *b = sB + buf * BM * BIG_BK + cm * (BM / 2) * BIG_BK + frag_lane_off(lane);
+        half8 af[2][4], bf[2][TM];
         auto fetch = [&](int kk) __attribute__((always_inline)) {
 #pragma unroll
             for (int tn = 0; tn < 4; ++tn) af[kk][tn] = *(const half8 *)&a[(tn * 2 + kk) * 512];
 #pragma unroll
-            for (int tm = 0; tm < 8; ++tm) bf[kk][tm] = *(const half8 *)&b[(tm * 2 + kk) * 512];
+            for (int tm = 0; tm < TM; ++tm) bf[kk][tm] = *(const half8 *)&b[(tm * 2 + kk) * 512];
         };
         auto mma = [&](int kk) __attribute__((always_inline)) {
 #pragma unroll
             for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
-                for (int tm = 0; tm < 8; ++tm)
+                for (int tm = 0; tm < TM; ++tm)
                     acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[kk][tn], bf[kk][tm], acc[tn][tm], 0, 0, 0);
         };
         // the second half's operands are read while the first half's matrix instructions run
@@ -575,8 +578,8 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
 #pragma unroll
     for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
-        for (int tm = 0; tm < 8; ++tm) {
-            const int m = m0 + cm * 128 + tm * 16 + (lane & 15);
+        for (int tm = 0; tm < TM; ++tm) {
+            const int m = m0 + cm * (BM / 2) + tm * 16 + (lane & 15);
             const int n = n0 + cn * 64 + tn * 16 + 4 * (lane >> 4);
             if (m >= M) continue;
             float *dst = out + (size_t)m * N + n;
@@ -638,7 +641,7 @@ struct F16Job {
 
 template <class F, int BN, int BM, int WN, int WM, bool PC = false>
 static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, const _Float16 *xh, int64_t m) {
-    static_assert(!PC || (BN == 128 && BM == 256 && WN * WM == 8), "the role-split kernel is the 128 x 256 tile");
+    static_assert(!PC || (BN == 128 && (BM == 256 || BM == 128) && WN * WM == 8), "the role-split kernel's tiles");
     const int K = (int)jobs[0].w->cols;
     F16Group grp{};
     grp.count = count;
@@ -684,7 +687,7 @@ static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, cons
     constexpr size_t smem = (size_t)2 * (BN + BM) * BIG_BK * sizeof(_Float16);
     const bool epi_res = any_res && n_split == 1;
     void (*kern)(const F16Group, const _Float16 *, int, int, int, int, int, size_t);
-    if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, true> : k_mmq_f16_pc<F, false>;
+    if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, BM, true> : k_mmq_f16_pc<F, BM, false>;
     else kern = epi_res ? k_mmq_f16<F, BN, BM, WN, WM, true> : k_mmq_f16<F, BN, BM, WN, WM, false>;
     CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream, grp, xh, (int)m, K,
@@ -739,16 +742,19 @@ static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, con
     if (fmt == CANDY_HIP_Q8_0) CANDY_BIG_256(BigQ8_0);
     if (fmt == CANDY_HIP_Q4_0) CANDY_BIG_256(BigQ4_0<false>);
     if (fmt == CANDY_HIP_Q4_0_GGML) CANDY_BIG_256(BigQ4_0<true>);
-    // Q4_K. Up to 128 activation rows: 128 x 128 tiles (two workgroups per CU), K split over workgroups to fill the chip
+    // Q4_K. Up to 128 activation rows: 128 x 128 tiles, K split over workgroups to fill the chip
     const int shape = dev->opt.f16_shape;  // comparison runs
-    if (shape == 2 || m <= 128) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m);
+    auto small_tiles = [&]() {
+        return single ? launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m)
+                      : launch_big<BigQ4K, 128, 128, 2, 4, true>(dev, jobs, count, xh, m);
+    };
+    if (shape == 2 || m <= 128) return small_tiles();
     // up to 256 rows where the 128 x 128 tiles fill the chip and the 128 x 256 tiles would have to split K
     // (14336 x 4096 at 256 rows: 70.7 us against 80.3)
     int64_t n128 = 0;
     for (int s = 0; s < count; ++s) n128 += (jobs[s].w->rows + 127) / 128;
     const int64_t fill = (3 * (int64_t)dev->num_cus) / 4;
-    if (shape != 3 && m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill)
-        return launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m);
+    if (m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill) return small_tiles();
     CANDY_BIG_256(BigQ4K);
 #undef CANDY_BIG_256
 }

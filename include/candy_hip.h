@@ -90,7 +90,7 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   "mmq.i8_min_m"               0        5..15 rows: int8 tiles from this batch on (0: by measured cost model)
  *   "mmq.fp16_only"              0        every tile contraction on the single-buffered fp16 tiles
  *   "mmq.i8_grid_split"          1        int8 tiles split K over workgroups on small grids
- *   "mmq.f16_shape"              0        comparison runs: Q4_K fp16 tiles of 128 x 128 at every batch (2); 128 x 256 tiles
+ *   "mmq.f16_shape"              0        comparison runs: Q4_K fp16 tiles of 128 x 128 at every batch (2); fp16 tiles
  *                                         computed by the kernel whose wavefronts each dequantize and multiply (3)
  *                                         instead of the one that splits the two roles over wavefronts (0: by shape)
  *   "mmq.f16_split"              0        comparison runs: K split of the fp16 tile kernels over this many workgroups per

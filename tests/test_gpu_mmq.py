@@ -120,10 +120,12 @@ def test_big_fp16_tiles(dev, fmt, m, rows, cols):
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML])
 @pytest.mark.parametrize("m,rows,cols", [(256, 128, 256), (300, 129, 1024), (513, 1030, 768), (700, 130, 4352),
-                                         (260, 2100, 512)])
+                                         (260, 2100, 512), (96, 300, 2304), (128, 1030, 768), (200, 25000, 256)])
 def test_role_split_tiles_equal_the_single_role_tiles(dev, fmt, m, rows, cols):
-    # 128 x 256 tiles: producer / consumer wavefronts (the default) and the kernel whose wavefronts do both run
-    # the same multiply-adds in the same order on the same fp16 operands, with and without a K split
+    # 128 x 256 tiles (and Q4_K's 128 x 128 ones: up to 128 rows, and 129-256 rows on many weight rows): producer /
+    # consumer wavefronts (the default) and the kernel whose wavefronts do both run the same multiply-adds in the
+    # same order on the same fp16 operands, with and without a K split.  Below the fp16 threshold of a format both
+    # runs take the same int8 tiles.
     w = synth.random_weight(fmt, rows, cols, seed=rows + 3 * m)
     x = synth.random_activations(m, cols, seed=cols + m)
     q = dev.qtensor(fmt, rows, cols, w)
