@@ -30,6 +30,17 @@ def test_binding_covers_exactly_the_header():
     assert sorted(hip.SIGNATURES) == _declared_symbols()
 
 
+def test_header_documents_exactly_the_options_the_library_accepts():
+    # candy_hip_set_option's table in the header (one "key" default meaning line per switch) against the table the
+    # runtime looks keys up in: an undocumented switch or a documented one that does not exist fails here
+    header = open(os.path.join(ROOT, "include", "candy_hip.h")).read()
+    documented = set(re.findall(r'^ \*\s+"([a-z0-9_.]+)"\s+-?\d+\s', header, flags=re.M))
+    runtime = open(os.path.join(ROOT, "candy_amd", "csrc", "runtime.hip")).read()
+    accepted = set(re.findall(r'\{"([a-z0-9_.]+)", &candy::Options::', runtime))
+    assert len(accepted) >= 15
+    assert documented == accepted, (sorted(documented - accepted), sorted(accepted - documented))
+
+
 def test_format_tables():
     L = hip.lib()
     assert [L.candy_hip_block_bytes(f) for f in (hip.Q4_0, hip.Q8_0, hip.Q4_K, hip.Q6_K, hip.Q4_0_GGML)] == [18, 34, 144, 210, 18]
