@@ -65,7 +65,14 @@ struct BigQ4K {
     // A nibble n is placed in the mantissa of the half 1024 (bits 0x6400 | n = 1024 + n, exact), two nibbles per
     // instruction, and each value is one mixed-precision multiply-add (f16 operand, f32 scale and offset, f32
     // arithmetic, rounded once to fp16): (1024 + n) * (d*sc) + (-(dmin*m) - 1024 * (d*sc)) = (d*sc)*n - dmin*m.
+    // High nibbles stay where they are, four bits up (0x6400 | 16 n = 1024 + 16 n, exact as well), and take the
+    // scale d*sc / 16 and the offset -(dmin*m) - 64 * (d*sc): one shift per word instead of three.
     // The offset's own f32 rounding (2^-24 of 1024 d*sc) is a thirtieth of the fp16 rounding that follows.
+    __device__ static __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
+        uint32_t r;  // (x & mask) | bits in one instruction; the mask rides on the constant bus, the bits in a register
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(bits));
+        return r;
+    }
     __device__ static __forceinline__ void dequant(const Raw &r, int g, int c, half8 &o0, half8 &o1, int &k0, int &k1) {
         uint32_t sc2, m2;
         q4k_scale_min_pair(r.hdr.y, r.hdr.z, r.hdr.w, g, sc2, m2);
@@ -73,22 +80,23 @@ struct BigQ4K {
         const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
         const float d_lo = d * (float)(sc2 & 0xFF), d_hi = d * (float)((sc2 >> 8) & 0xFF);
         const float c_lo = fmaf(-1024.0f, d_lo, -(dmin * (float)(m2 & 0xFF)));
-        const float c_hi = fmaf(-1024.0f, d_hi, -(dmin * (float)((m2 >> 8) & 0xFF)));
+        const float c_hi = fmaf(-64.0f, d_hi, -(dmin * (float)((m2 >> 8) & 0xFF)));
+        const float d_hi16 = d_hi * 0.0625f;
         const u32x2 q = r.q[g];
+        const uint32_t MAGIC = 0x64006400u, LO = 0x000F000Fu, HI = 0x00F000F0u;
 #pragma unroll
         for (int wi = 0; wi < 2; ++wi) {
-            const uint32_t w = wi ? q.y : q.x;
-            const uint32_t MAGIC = 0x64006400u, M = 0x000F000Fu;
-            const half2v l02 = bits_h2((w & M) | MAGIC), l13 = bits_h2(((w >> 8) & M) | MAGIC);
-            const half2v h02 = bits_h2(((w >> 4) & M) | MAGIC), h13 = bits_h2(((w >> 12) & M) | MAGIC);
+            const uint32_t w = wi ? q.y : q.x, w8 = w >> 8;
+            const half2v l02 = bits_h2(and_or(w, LO, MAGIC)), l13 = bits_h2(and_or(w8, LO, MAGIC));
+            const half2v h02 = bits_h2(and_or(w, HI, MAGIC)), h13 = bits_h2(and_or(w8, HI, MAGIC));
             o0[4 * wi + 0] = (_Float16)fmaf((float)l02[0], d_lo, c_lo);
             o0[4 * wi + 1] = (_Float16)fmaf((float)l13[0], d_lo, c_lo);
             o0[4 * wi + 2] = (_Float16)fmaf((float)l02[1], d_lo, c_lo);
             o0[4 * wi + 3] = (_Float16)fmaf((float)l13[1], d_lo, c_lo);
-            o1[4 * wi + 0] = (_Float16)fmaf((float)h02[0], d_hi, c_hi);
-            o1[4 * wi + 1] = (_Float16)fmaf((float)h13[0], d_hi, c_hi);
-            o1[4 * wi + 2] = (_Float16)fmaf((float)h02[1], d_hi, c_hi);
-            o1[4 * wi + 3] = (_Float16)fmaf((float)h13[1], d_hi, c_hi);
+            o1[4 * wi + 0] = (_Float16)fmaf((float)h02[0], d_hi16, c_hi);
+            o1[4 * wi + 1] = (_Float16)fmaf((float)h13[0], d_hi16, c_hi);
+            o1[4 * wi + 2] = (_Float16)fmaf((float)h02[1], d_hi16, c_hi);
+            o1[4 * wi + 3] = (_Float16)fmaf((float)h13[1], d_hi16, c_hi);
         }
         k0 = c * 8;
         k1 = 32 + c * 8;
