@@ -188,6 +188,16 @@ __device__ __forceinline__ half4v q8_lane4_to_half(uint32_t packed, __half d_hal
     return r;
 }
 
+// Where those 4 values go.  The fp16 image of an activation matrix [rows][K] lies in memory as the B operands of
+// 16x16x32 matrix instructions: fragments of 16 rows x 32 values (1 KB), [row block][32-value block of K], 64
+// bytes per row inside a fragment.  The 64 lanes of a wavefront (lane l: row l & 15, values 8 (l >> 4) .. + 7) load
+// a fragment with one 128-bit load each, 1 KB of consecutive memory, straight into the operand registers; a
+// quantizer writes a row's 32-value block as 64 consecutive bytes.  Index in units of 4 halves of values
+// 4 c4 .. 4 c4 + 3 of `row`; rows are padded to a multiple of 16 by the caller's allocation, K is a multiple of 32.
+__host__ __device__ __forceinline__ int64_t xh_index4(int64_t row, int64_t c4, int64_t K) {
+    return ((row >> 4) * (K >> 5) + (c4 >> 3)) * 128 + (row & 15) * 8 + (c4 & 7);
+}
+
 // Same quantization with one value per lane: the 32 lanes of a block are consecutive lanes
 // (lane % 32 == position in the block), all active.
 __device__ __forceinline__ int quantize_q8_lane1(float v, __half &d_half, int &bsum) {

@@ -173,8 +173,8 @@ int launch_matvec_multi(candy_hip_device *dev, const candy_hip_qtensor *const *w
 int64_t mmq_m_pad(int64_t m);
 // Whether launch_mmq / launch_contract add `res` in the contraction's own epilogue (then res may alias y).
 bool mmq_fuses_residual(const candy_hip_qtensor *w, int64_t m);
-// xh_ready (optional): the activations already expanded to fp16 [>= mmq_m_pad(m) rows][cols] (rows past m
-// may hold anything); res (optional, may alias y): y = res + x . W^T.
+// xh_ready (optional): the activations already expanded to fp16, >= mmq_m_pad(m) rows of `cols` values in the
+// fragment order of xh_index4 (rows past m may hold anything); res (optional, may alias y): y = res + x . W^T.
 // f16_min_m: batch from which the fp16 big tiles may answer (0: the decoder's threshold, opt.f16_big_min_m)
 int launch_mmq(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                const Q8Scale *scales, int64_t m, float *y, void *half_ws, const _Float16 *xh_ready = nullptr,
@@ -188,7 +188,8 @@ int launch_mmv(candy_hip_device *dev, const candy_hip_qtensor *w, const float *x
                float *y, void *ws);
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,
                   const Q8Scale *scales, int64_t m, float *y);
-// mmq_f16.hip: Q4_K with prompt-sized batches on big fp16 tiles. xh: fp16 activations [mmq_m_pad(m)][K].
+// mmq_f16.hip: prompt-sized batches on big fp16 tiles. xh: fp16 activations, mmq_m_pad(m) rows in the fragment order
+// of xh_index4.
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m = 0);
 int launch_mmq_f16_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _Float16 *xh, int64_t m, float *y,
                        const float *res = nullptr);
@@ -199,8 +200,8 @@ int launch_mmq_f16_group(candy_hip_device *dev, const candy_hip_qtensor *const *
 // ops.hip: fused decode-step stages (all enqueue on dev->stream, no allocation, no sync).
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
                           int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales, _Float16 *xh = nullptr);
-int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *act_out,
-                          int8_t *qs, Q8Scale *scales, _Float16 *xh = nullptr);
+int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t rows, int64_t cols,
+                          float *act_out, int8_t *qs, Q8Scale *scales, _Float16 *xh = nullptr);
 // fused.hip: batch-1 contraction of one activation row with up to three weights, with optional
 // RMSNorm+quantize prologue (x != nullptr, else planar Q8_0 in xq/xs), residuals, or the
 // gate/up SiLU*Mul+quantize epilogue (pair). Returns CANDY_HIP_ERR_UNSUPPORTED when the shape

@@ -351,7 +351,7 @@ static int llama_enqueue_step(candy_hip_llama *m) {
                 const candy_hip_qtensor *ws[2] = {L.gate, L.up};
                 float *ys[2] = {m->gate_o, m->up_o};
                 if ((rc = norm_linear(m, L.ffn_norm, ws, ys, 2))) return rc;
-                rc = launch_silu_mul_quant(dev, m->gate_o, m->up_o, c.d_ffn, nullptr, m->xq, m->xs);
+                rc = launch_silu_mul_quant(dev, m->gate_o, m->up_o, 1, c.d_ffn, nullptr, m->xq, m->xs);
             }
             if (rc) return rc;
         }
@@ -492,7 +492,7 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
             if ((rc = launch_contract(dev, L.gate, P.xq, P.xs, n, P.gate, xh_for(L.gate)))) return rc;
             if ((rc = launch_contract(dev, L.up, P.xq, P.xs, n, P.up, xh_for(L.up)))) return rc;
         }
-        if ((rc = launch_silu_mul_quant(dev, P.gate, P.up, (int64_t)n * c.d_ffn, nullptr, P.xq, P.xs, xh_for(L.down))))
+        if ((rc = launch_silu_mul_quant(dev, P.gate, P.up, n, c.d_ffn, nullptr, P.xq, P.xs, xh_for(L.down))))
             return rc;
         if ((rc = add_linear(L.down))) return rc;  // h += Wdown . act
     }

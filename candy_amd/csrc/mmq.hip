@@ -178,7 +178,9 @@ struct MmqMore {
 };
 
 // ------------------------------------------------------------------ activation expansion
-// planar Q8_0 -> fp16 [m_pad, K]; rows m..m_pad-1 are zero so the tile kernel needs no row guard.
+// planar Q8_0 -> fp16 [m_pad, K]; rows m..m_pad-1 are zero so the tile kernel needs no row guard.  FRAG: in the
+// fragment order of xh_index4 (what the big fp16 tiles read) instead of row by row (k_mmq below).
+template <bool FRAG>
 __global__ __launch_bounds__(256) void k_q8_to_half(const int8_t *__restrict__ qs, const Q8Scale *__restrict__ sc,
                                                     int64_t m, int64_t m_pad, int64_t K, half8 *__restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one 8-value run
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(256) void k_q8_to_half(const int8_t *__restrict__ q
         for (int l = 0; l < 8; ++l) v[l] = d * (float)(int8_t)(((l < 4 ? q.x : q.y) >> (8 * (l & 3))) & 0xFF);
         h = to_half8(v);
     }
-    out[i] = h;
+    out[FRAG ? xh_index4(row, 2 * c, K) >> 1 : i] = h;
 }
 
 // ------------------------------------------------------------------ tile kernel
@@ -357,8 +359,8 @@ static int mmq_dispatch(candy_hip_device *dev, const candy_hip_qtensor *w, const
     CANDY_REQUIRE(half_ws, "internal: no workspace for the fp16 activations");
     const int64_t m_pad = mmq_m_pad(m);
     const int64_t runs = m_pad * (K >> 3);
-    hipLaunchKernelGGL(k_q8_to_half, dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, dev->stream, qs, scales, m,
-                       m_pad, K, (half8 *)half_ws);
+    hipLaunchKernelGGL(big ? k_q8_to_half<true> : k_q8_to_half<false>, dim3((unsigned)((runs + 255) / 256)), dim3(256), 0,
+                       dev->stream, qs, scales, m, m_pad, K, (half8 *)half_ws);
     CANDY_LAUNCH_CHECK();
     const _Float16 *xh = (const _Float16 *)half_ws;
     if (big) {

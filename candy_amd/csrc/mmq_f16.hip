@@ -288,11 +288,11 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wn = wave % WN, wm = wave / WN;
-    // Staging lane maps: neighbouring lanes take neighbouring pieces of a row (global loads of whole 64- and 128-byte
+    // Weight staging lane map: neighbouring lanes take neighbouring quarters of a row (global loads of whole 64-byte
     // runs); the 32 lanes of a half-wavefront take rows {x, x+4, x+8, x+12}, which the row ^ piece term of the
-    // layout spreads over all 16 bank windows.
+    // layout spreads over all 16 bank windows.  The activations lie in memory fragment by fragment (xh_index4): the
+    // tile's share of a step is 2 KB per 16 rows, copied piece by piece into the LDS order.
     const int a_c = lane & 3, a_r = 4 * ((lane >> 2) & 3) + (lane >> 4);
-    const int b_kc = lane & 7, b_r = 4 * ((lane >> 3) & 3) + (lane >> 5);  // + 2 (i & 1)
 
     // tile numbering: the hardware deals workgroups round-robin to the 8 XCDs; give each XCD a
     // contiguous run of weight tiles inside one activation tile
@@ -310,9 +310,10 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
     const int n_sb = min(K >> 8, sb0 + sb_per) - sb0;  // >= 1 by construction of the grid
     const int steps = n_sb * 4;
     const uint8_t *__restrict__ W = seg.W + (size_t)sb0 * F::BLOCK;
-    xh += (size_t)sb0 * 256;
+    xh += (size_t)sb0 * 8 * 512;  // 8 fragments of 32 values further along K, in every row block
     float *out = seg.out + (size_t)split * split_stride;
     const float *res = seg.res;
+    const _Float16 *xtile = xh + (size_t)(m0 >> 4) * (K >> 5) * 512;
 
     typename F::Raw raw[2][ATK];
     u32x4 xr[2][BCH];
@@ -326,8 +327,11 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
     auto gload_b = [&](int ks, int slot) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < BCH; ++i) {
-            const int r = (wave + (T / 64) * (i >> 1)) * 16 + 2 * (i & 1) + b_r;
-            xr[slot][i] = *(const u32x4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BIG_BK + b_kc * 8);
+            // LDS piece q of the tile: 16-row block q >> 7, half of the step (q >> 6) & 1, piece p = (q >> 4) & 3 of row
+            // (q & 15) ^ p; in memory a fragment is 16 rows of 64 bytes
+            const int q = tid + i * T, pc = (q >> 4) & 3, row = (q & 15) ^ pc;
+            xr[slot][i] = *(const u32x4 *)(xtile + ((size_t)(q >> 7) * (K >> 5) + (size_t)ks * 2 + ((q >> 6) & 1)) * 512 +
+                                           row * 32 + pc * 8);
         }
     };
     auto stage = [&](int g, int aslot, int bslot, int buf) __attribute__((always_inline)) {
@@ -343,10 +347,7 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
             *(half8 *)&a[frag_off(row, k1)] = o1;
         }
 #pragma unroll
-        for (int i = 0; i < BCH; ++i) {
-            const int r = (wave + (T / 64) * (i >> 1)) * 16 + 2 * (i & 1) + b_r;
-            *(u32x4 *)&b[frag_off(r, b_kc * 8)] = xr[bslot][i];
-        }
+        for (int i = 0; i < BCH; ++i) *(u32x4 *)&b[(tid + i * T) * 8] = xr[bslot][i];
     };
 
     float4v acc[TN][TM];
@@ -433,25 +434,30 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
 // ------------------------------------------------------------------ the same tile with the work split by role
 // 128 weight rows x BM (256 or 128) activation rows, 8 wavefronts: wavefronts 0-3 (one per SIMD) are producers, 4-7
 // consumers.
-// Producers request weights and activations, dequantize and fill the LDS buffers of step s + 1 while the
-// consumers read the operands of step s (each a 64 x BM / 2 sub-tile; at BM = 256 that is 24 KB of LDS reads per step
-// instead of the 4 x 8 KB that two 64 x 64 wavefronts of a SIMD read for the same matrix work) and issue its matrix
-// instructions; one workgroup barrier per step hands a buffer over.  In the single-role kernel every wavefront
-// walks the same phases in step (operand reads, matrix instructions, dequantization, LDS writes), so the LDS port,
-// the matrix cores and the vector ALU take turns; here a SIMD's two wavefronts are in different phases by
-// construction.  The two roles are separate loops with the same number of barriers, so that their registers
-// (accumulators and operand fragments here, raw blocks and activation chunks there) share one allocation.
+// Producers request weights, dequantize them and fill the LDS weight buffer of step s + 1 (two buffers) while the
+// consumers contract step s; one workgroup barrier per step hands a buffer over.  The activations never touch LDS:
+// their fp16 image lies in memory fragment by fragment, 1 KB per B operand of a matrix instruction (xh_index4), so a
+// consumer loads each fragment it needs with one 128-bit load per lane, 1 KB of consecutive memory per wavefront,
+// straight into operand registers, one step ahead.  Each consumer owns all 128 weight rows and a quarter of the tile's
+// activation rows, so every activation fragment is loaded by exactly one wavefront of the workgroup.
+//   Why: with the activations staged through LDS by the producers (8 loads and 8 LDS writes per thread and step for
+//   BM = 256), disabling parts of the kernel showed the producers alone taking 72 of the kernel's 81 us at
+//   14336 x 4096 x 512 - 23 us of that the activation copy, 12 us the dequantization - against 55 us for the consumers
+//   alone: moving a step's 32 KB of activations into the CU costs 700 to 950 cycles whichever wavefronts do it, and
+//   LDS carried 144 KB per step (now 80 KB: 16 KB of weight tile written, 4 x 16 KB read).
+// A consumer walks a step in four phases (two halves of K x two halves of the weight rows) of 16 or 8 matrix
+// instructions, reading the next phase's four weight fragments from LDS while the current phase's instructions run.
+// The two roles are separate loops with the same number of barriers, so that their registers (accumulators and
+// operand fragments here, raw blocks there) share one allocation.
 template <class F, int BM, bool RES>
 __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _Float16 *__restrict__ xh, int M, int K,
                                                     int n_tiles, int m_tiles, int sb_per, size_t split_stride) {
     constexpr int BN = 128, PT = 256;
     constexpr int ATK = BN * 4 / PT;  // dequantization tasks per producer thread per step
-    constexpr int BCH = BM * 8 / PT;  // 16-byte activation chunks per producer thread per step
-    constexpr int TM = BM / 32;       // 16-row activation fragments of a consumer's sub-tile
+    constexpr int TM = BM / 64;       // 16-row activation fragments of a consumer's sub-tile (its rows: BM / 4)
     static_assert(BM == 256 || BM == 128, "activation rows per tile");
     extern __shared__ __align__(16) uint8_t smem_raw[];
     _Float16 *sA = (_Float16 *)smem_raw;               // [2][BN / 16][2] fragments
-    _Float16 *sB = sA + 2 * BN * BIG_BK;               // [2][BM / 16][2] fragments
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -470,32 +476,22 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
     const int n_sb = min(K >> 8, sb0 + sb_per) - sb0;  // >= 1 by construction of the grid
     const int steps = n_sb * 4;
     const uint8_t *__restrict__ W = seg.W + (size_t)sb0 * F::BLOCK;
-    xh += (size_t)sb0 * 256;
+    xh += (size_t)sb0 * 8 * 512;  // 8 fragments of 32 values further along K, in every row block
     float *out = seg.out + (size_t)split * split_stride;
     const float *res = seg.res;
 
     if (wave < 4) {
-        // ---------------- producers
+        // ---------------- producers: the weight tile of step ks + 1 while step ks is contracted
         typename F::Raw raw[2][ATK];
-        u32x4 xr[2][BCH];
-        // neighbouring lanes take neighbouring pieces of a row; a half-wavefront takes rows {x, x+4, x+8, x+12}
+        // neighbouring lanes take neighbouring quarters of a row; a half-wavefront takes rows {x, x+4, x+8, x+12}
         const int a_c = lane & 3, a_row = 16 * wave + 4 * ((lane >> 2) & 3) + (lane >> 4);   // + 64 i
-        const int b_kc = lane & 7, b_row = 4 * ((lane >> 3) & 3) + (lane >> 5);              // + 16 block + 2 half
         auto gload_a = [&](int sb, int slot) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < ATK; ++i)
                 F::load(W + (size_t)min(n0 + a_row + 64 * i, N - 1) * rb + (size_t)sb * F::BLOCK, a_c, raw[slot][i]);
         };
-        auto gload_b = [&](int ks, int slot) __attribute__((always_inline)) {
-#pragma unroll
-            for (int i = 0; i < BCH; ++i) {
-                const int r = 16 * (wave * (BCH / 2) + (i >> 1)) + 2 * (i & 1) + b_row;
-                xr[slot][i] = *(const u32x4 *)(xh + (size_t)(m0 + r) * K + (size_t)ks * BIG_BK + b_kc * 8);
-            }
-        };
-        auto stage = [&](int g, int aslot, int bslot, int buf) __attribute__((always_inline)) {
+        auto stage = [&](int g, int aslot, int buf) __attribute__((always_inline)) {
             _Float16 *a = sA + buf * BN * BIG_BK;
-            _Float16 *b = sB + buf * BM * BIG_BK;
 #pragma unroll
             for (int i = 0; i < ATK; ++i) {
                 half8 o0, o1;
@@ -504,18 +500,10 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
                 *(half8 *)&a[frag_off(a_row + 64 * i, k0)] = o0;
                 *(half8 *)&a[frag_off(a_row + 64 * i, k1)] = o1;
             }
-#pragma unroll
-            for (int i = 0; i < BCH; ++i) {
-                const int r = 16 * (wave * (BCH / 2) + (i >> 1)) + 2 * (i & 1) + b_row;
-                *(u32x4 *)&b[frag_off(r, b_kc * 8)] = xr[bslot][i];
-            }
         };
         gload_a(0, 0);
-        gload_b(0, 0);
-        gload_b(1, 1);
         gload_a(min(1, n_sb - 1), 1);
-        stage(0, 0, 0, 0);
-        gload_b(2, 0);
+        stage(0, 0, 0);
         __syncthreads();
         for (int sb2 = 0; sb2 < n_sb; sb2 += 2) {
 #pragma unroll
@@ -524,11 +512,9 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
                 if (sb >= n_sb) break;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int ks = sb * 4 + g;
-                    // while the consumers contract step ks from buffer g & 1: fill the other buffer with step ks + 1
-                    if (g < 3) stage(g + 1, half, (g + 1) & 1, (g + 1) & 1);
-                    else stage(0, half ^ 1, 0, 0);
-                    gload_b(min(ks + 3, steps - 1), (g + 1) & 1);
+                    // while the consumers contract step 4 sb + g from buffer g & 1: fill the other buffer with the next step
+                    if (g < 3) stage(g + 1, half, (g + 1) & 1);
+                    else stage(0, half ^ 1, 0);
                     if (g == 3) gload_a(min(sb + 2, n_sb - 1), half);
                     __syncthreads();
                 }
@@ -537,37 +523,50 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
         return;
     }
 
-    // ---------------- consumers: 2 x 2 wavefronts of 64 weight rows x BM / 2 activation rows
-    const int cw = wave - 4, cn = cw & 1, cm = cw >> 1;
-    float4v acc[4][TM];
+    // ---------------- consumers: wavefront cw owns 128 weight rows x activation rows [cw * BM / 4, + BM / 4)
+    const int cw = wave - 4;
+    float4v acc[8][TM];
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < 8; ++a)
 #pragma unroll
         for (int b = 0; b < TM; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
-    auto compute = [&](int buf) __attribute__((always_inline)) {
-        const _Float16 *a = sA + buf * BN * BIG_BK + cn * 64 * BIG_BK + frag_lane_off(lane);
-        const _Float16 *b = sB + buf * BM * BIG_BK + cm * (BM / 2) * BIG_BK + frag_lane_off(lane);
-        half8 af[2][4], bf[2][TM];
-        auto fetch = [&](int kk) __attribute__((always_inline)) {
+    // activation fragment (16-row block rbk of the tile, 32-value block kb of K): 1 KB at ((m0 / 16 + rbk) * (K / 32) + kb)
+    // * 1 KB; lane l takes row l & 15, values 8 (l >> 4) .. + 7: the wavefront's 64 loads cover the fragment once
+    const _Float16 *xfrag = xh + ((size_t)((m0 >> 4) + cw * TM) * (K >> 5)) * 512 + (lane & 15) * 32 + (lane >> 4) * 8;
+    half8 bf[2][2][TM];  // [step parity][half of the step][fragment]
+    auto load_b = [&](int ks, int slot) __attribute__((always_inline)) {
 #pragma unroll
-            for (int tn = 0; tn < 4; ++tn) af[kk][tn] = *(const half8 *)&a[(tn * 2 + kk) * 512];
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) bf[kk][tm] = *(const half8 *)&b[(tm * 2 + kk) * 512];
+            for (int tm = 0; tm < TM; ++tm)
+                bf[slot][kk][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ks * 2 + kk) * 512);
+    };
+    auto compute = [&](int abuf, int bslot) __attribute__((always_inline)) {
+        const _Float16 *a = sA + abuf * BN * BIG_BK + frag_lane_off(lane);
+        half8 af[2][4];
+        // phase p = 2 * kk + h: weight rows 64 h .. 64 h + 63, values 32 kk .. 32 kk + 31 of the step
+        auto fetch = [&](int p) __attribute__((always_inline)) {
+#pragma unroll
+            for (int tn = 0; tn < 4; ++tn) af[p & 1][tn] = *(const half8 *)&a[(((p & 1) * 4 + tn) * 2 + (p >> 1)) * 512];
         };
-        auto mma = [&](int kk) __attribute__((always_inline)) {
+        auto mma = [&](int p) __attribute__((always_inline)) {
 #pragma unroll
             for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
                 for (int tm = 0; tm < TM; ++tm)
-                    acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[kk][tn], bf[kk][tm], acc[tn][tm], 0, 0, 0);
+                    acc[(p & 1) * 4 + tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[p & 1][tn], bf[bslot][p >> 1][tm],
+                                                                                     acc[(p & 1) * 4 + tn][tm], 0, 0, 0);
         };
-        // the second half's operands are read while the first half's matrix instructions run
         fetch(0);
-        fetch(1);
-        __builtin_amdgcn_sched_barrier(0);
-        mma(0);
-        mma(1);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            if (p < 3) fetch(p + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(p);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
+    load_b(0, 0);
     __syncthreads();
     for (int sb2 = 0; sb2 < n_sb; sb2 += 2) {
 #pragma unroll
@@ -576,7 +575,9 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             if (sb >= n_sb) break;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                compute(g & 1);
+                const int ks = sb * 4 + g;
+                load_b(min(ks + 1, steps - 1), (g + 1) & 1);  // the next step's activations, in flight during this one
+                compute(g & 1, g & 1);
                 __syncthreads();
             }
         }
@@ -584,11 +585,11 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
 
     // C layout of a 16x16 tile: lane holds activation row (lane & 15) and weight rows 4*(lane>>4)..+3
 #pragma unroll
-    for (int tn = 0; tn < 4; ++tn)
+    for (int tn = 0; tn < 8; ++tn)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
-            const int m = m0 + cm * (BM / 2) + tm * 16 + (lane & 15);
-            const int n = n0 + cn * 64 + tn * 16 + 4 * (lane >> 4);
+            const int m = m0 + cw * (BM / 4) + tm * 16 + (lane & 15);
+            const int n = n0 + tn * 16 + 4 * (lane >> 4);
             if (m >= M) continue;
             float *dst = out + (size_t)m * N + n;
             const float *r = RES && res ? res + (size_t)m * N + n : nullptr;  // may alias dst: read before the store
@@ -692,7 +693,7 @@ static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, cons
             off += (size_t)m * (size_t)jobs[s].w->rows;
         }
     }
-    constexpr size_t smem = (size_t)2 * (BN + BM) * BIG_BK * sizeof(_Float16);
+    constexpr size_t smem = (size_t)2 * (BN + (PC ? 0 : BM)) * BIG_BK * sizeof(_Float16);  // role-split: weight tiles only
     const bool epi_res = any_res && n_split == 1;
     void (*kern)(const F16Group, const _Float16 *, int, int, int, int, int, size_t);
     if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, BM, true> : k_mmq_f16_pc<F, BM, false>;

@@ -237,7 +237,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict_
         const size_t i = (size_t)blockIdx.x * n4 + c;
         if (xn_out) ((float4 *)xn_out)[i] = v;
         qs[i] = packed;
-        if (xh) xh[i] = q8_lane4_to_half(packed, h);
+        if (xh) xh[xh_index4(blockIdx.x, c, cols)] = q8_lane4_to_half(packed, h);
         if ((c & 7) == 0) {
             Q8Scale sc;
             sc.d = __half2float(h);
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict_
 
 // silu(gate) * up, then Q8_0 quantization. n % 32 == 0.
 __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict__ gate, const float4 *__restrict__ up,
-                                                        int64_t n4, float4 *__restrict__ act_out,
+                                                        int64_t n4, int64_t row_n4, float4 *__restrict__ act_out,
                                                         uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
                                                         half4v *__restrict__ xh) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict
     if (!live) return;
     if (act_out) act_out[i] = v;
     qs[i] = packed;
-    if (xh) xh[i] = q8_lane4_to_half(packed, h);
+    if (xh) xh[xh_index4(i / row_n4, i % row_n4, 4 * row_n4)] = q8_lane4_to_half(packed, h);
     if ((i & 7) == 0) {
         Q8Scale sc;
         sc.d = __half2float(h);
@@ -284,12 +284,12 @@ int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *al
     return CANDY_HIP_OK;
 }
 
-int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t n, float *act_out,
-                          int8_t *qs, Q8Scale *scales, _Float16 *xh) {
-    CANDY_REQUIRE(n % 32 == 0 && n > 0, "silu_mul_quant needs n %% 32 == 0");
-    const int64_t n4 = n >> 2;
+int launch_silu_mul_quant(candy_hip_device *dev, const float *gate, const float *up, int64_t rows, int64_t cols,
+                          float *act_out, int8_t *qs, Q8Scale *scales, _Float16 *xh) {
+    CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0, "silu_mul_quant needs cols %% 32 == 0");
+    const int64_t n4 = rows * cols >> 2;
     hipLaunchKernelGGL(k_silu_mul_quant, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, dev->stream,
-                       (const float4 *)gate, (const float4 *)up, n4, (float4 *)act_out, (uint32_t *)qs, scales,
+                       (const float4 *)gate, (const float4 *)up, n4, cols >> 2, (float4 *)act_out, (uint32_t *)qs, scales,
                        (half4v *)xh);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;

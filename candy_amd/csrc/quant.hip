@@ -12,7 +12,7 @@ namespace candy {
 //   amax = max|x|, d = amax / 127 (IEEE f32 division), q = amax == 0 ? 0 : roundf(x / d),
 // the stored scale is fp16(d) while q uses the unrounded d.
 // One lane owns 4 consecutive values; the 8 lanes of a block reduce with cross-lane xor.
-__global__ __launch_bounds__(256) void k_quantize_q8_0(const float4 *__restrict__ x, int64_t n4,
+__global__ __launch_bounds__(256) void k_quantize_q8_0(const float4 *__restrict__ x, int64_t n4, int64_t row_n4,
                                                        uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
                                                        uint8_t *__restrict__ blocks, half4v *__restrict__ xh) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void k_quantize_q8_0(const float4 *__restrict_
     const int64_t b = i >> 3;
     const int part = (int)(i & 7);
     if (qs) qs[i] = packed;
-    if (xh) xh[i] = q8_lane4_to_half(packed, h);
+    if (xh) xh[xh_index4(i / row_n4, i % row_n4, 4 * row_n4)] = q8_lane4_to_half(packed, h);
     if (scales && part == 0) {
         Q8Scale sc;
         sc.d = __half2float(h);
@@ -69,7 +69,7 @@ int launch_quantize_q8(candy_hip_device *dev, const float *x, int64_t rows, int6
     if (n4 == 0) return CANDY_HIP_OK;
     const int64_t grid = (n4 + 255) / 256;
     CANDY_REQUIRE(grid <= 0x7FFFFFFF, "activation too large");
-    hipLaunchKernelGGL(k_quantize_q8_0, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const float4 *)x, n4,
+    hipLaunchKernelGGL(k_quantize_q8_0, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const float4 *)x, n4, cols / 4,
                        (uint32_t *)qs, scales, (uint8_t *)blocks, (half4v *)xh);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
