@@ -456,8 +456,13 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
     constexpr int ATK = BN * 4 / PT;  // dequantization tasks per producer thread per step
     constexpr int TM = BM / 64;       // 16-row activation fragments of a consumer's sub-tile (its rows: BM / 4)
     static_assert(BM == 256 || BM == 128, "activation rows per tile");
+    // BM = 256: the producers work two steps ahead into the third of three weight buffers, and a consumer reads the
+    // first weight fragments of step s + 1 during the last matrix instructions of step s (16 per phase cover the
+    // read).  BM = 128 (8 matrix instructions per phase) is faster one step ahead with two buffers: 33.8 against
+    // 35.2 us at 14336 x 4096 x 128.
+    constexpr int LEAD = BM == 256 ? 2 : 1, NB = LEAD + 1;
     extern __shared__ __align__(16) uint8_t smem_raw[];
-    _Float16 *sA = (_Float16 *)smem_raw;               // [2][BN / 16][2] fragments
+    _Float16 *sA = (_Float16 *)smem_raw;               // [NB][BN / 16][2] fragments
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -481,7 +486,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
     const float *res = seg.res;
 
     if (wave < 4) {
-        // ---------------- producers: the weight tile of step ks + 1 while step ks is contracted
+        // ---------------- producers: the weight tile of step t + LEAD (buffer (t + LEAD) % NB) while step t is contracted
         typename F::Raw raw[2][ATK];
         // neighbouring lanes take neighbouring quarters of a row; a half-wavefront takes rows {x, x+4, x+8, x+12}
         const int a_c = lane & 3, a_row = 16 * wave + 4 * ((lane >> 2) & 3) + (lane >> 4);   // + 64 i
@@ -504,20 +509,21 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
         gload_a(0, 0);
         gload_a(min(1, n_sb - 1), 1);
         stage(0, 0, 0);
+        if (LEAD == 2) stage(1, 0, 1);
         __syncthreads();
-        for (int sb2 = 0; sb2 < n_sb; sb2 += 2) {
+        // Iteration t = 8 j + u stages step t + LEAD (past the end: a clamped super-block, into a buffer nobody
+        // reads): super-blocks alternate between the two raw slots, so u fixes group and slot of the staged step.
+        int buf = LEAD % NB;
+        for (int t8 = 0; t8 < steps; t8 += 8) {
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int sb = sb2 + half;
-                if (sb >= n_sb) break;
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    // while the consumers contract step 4 sb + g from buffer g & 1: fill the other buffer with the next step
-                    if (g < 3) stage(g + 1, half, (g + 1) & 1);
-                    else stage(0, half ^ 1, 0);
-                    if (g == 3) gload_a(min(sb + 2, n_sb - 1), half);
-                    __syncthreads();
-                }
+            for (int u = 0; u < 8; ++u) {
+                const int t = t8 + u;
+                if ((u & 3) == 0 && t >= steps) break;  // steps is a multiple of 4
+                const int g = (u + LEAD) & 3, slot = ((u + LEAD) >> 2) & 1;
+                stage(g, slot, NB == 2 ? ((u + LEAD) & 1) : buf);  // two buffers: a constant of the unrolled body
+                buf = buf == NB - 1 ? 0 : buf + 1;
+                if (g == 3) gload_a(min(((t + LEAD) >> 2) + 2, n_sb - 1), slot);
+                __syncthreads();
             }
         }
         return;
@@ -541,33 +547,26 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             for (int tm = 0; tm < TM; ++tm)
                 bf[slot][kk][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ks * 2 + kk) * 512);
     };
-    auto compute = [&](int abuf, int bslot) __attribute__((always_inline)) {
+    half8 af[2][4];
+    // phase p = 2 * kk + h of a step: weight rows 64 h .. 64 h + 63, values 32 kk .. 32 kk + 31
+    auto fetch = [&](int abuf, int p) __attribute__((always_inline)) {
         const _Float16 *a = sA + abuf * BN * BIG_BK + frag_lane_off(lane);
-        half8 af[2][4];
-        // phase p = 2 * kk + h: weight rows 64 h .. 64 h + 63, values 32 kk .. 32 kk + 31 of the step
-        auto fetch = [&](int p) __attribute__((always_inline)) {
 #pragma unroll
-            for (int tn = 0; tn < 4; ++tn) af[p & 1][tn] = *(const half8 *)&a[(((p & 1) * 4 + tn) * 2 + (p >> 1)) * 512];
-        };
-        auto mma = [&](int p) __attribute__((always_inline)) {
+        for (int tn = 0; tn < 4; ++tn) af[p & 1][tn] = *(const half8 *)&a[(((p & 1) * 4 + tn) * 2 + (p >> 1)) * 512];
+    };
+    auto mma = [&](int bslot, int p) __attribute__((always_inline)) {
 #pragma unroll
-            for (int tn = 0; tn < 4; ++tn)
+        for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
-                for (int tm = 0; tm < TM; ++tm)
-                    acc[(p & 1) * 4 + tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[p & 1][tn], bf[bslot][p >> 1][tm],
-                                                                                     acc[(p & 1) * 4 + tn][tm], 0, 0, 0);
-        };
-        fetch(0);
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            if (p < 3) fetch(p + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(p);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+            for (int tm = 0; tm < TM; ++tm)
+                acc[(p & 1) * 4 + tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[p & 1][tn], bf[bslot][p >> 1][tm],
+                                                                                 acc[(p & 1) * 4 + tn][tm], 0, 0, 0);
     };
     load_b(0, 0);
-    __syncthreads();
+    __syncthreads();  // the weight tiles of the first LEAD steps are in LDS
+    constexpr bool AHEAD = LEAD == 2;
+    if (AHEAD) fetch(0, 0);
+    int abuf = 0;
     for (int sb2 = 0; sb2 < n_sb; sb2 += 2) {
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -576,8 +575,21 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int ks = sb * 4 + g;
+                const int anext = abuf == NB - 1 ? 0 : abuf + 1;
+                const int acur = NB == 2 ? (g & 1) : abuf;  // two buffers: a constant of the unrolled body
                 load_b(min(ks + 1, steps - 1), (g + 1) & 1);  // the next step's activations, in flight during this one
-                compute(g & 1, g & 1);
+                if (!AHEAD) fetch(acur, 0);
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    // the next phase's weight fragments - after the last phase: the next step's first, whose buffer
+                    // has been complete since the barrier before this step - are read while this phase multiplies
+                    if (p < 3) fetch(acur, p + 1);
+                    else if (AHEAD) fetch(anext, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mma(g & 1, p);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                abuf = anext;
                 __syncthreads();
             }
         }
@@ -693,7 +705,7 @@ static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, cons
             off += (size_t)m * (size_t)jobs[s].w->rows;
         }
     }
-    constexpr size_t smem = (size_t)2 * (BN + (PC ? 0 : BM)) * BIG_BK * sizeof(_Float16);  // role-split: weight tiles only
+    constexpr size_t smem = (size_t)(PC ? 3 * BN : 2 * (BN + BM)) * BIG_BK * sizeof(_Float16);  // role-split: weight tiles only
     const bool epi_res = any_res && n_split == 1;
     void (*kern)(const F16Group, const _Float16 *, int, int, int, int, int, size_t);
     if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, BM, true> : k_mmq_f16_pc<F, BM, false>;
