@@ -567,31 +567,26 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
     constexpr bool AHEAD = LEAD == 2;
     if (AHEAD) fetch(0, 0);
     int abuf = 0;
-    for (int sb2 = 0; sb2 < n_sb; sb2 += 2) {
+    for (int sb = 0; sb < n_sb; ++sb) {  // four steps per iteration: no exit inside the unrolled body
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int sb = sb2 + half;
-            if (sb >= n_sb) break;
+        for (int g = 0; g < 4; ++g) {
+            const int ks = sb * 4 + g;
+            const int anext = abuf == NB - 1 ? 0 : abuf + 1;
+            const int acur = NB == 2 ? (g & 1) : abuf;  // two buffers: a constant of the unrolled body
+            load_b(min(ks + 1, steps - 1), (g + 1) & 1);  // the next step's activations, in flight during this one
+            if (!AHEAD) fetch(acur, 0);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int ks = sb * 4 + g;
-                const int anext = abuf == NB - 1 ? 0 : abuf + 1;
-                const int acur = NB == 2 ? (g & 1) : abuf;  // two buffers: a constant of the unrolled body
-                load_b(min(ks + 1, steps - 1), (g + 1) & 1);  // the next step's activations, in flight during this one
-                if (!AHEAD) fetch(acur, 0);
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    // the next phase's weight fragments - after the last phase: the next step's first, whose buffer
-                    // has been complete since the barrier before this step - are read while this phase multiplies
-                    if (p < 3) fetch(acur, p + 1);
-                    else if (AHEAD) fetch(anext, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    mma(g & 1, p);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                abuf = anext;
-                __syncthreads();
+            for (int p = 0; p < 4; ++p) {
+                // the next phase's weight fragments - after the last phase: the next step's first, whose buffer has
+                // been complete since the barrier before this step - are read while this phase multiplies
+                if (p < 3) fetch(acur, p + 1);
+                else if (AHEAD) fetch(anext, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                mma(g & 1, p);
+                __builtin_amdgcn_sched_barrier(0);
             }
+            abuf = anext;
+            __syncthreads();
         }
     }
 
