@@ -334,6 +334,10 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the other shapes of the batch-1 sweep")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the batched-prefill (MFMA) leg")
+    ap.add_argument("--prefill-steps", type=int, default=1000, help="timed calls per batch size of the prefill leg")
+    ap.add_argument("--prefill-warmup-ms", type=float, default=150.0,
+                    help="untimed calls in front of them, as milliseconds of work (the matrix-core kernels run 10-20 %% "
+                         "slower until the chip has raised its clocks); a counter run wants few dispatches: 0")
     ap.add_argument("--no-llama3", action="store_true", help="skip the Llama-3-8B-shaped prefill + decode leg")
     ap.add_argument("--decode-steps", type=int, default=32)
     ap.add_argument("--eager", action="store_true",
@@ -511,7 +515,8 @@ def main():
         big_min = dev.get_option("mmq.f16_api_min_m")
         for m in (16, 128, 512):
             # warm-up of about 150 ms: the matrix-core kernels run 10 % slower until the chip has raised its clocks
-            ms, _ = time_matvec(dev, synth.Q4_K, r, k, 1000, {16: 2000, 128: 4000, 512: 2000}[m], quantize_each=True, seed=m, m=m)
+            warm = max(5, int({16: 2000, 128: 4000, 512: 2000}[m] * args.prefill_warmup_ms / 150.0))
+            ms, _ = time_matvec(dev, synth.Q4_K, r, k, args.prefill_steps, warm, quantize_each=True, seed=m, m=m)
             flops = 2.0 * m * r * k
             byts = algorithmic_bytes(synth.Q4_K, r, k, m)
             int8 = m < big_min
