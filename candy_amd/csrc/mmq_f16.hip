@@ -771,6 +771,11 @@ static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, con
     for (int s = 0; s < count; ++s) n128 += (jobs[s].w->rows + 127) / 128;
     const int64_t fill = (3 * (int64_t)dev->num_cus) / 4;
     if (m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill) return small_tiles();
+    // short K (at most 16 super-blocks) on a grid that 128 x 256 tiles would have to split: 128 x 128 tiles halve the
+    // split as long as they still fit one round (4096 x 4096 at 512 rows 35.5 against 36.8 us, at 1024 rows 50.9 against
+    // 54.2; 6144 x 4096 at 512 rows 44.8 against 47.1; with K = 14336 the split is cheap and the wider tile wins)
+    if (shape == 0 && jobs[0].w->cols <= 4096 && n128 * ((m + 255) / 256) < fill && n128 * ((m + 127) / 128) <= dev->num_cus)
+        return small_tiles();
     CANDY_BIG_256(BigQ4K);
 #undef CANDY_BIG_256
 }
