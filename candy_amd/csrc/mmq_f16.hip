@@ -1,4 +1,4 @@
-// Prompt-sized batches (m >= 256) of Q4_K and Q6_K on the fp16 matrix cores: y[m, N] = x[m, K] . W^T.
+// Prompt-sized batches of Q4_K, Q5_K, Q6_K, Q8_0 and Q4_0 on the fp16 matrix cores: y[m, N] = x[m, K] . W^T.
 //
 // Replaces mul_mat_q / load_tiles_q4_K / load_tiles_q6_K (tensor/internal/cuda/kernels/quantized.cu
 // :455-578, :4116-4205) for prompt-sized batches.  With hundreds of activation rows the contraction
@@ -12,16 +12,19 @@
 // Both roundings are 2^-12 relative per element; the result stays a few 1e-4 (max-norm) from the
 // CPU contraction, inside the 1e-3 bar.
 //
-// Tiling: a workgroup owns 128 weight rows x 256 activation rows and walks K in steps of 64.  Every
-// thread dequantizes 16 weights per step into an LDS tile, the fp16 activations go into a second
-// LDS tile, both double-buffered so one barrier per step suffices.  Global requests run ahead in
-// registers: a thread's share of a whole super-block of weights four steps ahead (HBM), the
-// activations two steps ahead (L2).  Each of the 8 wavefronts owns a 64 x 64 sub-tile; LDS rows are
-// padded to 144 bytes so that the 16-byte operand reads of a wavefront spread over all banks.
-// Workgroups are numbered so that those sharing an XCD (and its L2) work on neighbouring weight
-// tiles of the same activation tile.  When the output has too few tiles to fill the chip
-// (N = 4096 or 1024 projections), K is split over several workgroups per tile; their partial sums
-// go to a scratch buffer and a second kernel adds them in a fixed order (bitwise reproducible).
+// Tiling: a workgroup owns 128 weight rows x 256 (or 128) activation rows and walks K in steps of 64.
+//   k_mmq_f16_pc (what runs): four producer wavefronts dequantize 16 weights per thread and step into an LDS tile
+//     (two or three buffers, one barrier per step); four consumer wavefronts read the weight fragments from LDS,
+//     load their activation fragments straight from memory into operand registers (the fp16 image is stored
+//     fragment by fragment, xh_index4) and issue the matrix instructions.
+//   k_mmq_f16 (comparison: option mmq.f16_shape 3): every wavefront dequantizes, copies activations into a second LDS
+//     tile and multiplies a 64 x 64 sub-tile.
+// Global requests run ahead in registers: a thread's share of a whole super-block of weights four steps ahead
+// (HBM), the activations one or two steps ahead (L2).  Workgroups are numbered so that those sharing an XCD (and its
+// L2) work on neighbouring weight tiles of the same activation tile.  When the output has too few tiles to fill the
+// chip (N = 4096 or 1024 projections), K is split over several workgroups per tile; their partial sums go to a
+// scratch buffer and a second kernel adds them in a fixed order (bitwise reproducible).  One launch can serve up to
+// three weight tensors that share their activations (q / k / v, gate / up).
 #include <cstdlib>
 
 #include "blocks.h"
