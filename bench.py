@@ -523,7 +523,7 @@ def main():
             peak = MFMA_I8_PEAK_TOPS if int8 else MFMA_F16_PEAK_TFLOPS
             roof_us = max(byts / (HBM_PEAK_GBPS * 1e9), flops / (peak * 1e12)) * 1e6
             pre.append({"m": m, "kernel": "k_mmv_q4k<1,2,2,8> (int8 MFMA, one pass)" if m <= 16 else
-                        ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else ("k_mmq_f16_pc<BigQ4K,%d> (fp16 MFMA, 128x%d tiles)" % ((128, 128) if m <= 128 else (256, 256))),
+                        ("k_mmq_i8<TileQ4K,%d,1,1> (int8 MFMA)" % (1 if m <= 32 else 4)) if int8 else ("k_mmq_f16_pc<BigQ4K,112,%d> (fp16 MFMA, 112x%d tiles)" % ((128, 128) if m <= 128 else (256, 256))),
                         "us": round(ms * 1e3, 2), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1),
                         "mfma_peak_TFLOPs": peak, "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / peak, 4),
                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),

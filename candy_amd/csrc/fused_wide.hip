@@ -81,7 +81,9 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec_wide(const WideArgs a) {
     int job[R], jrow[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int g = min(start + wave + WAVES * r, a.total - 1);  // clamped: a valid row, dropped at the store
+        // slots past the workgroup's share repeat its own last row (dropped at the store): a row this CU fetches
+        // anyway, where one row for all workgroups would have every CU queue at the same few cache lines
+        const int g = min(start + wave + WAVES * r, end - 1);
         if (EPI == WEPI_PAIR) {
             job[r] = 0;
             jrow[r] = g;

@@ -52,13 +52,14 @@ struct Q8Scale {
 struct Options {
     int matvec_span = 1;         // batch-1 kernel of the 2-byte aligned formats: aligned 16-byte spans through LDS
     int small_batch_kernel = 1;  // 2..8 rows: the one-workgroup-per-CU kernel (0: the looping kernel only)
+    int even_two_rows = 1;       // Q4_K, 2 rows: the even-split vector kernel (0: the looping kernel)
     int i8_min_m = 0;            // 5..15 rows: int8 tiles from this batch on (0: whichever the fitted times say)
     int mmq_min_m = 16;          // batch from which the tile kernels take over from the matvec family (>= 16)
     int f16_big_min_m = 256;     // decoder prompt pass: batch from which the fp16 big tiles take over from the int8 tiles
     int f16_api_min_m = 96;      // candy_hip_qmatmul*: the same threshold for a single contraction (3e-4 per matmul)
     int mmq_fp16_only = 0;       // 1: every tile contraction on the single-buffered fp16 tiles
     int i8_grid_split = 1;       // int8 tiles: split K over workgroups on small grids
-    int f16_shape = 0;           // comparison runs: Q4_K fp16 tiles 128 x 128 (2); single-role 128 x 256 kernel (3)
+    int f16_shape = 0;           // comparison runs: Q4_K fp16 tiles 128 x 128 (2); single-role 128 x 256 kernel (3); never 112-row tiles (4)
     int f16_split = 0;           // comparison runs: workgroups that share one fp16 tile's K (0: by grid size)
     int mmv_min_m = 3;           // f32 x Q4_K with this many .. mmv_max_m rows: the one-pass int8 kernel
     int mmv_max_m = 32;          //   (0: never; more than 16 rows only for rows of up to 4096 values)
@@ -184,6 +185,7 @@ bool mmq_i8_covers(const candy_hip_qtensor *w, const int8_t *qs);
 // mmv_i8.hip: 2 .. 32 activation rows against a Q4_K weight, one pass over the weights on the int8 matrix cores
 size_t mmv_workspace_bytes(int64_t K);
 bool mmv_covers(const candy_hip_qtensor *w, int64_t m);
+bool matvec_even_covers(const candy_hip_qtensor *w, int64_t m);  // the even-split vector kernel takes this batch
 int launch_mmv(candy_hip_device *dev, const candy_hip_qtensor *w, const float *x, const void *q8_blocks, int64_t m,
                float *y, void *ws);
 int launch_mmq_i8(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs,

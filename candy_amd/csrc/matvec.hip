@@ -466,6 +466,131 @@ static int launch_mb(candy_hip_device *dev, const candy_hip_qtensor *w, const in
 #undef CANDY_MB
 }
 
+// Two activation rows, even split: the weight rows dealt evenly (to within one row) to two workgroups of 8 wavefronts
+// per CU; a wavefront requests all of its R rows before the NB = 2 quantized activation rows are staged in LDS, so the
+// whole share of a CU is in flight at once, as in the batch-1 kernel, and the dots of a row (its weight-only part
+// prepared once, then one dot per activation row) start as its bytes arrive.  Per row and activation row the
+// additions are those of the other vector kernels: a lane's units in ascending order, then the wavefront sum - the
+// same bits.  The role of mul_mat_vec_q<2> (quantized.cu:2787-2871).  Measured with more images (us per call with the
+// quantizer, 4096 x 11008): 2 rows 12.2 against 14.5 on the looping kernel; 3 and 4 rows 15.6 and 16.3 against 14.0 on
+// the one-pass matrix-core kernel - every further image costs a CU 1.7 us of dot4 arithmetic that starts only when
+// the rows have arrived - so only the two-image form is built.
+template <class U, int ITER, int R, int NB>
+__global__ __launch_bounds__(512, 4) void k_matvec_even(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
+                                                     const Q8Scale *__restrict__ xs, float *__restrict__ y, int N, int K,
+                                                     int m) {
+    constexpr int WAVES = 8;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int units = K / U::ELEMS;
+    const size_t rb = U::row_bytes(K);
+    const int q_bytes = skewed(K), blocks_per_row = K >> 5;
+    int8_t *sq = (int8_t *)smem;
+    Q8Scale *ss = (Q8Scale *)(smem + NB * q_bytes);
+    const int G = gridDim.x;
+    const int start = (int)(((long long)blockIdx.x * N) / G), end = (int)(((long long)(blockIdx.x + 1) * N) / G);
+
+    typename U::W w[R][ITER];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        // slots past the share repeat its last row (not stored): a row this workgroup fetches anyway
+        const uint8_t *rp = W + (size_t)min(start + wave + WAVES * r, end - 1) * rb;
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) U::load(rp, min(it * 64 + lane, units - 1), w[r][it]);
+    }
+    {
+        const int chunks = K >> 4;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int src_row = min(nb, m - 1);  // images past m: a copy of the last row, not stored
+            const uint4 *src = (const uint4 *)(xq + (size_t)src_row * K);
+            uint4 *dst = (uint4 *)(sq + nb * q_bytes);
+            for (int c = tid; c < chunks; c += WAVES * 64) dst[c + (c >> 4)] = src[c];
+            const uint2 *s2 = (const uint2 *)(xs + (size_t)src_row * blocks_per_row);
+            uint2 *d2 = (uint2 *)(ss + nb * blocks_per_row);
+            for (int i = tid; i < blocks_per_row; i += WAVES * 64) d2[i] = s2[i];
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float acc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = 0.0f;
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int u = it * 64 + lane;
+            const bool live = u < units;
+            const int uc = live ? u : units - 1;
+            typename Prepped<U>::P pw;
+            Prepped<U>::prep(w[r][it], uc, pw);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const float v = Prepped<U>::dot(pw, uc, sq + nb * q_bytes, ss + nb * blocks_per_row);
+                acc[nb] += live ? v : 0.0f;
+                // one dot's activations in registers at a time: the sum is pinned here and no LDS read crosses (the
+                // reads of every image and round hoisted cost registers; the SIMD's other wavefronts cover the latency)
+                asm volatile("" : "+v"(acc[nb]) : : "memory");
+            }
+        }
+        const int row = start + wave + WAVES * r;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const float sum = wave_sum(acc[nb]);
+            if (lane == 0 && nb < m && row < end) y[(size_t)nb * N + row] = sum;
+        }
+    }
+}
+
+template <class U, int ITER, int R, int NB>
+static int launch_even_cfg(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int m,
+                           float *y, int grid) {
+    const int N = (int)w->rows, K = (int)w->cols;
+    const size_t smem = mb_lds_bytes(NB, K);
+    auto kern = k_matvec_even<U, ITER, R, NB>;
+    if (smem > 48 * 1024)
+        CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, dev->stream, (const uint8_t *)w->data, qs, scales, y, N,
+                       K, m);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+// Rows of a weight per wavefront (R) in the even-split kernel, or 0 where it does not apply: two activation rows,
+// Q4_K with rows of up to four rounds of units, at least 16 weight rows per CU and at most R * rounds = 3 or 4 units
+// per lane (measured, us per call with the quantizer, against the looping kernel: 4096 x 14336 14.3 / 17.4, 4096 x
+// 11008 12.2 / 14.5, 4096 x 4096 7.3 / 7.9, 11008 x 4096 11.8 / 12.2; with four rows per wavefront 14336 x 4096 13.9 /
+// 13.2), and the images of two workgroups fitting a CU's LDS.
+static int even_rows_per_wave(const candy_hip_qtensor *w, int64_t m) {
+    const candy_hip_device *dev = w->dev;
+    if (w->fmt != CANDY_HIP_Q4_K || m != 2 || !dev->opt.even_two_rows || ((uintptr_t)w->data & 15) != 0) return 0;
+    const int64_t K = w->cols;
+    if (K % 256 != 0 || K > 16384 || w->rows < 16 * (int64_t)dev->num_cus || w->rows > 0x3FFFFFFF) return 0;
+    if (2 * mb_lds_bytes(2, K) > MB_LDS_MAX) return 0;
+    const int iter = (int)((K / UnitQ4K::ELEMS + 63) / 64);
+    const int64_t per2 = (w->rows + 2 * dev->num_cus - 1) / (2 * dev->num_cus);
+    const int r = (int)((per2 + 7) / 8);
+    return r <= (iter == 1 ? 3 : 1) ? r : 0;
+}
+bool matvec_even_covers(const candy_hip_qtensor *w, int64_t m) { return even_rows_per_wave(w, m) != 0; }
+
+static int launch_even(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales, int m,
+                       float *y) {
+    typedef UnitQ4K U;
+    const int r = even_rows_per_wave(w, m);
+    if (!r) return CANDY_HIP_ERR_UNSUPPORTED;
+    const int iter = (int)((w->cols / U::ELEMS + 63) / 64), grid = 2 * dev->num_cus;
+    if (iter == 1) {
+        if (r == 1) return launch_even_cfg<U, 1, 1, 2>(dev, w, qs, scales, m, y, grid);
+        if (r == 2) return launch_even_cfg<U, 1, 2, 2>(dev, w, qs, scales, m, y, grid);
+        return launch_even_cfg<U, 1, 3, 2>(dev, w, qs, scales, m, y, grid);
+    }
+    if (iter == 2) return launch_even_cfg<U, 2, 1, 2>(dev, w, qs, scales, m, y, grid);
+    if (iter == 3) return launch_even_cfg<U, 3, 1, 2>(dev, w, qs, scales, m, y, grid);
+    return launch_even_cfg<U, 4, 1, 2>(dev, w, qs, scales, m, y, grid);
+}
+
 template <class U, int NB, int R, int WAVES>
 static int launch_one(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                       float *y, int m = NB) {
@@ -513,6 +638,11 @@ static int launch_fmt(candy_hip_device *dev, const candy_hip_qtensor *w, const i
         const Q8Scale *s = scales + done * sstride;
         float *yo = y + done * N;
         int rc;
+        if (!old_small && matvec_even_covers(w, left)) {  // what is left in one pass of the even-split kernel
+            rc = launch_even(dev, w, q, s, (int)left, yo);
+            if (rc == CANDY_HIP_OK) { done += left; continue; }
+            if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+        }
         {
             // The looping kernel below takes up to 8, 4, 2 or 1 rows per launch (fewer the longer the row is); where that
             // covers what is left in as few launches as this kernel's 8 per pass, it is as fast or a little faster
@@ -679,7 +809,7 @@ static int qmatmul_f32(candy_hip_device *dev, const candy_hip_qtensor *w, const 
         const int rc = launch_matvec_wide(dev, Wd);
         if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     }
-    if (a.mmv_ws && mmv_covers(w, m)) return launch_mmv(dev, w, dev_x, nullptr, m, dev_y, a.mmv_ws);
+    if (a.mmv_ws && mmv_covers(w, m) && !matvec_even_covers(w, m)) return launch_mmv(dev, w, dev_x, nullptr, m, dev_y, a.mmv_ws);
     if (a.half_ws && m >= mmq_min_m(dev) && !dev->opt.mmq_fp16_only && mmq_f16_big_covers(w, m, dev->opt.f16_api_min_m)) {
         // the fp16 tiles read d * q as fp16: the quantizer writes that image directly (one launch, no int8 copy)
         if (int rc = launch_quantize_q8(dev, dev_x, m, w->cols, nullptr, nullptr, nullptr, (_Float16 *)a.half_ws)) return rc;
@@ -730,7 +860,7 @@ int candy_hip_qmatmul_q8(candy_hip_device *dev, const candy_hip_qtensor *w, cons
     if (int rc = use_device(dev)) return rc;
     ActWorkspace a;
     if (int rc = act_workspace(dev, m, w->cols, true, &a)) return rc;
-    if (a.mmv_ws && mmv_covers(w, m)) return launch_mmv(dev, w, nullptr, dev_x_q8_0, m, dev_y, a.mmv_ws);
+    if (a.mmv_ws && mmv_covers(w, m) && !matvec_even_covers(w, m)) return launch_mmv(dev, w, nullptr, dev_x_q8_0, m, dev_y, a.mmv_ws);
     if (int rc = launch_q8_blocks_to_planar(dev, dev_x_q8_0, m * (w->cols >> 5), a.qs, a.scales)) return rc;
     return contract(dev, w, a, m, dev_y);
 }

@@ -452,11 +452,17 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
 // instructions, reading the next phase's four weight fragments from LDS while the current phase's instructions run.
 // The two roles are separate loops with the same number of barriers, so that their registers (accumulators and
 // operand fragments here, raw blocks there) share one allocation.
-template <class F, int BM, bool RES>
+// BN = 112 (seven 16-row fragments: the second half of the weight rows is three fragments instead of four) is for
+// row counts that are a multiple of 7 * 16 and not of 256 * 128: 14336 = 128 * 112 rows are 128 tiles, one or two per
+// CU, where 112 tiles of 128 rows leave an eighth of the chip idle or wait for a short last round.  The LDS buffers
+// keep room for 128 rows; the producer wavefront whose second task would fall on rows 112 .. 127 repeats its first.
+template <class F, int BN, int BM, bool RES>
 __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _Float16 *__restrict__ xh, int M, int K,
                                                     int n_tiles, int m_tiles, int sb_per, size_t split_stride) {
-    constexpr int BN = 128, PT = 256;
-    constexpr int ATK = BN * 4 / PT;  // dequantization tasks per producer thread per step
+    constexpr int PT = 256, BNB = 128;  // BNB: weight rows an LDS buffer has room for
+    constexpr int ATK = BNB * 4 / PT;   // dequantization tasks per producer thread per step
+    constexpr int TNF = BN / 16;        // 16-row weight fragments of the tile
+    static_assert(BN == 128 || BN == 112, "weight rows per tile");
     constexpr int TM = BM / 64;       // 16-row activation fragments of a consumer's sub-tile (its rows: BM / 4)
     static_assert(BM == 256 || BM == 128, "activation rows per tile");
     // BM = 256: the producers work two steps ahead into the third of three weight buffers, and a consumer reads the
@@ -465,7 +471,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
     // 35.2 us at 14336 x 4096 x 128.
     constexpr int LEAD = BM == 256 ? 2 : 1, NB = LEAD + 1;
     extern __shared__ __align__(16) uint8_t smem_raw[];
-    _Float16 *sA = (_Float16 *)smem_raw;               // [NB][BN / 16][2] fragments
+    _Float16 *sA = (_Float16 *)smem_raw;               // [NB][BNB / 16][2] fragments
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -492,21 +498,22 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
         // ---------------- producers: the weight tile of step t + LEAD (buffer (t + LEAD) % NB) while step t is contracted
         typename F::Raw raw[2][ATK];
         // neighbouring lanes take neighbouring quarters of a row; a half-wavefront takes rows {x, x+4, x+8, x+12}
-        const int a_c = lane & 3, a_row = 16 * wave + 4 * ((lane >> 2) & 3) + (lane >> 4);   // + 64 i
+        const int a_c = lane & 3, a_row = 16 * wave + 4 * ((lane >> 2) & 3) + (lane >> 4);   // + a_step i
+        const int a_step = BN == 112 && wave == 3 ? 0 : 64;
         auto gload_a = [&](int sb, int slot) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < ATK; ++i)
-                F::load(W + (size_t)min(n0 + a_row + 64 * i, N - 1) * rb + (size_t)sb * F::BLOCK, a_c, raw[slot][i]);
+                F::load(W + (size_t)min(n0 + a_row + a_step * i, N - 1) * rb + (size_t)sb * F::BLOCK, a_c, raw[slot][i]);
         };
         auto stage = [&](int g, int aslot, int buf) __attribute__((always_inline)) {
-            _Float16 *a = sA + buf * BN * BIG_BK;
+            _Float16 *a = sA + buf * BNB * BIG_BK;
 #pragma unroll
             for (int i = 0; i < ATK; ++i) {
                 half8 o0, o1;
                 int k0, k1;
                 F::dequant(raw[aslot][i], g, a_c, o0, o1, k0, k1);
-                *(half8 *)&a[frag_off(a_row + 64 * i, k0)] = o0;
-                *(half8 *)&a[frag_off(a_row + 64 * i, k1)] = o1;
+                *(half8 *)&a[frag_off(a_row + a_step * i, k0)] = o0;
+                *(half8 *)&a[frag_off(a_row + a_step * i, k1)] = o1;
             }
         };
         gload_a(0, 0);
@@ -532,11 +539,11 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
         return;
     }
 
-    // ---------------- consumers: wavefront cw owns 128 weight rows x activation rows [cw * BM / 4, + BM / 4)
+    // ---------------- consumers: wavefront cw owns the BN weight rows x activation rows [cw * BM / 4, + BM / 4)
     const int cw = wave - 4;
-    float4v acc[8][TM];
+    float4v acc[TNF][TM];
 #pragma unroll
-    for (int a = 0; a < 8; ++a)
+    for (int a = 0; a < TNF; ++a)
 #pragma unroll
         for (int b = 0; b < TM; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
     // activation fragment (16-row block rbk of the tile, 32-value block kb of K): 1 KB at ((m0 / 16 + rbk) * (K / 32) + kb)
@@ -551,19 +558,21 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
                 bf[slot][kk][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ks * 2 + kk) * 512);
     };
     half8 af[2][4];
-    // phase p = 2 * kk + h of a step: weight rows 64 h .. 64 h + 63, values 32 kk .. 32 kk + 31
+    // phase p = 2 * kk + h of a step: weight rows 64 h .. min(64 h + 63, BN - 1), values 32 kk .. 32 kk + 31
     auto fetch = [&](int abuf, int p) __attribute__((always_inline)) {
-        const _Float16 *a = sA + abuf * BN * BIG_BK + frag_lane_off(lane);
+        const _Float16 *a = sA + abuf * BNB * BIG_BK + frag_lane_off(lane);
 #pragma unroll
-        for (int tn = 0; tn < 4; ++tn) af[p & 1][tn] = *(const half8 *)&a[(((p & 1) * 4 + tn) * 2 + (p >> 1)) * 512];
+        for (int tn = 0; tn < 4; ++tn)
+            if ((p & 1) * 4 + tn < TNF) af[p & 1][tn] = *(const half8 *)&a[(((p & 1) * 4 + tn) * 2 + (p >> 1)) * 512];
     };
     auto mma = [&](int bslot, int p) __attribute__((always_inline)) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm)
-                acc[(p & 1) * 4 + tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[p & 1][tn], bf[bslot][p >> 1][tm],
-                                                                                 acc[(p & 1) * 4 + tn][tm], 0, 0, 0);
+                if ((p & 1) * 4 + tn < TNF)
+                    acc[(p & 1) * 4 + tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        af[p & 1][tn], bf[bslot][p >> 1][tm], acc[(p & 1) * 4 + tn][tm], 0, 0, 0);
     };
     load_b(0, 0);
     __syncthreads();  // the weight tiles of the first LEAD steps are in LDS
@@ -595,7 +604,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
 
     // C layout of a 16x16 tile: lane holds activation row (lane & 15) and weight rows 4*(lane>>4)..+3
 #pragma unroll
-    for (int tn = 0; tn < 8; ++tn)
+    for (int tn = 0; tn < TNF; ++tn)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
             const int m = m0 + cw * (BM / 4) + tm * 16 + (lane & 15);
@@ -658,9 +667,25 @@ struct F16Job {
     const float *res;
 };
 
+// Workgroups per tile along K: split K until the grid covers the chip, keeping at least two super-blocks (8 steps)
+// per workgroup: as many workgroups per tile as leave every workgroup a CU of its own (measured against rounding up:
+// 14336 x 4096 at 128 rows 44.8 us with 2 against 47.6 with 3; 11008 x 4096 at 256 rows 57.4 with 2 against 66.6 with
+// 3, at 512 rows 88.8 with 1 against 105.7 with 2)
+static int plan_split(const candy_hip_device *dev, int tiles, int n_sb) {
+    int n_split = 1;
+    if (tiles < (3 * dev->num_cus) / 4) {
+        n_split = dev->num_cus / tiles;
+        if (n_split > n_sb / 2) n_split = n_sb / 2;
+        if (n_split > 16) n_split = 16;
+        if (n_split < 1) n_split = 1;
+    }
+    if (dev->opt.f16_split > 0) n_split = std::min(dev->opt.f16_split, n_sb);  // comparison runs
+    return n_split;
+}
+
 template <class F, int BN, int BM, int WN, int WM, bool PC = false>
 static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, const _Float16 *xh, int64_t m) {
-    static_assert(!PC || (BN == 128 && (BM == 256 || BM == 128) && WN * WM == 8), "the role-split kernel's tiles");
+    static_assert(!PC || ((BN == 128 || BN == 112) && (BM == 256 || BM == 128) && WN * WM == 8), "the role-split kernel's tiles");
     const int K = (int)jobs[0].w->cols;
     F16Group grp{};
     grp.count = count;
@@ -675,18 +700,7 @@ static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, cons
     }
     const int m_tiles = (int)((m + BM - 1) / BM);
     const int tiles = n_tiles * m_tiles, n_sb = K >> 8;
-    // split K until the grid covers the chip, keeping at least two super-blocks (8 steps) per workgroup: as many
-    // workgroups per tile as leave every workgroup a CU of its own (measured against rounding up: 14336 x 4096 at
-    // 128 rows 44.8 us with 2 against 47.6 with 3; 11008 x 4096 at 256 rows 57.4 with 2 against 66.6 with 3, at 512
-    // rows 88.8 with 1 against 105.7 with 2)
-    int n_split = 1;
-    if (tiles < (3 * dev->num_cus) / 4) {
-        n_split = dev->num_cus / tiles;
-        if (n_split > n_sb / 2) n_split = n_sb / 2;
-        if (n_split > 16) n_split = 16;
-        if (n_split < 1) n_split = 1;
-    }
-    if (dev->opt.f16_split > 0) n_split = std::min(dev->opt.f16_split, n_sb);  // comparison runs
+    int n_split = plan_split(dev, tiles, n_sb);
     const int sb_per = (n_sb + n_split - 1) / n_split;
     n_split = (n_sb + sb_per - 1) / sb_per;  // no empty splits
     const size_t split_stride = (size_t)m * (size_t)n_total;
@@ -703,10 +717,10 @@ static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, cons
             off += (size_t)m * (size_t)jobs[s].w->rows;
         }
     }
-    constexpr size_t smem = (size_t)(PC ? 3 * BN : 2 * (BN + BM)) * BIG_BK * sizeof(_Float16);  // role-split: weight tiles only
+    constexpr size_t smem = (size_t)(PC ? 3 * 128 : 2 * (BN + BM)) * BIG_BK * sizeof(_Float16);  // role-split: weight tiles only
     const bool epi_res = any_res && n_split == 1;
     void (*kern)(const F16Group, const _Float16 *, int, int, int, int, int, size_t);
-    if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, BM, true> : k_mmq_f16_pc<F, BM, false>;
+    if constexpr (PC) kern = epi_res ? k_mmq_f16_pc<F, BN, BM, true> : k_mmq_f16_pc<F, BN, BM, false>;
     else kern = epi_res ? k_mmq_f16<F, BN, BM, WN, WM, true> : k_mmq_f16<F, BN, BM, WN, WM, false>;
     CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream, grp, xh, (int)m, K,
@@ -763,9 +777,29 @@ static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, con
     if (fmt == CANDY_HIP_Q4_0_GGML) CANDY_BIG_256(BigQ4_0<true>);
     // Q4_K. Up to 128 activation rows: 128 x 128 tiles, K split over workgroups to fill the chip
     const int shape = dev->opt.f16_shape;  // comparison runs
+    // Tiles of 112 weight rows where every tensor's rows divide by 112 and the grid then takes fewer row-steps of its
+    // busiest CU: rounds of workgroups x rows per tile x super-blocks per workgroup (14336 rows: 128 tiles instead of
+    // 112, so 256 instead of 224 workgroups at 512 activation rows, 512 instead of 448 for a gate / up pair).
+    auto narrow = [&](int bm) {
+        if (single || shape == 4) return false;
+        const int n_sb = (int)(jobs[0].w->cols >> 8), m_tiles = (int)((m + bm - 1) / bm);
+        int64_t t112 = 0, t128 = 0;
+        for (int s = 0; s < count; ++s) {
+            if (jobs[s].w->rows % 112 != 0) return false;
+            t112 += jobs[s].w->rows / 112;
+            t128 += (jobs[s].w->rows + 127) / 128;
+        }
+        auto cost = [&](int64_t tiles, int bn) {
+            const int ns = plan_split(dev, (int)(tiles * m_tiles), n_sb), sb_per = (n_sb + ns - 1) / ns;
+            const int64_t wgs = tiles * m_tiles * ((n_sb + sb_per - 1) / sb_per);
+            return ((wgs + dev->num_cus - 1) / dev->num_cus) * bn * sb_per;
+        };
+        return cost(t112, 112) < cost(t128, 128);
+    };
     auto small_tiles = [&]() {
-        return single ? launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m)
-                      : launch_big<BigQ4K, 128, 128, 2, 4, true>(dev, jobs, count, xh, m);
+        if (single) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m);
+        if (narrow(128)) return launch_big<BigQ4K, 112, 128, 2, 4, true>(dev, jobs, count, xh, m);
+        return launch_big<BigQ4K, 128, 128, 2, 4, true>(dev, jobs, count, xh, m);
     };
     if (shape == 2 || m <= 128) return small_tiles();
     // up to 256 rows where the 128 x 128 tiles fill the chip and the 128 x 256 tiles would have to split K
@@ -779,6 +813,7 @@ static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, con
     // 54.2; 6144 x 4096 at 512 rows 44.8 against 47.1; with K = 14336 the split is cheap and the wider tile wins)
     if (shape == 0 && jobs[0].w->cols <= 4096 && n128 * ((m + 255) / 256) < fill && n128 * ((m + 127) / 128) <= dev->num_cus)
         return small_tiles();
+    if (narrow(256)) return launch_big<BigQ4K, 112, 256, 2, 4, true>(dev, jobs, count, xh, m);
     CANDY_BIG_256(BigQ4K);
 #undef CANDY_BIG_256
 }

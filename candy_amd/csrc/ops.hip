@@ -101,22 +101,24 @@ __global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ src, 
     float best = -3.402823466e+38f;
     uint32_t bi = 0xFFFFFFFFu;
     if ((cols & 3) == 0 && ((uintptr_t)xr & 15) == 0) {
-        // four independent 16-byte loads in flight per thread: one block has to cover a whole vocabulary row
+        // sixteen independent 16-byte loads in flight per thread: one block has to cover a whole vocabulary row, and
+        // every round of loads is a memory latency (128256 logits: two rounds; with four loads per round 13 us)
+        constexpr int U = 16;
         const float4 *x4 = (const float4 *)xr;
         const int n4 = cols >> 2, step = (int)blockDim.x;
-        for (int c0 = threadIdx.x; c0 < n4; c0 += 4 * step) {
-            float4 v[4];
+        for (int c0 = threadIdx.x; c0 < n4; c0 += U * step) {
+            float4 v[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = x4[min(c0 + u * step, n4 - 1)];
+            for (int u = 0; u < U; ++u) v[u] = x4[min(c0 + u * step, n4 - 1)];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int c = c0 + u * step;
-                if (c >= n4) break;
+                const bool in = c < n4;  // past the row: the clamped load is a value already seen at a lower index
                 // ascending index within the thread, strict >: the first maximum wins
-                if (v[u].x > best) { best = v[u].x; bi = (uint32_t)(4 * c); }
-                if (v[u].y > best) { best = v[u].y; bi = (uint32_t)(4 * c + 1); }
-                if (v[u].z > best) { best = v[u].z; bi = (uint32_t)(4 * c + 2); }
-                if (v[u].w > best) { best = v[u].w; bi = (uint32_t)(4 * c + 3); }
+                if (in && v[u].x > best) { best = v[u].x; bi = (uint32_t)(4 * c); }
+                if (in && v[u].y > best) { best = v[u].y; bi = (uint32_t)(4 * c + 1); }
+                if (in && v[u].z > best) { best = v[u].z; bi = (uint32_t)(4 * c + 2); }
+                if (in && v[u].w > best) { best = v[u].w; bi = (uint32_t)(4 * c + 3); }
             }
         }
     } else {

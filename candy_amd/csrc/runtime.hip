@@ -344,13 +344,14 @@ struct OptionKey {
 const OptionKey OPTION_KEYS[] = {
     {"matvec.span", &candy::Options::matvec_span, 0, 1},
     {"matvec.small_batch_kernel", &candy::Options::small_batch_kernel, 0, 1},
+    {"matvec.even_two_rows", &candy::Options::even_two_rows, 0, 1},
     {"mmq.i8_min_m", &candy::Options::i8_min_m, 0, 1 << 20},
     {"mmq.min_m", &candy::Options::mmq_min_m, 16, 1 << 20},
     {"mmq.f16_big_min_m", &candy::Options::f16_big_min_m, 16, 1 << 30},
     {"mmq.f16_api_min_m", &candy::Options::f16_api_min_m, 16, 1 << 30},
     {"mmq.fp16_only", &candy::Options::mmq_fp16_only, 0, 1},
     {"mmq.i8_grid_split", &candy::Options::i8_grid_split, 0, 1},
-    {"mmq.f16_shape", &candy::Options::f16_shape, 0, 3},
+    {"mmq.f16_shape", &candy::Options::f16_shape, 0, 4},
     {"mmq.f16_split", &candy::Options::f16_split, 0, 16},
     {"mmv.min_m", &candy::Options::mmv_min_m, 2, 32},
     {"mmv.max_m", &candy::Options::mmv_max_m, 0, 32},

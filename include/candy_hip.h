@@ -87,12 +87,16 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   -- comparison / test only --
  *   "matvec.span"                1        batch-1 kernel of 2-byte aligned formats fetches aligned 16-byte spans
  *   "matvec.small_batch_kernel"  1        2..8 rows on the one-workgroup-per-CU kernel (0: looping kernel)
+ *   "matvec.even_two_rows"       1        Q4_K, 2 rows: the vector kernel that deals the weight rows evenly to two
+ *                                         workgroups per CU (0: looping kernel)
  *   "mmq.i8_min_m"               0        5..15 rows: int8 tiles from this batch on (0: by measured cost model)
  *   "mmq.fp16_only"              0        every tile contraction on the single-buffered fp16 tiles
  *   "mmq.i8_grid_split"          1        int8 tiles split K over workgroups on small grids
  *   "mmq.f16_shape"              0        comparison runs: Q4_K fp16 tiles of 128 x 128 at every batch (2); fp16 tiles
  *                                         computed by the kernel whose wavefronts each dequantize and multiply (3)
- *                                         instead of the one that splits the two roles over wavefronts (0: by shape)
+ *                                         instead of the one that splits the two roles over wavefronts; 128 weight
+ *                                         rows per tile also where 112 divide the rows and fill the chip better (4)
+ *                                         (0: by shape)
  *   "mmq.f16_split"              0        comparison runs: K split of the fp16 tile kernels over this many workgroups per
  *                                         tile, 1..16 (0: as many as fill the chip)
  *   "mmv.min_m"                  3        candy_hip_qmatmul on Q4_K: batches of this many .. "mmv.max_m" rows take the

@@ -138,6 +138,29 @@ def test_role_split_tiles_equal_the_single_role_tiles(dev, fmt, m, rows, cols):
     assert np.array_equal(got.view(np.uint32), single.view(np.uint32))
 
 
+@pytest.mark.parametrize("m,rows,cols", [(512, 1792, 1024), (128, 3584, 768), (300, 112, 512), (257, 2240, 2304),
+                                         (1000, 14336, 256)])
+@pytest.mark.parametrize("split", [1, 2])
+def test_tiles_of_112_weight_rows_equal_tiles_of_128(dev, m, rows, cols, split):
+    # Q4_K row counts that 112 divides (14336 = 128 * 112) take tiles of 112 weight rows where those fill the chip
+    # better: the same multiply-adds in the same order as the 128-row tiles when K is split the same way, and the
+    # oracle's values on every row (default split)
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=rows + m)
+    x = synth.random_activations(m, cols, seed=cols + 2 * m)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    dev.set_option("mmq.f16_split", split)
+    try:
+        got = dev.qmatmul(q, x)
+        dev.set_option("mmq.f16_shape", 4)
+        wide = dev.qmatmul(q, x)
+    finally:
+        dev.set_option("mmq.f16_shape", 0)
+        dev.set_option("mmq.f16_split", 0)
+    assert np.array_equal(got.view(np.uint32), wide.view(np.uint32))
+    if split == 1 and rows * m <= 1 << 20:
+        assert rel_err(dev.qmatmul(q, x), o.qmatmul(synth.Q4_K, w, rows, cols, x)) <= 5e-4
+
+
 def test_q8_0_wide_prompt_grid_takes_the_fp16_tiles(dev):
     # many weight rows and a prompt-sized batch: Q8_0 leaves the int8 tiles for the 128 x 128 fp16 tiles
     rows, cols, m = 8192, 256, 352
@@ -166,7 +189,7 @@ def test_config_prefill_q4k_14336x4096(dev, m):
     x = synth.random_activations(m, cols, seed=78 + m)
     q = dev.qtensor(synth.Q4_K, rows, cols, w)
     got = dev.qmatmul(q, x)
-    sub = np.arange(0, rows, 224)  # 64 rows
+    sub = np.arange(0, rows, 223)  # 65 rows, at varying places of the 16-, 112- and 128-row units the kernels tile by
     rb = synth.weight_nbytes(synth.Q4_K, 1, cols)
     want = o.qmatmul(synth.Q4_K, w.reshape(rows, rb)[sub].reshape(-1), len(sub), cols, x)
     assert rel_err(got[:, sub], want) <= TOL

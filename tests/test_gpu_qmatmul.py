@@ -82,6 +82,27 @@ def test_small_batch_one_pass_per_eight_rows(dev, monkeypatch, fmt, rows, cols):
         assert rel_err(got, old) <= 2e-6, m
 
 
+@pytest.mark.parametrize("rows,cols", [(4096, 256), (4100, 512), (11008, 4096), (4096, 11008), (4096, 8192),
+                                       (4096, 14336), (12288, 1024), (9000, 2048)])
+def test_two_rows_even_split_kernel(dev, rows, cols):
+    # two activation rows against a Q4_K weight with 16 .. 48 rows per CU: the weight rows dealt evenly to two
+    # workgroups per CU, one to three rows per wavefront, one to four rounds of units per row, row counts that do not
+    # divide by the grid.  Same additions in the same order as the looping kernel: same bits.
+    w = synth.random_weight(synth.Q4_K, rows, cols, seed=rows + cols)
+    q = dev.qtensor(synth.Q4_K, rows, cols, w)
+    sub = np.unique(np.concatenate([np.arange(0, rows, 97), np.arange(rows - 40, rows)]))
+    wsub = w.reshape(rows, -1)[sub].reshape(-1)
+    x = synth.random_activations(2, cols, seed=22 + cols)
+    got = dev.qmatmul(q, x)
+    try:
+        dev.set_option("matvec.even_two_rows", 0)
+        old = dev.qmatmul(q, x)
+    finally:
+        dev.set_option("matvec.even_two_rows", 1)
+    assert np.array_equal(got.view(np.uint32), old.view(np.uint32))
+    assert rel_err(got[:, sub], o.qmatmul(synth.Q4_K, wsub, len(sub), cols, x)) <= 2e-5
+
+
 def test_config_q4_0_4096x4096(dev):
     # the single-QMatMul configuration: Q4_0 4096x4096, one f32 N(0,1) vector, seeded
     rows = cols = 4096
