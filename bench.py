@@ -507,8 +507,8 @@ def main():
 
     if not args.no_prefill:
         # batched prefill: Q4_K 14336x4096 x f32 [M, 4096], f32 in -> f32 out (activation quantization included).
-        # m <= 16 is one pass over the weights on the int8 matrix cores (k_mmv_q4k), 16 < m < 96 the int8 tile kernel
-        # (both exact integer dots; peak 5.0 POP/s), m >= 96 fp16 tiles
+        # m <= 16 is one pass over the weights on the int8 matrix cores (k_mmv_q4k), 16 < m < 33 the int8 tile kernel
+        # (both exact integer dots; peak 5.0 POP/s), m >= 33 fp16 tiles
         # (operands rounded to fp16, 3e-4 per matmul; peak 2.5 PFLOP/s).  roofline_us = the larger of the bytes at 8 TB/s and the contraction at that peak.
         pre = []
         r, k = 14336, 4096

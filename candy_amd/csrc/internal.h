@@ -56,7 +56,7 @@ struct Options {
     int i8_min_m = 0;            // 5..15 rows: int8 tiles from this batch on (0: whichever the fitted times say)
     int mmq_min_m = 16;          // batch from which the tile kernels take over from the matvec family (>= 16)
     int f16_big_min_m = 256;     // decoder prompt pass: batch from which the fp16 big tiles take over from the int8 tiles
-    int f16_api_min_m = 96;      // candy_hip_qmatmul*: the same threshold for a single contraction (3e-4 per matmul)
+    int f16_api_min_m = 33;      // candy_hip_qmatmul*: the same for a single contraction (Q4_K, Q6_K; the others from 65)
     int mmq_fp16_only = 0;       // 1: every tile contraction on the single-buffered fp16 tiles
     int i8_grid_split = 1;       // int8 tiles: split K over workgroups on small grids
     int f16_shape = 0;           // comparison runs: Q4_K fp16 tiles 128 x 128 (2); single-role 128 x 256 kernel (3); never 112-row tiles (4)

@@ -25,7 +25,9 @@
 // chip (N = 4096 or 1024 projections), K is split over several workgroups per tile; their partial sums go to a
 // scratch buffer and a second kernel adds them in a fixed order (bitwise reproducible).  One launch can serve up to
 // three weight tensors that share their activations (q / k / v, gate / up).
+#include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "blocks.h"
 #include "internal.h"
@@ -754,9 +756,14 @@ static int launch_big(candy_hip_device *dev, const candy_hip_qtensor *w, const _
 }
 
 bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m) {
-    // a lower threshold (single contractions through the API) holds for Q4_K only: its tiles have the cheap
-    // dequantization and the 128 x 128 shape; the other formats' int8 tiles stay ahead up to the decoder's threshold
-    if (min_m <= 0 || w->fmt != CANDY_HIP_Q4_K) min_m = w->dev->opt.f16_big_min_m;
+    // A lower threshold than the decoder's holds for single contractions through the API: Q4_K and Q6_K from `min_m`
+    // rows, the other formats from 65: up to 64 rows are one tile of the int8 kernel, which is level with the fp16 tiles
+    // there for Q8_0, Q4_0 and Q5_K (and exact).  Measured, us per call, int8 / fp16 tiles: Q6_K 14336 x 4096 at 33 rows
+    // 43.8 / 36.6, 4096 x 14336 at 96 rows 71.5 / 39.2, at 255 rows 133 / 57; Q8_0 14336 x 4096 at 48 rows 46.2 / 41.9
+    // (4096 x 4096 22.4 / 22.6), at 96 rows 77.8 / 44.7, at 255 rows 121 / 61; Q4_0 at 48 rows 38.9 / 38.0 (4096 x 4096
+    // 19.9 / 22.4), at 96 rows 64.3 / 48.7; Q5_K 36.9 / 35.1 (19.9 / 19.9) and 58.6 / 47.2.
+    if (min_m <= 0) min_m = w->dev->opt.f16_big_min_m;
+    else if (w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K) min_m = std::min(std::max(min_m, 65), w->dev->opt.f16_big_min_m);
     if (m < min_m || w->cols % 256 != 0) return false;
     if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
     if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML)
@@ -764,24 +771,19 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m) {
     return false;
 }
 
-static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, const _Float16 *xh, int64_t m) {
-    const int fmt = jobs[0].w->fmt;
-    const bool single = dev->opt.f16_shape == 3;  // comparison runs: every wavefront in both roles
-#define CANDY_BIG_256(F)                                                                      \
-    return single ? launch_big<F, 128, 256, 2, 4>(dev, jobs, count, xh, m)                  \
-                  : launch_big<F, 128, 256, 2, 4, true>(dev, jobs, count, xh, m)
-    if (fmt == CANDY_HIP_Q6_K) CANDY_BIG_256(BigQ6K);
-    if (fmt == CANDY_HIP_Q5_K) CANDY_BIG_256(BigQ5K);
-    if (fmt == CANDY_HIP_Q8_0) CANDY_BIG_256(BigQ8_0);
-    if (fmt == CANDY_HIP_Q4_0) CANDY_BIG_256(BigQ4_0<false>);
-    if (fmt == CANDY_HIP_Q4_0_GGML) CANDY_BIG_256(BigQ4_0<true>);
-    // Q4_K. Up to 128 activation rows: 128 x 128 tiles, K split over workgroups to fill the chip
+// Tile shape by batch and grid.  Every format: 128 x 128 tiles up to 128 activation rows, 128 x 256 above.  Q4_K, whose
+// dequantization is the cheapest, also takes the narrower tiles on some grids above 128 rows (with the heavier formats
+// the producers then set the pace: Q6_K 14336 x 4096 at 192 rows 58.3 us on 128 x 128 tiles against 53.8, Q8_0 68.5
+// against 58.6), and tiles of 112 weight rows.
+template <class F>
+static int launch_shapes(candy_hip_device *dev, const F16Job *jobs, int count, const _Float16 *xh, int64_t m) {
     const int shape = dev->opt.f16_shape;  // comparison runs
+    const bool single = shape == 3;        // every wavefront in both roles
     // Tiles of 112 weight rows where every tensor's rows divide by 112 and the grid then takes fewer row-steps of its
     // busiest CU: rounds of workgroups x rows per tile x super-blocks per workgroup (14336 rows: 128 tiles instead of
     // 112, so 256 instead of 224 workgroups at 512 activation rows, 512 instead of 448 for a gate / up pair).
     auto narrow = [&](int bm) {
-        if (single || shape == 4) return false;
+        if (!std::is_same<F, BigQ4K>::value || single || shape == 4) return false;
         const int n_sb = (int)(jobs[0].w->cols >> 8), m_tiles = (int)((m + bm - 1) / bm);
         int64_t t112 = 0, t128 = 0;
         for (int s = 0; s < count; ++s) {
@@ -797,25 +799,40 @@ static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, con
         return cost(t112, 112) < cost(t128, 128);
     };
     auto small_tiles = [&]() {
-        if (single) return launch_big<BigQ4K, 128, 128, 2, 4>(dev, jobs, count, xh, m);
-        if (narrow(128)) return launch_big<BigQ4K, 112, 128, 2, 4, true>(dev, jobs, count, xh, m);
-        return launch_big<BigQ4K, 128, 128, 2, 4, true>(dev, jobs, count, xh, m);
+        if (single) return launch_big<F, 128, 128, 2, 4>(dev, jobs, count, xh, m);
+        if constexpr (std::is_same<F, BigQ4K>::value)
+            if (narrow(128)) return launch_big<F, 112, 128, 2, 4, true>(dev, jobs, count, xh, m);
+        return launch_big<F, 128, 128, 2, 4, true>(dev, jobs, count, xh, m);
     };
+    // up to 128 activation rows: 128 x 128 tiles, K split over workgroups to fill the chip
     if (shape == 2 || m <= 128) return small_tiles();
+    constexpr bool q4k = std::is_same<F, BigQ4K>::value;
     // up to 256 rows where the 128 x 128 tiles fill the chip and the 128 x 256 tiles would have to split K
-    // (14336 x 4096 at 256 rows: 70.7 us against 80.3)
+    // (Q4_K 14336 x 4096 at 256 rows: 70.7 us against 80.3)
     int64_t n128 = 0;
     for (int s = 0; s < count; ++s) n128 += (jobs[s].w->rows + 127) / 128;
     const int64_t fill = (3 * (int64_t)dev->num_cus) / 4;
-    if (m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill) return small_tiles();
+    if (q4k && m <= 256 && n128 * ((m + 127) / 128) >= fill && n128 * ((m + 255) / 256) < fill) return small_tiles();
     // short K (at most 16 super-blocks) on a grid that 128 x 256 tiles would have to split: 128 x 128 tiles halve the
-    // split as long as they still fit one round (4096 x 4096 at 512 rows 35.5 against 36.8 us, at 1024 rows 50.9 against
-    // 54.2; 6144 x 4096 at 512 rows 44.8 against 47.1; with K = 14336 the split is cheap and the wider tile wins)
-    if (shape == 0 && jobs[0].w->cols <= 4096 && n128 * ((m + 255) / 256) < fill && n128 * ((m + 127) / 128) <= dev->num_cus)
+    // split as long as they still fit one round (Q4_K 4096 x 4096 at 512 rows 35.5 against 36.8 us, at 1024 rows 50.9
+    // against 54.2; 6144 x 4096 at 512 rows 44.8 against 47.1; with K = 14336 the split is cheap and the wider tile wins)
+    if (q4k && shape == 0 && jobs[0].w->cols <= 4096 && n128 * ((m + 255) / 256) < fill && n128 * ((m + 127) / 128) <= dev->num_cus)
         return small_tiles();
-    if (narrow(256)) return launch_big<BigQ4K, 112, 256, 2, 4, true>(dev, jobs, count, xh, m);
-    CANDY_BIG_256(BigQ4K);
-#undef CANDY_BIG_256
+    if (single) return launch_big<F, 128, 256, 2, 4>(dev, jobs, count, xh, m);
+    if constexpr (std::is_same<F, BigQ4K>::value)
+        if (narrow(256)) return launch_big<F, 112, 256, 2, 4, true>(dev, jobs, count, xh, m);
+    return launch_big<F, 128, 256, 2, 4, true>(dev, jobs, count, xh, m);
+}
+
+static int launch_jobs(candy_hip_device *dev, const F16Job *jobs, int count, const _Float16 *xh, int64_t m) {
+    switch (jobs[0].w->fmt) {
+    case CANDY_HIP_Q6_K: return launch_shapes<BigQ6K>(dev, jobs, count, xh, m);
+    case CANDY_HIP_Q5_K: return launch_shapes<BigQ5K>(dev, jobs, count, xh, m);
+    case CANDY_HIP_Q8_0: return launch_shapes<BigQ8_0>(dev, jobs, count, xh, m);
+    case CANDY_HIP_Q4_0: return launch_shapes<BigQ4_0<false>>(dev, jobs, count, xh, m);
+    case CANDY_HIP_Q4_0_GGML: return launch_shapes<BigQ4_0<true>>(dev, jobs, count, xh, m);
+    default: return launch_shapes<BigQ4K>(dev, jobs, count, xh, m);
+    }
 }
 
 // xh: fp16 activations [mmq_m_pad(m)][K], rows past m zero.

@@ -83,7 +83,9 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   "mmq.min_m"                  16       batch from which tile kernels replace the matvec family (>= 16)
  *   "mmq.f16_big_min_m"          256      decoder prompt pass: batch from which fp16 big tiles (3e-4 per matmul) replace the
  *                                         exact int8 tiles (below it the pass holds the decode step's 1e-3 end to end)
- *   "mmq.f16_api_min_m"          96       the same for Q4_K through candy_hip_qmatmul / candy_hip_qmatmul_q8 (one matmul: 3e-4 < 1e-3)
+ *   "mmq.f16_api_min_m"          33       the same for one contraction through candy_hip_qmatmul / candy_hip_qmatmul_q8 (one
+ *                                         matmul: 3e-4 < 1e-3): Q4_K and Q6_K from this many rows, the other formats from 65
+ *                                         or this if larger
  *   -- comparison / test only --
  *   "matvec.span"                1        batch-1 kernel of 2-byte aligned formats fetches aligned 16-byte spans
  *   "matvec.small_batch_kernel"  1        2..8 rows on the one-workgroup-per-CU kernel (0: looping kernel)

@@ -48,23 +48,23 @@ def test_int8_tiles_are_integer_exact(dev, fmt, m, rows, cols):
     # rows off every 4/16/64 boundary, block counts off every stage length, m off every tile height
     w = synth.random_weight(fmt, rows, cols, seed=rows + m)
     x = synth.random_activations(m, cols, seed=cols + m)
-    # single Q4_K contractions move to the fp16 tiles from 96 rows on; here the int8 tiles are asked for up to the
+    # single Q4_K contractions move to the fp16 tiles from 33 rows on; here the int8 tiles are asked for up to the
     # decoder's threshold (what its prompt pass uses)
     dev.set_option("mmq.f16_api_min_m", 256)
     try:
         got = dev.qmatmul(dev.qtensor(fmt, rows, cols, w), x)
     finally:
-        dev.set_option("mmq.f16_api_min_m", 96)
+        dev.set_option("mmq.f16_api_min_m", 33)
     want = o.qmatmul(fmt, w, rows, cols, x)
     assert got.shape == (m, rows)
     # 256 activation rows or more run on the fp16 tiles (operands rounded to fp16)
     assert rel_err(got, want) <= (5e-4 if m >= 256 and fmt in (synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML) else 2e-5)
 
 
-@pytest.mark.parametrize("m", [96, 97, 100, 128, 129, 200, 255])
+@pytest.mark.parametrize("m", [33, 48, 64, 65, 96, 100, 128, 129, 200, 255])
 @pytest.mark.parametrize("rows,cols", [(1, 256), (127, 512), (129, 1024), (300, 2304), (1030, 768), (130, 4352)])
-def test_q4k_fp16_tiles_from_96_rows(dev, m, rows, cols):
-    # a single Q4_K contraction of 96 .. 255 rows: 128 x 128 tiles up to 128 rows, 128 x 256 above, K split over
+def test_q4k_fp16_tiles_from_33_rows(dev, m, rows, cols):
+    # a single Q4_K contraction of 33 .. 255 rows: 128 x 128 tiles up to 128 rows, 128 x 256 above, K split over
     # workgroups on small grids; fp16 operands (the bar of the big tiles), the same bits from call to call
     w = synth.random_weight(synth.Q4_K, rows, cols, seed=7 * rows + m)
     x = synth.random_activations(m, cols, seed=cols + 3 * m)
@@ -72,6 +72,24 @@ def test_q4k_fp16_tiles_from_96_rows(dev, m, rows, cols):
     got = dev.qmatmul(q, x)
     err = rel_err(got, o.qmatmul(synth.Q4_K, w, rows, cols, x))
     assert err <= 5e-4, err
+    assert np.array_equal(got, dev.qmatmul(q, x))
+
+
+@pytest.mark.parametrize("fmt", [synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML])
+@pytest.mark.parametrize("m", [33, 64, 65, 128, 129, 255])
+@pytest.mark.parametrize("rows,cols", [(127, 512), (300, 2304), (1030, 768)])
+def test_other_formats_fp16_tiles_from_65_rows(dev, fmt, m, rows, cols):
+    # a single contraction of the other formats: up to 64 rows one tile of the integer-exact kernel, from 65 rows the
+    # fp16 tiles (128 x 128 up to 128 rows), at their bar and not at the exact kernel's
+    w = synth.random_weight(fmt, rows, cols, seed=5 * rows + m + fmt)
+    x = synth.random_activations(m, cols, seed=cols + m)
+    q = dev.qtensor(fmt, rows, cols, w)
+    got = dev.qmatmul(q, x)
+    err = rel_err(got, o.qmatmul(fmt, w, rows, cols, x))
+    if m <= 64 and fmt != synth.Q6_K:  # Q6_K is on the fp16 tiles from 33 rows, like Q4_K
+        assert err <= 2e-5, err
+    else:
+        assert 2e-6 < err <= 5e-4, err
     assert np.array_equal(got, dev.qmatmul(q, x))
 
 
@@ -84,6 +102,7 @@ def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, 
     w = synth.random_weight(fmt, rows, cols, seed=rows + cols + fmt)
     q = dev.qtensor(fmt, rows, cols, w)
     dev.set_option("mmv.max_m", 0)  # 16 .. 32 rows of Q4_K on the tile kernel here, not on the one-pass kernel
+    dev.set_option("mmq.f16_api_min_m", 256)  # ... and 33 rows and more not on the fp16 tiles
     try:
         for m in (16, 24, 33, 64, 130):
             x = synth.random_activations(m, cols, seed=m * 7 + fmt)
@@ -99,6 +118,7 @@ def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, 
             assert rel_err(got, whole) <= 2e-6, m
     finally:
         dev.set_option("mmv.max_m", 32)
+        dev.set_option("mmq.f16_api_min_m", 33)
 
 
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0, synth.Q4_0_GGML])
@@ -219,18 +239,18 @@ def test_mixed_format_prefill_q6k_down_proj(dev, m):
 def test_batch_size_boundaries_agree_within_their_bars(dev):
     # Which kernel contracts depends on the number of activation rows.  Rows computed in a batch of one size and
     # again in a batch across the next boundary agree to f32 summation order where both kernels are integer-exact
-    # (2 | 3: vector | one-pass; 16 | 17: one tile | two tiles; 32 | 33: one-pass | int8 tiles) and to the
-    # fp16-operand bar across the fp16 threshold (95 | 96 for a single Q4_K contraction).
+    # (2 | 3: vector | one-pass; 16 | 17: one tile | two tiles) and to the fp16-operand bar across the fp16
+    # threshold (32 | 33 for a single Q4_K contraction).
     rows, cols = 512, 2048
     w = synth.random_weight(synth.Q4_K, rows, cols, seed=41)
     q = dev.qtensor(synth.Q4_K, rows, cols, w)
-    x = synth.random_activations(96, cols, seed=42)
+    x = synth.random_activations(33, cols, seed=42)
     want = o.qmatmul(synth.Q4_K, w, rows, cols, x)
-    for lo, hi, bar in ((2, 3, 2e-6), (16, 17, 2e-6), (32, 33, 2e-6), (95, 96, 1e-3)):
+    for lo, hi, bar in ((2, 3, 2e-6), (16, 17, 2e-6), (32, 33, 1e-3)):
         a, b = dev.qmatmul(q, x[:lo]), dev.qmatmul(q, x[:hi])
         d = rel_err(b[:lo], a.astype(np.float64))
         assert d <= bar, (lo, hi, d)
         assert rel_err(a, want[:lo]) <= 2e-5                      # below the threshold: exact kernels
-        assert rel_err(b, want[:hi]) <= (5e-4 if hi >= 96 else 2e-5)
-    a, b = dev.qmatmul(q, x[:95]), dev.qmatmul(q, x[:96])
-    assert rel_err(b[:95], a.astype(np.float64)) > 1e-6           # and it IS another kernel: not the same bits
+        assert rel_err(b, want[:hi]) <= (5e-4 if hi >= 33 else 2e-5)
+    a, b = dev.qmatmul(q, x[:32]), dev.qmatmul(q, x[:33])
+    assert rel_err(b[:32], a.astype(np.float64)) > 1e-6           # and it IS another kernel: not the same bits
