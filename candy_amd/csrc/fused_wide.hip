@@ -46,8 +46,13 @@ __device__ __forceinline__ int wide_start(int g, int total, int G) { return (int
 // The workgroup that item p falls to under wide_start.
 __device__ __forceinline__ int wide_owner(int p, int total, int G) { return (int)((((long long)p + 1) * G - 1) / total); }
 
+// Two workgroups of 8 wavefronts (or one of 16) per CU are four wavefronts per SIMD: 128 registers each.  The shapes
+// that hold up to eight rows of weights per lane are held to that (gate / up with four pairs per wavefront came to
+// 130 registers without it, one workgroup per CU at a time and two rounds: 22.5 us per launch on a 2 x 14336 x 4096
+// pair); the one-workgroup-per-CU shape with sixteen rows per lane keeps its 226.
 template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void k_matvec_wide(const WideArgs a) {
+__global__ __launch_bounds__(WAVES * 64, ((EPI == WEPI_PAIR ? 2 : 1) * R * ITER <= 8 ? 4 : 2))
+void k_matvec_wide(const WideArgs a) {
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;   // activation values the LDS image is sized for
     constexpr int XF = (CAP / 4 + T - 1) / T;   // float4 of prologue input per thread
