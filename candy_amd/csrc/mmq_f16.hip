@@ -543,6 +543,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
 
     // ---------------- consumers: wavefront cw owns the BN weight rows x activation rows [cw * BM / 4, + BM / 4)
     const int cw = wave - 4;
+    __builtin_amdgcn_s_setprio(3);
     float4v acc[TNF][TM];
 #pragma unroll
     for (int a = 0; a < TNF; ++a)
@@ -587,10 +588,15 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             const int ks = sb * 4 + g;
             const int anext = abuf == NB - 1 ? 0 : abuf + 1;
             const int acur = NB == 2 ? (g & 1) : abuf;  // two buffers: a constant of the unrolled body
-            load_b(min(ks + 1, steps - 1), (g + 1) & 1);  // the next step's activations, in flight during this one
-            if (!AHEAD) fetch(acur, 0);
+            const int ksn = min(ks + 1, steps - 1);  // the next step's activations, in flight during this one:
+            if (!AHEAD) fetch(acur, 0);               // a quarter of them requested in front of each phase
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
+#pragma unroll
+                for (int t = 0; t < TM / 2; ++t) {
+                    const int tm = (p & 1) * (TM / 2) + t;
+                    bf[(g + 1) & 1][p >> 1][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ksn * 2 + (p >> 1)) * 512);
+                }
                 // the next phase's weight fragments - after the last phase: the next step's first, whose buffer has
                 // been complete since the barrier before this step - are read while this phase multiplies
                 if (p < 3) fetch(acur, p + 1);
