@@ -106,6 +106,53 @@ struct BigQ4K {
         k0 = c * 8;
         k1 = 32 + c * 8;
     }
+    // The same in two parts for the kernel whose four neighbouring lanes hold the four quarters of one row: the scale
+    // and offset of group g are the same for all four, so lane c works out those of group c once per super-block
+    // (prepare) and each step fetches its group's from the lane that has them (four cross-lane moves instead of the
+    // unpacking and six multiplies).  The same operations on the same values as dequant(): the same bits.
+    struct Pre { float d_lo, d_hi16, c_lo, c_hi; };
+    __device__ static __forceinline__ void prepare(const Raw &r, int c, Pre &p) {
+        uint32_t sc2, m2;
+        q4k_scale_min_pair(r.hdr.y, r.hdr.z, r.hdr.w, c, sc2, m2);
+        const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
+        const float d_lo = d * (float)(sc2 & 0xFF), d_hi = d * (float)((sc2 >> 8) & 0xFF);
+        p.c_lo = fmaf(-1024.0f, d_lo, -(dmin * (float)(m2 & 0xFF)));
+        p.c_hi = fmaf(-64.0f, d_hi, -(dmin * (float)((m2 >> 8) & 0xFF)));
+        p.d_lo = d_lo;
+        p.d_hi16 = d_hi * 0.0625f;
+    }
+    __device__ static __forceinline__ float quad_lane(float v, int g) {  // the value lane g of this lane's quad holds
+        switch (g) {
+        case 0: return dpp_move<0x00>(v);
+        case 1: return dpp_move<0x55>(v);
+        case 2: return dpp_move<0xAA>(v);
+        default: return dpp_move<0xFF>(v);
+        }
+    }
+    __device__ static __forceinline__ void dequant_pre(const Raw &r, const Pre &p, int g, int c, half8 &o0, half8 &o1,
+                                                       int &k0, int &k1) {
+        const float d_lo = quad_lane(p.d_lo, g), d_hi16 = quad_lane(p.d_hi16, g);
+        const float c_lo = quad_lane(p.c_lo, g), c_hi = quad_lane(p.c_hi, g);
+        const u32x2 q = r.q[g];
+        const uint32_t MAGIC = 0x64006400u, LO = 0x000F000Fu, HI = 0x00F000F0u;
+#pragma unroll
+        for (int wi = 0; wi < 2; ++wi) {
+            const uint32_t w = wi ? q.y : q.x, w8 = w >> 8;
+            const half2v l02 = bits_h2(and_or(w, LO, MAGIC)), l13 = bits_h2(and_or(w8, LO, MAGIC));
+            const half2v h02 = bits_h2(and_or(w, HI, MAGIC)), h13 = bits_h2(and_or(w8, HI, MAGIC));
+            o0[4 * wi + 0] = (_Float16)fmaf((float)l02[0], d_lo, c_lo);
+            o0[4 * wi + 1] = (_Float16)fmaf((float)l13[0], d_lo, c_lo);
+            o0[4 * wi + 2] = (_Float16)fmaf((float)l02[1], d_lo, c_lo);
+            o0[4 * wi + 3] = (_Float16)fmaf((float)l13[1], d_lo, c_lo);
+            o1[4 * wi + 0] = (_Float16)fmaf((float)h02[0], d_hi16, c_hi);
+            o1[4 * wi + 1] = (_Float16)fmaf((float)h13[0], d_hi16, c_hi);
+            o1[4 * wi + 2] = (_Float16)fmaf((float)h02[1], d_hi16, c_hi);
+            o1[4 * wi + 3] = (_Float16)fmaf((float)h13[1], d_hi16, c_hi);
+        }
+        k0 = c * 8;
+        k1 = 32 + c * 8;
+    }
 };
 
 // Q5_K: Q4_K's layout with 32 bytes of fifth bits between the header and the nibbles (quantized.cu:1044-1080):
@@ -260,6 +307,18 @@ struct BigQ6K {
 // ------------------------------------------------------------------ tile kernel
 // One launch may serve up to three weight tensors that share the activations (q / k / v of a prompt pass): weight
 // tiles [tile0, next tile0) belong to segment s, which has its own weights, row count, output and residual.
+// Whether a policy offers the two-part dequantization (Pre, prepare, dequant_pre)
+template <class F, class = void>
+struct F16Pre {
+    struct type {};
+    static constexpr bool value = false;
+};
+template <class F>
+struct F16Pre<F, std::void_t<typename F::Pre>> {
+    typedef typename F::Pre type;
+    static constexpr bool value = true;
+};
+
 struct F16Seg {
     const uint8_t *W;
     float *out;
@@ -451,7 +510,9 @@ __global__ __launch_bounds__(WN * WM * 64) void k_mmq_f16(const F16Group grp, co
 //   alone: moving a step's 32 KB of activations into the CU costs 700 to 950 cycles whichever wavefronts do it, and
 //   LDS carried 144 KB per step (now 80 KB: 16 KB of weight tile written, 4 x 16 KB read).
 // A consumer walks a step in four phases (two halves of K x two halves of the weight rows) of 16 or 8 matrix
-// instructions, reading the next phase's four weight fragments from LDS while the current phase's instructions run.
+// instructions, reading the next phase's four weight fragments from LDS and requesting a quarter of the next step's
+// activation fragments while the current phase's instructions run; it runs at raised priority, so that its matrix
+// instruction goes ahead of a producer's vector instruction when both are ready.
 // The two roles are separate loops with the same number of barriers, so that their registers (accumulators and
 // operand fragments here, raw blocks there) share one allocation.
 // BN = 112 (seven 16-row fragments: the second half of the weight rows is three fragments instead of four) is for
@@ -499,6 +560,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
     if (wave < 4) {
         // ---------------- producers: the weight tile of step t + LEAD (buffer (t + LEAD) % NB) while step t is contracted
         typename F::Raw raw[2][ATK];
+        typename F16Pre<F>::type pre[2][ATK];
         // neighbouring lanes take neighbouring quarters of a row; a half-wavefront takes rows {x, x+4, x+8, x+12}
         const int a_c = lane & 3, a_row = 16 * wave + 4 * ((lane >> 2) & 3) + (lane >> 4);   // + a_step i
         const int a_step = BN == 112 && wave == 3 ? 0 : 64;
@@ -513,7 +575,12 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             for (int i = 0; i < ATK; ++i) {
                 half8 o0, o1;
                 int k0, k1;
-                F::dequant(raw[aslot][i], g, a_c, o0, o1, k0, k1);
+                if constexpr (F16Pre<F>::value) {
+                    if (g == 0) F::prepare(raw[aslot][i], a_c, pre[aslot][i]);  // a super-block's first step
+                    F::dequant_pre(raw[aslot][i], pre[aslot][i], g, a_c, o0, o1, k0, k1);
+                } else {
+                    F::dequant(raw[aslot][i], g, a_c, o0, o1, k0, k1);
+                }
                 *(half8 *)&a[frag_off(a_row + a_step * i, k0)] = o0;
                 *(half8 *)&a[frag_off(a_row + a_step * i, k1)] = o1;
             }
@@ -560,22 +627,27 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             for (int tm = 0; tm < TM; ++tm)
                 bf[slot][kk][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ks * 2 + kk) * 512);
     };
-    half8 af[2][4];
-    // phase p = 2 * kk + h of a step: weight rows 64 h .. min(64 h + 63, BN - 1), values 32 kk .. 32 kk + 31
+    // A step is four phases, phase p = 2 * kk + h: weight rows 64 h .. min(64 h + 63, BN - 1), values 32 kk .. 32 kk + 31
+    // (two phases of all the weight rows for the 128-row tiles, whose phases have 8 matrix instructions: 34.4 against
+    // 33.8 us at 14336 x 4096 x 128; eight producer wavefronts for them: 33.6 against 33.0)
+    constexpr int PH = 4, HN = 4;  // phases per step, weight fragments per phase
+    half8 af[2][HN];
     auto fetch = [&](int abuf, int p) __attribute__((always_inline)) {
         const _Float16 *a = sA + abuf * BNB * BIG_BK + frag_lane_off(lane);
+        const int kk = PH == 4 ? p >> 1 : p, t0 = PH == 4 ? (p & 1) * 4 : 0;
 #pragma unroll
-        for (int tn = 0; tn < 4; ++tn)
-            if ((p & 1) * 4 + tn < TNF) af[p & 1][tn] = *(const half8 *)&a[(((p & 1) * 4 + tn) * 2 + (p >> 1)) * 512];
+        for (int tn = 0; tn < HN; ++tn)
+            if (t0 + tn < TNF) af[p & 1][tn] = *(const half8 *)&a[((t0 + tn) * 2 + kk) * 512];
     };
     auto mma = [&](int bslot, int p) __attribute__((always_inline)) {
+        const int kk = PH == 4 ? p >> 1 : p, t0 = PH == 4 ? (p & 1) * 4 : 0;
 #pragma unroll
-        for (int tn = 0; tn < 4; ++tn)
+        for (int tn = 0; tn < HN; ++tn)
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm)
-                if ((p & 1) * 4 + tn < TNF)
-                    acc[(p & 1) * 4 + tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        af[p & 1][tn], bf[bslot][p >> 1][tm], acc[(p & 1) * 4 + tn][tm], 0, 0, 0);
+                if (t0 + tn < TNF)
+                    acc[t0 + tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[p & 1][tn], bf[bslot][kk][tm],
+                                                                            acc[t0 + tn][tm], 0, 0, 0);
     };
     load_b(0, 0);
     __syncthreads();  // the weight tiles of the first LEAD steps are in LDS
@@ -591,15 +663,15 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             const int ksn = min(ks + 1, steps - 1);  // the next step's activations, in flight during this one:
             if (!AHEAD) fetch(acur, 0);               // a quarter of them requested in front of each phase
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
+            for (int p = 0; p < PH; ++p) {
 #pragma unroll
-                for (int t = 0; t < TM / 2; ++t) {
-                    const int tm = (p & 1) * (TM / 2) + t;
-                    bf[(g + 1) & 1][p >> 1][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ksn * 2 + (p >> 1)) * 512);
+                for (int t = 0; t < 2 * TM / PH; ++t) {
+                    const int l = p * (2 * TM / PH) + t, kk = l / TM, tm = l % TM;
+                    bf[(g + 1) & 1][kk][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ksn * 2 + kk) * 512);
                 }
                 // the next phase's weight fragments - after the last phase: the next step's first, whose buffer has
                 // been complete since the barrier before this step - are read while this phase multiplies
-                if (p < 3) fetch(acur, p + 1);
+                if (p < PH - 1) fetch(acur, p + 1);
                 else if (AHEAD) fetch(anext, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 mma(g & 1, p);
