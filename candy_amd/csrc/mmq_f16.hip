@@ -841,7 +841,7 @@ bool mmq_f16_big_covers(const candy_hip_qtensor *w, int64_t m, int min_m) {
     // (4096 x 4096 22.4 / 22.6), at 96 rows 77.8 / 44.7, at 255 rows 121 / 61; Q4_0 at 48 rows 38.9 / 38.0 (4096 x 4096
     // 19.9 / 22.4), at 96 rows 64.3 / 48.7; Q5_K 36.9 / 35.1 (19.9 / 19.9) and 58.6 / 47.2.
     if (min_m <= 0) min_m = w->dev->opt.f16_big_min_m;
-    else if (w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K) min_m = std::min(std::max(min_m, 65), w->dev->opt.f16_big_min_m);
+    else if (w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K) min_m = std::max(min_m, 65);
     if (m < min_m || w->cols % 256 != 0) return false;
     if (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q5_K) return ((uintptr_t)w->data & 15) == 0;
     if (w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q8_0 || w->fmt == CANDY_HIP_Q4_0 || w->fmt == CANDY_HIP_Q4_0_GGML)

@@ -93,6 +93,22 @@ def test_other_formats_fp16_tiles_from_65_rows(dev, fmt, m, rows, cols):
     assert np.array_equal(got, dev.qmatmul(q, x))
 
 
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K, synth.Q5_K, synth.Q8_0, synth.Q4_0])
+def test_single_contractions_stay_exact_on_request(dev, fmt):
+    # "mmq.f16_api_min_m" = 1 << 30 keeps candy_hip_qmatmul on the integer-exact kernels at every batch size
+    rows, cols, m = 300, 1024, 400
+    w = synth.random_weight(fmt, rows, cols, seed=fmt + 1)
+    x = synth.random_activations(m, cols, seed=fmt + 2)
+    q = dev.qtensor(fmt, rows, cols, w)
+    want = o.qmatmul(fmt, w, rows, cols, x)
+    assert rel_err(dev.qmatmul(q, x), want) > 2e-6  # by default: fp16 tiles
+    dev.set_option("mmq.f16_api_min_m", 1 << 30)
+    try:
+        assert rel_err(dev.qmatmul(q, x), want) <= 2e-6
+    finally:
+        dev.set_option("mmq.f16_api_min_m", 33)
+
+
 @pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q6_K])
 @pytest.mark.parametrize("rows,cols", [(200, 11008), (64, 4352), (1000, 2560)])
 def test_int8_tiles_split_the_contraction_on_small_grids(dev, monkeypatch, fmt, rows, cols):
