@@ -619,7 +619,10 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
     // activation fragment (16-row block rbk of the tile, 32-value block kb of K): 1 KB at ((m0 / 16 + rbk) * (K / 32) + kb)
     // * 1 KB; lane l takes row l & 15, values 8 (l >> 4) .. + 7: the wavefront's 64 loads cover the fragment once
     const _Float16 *xfrag = xh + ((size_t)((m0 >> 4) + cw * TM) * (K >> 5)) * 512 + (lane & 15) * 32 + (lane >> 4) * 8;
-    half8 bf[2][2][TM];  // [step parity][half of the step][fragment]
+    // steps the activation loads run ahead, and register slots for them: two steps for the 128-row tiles, whose steps
+    // are shorter than a load from L2 under this traffic takes (14336 x 4096 x 128: 31.5 us; one step 32.2, three 32.6)
+    constexpr int BD = BM == 128 ? 2 : 1, NS = 2 * BD;
+    half8 bf[NS][2][TM];  // [step % NS][half of the step][fragment]
     auto load_b = [&](int ks, int slot) __attribute__((always_inline)) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
@@ -650,6 +653,7 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
                                                                             acc[t0 + tn][tm], 0, 0, 0);
     };
     load_b(0, 0);
+    if (BD == 2) load_b(min(1, steps - 1), 1);
     __syncthreads();  // the weight tiles of the first LEAD steps are in LDS
     constexpr bool AHEAD = LEAD == 2;
     if (AHEAD) fetch(0, 0);
@@ -660,21 +664,21 @@ __global__ __launch_bounds__(512) void k_mmq_f16_pc(const F16Group grp, const _F
             const int ks = sb * 4 + g;
             const int anext = abuf == NB - 1 ? 0 : abuf + 1;
             const int acur = NB == 2 ? (g & 1) : abuf;  // two buffers: a constant of the unrolled body
-            const int ksn = min(ks + 1, steps - 1);  // the next step's activations, in flight during this one:
+            const int ksn = min(ks + BD, steps - 1);  // a later step's activations, in flight during this one:
             if (!AHEAD) fetch(acur, 0);               // a quarter of them requested in front of each phase
 #pragma unroll
             for (int p = 0; p < PH; ++p) {
 #pragma unroll
                 for (int t = 0; t < 2 * TM / PH; ++t) {
                     const int l = p * (2 * TM / PH) + t, kk = l / TM, tm = l % TM;
-                    bf[(g + 1) & 1][kk][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ksn * 2 + kk) * 512);
+                    bf[(g + BD) & (NS - 1)][kk][tm] = *(const half8 *)(xfrag + ((size_t)tm * (K >> 5) + (size_t)ksn * 2 + kk) * 512);
                 }
                 // the next phase's weight fragments - after the last phase: the next step's first, whose buffer has
                 // been complete since the barrier before this step - are read while this phase multiplies
                 if (p < PH - 1) fetch(acur, p + 1);
                 else if (AHEAD) fetch(anext, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                mma(g & 1, p);
+                mma(g & (NS - 1), p);
                 __builtin_amdgcn_sched_barrier(0);
             }
             abuf = anext;
