@@ -276,10 +276,12 @@ __global__ __launch_bounds__(HD) void k_attn_merge(const float *__restrict__ par
 }
 
 int attention_splits(const candy_hip_device *dev, int64_t n_kv_heads, int64_t max_pos) {
-    // enough workgroups to fill the chip a few times over, at least 64 positions per split,
-    // at most 64 splits (the merge kernel gives each split a lane)
+    // enough workgroups to fill the chip a few times over (twice as many measured slower: 7B shape at 2048 positions
+    // 531 against 539 tokens/s), at least 32 positions per split - one batch of rows per wavefront (Llama-3-8B shape at
+    // 512-640 positions: 503 tokens/s against 489 with 64 and 491 with 16) -, at most 64 splits (the merge kernel
+    // gives each split a lane)
     int n_splits = (int)((4 * (int64_t)dev->num_cus + n_kv_heads - 1) / n_kv_heads);
-    const int max_splits = (int)((max_pos + 63) / 64);
+    const int max_splits = (int)((max_pos + 31) / 32);
     if (n_splits > max_splits) n_splits = max_splits;
     if (n_splits > 64) n_splits = 64;
     return n_splits < 1 ? 1 : n_splits;
