@@ -289,6 +289,11 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
             const int per2 = (a.total + 2 * cus - 1) / (2 * cus);
             if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
             if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+            // four pairs per wavefront need every register: three workgroups of three pairs per CU instead, the third
+            // starting when the first is done (2 x 14336 x 4096: 508 against 502 tokens/s on the Llama-3-8B shape; the
+            // same step from three pairs to two loses, 509 against 539 on the 7B shape: more blocks are shared)
+            if (per2 <= 32 && (a.total + 3 * cus - 1) / (3 * cus) <= 24)
+                return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 3 * cus);
             if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
         }
         if (iter == 1) {

@@ -245,12 +245,14 @@ def test_full_depth_7b_step_within_activation_noise(dev):
     model.free()
 
 
-def test_long_cache_step_on_the_even_split_kernels(dev):
+@pytest.mark.parametrize("d_ffn", [11008, 14336])
+def test_long_cache_step_on_the_even_split_kernels(dev, d_ffn):
     # One full-width 7B layer over a cache of 600 positions with q/k/v and gate/up on the kernels that deal the rows
-    # evenly over the CUs (two workgroups of eight wavefronts per CU, or one of sixteen), against the CPU composition
+    # evenly over the CUs (two workgroups of eight wavefronts per CU, or one of sixteen; three of eight for the 14336
+    # pairs of the wider FFN, where a 32-value block can belong to three workgroups), against the CPU composition
     # and against the same step on the narrower kernels (the RMS sum runs in another order, so not the same bits).
     n_pos = 600
-    cfg = dict(n_layers=1, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=11008, vocab=512,
+    cfg = dict(n_layers=1, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=d_ffn, vocab=512,
                max_pos=n_pos + 8, rms_eps=1e-5, rope_base=10000.0)
     fmts = {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}
     host, model = build(dev, cfg, fmts, seed=91)
@@ -570,7 +572,7 @@ def test_prompt_chunks_on_either_side_of_the_fp16_threshold(dev):
     assert 0 < rel(kb[0, :, :255], ka[0, :, :255].astype(np.float64)) <= 1e-3
 
 
-@pytest.mark.parametrize("d_ffn", [11008, 1024 + 256])
+@pytest.mark.parametrize("d_ffn", [11008, 14336, 1024 + 256])
 def test_gate_up_block_parts_give_the_same_bits(dev, monkeypatch, d_ffn):
     # the fused gate/up kernel lets a workgroup own a whole 32-value block of the FFN activation or a half / quarter
     # of one (whichever divides the rows evenly over the CUs); the block is quantized from the same 32 f32 values
