@@ -276,11 +276,14 @@ static int norm_linear(candy_hip_llama *m, const float *alpha, const candy_hip_q
     Wd.x = m->h; Wd.alpha = alpha; Wd.eps = c.rms_eps;
     rc = launch_matvec_wide(m->dev, Wd);
     if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
+    // a vocabulary-sized Q6_K head: the norm as a launch of its own and the batch-1 kernel stream the rows faster than
+    // the fused kernel, whose thousands of workgroups each repeat the prologue
+    const bool plain_head = n == 1 && ws[0]->fmt == CANDY_HIP_Q6_K && ws[0]->rows >= 16384;
     FusedLaunch F;
     F.n = n;
     for (int i = 0; i < n; ++i) { F.w[i] = ws[i]; F.y[i] = ys[i]; }
     F.x = m->h; F.alpha = alpha; F.eps = c.rms_eps;
-    rc = launch_matvec_fused(m->dev, F);
+    rc = plain_head ? CANDY_HIP_ERR_UNSUPPORTED : launch_matvec_fused(m->dev, F);
     if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
     if ((rc = launch_rms_norm_quant(m->dev, m->h, alpha, c.rms_eps, 1, c.d_model, nullptr, m->xq, m->xs))) return rc;
     return launch_matvec_multi(m->dev, ws, ys, nullptr, n, m->xq, m->xs);
