@@ -715,9 +715,13 @@ int act_workspace(candy_hip_device *dev, int64_t m, int64_t cols, bool need_quan
 int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_t *qs, const Q8Scale *scales,
                   int64_t m, float *y, bool vector_only) {
     CANDY_REQUIRE(w->rows <= 0x7FFFFFFF && w->cols <= 0x7FFFFFFF, "matrix too large");
-    // the 32-value formats: the vector kernels match the tile kernel up to 8 rows (one pass); from 9 rows on they need two
-    if (!vector_only && m >= 9 && w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K && w->fmt != CANDY_HIP_Q5_K &&
-        dev->opt.i8_min_m == 0 && mmq_i8_covers(w, qs))
+    // the 32-value formats: the vector kernels match the tile kernel up to 8 rows (one pass) on small weights; from 9
+    // rows on they need two passes, and on weights of 40 M values and more the tile kernel is level or ahead from 5 rows
+    // (us per call, 5-8 rows on the vector kernels / 9 rows on the tiles: Q8_0 32000 x 4096 50.5-51.4 / 46.3, 4096 x 11008
+    // 26 / 25.3; Q4_0 32000 x 4096 49.2-50.3 / 40.2, 4096 x 11008 24.8-25.9 / 23.1; but 4096 x 4096 13.4-15.0 / 15.1)
+    const bool big_weight = (double)w->rows * (double)w->cols >= 4.0e7;
+    if (!vector_only && (m >= 9 || (m >= 5 && big_weight)) && w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K &&
+        w->fmt != CANDY_HIP_Q5_K && dev->opt.i8_min_m == 0 && mmq_i8_covers(w, qs))
         return launch_mmq_i8(dev, w, qs, scales, m, y);
     if (!vector_only && m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q5_K) && mmq_i8_covers(w, qs)) {
         // 5 .. 15 rows: the vector kernels below (one or two passes of up to 8 rows) or one pass of the int8 tile

@@ -103,6 +103,28 @@ def test_two_rows_even_split_kernel(dev, rows, cols):
     assert rel_err(got[:, sub], o.qmatmul(synth.Q4_K, wsub, len(sub), cols, x)) <= 2e-5
 
 
+@pytest.mark.parametrize("fmt", [synth.Q8_0, synth.Q4_0, synth.Q5_1])
+def test_five_to_eight_rows_on_a_big_weight_take_the_tile_kernel(dev, fmt):
+    # 32-value formats, weights of 40 M values and more: 5 .. 8 rows run on the int8 tile kernel (integer-exact, like
+    # the vector kernels they replace there: the two differ by f32 summation order only)
+    rows, cols = 4096, 11008
+    w = synth.random_weight(fmt, rows, cols, seed=fmt + 50)
+    q = dev.qtensor(fmt, rows, cols, w)
+    sub = np.arange(3, rows, 61)
+    wsub = w.reshape(rows, -1)[sub].reshape(-1)
+    for m in (5, 8):
+        x = synth.random_activations(m, cols, seed=m + fmt)
+        got = dev.qmatmul(q, x)
+        assert rel_err(got[:, sub], o.qmatmul(fmt, wsub, len(sub), cols, x)) <= 2e-5, m
+        try:
+            dev.set_option("mmq.i8_min_m", 99)  # the vector kernels
+            vector = dev.qmatmul(q, x)
+        finally:
+            dev.set_option("mmq.i8_min_m", 0)
+        assert rel_err(got, vector) <= 2e-6, m
+        assert not np.array_equal(got, vector), m  # another kernel did run
+
+
 def test_config_q4_0_4096x4096(dev):
     # the single-QMatMul configuration: Q4_0 4096x4096, one f32 N(0,1) vector, seeded
     rows = cols = 4096
