@@ -723,20 +723,34 @@ int launch_matvec(candy_hip_device *dev, const candy_hip_qtensor *w, const int8_
     if (!vector_only && (m >= 9 || (m >= 5 && big_weight)) && w->fmt != CANDY_HIP_Q4_K && w->fmt != CANDY_HIP_Q6_K &&
         w->fmt != CANDY_HIP_Q5_K && dev->opt.i8_min_m == 0 && mmq_i8_covers(w, qs))
         return launch_mmq_i8(dev, w, qs, scales, m, y);
-    if (!vector_only && m >= 5 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q5_K) && mmq_i8_covers(w, qs)) {
-        // 5 .. 15 rows: the vector kernels below (one or two passes of up to 8 rows) or one pass of the int8 tile
-        // kernel with a 16-row tile, whichever a fit to measurements on this chip says is shorter, in us.  The tile
-        // kernel's time hardly depends on m: Q4_K 4096x4096 12.7, 11008x4096 19.6, 4096x11008 19.3, 32000x4096 31.5;
-        // Q6_K 14.0, 23.2, 21.5, 41.3 (short rows: a few us per super-block); the vector kernels' follows rows x
-        // columns x batch.
-        const bool q6 = w->fmt != CANDY_HIP_Q4_K;  // Q6_K and Q5_K: the looping vector kernel, a heavier tile
+    if (!vector_only && m >= 3 && (w->fmt == CANDY_HIP_Q4_K || w->fmt == CANDY_HIP_Q6_K || w->fmt == CANDY_HIP_Q5_K) && mmq_i8_covers(w, qs)) {
+        // 3 .. 15 rows: the vector kernels below or one pass of the int8 tile kernel with a 16-row tile, whichever a
+        // fit to measurements on this chip says is shorter, in us.  The tile kernel's time hardly depends on m: Q4_K
+        // 4096x4096 12.7, 11008x4096 19.6, 4096x11008 19.3, 32000x4096 31.5; Q6_K 10.9, 20.8, 19.0, 38.3, 4096x14336
+        // 22.0, 128256x4096 132 (short rows: a few us per super-block).  Q6_K and Q5_K have only the looping vector
+        // kernel, which takes 8, 4, 2 or 1 activation rows per launch the longer the weight rows are and costs their
+        // padded count: 0.07 us per M values and image with rows of up to 5632 values, 0.105 beyond (Q6_K at 3 / 5 rows:
+        // 4096x4096 9.2 / 15.1, 11008x4096 16.8 / 31.5, 4096x11008 22.6 / 33.8, 32000x4096 39.7 / 77.5, 4096x14336
+        // 33.8 / 51.2, 128256x4096 151 / 273).
+        const bool q6 = w->fmt != CANDY_HIP_Q4_K;
         const double nsb = (double)(w->cols >> 8), mnk = (double)w->rows * (double)w->cols * 1e-6;
-        const int m_pad = q6 ? (int)m : (int)((m + 3) / 4 * 4);
-        const double t_tiles = q6 ? std::min(3.5 + 2.5 * nsb * (1.0 + mnk / 40.0), 11.5 + 0.23 * mnk)
-                                  : std::min(3.5 + 2.0 * nsb * (1.0 + mnk / 40.0), 11.0 + 0.16 * mnk);
-        const double t_vector = 4.0 + (m > 8 ? 2.0 : 0.0) + (q6 ? 0.1 : 0.052) * mnk * m_pad;
+        double t_tiles, t_vector;
+        if (q6) {
+            t_tiles = std::min(3.5 + 2.5 * nsb * (1.0 + mnk / 40.0), 7.0 + 0.24 * mnk);
+            const double per_image = (w->cols > 5632 ? 0.105 : 0.07) * mnk;
+            t_vector = 0.0;
+            for (int64_t left = m; left > 0;) {
+                const int nb = looping_rows(left, w->cols);
+                t_vector += 4.0 + per_image * nb;
+                left -= std::min<int64_t>(left, nb);
+            }
+        } else {
+            const int m_pad = (int)((m + 3) / 4 * 4);
+            t_tiles = std::min(3.5 + 2.0 * nsb * (1.0 + mnk / 40.0), 11.0 + 0.16 * mnk);
+            t_vector = m < 5 ? 0.0 : 4.0 + (m > 8 ? 2.0 : 0.0) + 0.052 * mnk * m_pad;  // Q4_K, 3 and 4 rows: vector
+        }
         const int from = dev->opt.i8_min_m;  // comparison runs: tiles from this batch size on
-        if (from ? m >= from : t_tiles < t_vector) return launch_mmq_i8(dev, w, qs, scales, m, y);
+        if (from ? m >= std::max(from, 3) : t_tiles < t_vector) return launch_mmq_i8(dev, w, qs, scales, m, y);
     }
     switch (w->fmt) {
     case CANDY_HIP_Q4_K: return launch_fmt<UnitQ4K>(dev, w, qs, scales, m, y);
