@@ -125,6 +125,28 @@ def test_five_to_eight_rows_on_a_big_weight_take_the_tile_kernel(dev, fmt):
         assert not np.array_equal(got, vector), m  # another kernel did run
 
 
+@pytest.mark.parametrize("fmt", [synth.Q6_K, synth.Q5_K])
+def test_three_and_four_rows_on_long_weight_rows_take_the_tile_kernel(dev, fmt):
+    # Q6_K / Q5_K with weight rows so long that the looping kernel holds one or two activation rows per launch:
+    # 3 and 4 rows run as one 16-row int8 tile; on 4096-long weight rows the vector kernel keeps them
+    for rows, cols, tiles in ((4096, 14336, True), (1024, 4096, False)):
+        w = synth.random_weight(fmt, rows, cols, seed=fmt + 70)
+        q = dev.qtensor(fmt, rows, cols, w)
+        sub = np.arange(5, rows, 67)
+        wsub = w.reshape(rows, -1)[sub].reshape(-1)
+        for m in (3, 4):
+            x = synth.random_activations(m, cols, seed=m + fmt + cols)
+            got = dev.qmatmul(q, x)
+            assert rel_err(got[:, sub], o.qmatmul(fmt, wsub, len(sub), cols, x)) <= 2e-5, (cols, m)
+            try:
+                dev.set_option("mmq.i8_min_m", 99)  # the vector kernels
+                vector = dev.qmatmul(q, x)
+            finally:
+                dev.set_option("mmq.i8_min_m", 0)
+            assert rel_err(got, vector) <= 2e-6, (cols, m)
+            assert np.array_equal(got, vector) != tiles, (cols, m)
+
+
 def test_config_q4_0_4096x4096(dev):
     # the single-QMatMul configuration: Q4_0 4096x4096, one f32 N(0,1) vector, seeded
     rows = cols = 4096
