@@ -66,6 +66,7 @@ struct Options {
     int mmv_variant = 0;         // comparison runs: 1 = one 16-row strip per wavefront, 2 = two
     int pair_rows = 0;           // fused gate/up: row pairs per workgroup, 32 / 16 / 8 (0: the most even split)
     int rms_rows = 0;            // fused RMSNorm prologue: rows per workgroup, 16 / 24 (0: the most even split)
+    int prefill_split_norm = 1;      // prompt pass: split-K copies of o / down summed inside the following norm launch
     int prefill_qkv_group = 1;       // prompt pass: q / k / v (and gate / up) on one grid each where they run on the fp16 tiles
     int prefill_attention_valu = 0;  // prompt attention for head_dim 128 on the vector ALU instead of the matrix cores
     int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
@@ -73,6 +74,17 @@ struct Options {
     int wide_waves = 8;          // wavefronts per workgroup of those kernels: 8 (two workgroups per CU) or 16 (one)
 };
 
+}  // namespace candy
+
+namespace candy {
+// y = res + (part[0] + part[1] + ...), `count` floats, copies `stride` floats apart: a split sum not yet launched
+struct SplitPending {
+    const float *part = nullptr;
+    float *y = nullptr;
+    const float *res = nullptr;
+    size_t count = 0, stride = 0;
+    int n_split = 0;  // 0: nothing pending
+};
 }  // namespace candy
 
 struct candy_hip_device {
@@ -91,6 +103,9 @@ struct candy_hip_device {
     // One word of pinned host memory that kernels raise when they meet an index outside its table (the condition
     // the CPU path panics on); check_fault() reports and clears it after a synchronisation.
     int *fault = nullptr;
+    // While this points at a record, a single fp16-tile contraction that splits K leaves its partial copies unsummed
+    // and describes them there; the caller's next launch adds them up (the prompt pass: inside its norm kernel).
+    candy::SplitPending *defer_split = nullptr;
     // This GPU's copy of the library's file-scope scratch array (matvec.hip), resolved when the handle is opened.
     void *noalloc_scratch = nullptr;
 };
@@ -140,7 +155,11 @@ int workspace(candy_hip_device *dev, size_t bytes, void **out);
 // Second buffer, for the split-K partial sums (lives beside the activation workspace).
 int splitk_workspace(candy_hip_device *dev, size_t bytes, void **out);
 // mmq_f16.hip: y[i] = (res[i] +) part[0][i] + part[1][i] + ... in that order (count floats per part)
-int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split);
+int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split,
+                      size_t stride = 0);  // copies `stride` floats apart (0: count)
+// ops.hip: the pending sum, the residual add, RMSNorm and Q8_0 quantization of the rows in one launch
+int launch_split_rms_norm_quant(candy_hip_device *dev, const SplitPending &sp, const float *alpha, float eps, int64_t rows,
+                                int64_t cols, int8_t *qs, Q8Scale *scales, _Float16 *xh);
 // Formats the batch-1 kernel contracts (residual epilogue, several weights per launch): all that have a vec-dot.
 // The fused decode kernels exist for Q4_K, Q6_K, Q8_0 and the two Q4_0 orders only.
 inline bool format_has_batch1_kernel(int fmt) {

@@ -454,6 +454,16 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
     const float scale = 1.0f / std::sqrt((float)c.head_dim);
     int rc;
     if ((rc = candy_hip_qindex_select(dev, m->embed, P.ids, n, P.h))) return rc;
+    // An o / down projection that splits K leaves its partial copies for the norm launch that follows, which sums them,
+    // adds the residual and writes P.h before it normalizes (one launch and one pass over P.h less each time).
+    SplitPending pend;
+    auto norm_quant = [&](const float *alpha, _Float16 *xh_out) -> int {
+        const int e = pend.n_split > 0
+                          ? launch_split_rms_norm_quant(dev, pend, alpha, c.rms_eps, n, c.d_model, P.xq, P.xs, xh_out)
+                          : launch_rms_norm_quant(dev, P.h, alpha, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs, xh_out);
+        pend.n_split = 0;
+        return e;
+    };
     for (int l = 0; l < c.n_layers; ++l) {
         const candy_hip_llama::Layer &L = m->layers[l];
         void *kc = layer_cache(m, m->k_cache, l), *vc = layer_cache(m, m->v_cache, l);
@@ -462,12 +472,17 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
         // projection's epilogue.
         auto xh_for = [&](const candy_hip_qtensor *w) { return mmq_f16_big_covers(w, n) ? P.xh : nullptr; };
         auto add_linear = [&](const candy_hip_qtensor *w) -> int {  // P.h += (quantized activations) . w^T
-            if (mmq_fuses_residual(w, n)) return launch_contract(dev, w, P.xq, P.xs, n, P.h, xh_for(w), P.h);
+            if (mmq_fuses_residual(w, n)) {
+                dev->defer_split = &pend;
+                const int e = launch_contract(dev, w, P.xq, P.xs, n, P.h, xh_for(w), P.h);
+                dev->defer_split = nullptr;
+                return e;
+            }
             if (int e = launch_contract(dev, w, P.xq, P.xs, n, P.tmp)) return e;
             return candy_hip_add(dev, P.h, P.tmp, (int64_t)n * c.d_model, P.h);
         };
         _Float16 *xh = (xh_for(L.wq) || xh_for(L.wk) || xh_for(L.wv)) ? P.xh : nullptr;
-        if ((rc = launch_rms_norm_quant(dev, P.h, L.attn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs, xh))) return rc;
+        if ((rc = norm_quant(L.attn_norm, xh))) return rc;
         const candy_hip_qtensor *qkv_w[3] = {L.wq, L.wk, L.wv};
         float *qkv_y[3] = {P.q, P.k, P.v};
         if (xh && mmq_f16_group_covers(qkv_w, 3, n)) {  // one grid for the three projections
@@ -486,7 +501,7 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
         if ((rc = launch_quantize_q8(dev, P.att, n, qd, P.xq, P.xs, nullptr, xh_for(L.wo)))) return rc;
         if ((rc = add_linear(L.wo))) return rc;  // h += Wo . att
         xh = (xh_for(L.gate) || xh_for(L.up)) ? P.xh : nullptr;
-        if ((rc = launch_rms_norm_quant(dev, P.h, L.ffn_norm, c.rms_eps, n, c.d_model, nullptr, P.xq, P.xs, xh))) return rc;
+        if ((rc = norm_quant(L.ffn_norm, xh))) return rc;
         const candy_hip_qtensor *gu_w[2] = {L.gate, L.up};
         float *gu_y[2] = {P.gate, P.up};
         if (xh && mmq_f16_group_covers(gu_w, 2, n)) {  // the second projection's tiles fill the first one's last round
@@ -499,6 +514,9 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
             return rc;
         if ((rc = add_linear(L.down))) return rc;  // h += Wdown . act
     }
+    if (pend.n_split > 0 &&
+        (rc = launch_splitk_sum(dev, pend.part, pend.y, pend.res, pend.count, pend.n_split, pend.stride)))
+        return rc;
     if ((rc = candy_hip_d2d(dev, m->h, P.h + (size_t)(n - 1) * c.d_model, (size_t)c.d_model * sizeof(float)))) return rc;
     const candy_hip_qtensor *ws[1] = {m->head};
     float *ys[1] = {m->logits};

@@ -736,9 +736,10 @@ __global__ __launch_bounds__(256) void k_splitk_sum(const float *__restrict__ pa
     }
 }
 
-int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split) {
+int launch_splitk_sum(candy_hip_device *dev, const float *part, float *y, const float *res, size_t count, int n_split,
+                      size_t stride) {
     hipLaunchKernelGGL(k_splitk_sum, dim3((unsigned)((count / 4 + 256) / 256)), dim3(256), 0, dev->stream, part, y, res,
-                       count, n_split, count);
+                       count, n_split, stride ? stride : count);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
@@ -810,7 +811,11 @@ static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, cons
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream, grp, xh, (int)m, K,
                        n_tiles, m_tiles, sb_per, split_stride);
     CANDY_LAUNCH_CHECK();
-    if (n_split > 1) {
+    if (n_split > 1 && count == 1 && dev->defer_split) {
+        SplitPending &sp = *dev->defer_split;  // the caller sums the copies
+        sp.part = part; sp.y = jobs[0].y; sp.res = jobs[0].res;
+        sp.count = split_stride; sp.stride = split_stride; sp.n_split = n_split;
+    } else if (n_split > 1) {
         // one sum per run of outputs that lie end to end (the prompt pass allocates q, k and v that way)
         size_t off = 0;
         for (int s = 0; s < count;) {

@@ -249,6 +249,78 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict_
     }
 }
 
+// The same for rows of up to 1024 * ITER values, the row held in registers between the two passes, and with the row
+// optionally assembled first from the partial copies a contraction split along K has left: x = res + (part[0] +
+// part[1] + ...), the additions in the order of the separate split sum, written back to x_out (res may alias x_out:
+// a thread reads what it overwrites).  With n_split == 0 the row is read from res.
+template <int ITER>
+__global__ __launch_bounds__(256) void k_rms_norm_quant_regs(const float *res, const float *__restrict__ part, int n_split,
+                                                             size_t stride, float *x_out,
+                                                             const float *__restrict__ alpha, float eps, int cols,
+                                                             uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
+                                                             half4v *__restrict__ xh) {
+    __shared__ float red[16];
+    const int n4 = cols >> 2;
+    const size_t row4 = (size_t)blockIdx.x * n4;
+    float4 v[ITER];
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int c = threadIdx.x + 256 * it;
+        v[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < n4) {
+            if (n_split > 0) {
+                float4 t = ((const float4 *)part)[row4 + c];
+                for (int k = 1; k < n_split; ++k) {
+                    const float4 u = ((const float4 *)(part + (size_t)k * stride))[row4 + c];
+                    t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+                }
+                if (res) {
+                    const float4 r = ((const float4 *)res)[row4 + c];
+                    t = make_float4(r.x + t.x, r.y + t.y, r.z + t.z, r.w + t.w);
+                }
+                v[it] = t;
+                ((float4 *)x_out)[row4 + c] = t;
+            } else {
+                v[it] = ((const float4 *)res)[row4 + c];
+            }
+        }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) s += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
+    s = block_reduce<false>(s, red);
+    const float mean = s / (float)cols;
+    const float scale = rms_inv_sqrt(mean + eps);
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int c = threadIdx.x + 256 * it;
+        if (256 * it >= n4) break;  // whole wavefronts take part in the cross-lane steps (n4 % 8 == 0)
+        const bool live = c < n4;
+        float4 w = v[it];
+        if (live) {
+            if (alpha) {
+                const float4 a = ((const float4 *)alpha)[c];
+                w = make_float4(scale * w.x * a.x, scale * w.y * a.y, scale * w.z * a.z, scale * w.w * a.w);
+            } else {
+                w = make_float4(scale * w.x, scale * w.y, scale * w.z, scale * w.w);
+            }
+        }
+        __half h;
+        int bsum;
+        const uint32_t packed = quantize_q8_lane4(w, h, bsum);
+        if (!live) continue;
+        const size_t i = row4 + c;
+        qs[i] = packed;
+        if (xh) xh[xh_index4(blockIdx.x, c, cols)] = q8_lane4_to_half(packed, h);
+        if ((c & 7) == 0) {
+            Q8Scale sc;
+            sc.d = __half2float(h);
+            sc.bsum = bsum;
+            scales[i >> 3] = sc;
+        }
+    }
+}
+
 // silu(gate) * up, then Q8_0 quantization. n % 32 == 0.
 __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict__ gate, const float4 *__restrict__ up,
                                                         int64_t n4, int64_t row_n4, float4 *__restrict__ act_out,
@@ -282,6 +354,24 @@ int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *al
     CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0 && cols <= 0x7FFFFFFF, "rms_norm_quant needs cols %% 32 == 0");
     hipLaunchKernelGGL(k_rms_norm_quant, dim3((unsigned)rows), dim3(256), 0, dev->stream, x, alpha, eps, (int)cols,
                        xn_out, (uint32_t *)qs, scales, (half4v *)xh);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+// RMSNorm + quantization of rows that a split contraction has left as partial copies (SplitPending, filled by the
+// fp16 tile launcher while dev->defer_split points at it): the sum, the residual add and the norm in one launch for
+// rows of up to 8192 values, the separate split sum first for longer ones.
+int launch_split_rms_norm_quant(candy_hip_device *dev, const SplitPending &sp, const float *alpha, float eps, int64_t rows,
+                                int64_t cols, int8_t *qs, Q8Scale *scales, _Float16 *xh) {
+    CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0 && cols <= 0x7FFFFFFF, "rms_norm_quant needs cols %% 32 == 0");
+    CANDY_REQUIRE(sp.count == (size_t)rows * (size_t)cols && sp.n_split > 0, "internal: pending split sum of another shape");
+    if (cols > 8192 || !dev->opt.prefill_split_norm) {
+        if (int rc = launch_splitk_sum(dev, sp.part, sp.y, sp.res, sp.count, sp.n_split, sp.stride)) return rc;
+        return launch_rms_norm_quant(dev, sp.y, alpha, eps, rows, cols, nullptr, qs, scales, xh);
+    }
+    auto kern = cols <= 4096 ? k_rms_norm_quant_regs<4> : k_rms_norm_quant_regs<8>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(256), 0, dev->stream, sp.res, sp.part, sp.n_split, sp.stride, sp.y,
+                       alpha, eps, (int)cols, (uint32_t *)qs, scales, (half4v *)xh);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }

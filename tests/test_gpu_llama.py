@@ -386,6 +386,29 @@ def test_prompt_pass_of_256_rows_and_more_matches_cpu(dev, n):
         tok = rt
 
 
+@pytest.mark.parametrize("n", [64, 256, 300, 512])
+def test_split_sums_inside_the_norm_launch_equal_separate_launches(dev, n):
+    # An o / down projection that splits K hands its partial copies to the RMSNorm + quantize launch behind it (the
+    # last layer's down projection to a split sum of its own).  Same additions in the same order as the separate
+    # split sum, residual add and norm: every cached k / v and the logits the same bits.
+    cfg, fmts = BIG_PROMPT_CFG, BIG_PROMPT_FMTS
+    _, a = build(dev, cfg, fmts, seed=72)
+    _, b = build(dev, cfg, fmts, seed=72)
+    tokens = [int(t) for t in np.random.default_rng(190 + n).integers(0, cfg["vocab"], n)]
+    ta, la = a.prefill(tokens, 0)
+    dev.set_option("prefill.split_norm", 0)
+    try:
+        tb, lb = b.prefill(tokens, 0)
+    finally:
+        dev.set_option("prefill.split_norm", 1)
+    shape = (cfg["n_layers"], cfg["n_kv_heads"], cfg["max_pos"], cfg["head_dim"])
+    ka, va = read_cache(dev, a, shape)
+    kb, vb = read_cache(dev, b, shape)
+    assert np.array_equal(ka.view(np.uint32), kb.view(np.uint32))
+    assert np.array_equal(va.view(np.uint32), vb.view(np.uint32))
+    assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)) and ta == tb
+
+
 @pytest.mark.parametrize("n", [256, 300, 512])
 def test_grouped_qkv_projection_agrees_with_separate_launches(dev, n):
     # From 256 rows on the q / k / v projections share one grid of fp16 tiles (their outputs lie end to end, one sum
