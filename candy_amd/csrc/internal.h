@@ -66,7 +66,7 @@ struct Options {
     int mmv_variant = 0;         // comparison runs: 1 = one 16-row strip per wavefront, 2 = two
     int pair_rows = 0;           // fused gate/up: row pairs per workgroup, 32 / 16 / 8 (0: the most even split)
     int rms_rows = 0;            // fused RMSNorm prologue: rows per workgroup, 16 / 24 (0: the most even split)
-    int prefill_split_norm = 1;      // prompt pass: split-K copies of o / down summed inside the following norm launch
+    int prefill_fold_split_sums = 1; // prompt pass: split-K copies summed inside the launch that follows (norm, rope)
     int prefill_qkv_group = 1;       // prompt pass: q / k / v (and gate / up) on one grid each where they run on the fp16 tiles
     int prefill_attention_valu = 0;  // prompt attention for head_dim 128 on the vector ALU instead of the matrix cores
     int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
@@ -303,9 +303,10 @@ int launch_contract(candy_hip_device *dev, const candy_hip_qtensor *w, const int
 // prefill.hip: prompt stages of the decoder (n tokens at positions pos0 ..).
 int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, const float *v, const float *cos_t,
                            const float *sin_t, void *k_cache, void *v_cache, bool kv_f16, int n, int pos0, int n_heads,
-                           int n_kv_heads, int head_dim, int64_t cache_stride);
+                           int n_kv_heads, int head_dim, int64_t cache_stride, const SplitPending *sp = nullptr);
 int launch_attn_prefill(candy_hip_device *dev, const float *q, const void *k_cache, const void *v_cache, bool kv_f16,
                         float *out, int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride,
-                        float scale);
+                        float scale, _Float16 *xh_out = nullptr);  // xh_out: the fp16 image of the quantized rows, not `out`
+bool attn_prefill_writes_half(const candy_hip_device *dev, int head_dim);
 
 }  // namespace candy

@@ -453,9 +453,12 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
     const int64_t qd = (int64_t)c.n_heads * c.head_dim;
     const float scale = 1.0f / std::sqrt((float)c.head_dim);
     int rc;
+    P.k = P.q + (size_t)n * qd;  // q, k and v of this pass end to end, whatever the buffer's capacity
+    P.v = P.k + (size_t)n * c.n_kv_heads * c.head_dim;
     if ((rc = candy_hip_qindex_select(dev, m->embed, P.ids, n, P.h))) return rc;
-    // An o / down projection that splits K leaves its partial copies for the norm launch that follows, which sums them,
-    // adds the residual and writes P.h before it normalizes (one launch and one pass over P.h less each time).
+    // A projection that splits K leaves its partial copies for the launch that follows: the norm launch behind o / down
+    // sums them, adds the residual and writes P.h before it normalizes, the rope launch behind q / k / v sums them on
+    // its way to the cache (one launch and one pass over the outputs less each time).
     SplitPending pend;
     auto norm_quant = [&](const float *alpha, _Float16 *xh_out) -> int {
         const int e = pend.n_split > 0
@@ -486,19 +489,24 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
         const candy_hip_qtensor *qkv_w[3] = {L.wq, L.wk, L.wv};
         float *qkv_y[3] = {P.q, P.k, P.v};
         if (xh && mmq_f16_group_covers(qkv_w, 3, n)) {  // one grid for the three projections
-            if ((rc = launch_mmq_f16_group(dev, qkv_w, qkv_y, 3, xh, n))) return rc;
+            dev->defer_split = &pend;  // q, k and v lie end to end: the rope launch sums their partial copies
+            rc = launch_mmq_f16_group(dev, qkv_w, qkv_y, 3, xh, n);
+            dev->defer_split = nullptr;
+            if (rc) return rc;
         } else {
             if ((rc = launch_contract(dev, L.wq, P.xq, P.xs, n, P.q, xh_for(L.wq)))) return rc;
             if ((rc = launch_contract(dev, L.wk, P.xq, P.xs, n, P.k, xh_for(L.wk)))) return rc;
             if ((rc = launch_contract(dev, L.wv, P.xq, P.xs, n, P.v, xh_for(L.wv)))) return rc;
         }
-        if ((rc = launch_prefill_rope_kv(dev, P.q, P.k, P.v, m->cos_t, m->sin_t, kc, vc, m->kv_f16, n, pos0, c.n_heads,
-                                         c.n_kv_heads, c.head_dim, cache_stride)))
-            return rc;
+        rc = launch_prefill_rope_kv(dev, P.q, P.k, P.v, m->cos_t, m->sin_t, kc, vc, m->kv_f16, n, pos0, c.n_heads,
+                                    c.n_kv_heads, c.head_dim, cache_stride, &pend);
+        pend.n_split = 0;
+        if (rc) return rc;
+        _Float16 *att_xh = xh_for(L.wo) && mmq_fuses_residual(L.wo, n) && attn_prefill_writes_half(dev, c.head_dim) ? P.xh : nullptr;
         if ((rc = launch_attn_prefill(dev, P.q, kc, vc, m->kv_f16, P.att, n, pos0, c.n_heads, c.n_kv_heads, c.head_dim,
-                                      cache_stride, scale)))
+                                      cache_stride, scale, att_xh)))
             return rc;
-        if ((rc = launch_quantize_q8(dev, P.att, n, qd, P.xq, P.xs, nullptr, xh_for(L.wo)))) return rc;
+        if (!att_xh && (rc = launch_quantize_q8(dev, P.att, n, qd, P.xq, P.xs, nullptr, xh_for(L.wo)))) return rc;
         if ((rc = add_linear(L.wo))) return rc;  // h += Wo . att
         xh = (xh_for(L.gate) || xh_for(L.up)) ? P.xh : nullptr;
         if ((rc = norm_quant(L.ffn_norm, xh))) return rc;

@@ -811,7 +811,10 @@ static int launch_big(candy_hip_device *dev, const F16Job *jobs, int count, cons
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * n_split)), dim3(WN * WM * 64), smem, dev->stream, grp, xh, (int)m, K,
                        n_tiles, m_tiles, sb_per, split_stride);
     CANDY_LAUNCH_CHECK();
-    if (n_split > 1 && count == 1 && dev->defer_split) {
+    bool one_run = true;  // outputs end to end, no residual but a single job's
+    for (int s = 1; s < count; ++s)
+        one_run = one_run && !jobs[0].res && !jobs[s].res && jobs[s].y == jobs[s - 1].y + (size_t)m * (size_t)jobs[s - 1].w->rows;
+    if (n_split > 1 && one_run && dev->defer_split) {
         SplitPending &sp = *dev->defer_split;  // the caller sums the copies
         sp.part = part; sp.y = jobs[0].y; sp.res = jobs[0].res;
         sp.count = split_stride; sp.stride = split_stride; sp.n_split = n_split;

@@ -365,7 +365,7 @@ int launch_split_rms_norm_quant(candy_hip_device *dev, const SplitPending &sp, c
                                 int64_t cols, int8_t *qs, Q8Scale *scales, _Float16 *xh) {
     CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0 && cols <= 0x7FFFFFFF, "rms_norm_quant needs cols %% 32 == 0");
     CANDY_REQUIRE(sp.count == (size_t)rows * (size_t)cols && sp.n_split > 0, "internal: pending split sum of another shape");
-    if (cols > 8192 || !dev->opt.prefill_split_norm) {
+    if (cols > 8192 || !dev->opt.prefill_fold_split_sums) {
         if (int rc = launch_splitk_sum(dev, sp.part, sp.y, sp.res, sp.count, sp.n_split, sp.stride)) return rc;
         return launch_rms_norm_quant(dev, sp.y, alpha, eps, rows, cols, nullptr, qs, scales, xh);
     }

@@ -66,6 +66,64 @@ __global__ __launch_bounds__(256) void k_prefill_rope_kv(float *__restrict__ q, 
     }
 }
 
+// The same four pairs per thread, for q, k and v rows that lie end to end in `src` ([n][q heads], [n][kv heads] twice),
+// optionally still as the n_split partial copies of a contraction split along K, `stride` floats apart, summed here in
+// the order of the separate split sum.  q is written to `q` (which may be `src`), k and v go to the cache only.
+template <class KV>
+__global__ __launch_bounds__(256) void k_prefill_rope_kv4(float *q, const float *src, int n_split, size_t stride,
+                                                          const float *__restrict__ cos_t,
+                                                          const float *__restrict__ sin_t, KV *__restrict__ k_cache,
+                                                          KV *__restrict__ v_cache, int n, int pos0, int n_heads,
+                                                          int n_kv_heads, int head_dim, int64_t cache_stride) {
+    const int half = head_dim >> 1, hq = half >> 2;
+    const int slots = n_heads + 2 * n_kv_heads;  // q heads, then k heads, then v heads
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t total = (int64_t)n * slots * hq;
+    if (idx >= total) return;
+    const int j = (int)(idx % hq) * 4;
+    const int slot = (int)((idx / hq) % slots);
+    const int i = (int)(idx / ((int64_t)hq * slots));
+    const int pos = pos0 + i;
+    auto load = [&](size_t off) {
+        float4 t = *(const float4 *)(src + off);
+        for (int k = 1; k < n_split; ++k) {
+            const float4 u = *(const float4 *)(src + (size_t)k * stride + off);
+            t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+        }
+        return t;
+    };
+    auto store = [&](KV *dst, float4 t) {  // 4-element aligned: head_dim % 8 == 0
+        typedef KV kv4 __attribute__((ext_vector_type(4)));
+        kv4 o;
+        o[0] = (KV)t.x; o[1] = (KV)t.y; o[2] = (KV)t.z; o[3] = (KV)t.w;
+        *(kv4 *)dst = o;
+    };
+    const size_t k_base = (size_t)n * n_heads * head_dim, v_base = k_base + (size_t)n * n_kv_heads * head_dim;
+    if (slot >= n_heads + n_kv_heads) {
+        const int h = slot - n_heads - n_kv_heads;
+        const size_t off = v_base + ((size_t)i * n_kv_heads + h) * head_dim + j;
+        KV *dst = v_cache + (size_t)h * cache_stride + (size_t)pos * head_dim + j;
+        store(dst, load(off));
+        store(dst + half, load(off + half));
+        return;
+    }
+    const float4 c = *(const float4 *)(cos_t + (size_t)pos * half + j), s = *(const float4 *)(sin_t + (size_t)pos * half + j);
+    const bool is_q = slot < n_heads;
+    const int h = is_q ? slot : slot - n_heads;
+    const size_t off = is_q ? ((size_t)i * n_heads + h) * head_dim + j : k_base + ((size_t)i * n_kv_heads + h) * head_dim + j;
+    const float4 a = load(off), b = load(off + half);
+    const float4 lo = make_float4(a.x * c.x - b.x * s.x, a.y * c.y - b.y * s.y, a.z * c.z - b.z * s.z, a.w * c.w - b.w * s.w);
+    const float4 hi = make_float4(a.x * s.x + b.x * c.x, a.y * s.y + b.y * c.y, a.z * s.z + b.z * c.z, a.w * s.w + b.w * c.w);
+    if (is_q) {
+        *(float4 *)(q + off) = lo;
+        *(float4 *)(q + off + half) = hi;
+    } else {
+        KV *dst = k_cache + (size_t)h * cache_stride + (size_t)pos * head_dim + j;
+        store(dst, lo);
+        store(dst + half, hi);
+    }
+}
+
 // grid (n_heads, ceil(n / 32)), 256 threads. Thread t serves query row t/8 throughout: in the score
 // phase it owns keys {t%8 + 8r}, in the output phase columns {4*(t%8) + 32r .. +3}; the 8 threads of
 // a row sit in adjacent lanes, so the row maximum and sum are three xor-shuffles.
@@ -207,7 +265,8 @@ template <class KV>
 __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restrict__ q, const KV *__restrict__ k_cache,
                                                            const KV *__restrict__ v_cache, float *__restrict__ out,
                                                            int n, int pos0, int n_heads, int n_kv_heads,
-                                                           int64_t cache_stride, float scale) {
+                                                           int64_t cache_stride, float scale,
+                                                           _Float16 *__restrict__ xh_out) {
     constexpr int HD = 128, QT = 64, KT = 32;
     constexpr int KP = HD + 8;   // K tile pitch in halves (272 bytes: the 16 rows of an operand read hit distinct banks)
     constexpr int VP = KT + 8;   // V^T tile pitch in halves (80 bytes, same property)
@@ -374,6 +433,24 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
         const int i = i0 + 16 * wave + 4 * c4 + j;
         if (i >= n) continue;
         const float inv = 1.0f / l_run[j];
+        if (xh_out) {
+            // The output row leaves as the fp16 image of its Q8_0 quantization (what the o projection's fp16 tiles
+            // contract with), the arithmetic of quantize_q8_lane4 + q8_lane4_to_half value by value: a 32-value block
+            // is columns 32 b .. 32 b + 31 = this 16-lane row's o[2 b] and o[2 b + 1].
+            const int K = n_heads * HD;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const float v0 = o[2 * b][j] * inv, v1 = o[2 * b + 1][j] * inv;
+                const float amax = row16_max(fmaxf(fabsf(v0), fabsf(v1)));
+                const float d = amax / 127.0f;
+                const int q0 = amax != 0.0f ? q8_level(v0, d) : 0, q1 = amax != 0.0f ? q8_level(v1, d) : 0;
+                const float df = __half2float(__float2half_rn(d));
+                const int col = head * HD + 32 * b + r16;
+                xh_out[xh_index4(i, col >> 2, K) * 4 + (col & 3)] = (_Float16)(df * (float)q0);
+                xh_out[xh_index4(i, (col + 16) >> 2, K) * 4 + (col & 3)] = (_Float16)(df * (float)q1);
+            }
+            continue;
+        }
         float *dst = out + ((size_t)i * n_heads + head) * HD + r16;
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) dst[dt * 16] = o[dt][j] * inv;
@@ -382,7 +459,30 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
 
 int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, const float *v, const float *cos_t,
                            const float *sin_t, void *k_cache, void *v_cache, bool kv_f16, int n, int pos0, int n_heads,
-                           int n_kv_heads, int head_dim, int64_t cache_stride) {
+                           int n_kv_heads, int head_dim, int64_t cache_stride, const SplitPending *sp) {
+    const size_t q_count = (size_t)n * n_heads * head_dim, kv_count = (size_t)n * n_kv_heads * head_dim;
+    const bool pending = sp && sp->n_split > 0;
+    if (pending) CANDY_REQUIRE(sp->y == q && !sp->res && sp->count == q_count + 2 * kv_count, "internal: pending split sum of another shape");
+    if (head_dim % 8 == 0 && k == q + q_count && v == k + kv_count && dev->opt.prefill_fold_split_sums) {
+        // q, k and v end to end: four pairs per thread, and the partial copies of a split contraction summed on the way
+        const int64_t total4 = (int64_t)n * (n_heads + 2 * n_kv_heads) * (head_dim / 8);
+        const dim3 grid4((unsigned)((total4 + 255) / 256));
+        const float *src = pending ? sp->part : q;
+        const int n_split = pending ? sp->n_split : 1;
+        const size_t stride = pending ? sp->stride : 0;
+        if (kv_f16)
+            hipLaunchKernelGGL(k_prefill_rope_kv4<_Float16>, grid4, dim3(256), 0, dev->stream, q, src, n_split, stride, cos_t,
+                               sin_t, (_Float16 *)k_cache, (_Float16 *)v_cache, n, pos0, n_heads, n_kv_heads, head_dim,
+                               cache_stride);
+        else
+            hipLaunchKernelGGL(k_prefill_rope_kv4<float>, grid4, dim3(256), 0, dev->stream, q, src, n_split, stride, cos_t,
+                               sin_t, (float *)k_cache, (float *)v_cache, n, pos0, n_heads, n_kv_heads, head_dim,
+                               cache_stride);
+        CANDY_LAUNCH_CHECK();
+        return CANDY_HIP_OK;
+    }
+    if (pending)
+        if (int rc = launch_splitk_sum(dev, sp->part, sp->y, nullptr, sp->count, sp->n_split, sp->stride)) return rc;
     const int64_t total = (int64_t)n * (n_heads + 2 * n_kv_heads) * (head_dim / 2);
     const dim3 grid((unsigned)((total + 255) / 256));
     if (kv_f16)
@@ -398,12 +498,12 @@ int launch_prefill_rope_kv(candy_hip_device *dev, float *q, const float *k, cons
 template <class KV>
 static void launch_attn_prefill_kv(candy_hip_device *dev, const float *q, const KV *k_cache, const KV *v_cache, float *out,
                                    int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride,
-                                   float scale) {
+                                   float scale, _Float16 *xh_out) {
     const dim3 grid((unsigned)n_heads, (unsigned)((n + 31) / 32));
     const bool valu_only = dev->opt.prefill_attention_valu != 0;  // comparison runs
     if (head_dim == 128 && !valu_only)
         hipLaunchKernelGGL(k_attn_prefill_mfma<KV>, dim3((unsigned)n_heads, (unsigned)((n + 63) / 64)), dim3(256), 0,
-                           dev->stream, q, k_cache, v_cache, out, n, pos0, n_heads, n_kv_heads, cache_stride, scale);
+                           dev->stream, q, k_cache, v_cache, out, n, pos0, n_heads, n_kv_heads, cache_stride, scale, xh_out);
     else if (head_dim == 128)
         hipLaunchKernelGGL((k_attn_prefill<128, KV>), grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n, pos0,
                            n_heads, n_kv_heads, cache_stride, scale);
@@ -412,17 +512,24 @@ static void launch_attn_prefill_kv(candy_hip_device *dev, const float *q, const 
                            n_heads, n_kv_heads, cache_stride, scale);
 }
 
+// The matrix-core kernel can leave its output as the fp16 image of the quantized rows instead of f32 (no separate
+// quantize launch in front of an o projection that runs on the fp16 tiles).
+bool attn_prefill_writes_half(const candy_hip_device *dev, int head_dim) {
+    return head_dim == 128 && !dev->opt.prefill_attention_valu && dev->opt.prefill_fold_split_sums;
+}
+
 int launch_attn_prefill(candy_hip_device *dev, const float *q, const void *k_cache, const void *v_cache, bool kv_f16,
                         float *out, int n, int pos0, int n_heads, int n_kv_heads, int head_dim, int64_t cache_stride,
-                        float scale) {
+                        float scale, _Float16 *xh_out) {
     CANDY_REQUIRE(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
     CANDY_REQUIRE(n > 0 && pos0 >= 0 && n_heads % n_kv_heads == 0, "invalid attention shape");
+    CANDY_REQUIRE(!xh_out || attn_prefill_writes_half(dev, head_dim), "internal: this attention kernel writes f32 only");
     if (kv_f16)
         launch_attn_prefill_kv(dev, q, (const _Float16 *)k_cache, (const _Float16 *)v_cache, out, n, pos0, n_heads,
-                               n_kv_heads, head_dim, cache_stride, scale);
+                               n_kv_heads, head_dim, cache_stride, scale, xh_out);
     else
         launch_attn_prefill_kv(dev, q, (const float *)k_cache, (const float *)v_cache, out, n, pos0, n_heads, n_kv_heads,
-                               head_dim, cache_stride, scale);
+                               head_dim, cache_stride, scale, xh_out);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }

@@ -359,7 +359,7 @@ const OptionKey OPTION_KEYS[] = {
     {"fused.pair_rows", &candy::Options::pair_rows, 0, 32},
     {"fused.rms_rows", &candy::Options::rms_rows, 0, 24},
     {"prefill.qkv_group", &candy::Options::prefill_qkv_group, 0, 1},
-    {"prefill.split_norm", &candy::Options::prefill_split_norm, 0, 1},
+    {"prefill.fold_split_sums", &candy::Options::prefill_fold_split_sums, 0, 1},
     {"prefill.attention_valu", &candy::Options::prefill_attention_valu, 0, 1},
     {"llama.graph", &candy::Options::llama_graph, 0, 1},
     {"fused.wide", &candy::Options::fused_wide, 0, 1},

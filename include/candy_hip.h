@@ -110,8 +110,9 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   "fused.wide_waves"           8        wavefronts per workgroup of those kernels: 8 (two workgroups per CU) or 16 (one)
  *   "prefill.qkv_group"          1        prompt pass: projections that share their input (q / k / v; gate / up) as one
  *                                         grid each where all of them run on the fp16 tiles (0: one launch each)
- *   "prefill.split_norm"         1        prompt pass: the partial copies of an o / down projection split along K summed by
- *                                         the RMSNorm + quantize launch that follows (0: a launch of its own sums them)
+ *   "prefill.fold_split_sums"    1        prompt pass: the partial copies a projection split along K leaves are summed by the
+ *                                         launch that follows (RMSNorm + quantize behind o / down, rope behind q / k / v;
+ *                                         0: a launch of its own sums them)
  *   "prefill.attention_valu"     0        prompt attention for head_dim 128 on the vector ALU */
 int candy_hip_set_option(candy_hip_device *dev, const char *key, int64_t value);
 int candy_hip_get_option(const candy_hip_device *dev, const char *key, int64_t *value);

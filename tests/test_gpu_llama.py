@@ -387,20 +387,21 @@ def test_prompt_pass_of_256_rows_and_more_matches_cpu(dev, n):
 
 
 @pytest.mark.parametrize("n", [64, 256, 300, 512])
-def test_split_sums_inside_the_norm_launch_equal_separate_launches(dev, n):
-    # An o / down projection that splits K hands its partial copies to the RMSNorm + quantize launch behind it (the
-    # last layer's down projection to a split sum of its own).  Same additions in the same order as the separate
-    # split sum, residual add and norm: every cached k / v and the logits the same bits.
+def test_split_sums_inside_the_following_launch_equal_separate_launches(dev, n):
+    # A projection that splits K hands its partial copies to the launch behind it: o / down to the RMSNorm + quantize
+    # launch (the last layer's down projection to a split sum of its own), the q / k / v grid to the rope launch.
+    # Same additions in the same order as the separate split sum, residual add, norm and rope: every cached k / v
+    # and the logits the same bits.
     cfg, fmts = BIG_PROMPT_CFG, BIG_PROMPT_FMTS
     _, a = build(dev, cfg, fmts, seed=72)
     _, b = build(dev, cfg, fmts, seed=72)
     tokens = [int(t) for t in np.random.default_rng(190 + n).integers(0, cfg["vocab"], n)]
     ta, la = a.prefill(tokens, 0)
-    dev.set_option("prefill.split_norm", 0)
+    dev.set_option("prefill.fold_split_sums", 0)
     try:
         tb, lb = b.prefill(tokens, 0)
     finally:
-        dev.set_option("prefill.split_norm", 1)
+        dev.set_option("prefill.fold_split_sums", 1)
     shape = (cfg["n_layers"], cfg["n_kv_heads"], cfg["max_pos"], cfg["head_dim"])
     ka, va = read_cache(dev, a, shape)
     kb, vb = read_cache(dev, b, shape)
