@@ -386,13 +386,18 @@ def test_prompt_pass_of_256_rows_and_more_matches_cpu(dev, n):
         tok = rt
 
 
-@pytest.mark.parametrize("n", [64, 256, 300, 512])
-def test_split_sums_inside_the_following_launch_equal_separate_launches(dev, n):
+WIDE_PROMPT_CFG = dict(n_layers=2, d_model=5120, n_heads=8, n_kv_heads=2, head_dim=128, d_ffn=1024, vocab=256,
+                       max_pos=300, rms_eps=1e-5, rope_base=10000.0)
+
+
+@pytest.mark.parametrize("n,wide", [(64, False), (256, False), (300, False), (512, False), (272, True)])
+def test_split_sums_inside_the_following_launch_equal_separate_launches(dev, n, wide):
     # A projection that splits K hands its partial copies to the launch behind it: o / down to the RMSNorm + quantize
     # launch (the last layer's down projection to a split sum of its own), the q / k / v grid to the rope launch.
     # Same additions in the same order as the separate split sum, residual add, norm and rope: every cached k / v
-    # and the logits the same bits.
-    cfg, fmts = BIG_PROMPT_CFG, BIG_PROMPT_FMTS
+    # and the logits the same bits.  `wide`: hidden rows of 5120 values (the norm launch then holds eight vectors a thread,
+    # five of them live).
+    cfg, fmts = (WIDE_PROMPT_CFG if wide else BIG_PROMPT_CFG), BIG_PROMPT_FMTS
     _, a = build(dev, cfg, fmts, seed=72)
     _, b = build(dev, cfg, fmts, seed=72)
     tokens = [int(t) for t in np.random.default_rng(190 + n).integers(0, cfg["vocab"], n)]
