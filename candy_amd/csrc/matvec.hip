@@ -51,9 +51,14 @@ __device__ __forceinline__ void stage_activations(const int8_t *__restrict__ xq,
 
 // Batch-1 kernel.  ITER = ceil(units / 64) is a compile-time bound: every weight load of the
 // wavefront's R rows is in flight before anything waits.  The grid covers all rows at once.
-template <class U, int ITER, int R, int WAVES>
+// The unit type this kernel loads and contracts with: Q4_K blocks with the header shared over a quad of lanes.
+template <class U> struct OnceUnit { typedef U type; };
+template <> struct OnceUnit<UnitQ4K> { typedef UnitQ4KQuad type; };
+
+template <class UT, int ITER, int R, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_matvec1(const MatvecJobs jobs, const int8_t *__restrict__ xq,
                                                         const Q8Scale *__restrict__ xs, int K) {
+    typedef typename OnceUnit<UT>::type U;
     // which of the (up to three) weights sharing this activation does the workgroup belong to
     const int ji = (int)(blockIdx.x >= (unsigned)jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)jobs.j[1].wg_end);
     const int wg = blockIdx.x - (ji > 0 ? jobs.j[ji - 1].wg_end : 0);

@@ -37,23 +37,28 @@ struct UnitQ4K {
     }
     // sum over the unit of w*x, with x = d_x * q_x: quantized.cu:2239-2263
     __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        return dot_parts(w.hdr, w.q0, w.q1, u, sq, ss);
+    }
+    // hdr: the block's 16-byte header; q0, q1: the unit's 32 bytes of nibbles
+    __device__ static __forceinline__ float dot_parts(const u32x4 &hdr, const u32x4 &q0, const u32x4 &q1, int u,
+                                                      const int8_t *sq, const Q8Scale *ss) {
         const uint4 *xa = (const uint4 *)(sq + skewed(u * 64));
         const uint4 x0 = xa[0], x1 = xa[1], x2 = xa[2], x3 = xa[3];
         const Q8Scale s0 = ss[2 * u], s1 = ss[2 * u + 1];
         uint32_t sc2, m2;
-        q4k_scale_min_pair(w.hdr.y, w.hdr.z, w.hdr.w, u & 3, sc2, m2);
+        q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, u & 3, sc2, m2);
         const uint32_t M = 0x0F0F0F0Fu;
         int lo = 0, hi = 0;
-        lo = dot4_i8(w.q0.x & M, x0.x, lo); hi = dot4_i8((w.q0.x >> 4) & M, x2.x, hi);
-        lo = dot4_i8(w.q0.y & M, x0.y, lo); hi = dot4_i8((w.q0.y >> 4) & M, x2.y, hi);
-        lo = dot4_i8(w.q0.z & M, x0.z, lo); hi = dot4_i8((w.q0.z >> 4) & M, x2.z, hi);
-        lo = dot4_i8(w.q0.w & M, x0.w, lo); hi = dot4_i8((w.q0.w >> 4) & M, x2.w, hi);
-        lo = dot4_i8(w.q1.x & M, x1.x, lo); hi = dot4_i8((w.q1.x >> 4) & M, x3.x, hi);
-        lo = dot4_i8(w.q1.y & M, x1.y, lo); hi = dot4_i8((w.q1.y >> 4) & M, x3.y, hi);
-        lo = dot4_i8(w.q1.z & M, x1.z, lo); hi = dot4_i8((w.q1.z >> 4) & M, x3.z, hi);
-        lo = dot4_i8(w.q1.w & M, x1.w, lo); hi = dot4_i8((w.q1.w >> 4) & M, x3.w, hi);
-        const float d = half_bits_to_float((uint16_t)(w.hdr.x & 0xFFFF));
-        const float dmin = half_bits_to_float((uint16_t)(w.hdr.x >> 16));
+        lo = dot4_i8(q0.x & M, x0.x, lo); hi = dot4_i8((q0.x >> 4) & M, x2.x, hi);
+        lo = dot4_i8(q0.y & M, x0.y, lo); hi = dot4_i8((q0.y >> 4) & M, x2.y, hi);
+        lo = dot4_i8(q0.z & M, x0.z, lo); hi = dot4_i8((q0.z >> 4) & M, x2.z, hi);
+        lo = dot4_i8(q0.w & M, x0.w, lo); hi = dot4_i8((q0.w >> 4) & M, x2.w, hi);
+        lo = dot4_i8(q1.x & M, x1.x, lo); hi = dot4_i8((q1.x >> 4) & M, x3.x, hi);
+        lo = dot4_i8(q1.y & M, x1.y, lo); hi = dot4_i8((q1.y >> 4) & M, x3.y, hi);
+        lo = dot4_i8(q1.z & M, x1.z, lo); hi = dot4_i8((q1.z >> 4) & M, x3.z, hi);
+        lo = dot4_i8(q1.w & M, x1.w, lo); hi = dot4_i8((q1.w >> 4) & M, x3.w, hi);
+        const float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
         // every factor fits 24 bits (|dot| <= 32*15*127, |bsum| <= 32*127, scales < 64): full-rate v_mul_i32_i24
         const float sd = s0.d * (float)__mul24(lo, (int)(sc2 & 0xFF)) + s1.d * (float)__mul24(hi, (int)(sc2 >> 8));
         const float sm = s0.d * (float)__mul24(s0.bsum, (int)(m2 & 0xFF)) + s1.d * (float)__mul24(s1.bsum, (int)(m2 >> 8));
@@ -92,6 +97,32 @@ struct UnitQ4K {
         const float sd = s0.d * (float)__mul24(lo, p.sc_lo) + s1.d * (float)__mul24(hi, p.sc_hi);
         const float sm = s0.d * (float)__mul24(s0.bsum, p.m_lo) + s1.d * (float)__mul24(s1.bsum, p.m_hi);
         return p.d * sd - p.dmin * sm;
+    }
+};
+
+// UnitQ4K for kernels that use a unit once and give lane l unit 64 i + l (whole quads live or clamped together): the
+// four units of a block sit in the four lanes of a quad, each lane loads one word of the block's 16-byte header and the
+// quad rebuilds it with broadcasts where the dot needs it.  A quarter of the header bytes requested and three
+// registers fewer held per unit (batch-1 kernel, 4096 x 11008: 6.53 -> 6.40 us; the fused decode kernels, which hold
+// many units per lane, were slower this way: 514 -> 506 tok/s on the Llama-3-8B shape).
+struct UnitQ4KQuad {
+    static constexpr int ELEMS = UnitQ4K::ELEMS, ROW_ALIGN = UnitQ4K::ROW_ALIGN, SPAN = 0;
+    struct W { uint32_t h; u32x4 q0, q1; };
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return UnitQ4K::row_bytes(K); }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const uint8_t *blk = row + (size_t)(u >> 2) * 144;
+        w.h = *(const uint32_t *)(blk + 4 * (u & 3));
+        const u32x4 *q = (const u32x4 *)(blk + 16 + (u & 3) * 32);
+        w.q0 = q[0];
+        w.q1 = q[1];
+    }
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        u32x4 hdr;
+        hdr.x = (uint32_t)dpp_move_i<0x00>((int)w.h);  // quad_perm [0,0,0,0] .. [3,3,3,3]
+        hdr.y = (uint32_t)dpp_move_i<0x55>((int)w.h);
+        hdr.z = (uint32_t)dpp_move_i<0xAA>((int)w.h);
+        hdr.w = (uint32_t)dpp_move_i<0xFF>((int)w.h);
+        return UnitQ4K::dot_parts(hdr, w.q0, w.q1, u, sq, ss);
     }
 };
 
