@@ -54,6 +54,7 @@ __device__ __forceinline__ void stage_activations(const int8_t *__restrict__ xq,
 // The unit type this kernel loads and contracts with: Q4_K blocks with the header shared over a quad of lanes.
 template <class U> struct OnceUnit { typedef U type; };
 template <> struct OnceUnit<UnitQ4K> { typedef UnitQ4KQuad type; };
+template <> struct OnceUnit<UnitQ6K> { typedef UnitQ6KQuad type; };
 
 template <class UT, int ITER, int R, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_matvec1(const MatvecJobs jobs, const int8_t *__restrict__ xq,

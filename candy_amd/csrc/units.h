@@ -215,6 +215,11 @@ struct UnitQ6K {
     // quantized.cu:2367-2389: d * sum over 16-value groups of d8 * (dot * scale); the -32 offset is
     // applied as dot(q,x) - 32*sum(x) in integers.
     __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        return dot_parts(w.ql0, w.ql1, w.qh, w.sc, w.d, u, sq, ss);
+    }
+    // sc: the unit's four scales, one per byte; d: the block's fp16 scale
+    __device__ static __forceinline__ float dot_parts(const u32x2 &wql0, const u32x2 &wql1, const u32x2 &wqh, uint32_t wsc,
+                                                      uint16_t wd, int u, const int8_t *sq, const Q8Scale *ss) {
         const int sb = u >> 3, ip = (u >> 2) & 1, j = u & 3;
         const int blk0 = sb * 8 + ip * 4;  // first of the four 32-value activation blocks
         float sumf = 0.0f;
@@ -222,18 +227,44 @@ struct UnitQ6K {
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
             const uint2 x = *(const uint2 *)(sq + skewed((blk0 + qd) * 32 + 8 * j));
-            const u32x2 ql = (qd & 1) ? w.ql1 : w.ql0;
+            const u32x2 ql = (qd & 1) ? wql1 : wql0;
             const uint32_t lx = (qd < 2) ? (ql.x & M) : ((ql.x >> 4) & M);
             const uint32_t ly = (qd < 2) ? (ql.y & M) : ((ql.y >> 4) & M);
-            const uint32_t vx = lx | (((w.qh.x >> (2 * qd)) << 4) & H);
-            const uint32_t vy = ly | (((w.qh.y >> (2 * qd)) << 4) & H);
+            const uint32_t vx = lx | (((wqh.x >> (2 * qd)) << 4) & H);
+            const uint32_t vy = ly | (((wqh.y >> (2 * qd)) << 4) & H);
             int dq = dot4_i8(vy, x.y, dot4_i8(vx, x.x, 0));
             const int sx = dot4_i8(ones, x.y, dot4_i8(ones, x.x, 0));
             dq -= 32 * sx;
-            const int scale = (int)(int8_t)((w.sc >> (8 * qd)) & 0xFF);
+            const int scale = (int)(int8_t)((wsc >> (8 * qd)) & 0xFF);
             sumf += ss[blk0 + qd].d * (float)__mul24(dq, scale);  // |dq| < 2^15, |scale| < 2^7
         }
-        return half_bits_to_float(w.d) * sumf;
+        return half_bits_to_float(wd) * sumf;
+    }
+};
+
+// UnitQ6K for kernels that use a unit once and give lane l unit 64 i + l (whole quads live or clamped together).  The
+// four lanes of a quad hold the units j = 0 .. 3 of one half ip of a block; between them they need the eight scale
+// bytes 8 ip .. 8 ip + 7 and d.  Lanes 0 and 1 load one word of scales each, lanes 2 and 3 the block's last word
+// (scales 14, 15 and d), and the quad hands them round with broadcasts in the dot: one 4-byte request per lane where
+// four single bytes and a half were five.
+struct UnitQ6KQuad {
+    static constexpr int ELEMS = UnitQ6K::ELEMS, ROW_ALIGN = UnitQ6K::ROW_ALIGN, SPAN = 0;
+    struct W { u32x2 ql0, ql1, qh; uint32_t h; };
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return UnitQ6K::row_bytes(K); }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const BlockQ6K *blk = (const BlockQ6K *)row + (u >> 3);
+        const int ip = (u >> 2) & 1, j = u & 3;
+        w.ql0 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 8 * j);
+        w.ql1 = *(const u32x2_a2 *)(blk->ql + 64 * ip + 32 + 8 * j);
+        w.qh = *(const u32x2_a2 *)(blk->qh + 32 * ip + 8 * j);
+        w.h = *(const u32_a2 *)((const uint8_t *)blk + (j < 2 ? 192 + 8 * ip + 4 * j : 206));
+    }
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        const uint32_t lo = (uint32_t)dpp_move_i<0x00>((int)w.h), hi = (uint32_t)dpp_move_i<0x55>((int)w.h);
+        const uint32_t last = (uint32_t)dpp_move_i<0xAA>((int)w.h);
+        // scales 8 ip + (j >> 1) + {0, 2, 4, 6}: the even or the odd bytes of the two words
+        const uint32_t sc = (u & 2) ? __builtin_amdgcn_perm(hi, lo, 0x07050301u) : __builtin_amdgcn_perm(hi, lo, 0x06040200u);
+        return UnitQ6K::dot_parts(w.ql0, w.ql1, w.qh, sc, (uint16_t)(last >> 16), u, sq, ss);
     }
 };
 
