@@ -207,10 +207,14 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1_span(const MatvecJobs jo
 
 // General kernel: NB activation rows (small batch) and any contraction length; each wavefront
 // owns R weight rows and walks the row 64 units at a time.
-template <class U, int NB, int R, int WAVES>
+template <class U> struct LoopUnit { typedef U type; };
+template <> struct LoopUnit<UnitQ6K> { typedef UnitQ6KQuad type; };
+
+template <class UT, int NB, int R, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
                                                        const Q8Scale *__restrict__ xs, float *__restrict__ y,
                                                        int N, int K, int m) {
+    typedef typename LoopUnit<UT>::type U;
     extern __shared__ __align__(16) uint8_t smem[];
     int8_t *sq;
     Q8Scale *ss;
