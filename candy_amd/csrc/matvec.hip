@@ -209,6 +209,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1_span(const MatvecJobs jo
 // owns R weight rows and walks the row 64 units at a time.
 template <class U> struct LoopUnit { typedef U type; };
 template <> struct LoopUnit<UnitQ6K> { typedef UnitQ6KQuad type; };
+template <> struct LoopUnit<UnitQ4K> { typedef UnitQ4KQuad type; };  // 2 rows: 4096 x 32768 41.1 -> 39.0 us, 32000 x 4096 23.1 -> 22.7
 
 template <class UT, int NB, int R, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_matvec(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
