@@ -236,19 +236,52 @@ struct UnitQ3K {
     }
     // level = two bits + 4 * mask bit - 4: sum level*x = sum (q | h << 2) x - 4 sum x
     __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        return dot_parts(w.q, w.h, w.sc, w.d, u, sq, ss);
+    }
+    // sc: the unit's four 6-bit scales, one per byte; d: the block's fp16 scale
+    __device__ static __forceinline__ float dot_parts(const u32x2 &wq, const u32x2 &wh, uint32_t wsc, uint16_t wd, int u,
+                                                      const int8_t *sq, const Q8Scale *ss) {
         const int sb = u >> 3, n = (u >> 2) & 1, j = u & 3;
         const int blk0 = sb * 8 + n * 4;
         float sumf = 0.0f;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const uint2 x = *(const uint2 *)(sq + skewed((blk0 + k) * 32 + 8 * j));
-            const uint32_t vx = ((w.q.x >> (2 * k)) & 0x03030303u) | (((w.h.x >> (4 * n + k)) & 0x01010101u) << 2);
-            const uint32_t vy = ((w.q.y >> (2 * k)) & 0x03030303u) | (((w.h.y >> (4 * n + k)) & 0x01010101u) << 2);
+            const uint32_t vx = ((wq.x >> (2 * k)) & 0x03030303u) | (((wh.x >> (4 * n + k)) & 0x01010101u) << 2);
+            const uint32_t vy = ((wq.y >> (2 * k)) & 0x03030303u) | (((wh.y >> (4 * n + k)) & 0x01010101u) << 2);
             const int dq = dot4_i8(vy, x.y, dot4_i8(vx, x.x, 0)) - 4 * sum4_i8(x.y, sum4_i8(x.x, 0));
-            const int sc = (int)((w.sc >> (8 * k)) & 0xFF) - 32;
+            const int sc = (int)((wsc >> (8 * k)) & 0xFF) - 32;
             sumf += ss[blk0 + k].d * (float)(dq * sc);
         }
-        return half_bits_to_float(w.d) * sumf;
+        return half_bits_to_float(wd) * sumf;
+    }
+};
+
+// UnitQ3K for kernels that give lane l unit 64 i + l: the quad that holds the units j = 0 .. 3 of one half n of a block
+// shares the twelve scale bytes and d.  Lanes 0, 1 and 2 load one word of scales each, lane 3 the block's last word
+// (scales 10, 11 and d); the dot takes them by quad broadcast and picks the unit's four 6-bit scales, groups
+// is = 8 n + 2 k + (j >> 1): low nibbles from the even or odd bytes of words 0 and 1 shifted by 4 n, high bit pairs from
+// bytes (is & 3) of word 2 shifted by 2 (is >> 2).  Three requests per unit where there were eleven.
+struct UnitQ3KQuad {
+    static constexpr int ELEMS = UnitQ3K::ELEMS, ROW_ALIGN = UnitQ3K::ROW_ALIGN, SPAN = 0;
+    struct W { u32x2 q, h; uint32_t s; };
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return UnitQ3K::row_bytes(K); }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const BlockQ3K *b = (const BlockQ3K *)(row + (size_t)(u >> 3) * 110);
+        const int n = (u >> 2) & 1, j = u & 3;
+        w.q = *(const u32x2_a2 *)(b->qs + 32 * n + 8 * j);
+        w.h = *(const u32x2_a2 *)(b->hmask + 8 * j);
+        w.s = load_u32_a2((const uint8_t *)b + (j < 3 ? 96 + 4 * j : 106));
+    }
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        const uint32_t w0 = (uint32_t)dpp_move_i<0x00>((int)w.s), w1 = (uint32_t)dpp_move_i<0x55>((int)w.s);
+        const uint32_t w2 = (uint32_t)dpp_move_i<0xAA>((int)w.s), last = (uint32_t)dpp_move_i<0xFF>((int)w.s);
+        const int n = (u >> 2) & 1;
+        const bool odd = (u & 2) != 0;
+        const uint32_t lo4 = ((odd ? __builtin_amdgcn_perm(w1, w0, 0x07050301u) : __builtin_amdgcn_perm(w1, w0, 0x06040200u)) >> (4 * n)) & 0x0F0F0F0Fu;
+        const uint32_t t = odd ? __builtin_amdgcn_perm(w2, w2, 0x03010301u) : __builtin_amdgcn_perm(w2, w2, 0x02000200u);
+        const uint32_t hi4 = ((t >> (4 * n)) & 0x00000303u) | ((t >> (4 * n + 2)) & 0x03030000u);
+        return UnitQ3K::dot_parts(w.q, w.h, lo4 | (hi4 << 4), (uint16_t)(last >> 16), u, sq, ss);
     }
 };
 
