@@ -319,15 +319,20 @@ struct UnitQ5K {
         w.q1 = q[1];
     }
     __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        const uint32_t h[8] = {w.h0.x, w.h0.y, w.h0.z, w.h0.w, w.h1.x, w.h1.y, w.h1.z, w.h1.w};
+        return dot_parts(w.hdr, h, w.q0, w.q1, u, sq, ss);
+    }
+    // hdr: the block's 16-byte header; h: its 32 bytes of fifth bits; q0, q1: the unit's 32 bytes of nibbles
+    __device__ static __forceinline__ float dot_parts(const u32x4 &hdr, const uint32_t (&h)[8], const u32x4 &q0,
+                                                      const u32x4 &q1, int u, const int8_t *sq, const Q8Scale *ss) {
         const uint4 *xa = (const uint4 *)(sq + skewed(u * 64));
         const uint4 x0 = xa[0], x1 = xa[1], x2 = xa[2], x3 = xa[3];
         const Q8Scale s0 = ss[2 * u], s1 = ss[2 * u + 1];
         const int p = u & 3;
         uint32_t sc2, m2;
-        q4k_scale_min_pair(w.hdr.y, w.hdr.z, w.hdr.w, p, sc2, m2);
+        q4k_scale_min_pair(hdr.y, hdr.z, hdr.w, p, sc2, m2);
         const uint32_t M = 0x0F0F0F0Fu, B = 0x01010101u;
-        const uint32_t q[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
-        const uint32_t h[8] = {w.h0.x, w.h0.y, w.h0.z, w.h0.w, w.h1.x, w.h1.y, w.h1.z, w.h1.w};
+        const uint32_t q[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
         const uint32_t xl[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
         const uint32_t xh[8] = {x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
         int lo = 0, hi = 0;
@@ -336,11 +341,41 @@ struct UnitQ5K {
             lo = dot4_i8((q[i] & M) | (((h[i] >> (2 * p)) & B) << 4), xl[i], lo);
             hi = dot4_i8(((q[i] >> 4) & M) | (((h[i] >> (2 * p + 1)) & B) << 4), xh[i], hi);
         }
-        const float d = half_bits_to_float((uint16_t)(w.hdr.x & 0xFFFF));
-        const float dmin = half_bits_to_float((uint16_t)(w.hdr.x >> 16));
+        const float d = half_bits_to_float((uint16_t)(hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_float((uint16_t)(hdr.x >> 16));
         const float sd = s0.d * (float)(lo * (int)(sc2 & 0xFF)) + s1.d * (float)(hi * (int)(sc2 >> 8));
         const float sm = s0.d * (float)(s0.bsum * (int)(m2 & 0xFF)) + s1.d * (float)(s1.bsum * (int)(m2 >> 8));
         return d * sd - dmin * sm;
+    }
+};
+
+// UnitQ5K for kernels that give lane l unit 64 i + l.  The four units of a block sit in the four lanes of a quad and all
+// need the block's first 48 bytes (header and fifth bits): lane j loads words 3 j .. 3 j + 2 of them and the dot takes
+// the twelve words by quad broadcast.  Two 16-byte and one 12-byte request per unit where there were five of 16 bytes.
+template <int LANE>
+__device__ __forceinline__ uint32_t quad_from(uint32_t v) {
+    return (uint32_t)dpp_move_i<LANE * 0x55>((int)v);  // quad_perm [LANE, LANE, LANE, LANE]
+}
+struct UnitQ5KQuad {
+    static constexpr int ELEMS = UnitQ5K::ELEMS, ROW_ALIGN = UnitQ5K::ROW_ALIGN, SPAN = 0;
+    struct W { uint32_t s0, s1, s2; u32x4 q0, q1; };
+    __host__ __device__ static __forceinline__ size_t row_bytes(int K) { return UnitQ5K::row_bytes(K); }
+    __device__ static __forceinline__ void load(const uint8_t *row, int u, W &w) {
+        const uint8_t *blk = row + (size_t)(u >> 2) * 176;
+        const uint32_t *s = (const uint32_t *)(blk + 12 * (u & 3));
+        w.s0 = s[0];
+        w.s1 = s[1];
+        w.s2 = s[2];
+        const u32x4 *q = (const u32x4 *)(blk + 48 + (u & 3) * 32);
+        w.q0 = q[0];
+        w.q1 = q[1];
+    }
+    __device__ static __forceinline__ float dot(const W &w, int u, const int8_t *sq, const Q8Scale *ss) {
+        u32x4 hdr;
+        hdr.x = quad_from<0>(w.s0); hdr.y = quad_from<0>(w.s1); hdr.z = quad_from<0>(w.s2); hdr.w = quad_from<1>(w.s0);
+        const uint32_t h[8] = {quad_from<1>(w.s1), quad_from<1>(w.s2), quad_from<2>(w.s0), quad_from<2>(w.s1),
+                               quad_from<2>(w.s2), quad_from<3>(w.s0), quad_from<3>(w.s1), quad_from<3>(w.s2)};
+        return UnitQ5K::dot_parts(hdr, h, w.q0, w.q1, u, sq, ss);
     }
 };
 

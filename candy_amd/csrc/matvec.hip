@@ -56,6 +56,7 @@ template <class U> struct OnceUnit { typedef U type; };
 template <> struct OnceUnit<UnitQ4K> { typedef UnitQ4KQuad type; };
 template <> struct OnceUnit<UnitQ6K> { typedef UnitQ6KQuad type; };
 template <> struct OnceUnit<UnitQ3K> { typedef UnitQ3KQuad type; };
+template <> struct OnceUnit<UnitQ5K> { typedef UnitQ5KQuad type; };
 
 template <class UT, int ITER, int R, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void k_matvec1(const MatvecJobs jobs, const int8_t *__restrict__ xq,
@@ -211,6 +212,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1_span(const MatvecJobs jo
 template <class U> struct LoopUnit { typedef U type; };
 template <> struct LoopUnit<UnitQ6K> { typedef UnitQ6KQuad type; };
 template <> struct LoopUnit<UnitQ3K> { typedef UnitQ3KQuad type; };
+template <> struct LoopUnit<UnitQ5K> { typedef UnitQ5KQuad type; };
 template <> struct LoopUnit<UnitQ4K> { typedef UnitQ4KQuad type; };  // 2 rows: 4096 x 32768 41.1 -> 39.0 us, 32000 x 4096 23.1 -> 22.7
 
 template <class UT, int NB, int R, int WAVES>
