@@ -31,30 +31,41 @@ __device__ __forceinline__ float half_wave_sum(float v) {
     return (threadIdx.x & 32) ? hi : lo;
 }
 
-struct AttnArgs {
+// What the first cache loads need are the kernel's plain leading arguments (14 dwords: they arrive in registers with
+// the wavefront, so the position can be fetched at once); the rest comes through the argument block.
+struct AttnHead {
+    const int *pos_ptr;    // optional: position of the new token in device memory
+    void *k_cache;         // [n_kv_heads, *, hd] of f32 or fp16 (the kernel's KV type), cache_stride elements between heads
+    void *v_cache;
     const float *q;        // [n_heads, hd]; pre-Rope when k_new is set
+    int64_t cache_stride;
+    int n_pos;             // used when pos_ptr is null: positions 0..n_pos-1 are in the cache
+    int n_splits;
+    float scale;
+    int fresh;             // the new token's k / v rows arrive in k_new / v_new (pre-Rope) and are appended here
+};
+struct AttnRest {
     const float *k_new;    // optional [n_kv_heads, hd] pre-Rope key of the new token
     const float *v_new;    // optional [n_kv_heads, hd]
     const float *cos_t;    // [max_pos, hd/2] (only with k_new)
     const float *sin_t;
-    void *k_cache;         // [n_kv_heads, *, hd] of f32 or fp16 (the kernel's KV type), cache_stride elements between heads
-    void *v_cache;
-    const int *pos_ptr;    // optional: position of the new token in device memory
-    int n_pos;             // used when pos_ptr is null: positions 0..n_pos-1 are in the cache
-    int64_t cache_stride;
-    float scale;
-    int n_splits;
     float *part_o;         // [n_heads, n_splits, hd]
     float *part_ml;        // [n_heads, n_splits, 2]
     float *out;            // optional [n_heads, hd]
     int8_t *oq;            // optional planar Q8_0 of the output
     Q8Scale *os;
 };
+struct AttnArgs {
+    AttnHead h;
+    AttnRest r;
+};
 
 // KV: float (candy's cache) or _Float16 (optional: half the bytes of the step's largest stream; the rows are
 // rounded once, when they enter the cache, and every product and sum stays f32).
 template <int GROUP, int VEC, class KV>
-__global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
+__global__ __launch_bounds__(256) void k_attn_decode(const int *__restrict__ pos_ptr, void *k_cache, void *v_cache,
+                                                     const float *__restrict__ q, int64_t cache_stride, int n_pos,
+                                                     int n_splits, float scale, int fresh_arg, const AttnRest a) {
     constexpr int HD = 32 * VEC;
     constexpr int UNR = 4;
     typedef float vecf __attribute__((ext_vector_type(VEC)));
@@ -62,13 +73,13 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hw = lane >> 5, hl = lane & 31;
     const int kvh = blockIdx.x, split = blockIdx.y;
-    const bool fresh = a.k_new != nullptr;                    // new token's k/v arrive in registers
-    const int pos = a.pos_ptr ? *a.pos_ptr : a.n_pos - 1;     // position of the new token
+    const bool fresh = fresh_arg != 0;                        // new token's k/v arrive in registers
+    const int pos = pos_ptr ? *pos_ptr : n_pos - 1;           // position of the new token
     const int n_cached = fresh ? pos : pos + 1;               // rows to read from the cache
-    const int per = (n_cached + a.n_splits - 1) / a.n_splits;
+    const int per = (n_cached + n_splits - 1) / n_splits;
     const int p0 = split * per, p1 = min(n_cached, p0 + per);
-    KV *kh = (KV *)a.k_cache + (size_t)kvh * a.cache_stride;
-    KV *vh = (KV *)a.v_cache + (size_t)kvh * a.cache_stride;
+    KV *kh = (KV *)k_cache + (size_t)kvh * cache_stride;
+    KV *vh = (KV *)v_cache + (size_t)kvh * cache_stride;
 
     // Rope pairs (i, i + HD/2) sit 16 lanes apart inside the half-wavefront
     vecf cs, sn;
@@ -90,7 +101,7 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
     vecf qv[GROUP];
 #pragma unroll
     for (int g = 0; g < GROUP; ++g) {
-        qv[g] = *(const vecf *)(a.q + (size_t)(kvh * GROUP + g) * HD + hl * VEC);
+        qv[g] = *(const vecf *)(q + (size_t)(kvh * GROUP + g) * HD + hl * VEC);
         if (fresh) qv[g] = rope(qv[g]);
     }
 
@@ -114,7 +125,7 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
                 float d = 0.0f;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) d += qv[g][j] * kv[u][j];
-                d = half_wave_sum(d) * a.scale;
+                d = half_wave_sum(d) * scale;
                 s[u] = valid[u] ? d : NEG_BIG;
                 m_new = fmaxf(m_new, s[u]);
             }
@@ -169,7 +180,7 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
     }
 
     // the new token: Rope its key, append both rows to the cache, attend to them from registers
-    if (fresh && split == a.n_splits - 1 && wave == 0) {
+    if (fresh && split == n_splits - 1 && wave == 0) {
         vecf kn = rope(*(const vecf *)(a.k_new + (size_t)kvh * HD + hl * VEC));
         vecf vn = *(const vecf *)(a.v_new + (size_t)kvh * HD + hl * VEC);
         const veckv kc = __builtin_convertvector(kn, veckv), vc = __builtin_convertvector(vn, veckv);
@@ -215,7 +226,7 @@ __global__ __launch_bounds__(256) void k_attn_decode(const AttnArgs a) {
             l += sl[w][g] * f;
             o += so[w][g][c] * f;
         }
-        const size_t ps = (size_t)(kvh * GROUP + g) * a.n_splits + split;
+        const size_t ps = (size_t)(kvh * GROUP + g) * n_splits + split;
         a.part_o[ps * HD + c] = o;
         if (c == 0) {
             a.part_ml[ps * 2 + 0] = m;
@@ -294,20 +305,23 @@ size_t attention_scratch_bytes(int n_heads, int n_kv_heads, int head_dim, int n_
 
 template <int GROUP, class KV>
 static int launch_group(candy_hip_device *dev, const AttnArgs &a, int n_kv_heads, int head_dim) {
-    dim3 grid((unsigned)n_kv_heads, (unsigned)a.n_splits);
+    dim3 grid((unsigned)n_kv_heads, (unsigned)a.h.n_splits);
+    const AttnHead &h = a.h;
     const unsigned n_heads = (unsigned)(n_kv_heads * GROUP);
     switch (head_dim) {
     case 64:
-        hipLaunchKernelGGL((k_attn_decode<GROUP, 2, KV>), grid, dim3(256), 0, dev->stream, a);
+        hipLaunchKernelGGL((k_attn_decode<GROUP, 2, KV>), grid, dim3(256), 0, dev->stream, h.pos_ptr, h.k_cache, h.v_cache,
+                           h.q, h.cache_stride, h.n_pos, h.n_splits, h.scale, h.fresh, a.r);
         CANDY_LAUNCH_CHECK();
-        hipLaunchKernelGGL((k_attn_merge<64>), dim3(n_heads), dim3(64), 0, dev->stream, a.part_o, a.part_ml, a.n_splits,
-                           a.out, a.oq, a.os);
+        hipLaunchKernelGGL((k_attn_merge<64>), dim3(n_heads), dim3(64), 0, dev->stream, a.r.part_o, a.r.part_ml, h.n_splits,
+                           a.r.out, a.r.oq, a.r.os);
         break;
     case 128:
-        hipLaunchKernelGGL((k_attn_decode<GROUP, 4, KV>), grid, dim3(256), 0, dev->stream, a);
+        hipLaunchKernelGGL((k_attn_decode<GROUP, 4, KV>), grid, dim3(256), 0, dev->stream, h.pos_ptr, h.k_cache, h.v_cache,
+                           h.q, h.cache_stride, h.n_pos, h.n_splits, h.scale, h.fresh, a.r);
         CANDY_LAUNCH_CHECK();
-        hipLaunchKernelGGL((k_attn_merge<128>), dim3(n_heads), dim3(128), 0, dev->stream, a.part_o, a.part_ml,
-                           a.n_splits, a.out, a.oq, a.os);
+        hipLaunchKernelGGL((k_attn_merge<128>), dim3(n_heads), dim3(128), 0, dev->stream, a.r.part_o, a.r.part_ml,
+                           h.n_splits, a.r.out, a.r.oq, a.r.os);
         break;
     default: return fail(CANDY_HIP_ERR_UNSUPPORTED, "head_dim %d unsupported (64 or 128)", head_dim);
     }
@@ -317,12 +331,13 @@ static int launch_group(candy_hip_device *dev, const AttnArgs &a, int n_kv_heads
 
 int launch_attention(candy_hip_device *dev, const AttnLaunch &L) {
     AttnArgs a{};
-    a.q = L.q; a.k_new = L.k_new; a.v_new = L.v_new; a.cos_t = L.cos_t; a.sin_t = L.sin_t;
-    a.k_cache = L.k_cache; a.v_cache = L.v_cache; a.pos_ptr = L.pos_ptr; a.n_pos = L.n_pos;
-    a.cache_stride = L.cache_stride; a.scale = L.scale; a.n_splits = L.n_splits;
-    a.part_o = (float *)L.scratch;
-    a.part_ml = a.part_o + (size_t)L.n_heads * L.n_splits * L.head_dim;
-    a.out = L.out; a.oq = L.oq; a.os = L.os;
+    a.h.q = L.q; a.r.k_new = L.k_new; a.r.v_new = L.v_new; a.r.cos_t = L.cos_t; a.r.sin_t = L.sin_t;
+    a.h.fresh = L.k_new != nullptr;
+    a.h.k_cache = L.k_cache; a.h.v_cache = L.v_cache; a.h.pos_ptr = L.pos_ptr; a.h.n_pos = L.n_pos;
+    a.h.cache_stride = L.cache_stride; a.h.scale = L.scale; a.h.n_splits = L.n_splits;
+    a.r.part_o = (float *)L.scratch;
+    a.r.part_ml = a.r.part_o + (size_t)L.n_heads * L.n_splits * L.head_dim;
+    a.r.out = L.out; a.r.oq = L.oq; a.r.os = L.os;
     const int group = L.n_heads / L.n_kv_heads;
     if (L.kv_f16) switch (group) {
         case 1: return launch_group<1, _Float16>(dev, a, L.n_kv_heads, L.head_dim);

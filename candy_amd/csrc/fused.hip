@@ -22,13 +22,18 @@ namespace candy {
 enum { PRO_Q8 = 0, PRO_RMS = 1 };
 enum { EPI_PLAIN = 0, EPI_PAIR = 1 };
 
-struct FusedArgs {
-    MatvecJobs jobs;        // PLAIN: up to 3 weights; PAIR: j[0] = gate, j[1] = up (same shape)
-    // prologue
-    const int8_t *xq;       // PRO_Q8: planar Q8_0 activations
-    const Q8Scale *xs;
-    const float *x;         // PRO_RMS: f32 input row, RMSNorm weight, epsilon
-    const float *alpha;
+// What a wavefront's first loads need - the input and the weights' addresses - are the kernel's plain leading
+// arguments (14 dwords: they arrive in registers with the wavefront); the rest comes through the argument block
+// while those loads are in flight.
+struct FusedHead {
+    const void *in0, *in1;  // PRO_Q8: planar Q8_0 activations (int8 quants, Q8Scale); PRO_RMS: f32 input row, RMSNorm weight
+    const uint8_t *W[3];    // PLAIN: up to 3 weights as one run of rows; PAIR: W[0] = gate, W[1] = up (same shape)
+    int K;
+    int e[3];               // PLAIN: each weight's END ROW in the run; PAIR: e[0] = rows of gate (and of up)
+};
+struct FusedRest {
+    float *y[3];
+    const float *res[3];
     float eps;
     // PAIR epilogue output: planar Q8_0 of silu(gate.x) * (up.x)
     int8_t *oq;
@@ -36,13 +41,20 @@ struct FusedArgs {
     // PAIR workgroups that own less than a 32-value block: their f32 results and one counter per block
     float *pair_act;
     unsigned *pair_tickets;
-    int K;
+};
+struct FusedArgs {
+    FusedHead h;
+    FusedRest r;
+    int n;      // host side only: weights in the launch
+    int N[3];   // host side only: rows of each weight
 };
 
 __device__ __forceinline__ float silu_exact(float x) { return x / (1.0f + expf(-x)); }
 
 template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
-__global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1) void k_matvec_fused(const FusedArgs a) {
+__global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1) void k_matvec_fused(
+    const void *__restrict__ in0, const void *__restrict__ in1, const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
+    const uint8_t *__restrict__ W2, int K, int e0, int e1, int e2, const FusedRest a) {
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;       // activation values the LDS image is sized for
     constexpr int AQ = (CAP / 16 + T - 1) / T;      // PRO_Q8: 16-byte chunks of quants per thread
@@ -57,7 +69,6 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
     __shared__ float s_act[32];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int K = a.K;
     const int units = K / U::ELEMS;
     const size_t rb = U::row_bytes(K);
 
@@ -67,7 +78,7 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
     // resolves each of its rows to a weight and a row of that weight (wavefront-uniform).  PAIR: blockIdx is the
     // group of S row pairs.
     const int wg = blockIdx.x;
-    const int N = a.jobs.j[0].N;  // PAIR: both weights have N rows
+    const int N = e0;  // PAIR: both weights have N rows
 
     // ---- inputs first (oldest entries of the in-order return queue)
     uint4 aq[AQ];
@@ -76,16 +87,16 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
     if (PRO == PRO_Q8) {
         const int qchunks = K >> 4, sblocks = K >> 5;
 #pragma unroll
-        for (int i = 0; i < AQ; ++i) aq[i] = ((const uint4 *)a.xq)[min(tid + i * T, qchunks - 1)];
+        for (int i = 0; i < AQ; ++i) aq[i] = ((const uint4 *)in0)[min(tid + i * T, qchunks - 1)];
 #pragma unroll
-        for (int i = 0; i < AS; ++i) as[i] = ((const uint2 *)a.xs)[min(tid + i * T, sblocks - 1)];
+        for (int i = 0; i < AS; ++i) as[i] = ((const uint2 *)in1)[min(tid + i * T, sblocks - 1)];
     } else {
         const int n4 = K >> 2;
 #pragma unroll
         for (int i = 0; i < XF; ++i) {
             const int c = min(tid + i * T, n4 - 1);
-            xv[i] = ((const float4 *)a.x)[c];
-            av[i] = ((const float4 *)a.alpha)[c];
+            xv[i] = ((const float4 *)in0)[c];
+            av[i] = ((const float4 *)in1)[c];
         }
     }
 
@@ -96,7 +107,6 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int g = row0 + r;
-        const int e0 = a.jobs.j[0].wg_end, e1 = a.jobs.j[1].wg_end, e2 = a.jobs.j[2].wg_end;
         const int ji = (int)(g >= e0) + (int)(g >= e1);
         job[r] = g < e2 ? ji : -1;
         jrow[r] = g < e2 ? g - (ji == 0 ? 0 : ji == 1 ? e0 : e1) : 0;
@@ -105,8 +115,8 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
     for (int m = 0; m < NW; ++m) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint8_t *row = EPI == EPI_PAIR ? a.jobs.j[m].W + (size_t)min(row0 + r, N - 1) * rb
-                                                 : a.jobs.j[max(job[r], 0)].W + (size_t)jrow[r] * rb;
+            const uint8_t *row = EPI == EPI_PAIR ? (m == 0 ? W0 : W1) + (size_t)min(row0 + r, N - 1) * rb
+                                                 : (job[r] <= 0 ? W0 : job[r] == 1 ? W1 : W2) + (size_t)jrow[r] * rb;
 #pragma unroll
             for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
         }
@@ -182,8 +192,8 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
         for (int r = 0; r < R; ++r) {
             const float v = wave_sum(acc[0][r]);
             if (lane == 0 && job[r] >= 0) {
-                float *y = a.jobs.j[job[r]].y;  // may alias res (h += W.x)
-                const float *res = a.jobs.j[job[r]].res;
+                float *y = a.y[job[r]];  // may alias res (h += W.x)
+                const float *res = a.res[job[r]];
                 y[jrow[r]] = res ? res[jrow[r]] + v : v;
             }
         }
@@ -245,16 +255,18 @@ static int launch_fused_cfg(candy_hip_device *dev, FusedArgs a) {
     const int rows_per_wg = R * WAVES;
     int total = 0;
     if (EPI == EPI_PAIR) {
-        total = a.jobs.j[0].N / rows_per_wg;
+        total = a.N[0] / rows_per_wg;
+        a.h.e[0] = a.h.e[1] = a.h.e[2] = a.N[0];
     } else {
         int rows = 0;
         for (int i = 0; i < 3; ++i) {
-            if (i < a.jobs.n) rows += a.jobs.j[i].N;
-            a.jobs.j[i].wg_end = rows;  // end row in the run; unused slots end where the last real one does
+            if (i < a.n) rows += a.N[i];
+            a.h.e[i] = rows;  // end row in the run; unused slots end where the last real one does
         }
         total = (rows + rows_per_wg - 1) / rows_per_wg;
     }
-    hipLaunchKernelGGL((k_matvec_fused<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)total), dim3(T), smem, dev->stream, a);
+    hipLaunchKernelGGL((k_matvec_fused<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)total), dim3(T), smem, dev->stream,
+                       a.h.in0, a.h.in1, a.h.W[0], a.h.W[1], a.h.W[2], a.h.K, a.h.e[0], a.h.e[1], a.h.e[2], a.r);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
@@ -290,8 +302,8 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
     if constexpr (sizeof(typename U::W) > 48) {
         if (epi == EPI_PAIR) {
             if constexpr (ITER <= 2) {
-                if (pro != PRO_RMS || !a.pair_act || !a.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
-                if (balanced_rows(a.jobs.j[0].N, dev->num_cus, 16, 8, dev->opt.pair_rows) == 8)
+                if (pro != PRO_RMS || !a.r.pair_act || !a.r.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
+                if (balanced_rows(a.N[0], dev->num_cus, 16, 8, dev->opt.pair_rows) == 8)
                     return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
                 return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
             } else {
@@ -307,7 +319,7 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
         if (epi == EPI_PAIR) {
             if constexpr (ITER <= 2) {  // two weights x 4 rows x ITER units must stay in registers
                 if (pro != PRO_RMS) return launch_fused_cfg<U, ITER, 4, 8, PRO_Q8, EPI_PAIR>(dev, a);
-                const int s = a.pair_act && a.pair_tickets ? balanced_rows(a.jobs.j[0].N, dev->num_cus, 32, 8, dev->opt.pair_rows) : 32;
+                const int s = a.r.pair_act && a.r.pair_tickets ? balanced_rows(a.N[0], dev->num_cus, 32, 8, dev->opt.pair_rows) : 32;
                 if (s == 16) return launch_fused_cfg<U, ITER, 1, 16, PRO_RMS, EPI_PAIR>(dev, a);
                 if (s == 8) return launch_fused_cfg<U, ITER, 1, 8, PRO_RMS, EPI_PAIR>(dev, a);
                 return launch_fused_cfg<U, ITER, 4, 8, PRO_RMS, EPI_PAIR>(dev, a);
@@ -319,7 +331,7 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
             if constexpr (ITER <= 2) {
                 // 16 rows per workgroup (4 x 4), or 24 (8 wavefronts x 3) where that leaves the fullest CU fewer rows
                 int rows = 0;
-                for (int i = 0; i < a.jobs.n; ++i) rows += a.jobs.j[i].N;
+                for (int i = 0; i < a.n; ++i) rows += a.N[i];
                 const int cus = dev->num_cus;
                 const long c16 = (long)((rows + 15) / 16 + cus - 1) / cus * 16, c24 = (long)((rows + 23) / 24 + cus - 1) / cus * 24;
                 const int forced = dev->opt.rms_rows;  // comparison runs
@@ -335,7 +347,7 @@ static int launch_fused_iter(candy_hip_device *dev, const FusedArgs &a, int pro,
 
 template <class U>
 static int launch_fused_fmt(candy_hip_device *dev, const FusedArgs &a, int pro, int epi) {
-    const int iter = (a.K / U::ELEMS + 63) / 64;
+    const int iter = (a.h.K / U::ELEMS + 63) / 64;
     switch (iter) {
     case 1: return launch_fused_iter<U, 1>(dev, a, pro, epi);
     case 2: return launch_fused_iter<U, 2>(dev, a, pro, epi);
@@ -357,17 +369,20 @@ int launch_matvec_fused(candy_hip_device *dev, const FusedLaunch &L) {
     if (L.pair && (n != 2 || L.w[0]->rows != L.w[1]->rows || w0->rows % 32 != 0)) return CANDY_HIP_ERR_UNSUPPORTED;
     if (w0->cols > 0x7FFFFFFF) return CANDY_HIP_ERR_UNSUPPORTED;
     FusedArgs a{};
-    a.jobs.n = n;
-    for (int i = 0; i < n; ++i) {
-        if (L.w[i]->rows > 0x7FFFFFFF) return CANDY_HIP_ERR_UNSUPPORTED;
-        a.jobs.j[i].W = (const uint8_t *)L.w[i]->data;
-        a.jobs.j[i].y = L.y[i];
-        a.jobs.j[i].res = L.res[i];
-        a.jobs.j[i].N = (int)L.w[i]->rows;
+    a.n = n;
+    for (int i = 0; i < 3; ++i) {
+        const int j = i < n ? i : n - 1;  // unused slots repeat the last weight: no row resolves to them
+        if (L.w[j]->rows > 0x7FFFFFFF) return CANDY_HIP_ERR_UNSUPPORTED;
+        a.h.W[i] = (const uint8_t *)L.w[j]->data;
+        a.r.y[i] = L.y[j];
+        a.r.res[i] = L.res[j];
+        a.N[i] = i < n ? (int)L.w[i]->rows : 0;
     }
-    a.xq = L.xq; a.xs = L.xs; a.x = L.x; a.alpha = L.alpha; a.eps = L.eps; a.oq = L.oq; a.os = L.os;
-    a.pair_act = L.pair_act; a.pair_tickets = L.pair_tickets;
-    a.K = (int)w0->cols;
+    if (L.x) { a.h.in0 = L.x; a.h.in1 = L.alpha; }
+    else { a.h.in0 = L.xq; a.h.in1 = L.xs; }
+    a.r.eps = L.eps; a.r.oq = L.oq; a.r.os = L.os;
+    a.r.pair_act = L.pair_act; a.r.pair_tickets = L.pair_tickets;
+    a.h.K = (int)w0->cols;
     switch (w0->fmt) {
     case CANDY_HIP_Q4_K: return launch_fused_fmt<UnitQ4K>(dev, a, pro, epi);
     case CANDY_HIP_Q8_0: return launch_fused_fmt<UnitQ8_0>(dev, a, pro, epi);

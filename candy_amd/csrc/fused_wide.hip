@@ -25,18 +25,29 @@ namespace candy {
 enum { WPRO_RMS = 0, WPRO_QUANT = 1 };
 enum { WEPI_PLAIN = 0, WEPI_PAIR = 1 };
 
-struct WideArgs {
-    MatvecJobs jobs;         // PLAIN: up to 3 weights, wg_end = END ROW of each in the run; PAIR: j[0] gate, j[1] up
+// What the first loads of a wavefront need - the prologue's input and the weights' addresses - are the kernel's plain
+// leading arguments (14 dwords: they arrive in registers with the wavefront); the rest comes through the argument
+// block while those loads are in flight.
+struct WideHead {
+    const float *x, *alpha;  // prologue input and (RMS) the norm weight
+    const uint8_t *W[3];     // PLAIN: up to 3 weights as one run of rows; PAIR: W[0] gate, W[1] up
     int total;               // rows of the run (PLAIN) or row pairs (PAIR)
     int K;
-    // RMS prologue
-    const float *x, *alpha;
+    int e0, e1;              // PLAIN: END ROW of the first and second weight in the run
+};
+struct WideRest {
+    float *y[3];
+    const float *res[3];
     float eps;
     // PAIR epilogue
     int8_t *oq;
     Q8Scale *os;
     float *pair_act;         // total floats of scratch
     unsigned *pair_tickets;  // total / 32 counters, zero before and after every launch
+};
+struct WideArgs {
+    WideHead h;
+    WideRest r;
 };
 
 __device__ __forceinline__ float wide_silu(float x) { return x / (1.0f + expf(-x)); }
@@ -52,7 +63,9 @@ __device__ __forceinline__ int wide_owner(int p, int total, int G) { return (int
 // pair); the one-workgroup-per-CU shape with sixteen rows per lane keeps its 226.
 template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
 __global__ __launch_bounds__(WAVES * 64, ((EPI == WEPI_PAIR ? 2 : 1) * R * ITER <= 8 ? 4 : 2))
-void k_matvec_wide(const WideArgs a) {
+void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha, const uint8_t *__restrict__ W0,
+                   const uint8_t *__restrict__ W1, const uint8_t *__restrict__ W2, int total, int K, int e0, int e1,
+                   const WideRest a) {
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;   // activation values the LDS image is sized for
     constexpr int XF = (CAP / 4 + T - 1) / T;   // float4 of prologue input per thread
@@ -65,11 +78,10 @@ void k_matvec_wide(const WideArgs a) {
     __shared__ float s_act[R * WAVES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int K = a.K;
     const int units = K / U::ELEMS;
     const size_t rb = U::row_bytes(K);
     const int G = gridDim.x;
-    const int start = wide_start(blockIdx.x, a.total, G), end = wide_start(blockIdx.x + 1, a.total, G);
+    const int start = wide_start(blockIdx.x, total, G), end = wide_start(blockIdx.x + 1, total, G);
     const int n4 = K >> 2;
 
     // ---- prologue inputs first (they return first)
@@ -77,8 +89,8 @@ void k_matvec_wide(const WideArgs a) {
 #pragma unroll
     for (int i = 0; i < XF; ++i) {
         const int c = min(tid + i * T, n4 - 1);
-        xv[i] = ((const float4 *)a.x)[c];
-        if (PRO == WPRO_RMS) av[i] = ((const float4 *)a.alpha)[c];
+        xv[i] = ((const float4 *)x)[c];
+        if (PRO == WPRO_RMS) av[i] = ((const float4 *)alpha)[c];
     }
 
     // ---- every weight load of the wavefront: items start + wave + WAVES * r
@@ -93,7 +105,6 @@ void k_matvec_wide(const WideArgs a) {
             job[r] = 0;
             jrow[r] = g;
         } else {
-            const int e0 = a.jobs.j[0].wg_end, e1 = a.jobs.j[1].wg_end;
             const int ji = (int)(g >= e0) + (int)(g >= e1);
             job[r] = ji;
             jrow[r] = g - (ji == 0 ? 0 : ji == 1 ? e0 : e1);
@@ -103,7 +114,8 @@ void k_matvec_wide(const WideArgs a) {
     for (int m = 0; m < NW; ++m)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint8_t *row = a.jobs.j[EPI == WEPI_PAIR ? m : job[r]].W + (size_t)jrow[r] * rb;
+            const uint8_t *Wj = EPI == WEPI_PAIR ? (m == 0 ? W0 : W1) : (job[r] == 0 ? W0 : job[r] == 1 ? W1 : W2);
+            const uint8_t *row = Wj + (size_t)jrow[r] * rb;
 #pragma unroll
             for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
         }
@@ -176,8 +188,8 @@ void k_matvec_wide(const WideArgs a) {
         for (int r = 0; r < R; ++r) {
             const float v = wave_sum(acc[0][r]);
             if (lane == 0 && start + wave + WAVES * r < end) {
-                float *y = a.jobs.j[job[r]].y;  // may alias res (h += W.x)
-                const float *res = a.jobs.j[job[r]].res;
+                float *y = a.y[job[r]];  // may alias res (h += W.x)
+                const float *res = a.res[job[r]];
                 y[jrow[r]] = res ? res[jrow[r]] + v : v;
             }
         }
@@ -209,7 +221,7 @@ void k_matvec_wide(const WideArgs a) {
             if (lane < 32 && first + lane >= lo && first + lane < hi)
                 __hip_atomic_store(a.pair_act + first + lane, s_act[first + lane - start], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            const unsigned expected = (unsigned)(wide_owner(first + 31, a.total, G) - wide_owner(first, a.total, G) + 1);
+            const unsigned expected = (unsigned)(wide_owner(first + 31, total, G) - wide_owner(first, total, G) + 1);
             unsigned old = 0;
             if (lane == 0) old = __hip_atomic_fetch_add(a.pair_tickets + blk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
@@ -238,7 +250,8 @@ static int launch_wide_cfg(candy_hip_device *dev, const WideArgs &a, int grid) {
     constexpr size_t QBYTES = (size_t)XF * T * 4;
     constexpr size_t smem = QBYTES + ((QBYTES >> 8) << 4) + ((size_t)XF * T / 8 + 1) * 8;
     static_assert(smem <= 48 * 1024, "LDS image too large");
-    hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a);
+    hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a.h.x,
+                       a.h.alpha, a.h.W[0], a.h.W[1], a.h.W[2], a.h.total, a.h.K, a.h.e0, a.h.e1, a.r);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
@@ -261,38 +274,36 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
     if (!L.x || ((uintptr_t)L.x & 15) != 0) return CANDY_HIP_ERR_UNSUPPORTED;
     if (quant && L.pair) return CANDY_HIP_ERR_UNSUPPORTED;
     WideArgs a{};
-    a.jobs.n = n;
-    int rows = 0;
+    int rows = 0, ends[3];
     for (int i = 0; i < 3; ++i) {
-        if (i < n) {
-            a.jobs.j[i].W = (const uint8_t *)L.w[i]->data;
-            a.jobs.j[i].y = L.y[i];
-            a.jobs.j[i].res = L.res[i];
-            a.jobs.j[i].N = (int)L.w[i]->rows;
-            rows += (int)L.w[i]->rows;
-        }
-        a.jobs.j[i].wg_end = rows;
+        // unused slots repeat the last weight and end where it does: no row resolves to them
+        a.h.W[i] = (const uint8_t *)L.w[i < n ? i : n - 1]->data;
+        a.r.y[i] = L.y[i < n ? i : n - 1];
+        a.r.res[i] = L.res[i < n ? i : n - 1];
+        if (i < n) rows += (int)L.w[i]->rows;
+        ends[i] = rows;
     }
-    a.K = (int)K;
-    a.x = L.x; a.alpha = L.alpha; a.eps = L.eps;
-    a.oq = L.oq; a.os = L.os; a.pair_act = L.pair_act; a.pair_tickets = L.pair_tickets;
+    a.h.e0 = ends[0]; a.h.e1 = ends[1];
+    a.h.K = (int)K;
+    a.h.x = L.x; a.h.alpha = L.alpha; a.r.eps = L.eps;
+    a.r.oq = L.oq; a.r.os = L.os; a.r.pair_act = L.pair_act; a.r.pair_tickets = L.pair_tickets;
     const int cus = dev->num_cus;
     if (L.pair) {
         if (n != 2 || L.w[0]->rows != L.w[1]->rows || w0->rows % 32 != 0 || !L.pair_act || !L.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
-        a.total = (int)w0->rows;
-        a.jobs.j[0].wg_end = a.jobs.j[1].wg_end = a.jobs.j[2].wg_end = a.total;
-        if (a.total < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
+        a.h.total = (int)w0->rows;
+        a.h.e0 = a.h.e1 = a.h.total;
+        if (a.h.total < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
         // one workgroup per CU; 16 wavefronts x 3 pairs while a CU's share fits, else 8 wavefronts x up to 8 pairs
         // (the weights of a wavefront's pairs stay in registers: 24 per pair and round of units)
-        const int per = (a.total + cus - 1) / cus;
+        const int per = (a.h.total + cus - 1) / cus;
         if (iter == 1 && dev->opt.wide_waves == 8) {  // two workgroups of eight wavefronts per CU
-            const int per2 = (a.total + 2 * cus - 1) / (2 * cus);
+            const int per2 = (a.h.total + 2 * cus - 1) / (2 * cus);
             if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
             if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
             // four pairs per wavefront need every register: three workgroups of three pairs per CU instead, the third
             // starting when the first is done (2 x 14336 x 4096: 508 against 502 tokens/s on the Llama-3-8B shape; the
             // same step from three pairs to two loses, 509 against 539 on the 7B shape: more blocks are shared)
-            if (per2 <= 32 && (a.total + 3 * cus - 1) / (3 * cus) <= 24)
+            if (per2 <= 32 && (a.h.total + 3 * cus - 1) / (3 * cus) <= 24)
                 return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 3 * cus);
             if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
         }
@@ -304,7 +315,7 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
         }
         return CANDY_HIP_ERR_UNSUPPORTED;
     }
-    a.total = rows;
+    a.h.total = rows;
     if (rows < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
     const int per = (rows + cus - 1) / cus;
     if (quant) {

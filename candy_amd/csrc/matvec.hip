@@ -58,17 +58,11 @@ template <> struct OnceUnit<UnitQ6K> { typedef UnitQ6KQuad type; };
 template <> struct OnceUnit<UnitQ3K> { typedef UnitQ3KQuad type; };
 template <> struct OnceUnit<UnitQ5K> { typedef UnitQ5KQuad type; };
 
+// The body: workgroup `wg` of weight W (N rows), output y (+ residual res, which may alias y: h += W.x).
 template <class UT, int ITER, int R, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_matvec1(const MatvecJobs jobs, const int8_t *__restrict__ xq,
-                                                        const Q8Scale *__restrict__ xs, int K) {
+__device__ __forceinline__ void matvec1_body(const uint8_t *__restrict__ W, float *y, const float *res, int N, int wg,
+                                             const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs, int K) {
     typedef typename OnceUnit<UT>::type U;
-    // which of the (up to three) weights sharing this activation does the workgroup belong to
-    const int ji = (int)(blockIdx.x >= (unsigned)jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)jobs.j[1].wg_end);
-    const int wg = blockIdx.x - (ji > 0 ? jobs.j[ji - 1].wg_end : 0);
-    const uint8_t *__restrict__ W = jobs.j[ji].W;
-    float *y = jobs.j[ji].y;  // may alias res (h += W.x)
-    const float *res = jobs.j[ji].res;
-    const int N = jobs.j[ji].N;
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;       // activation bytes the LDS image is sized for
     constexpr int AQ = (CAP / 16 + T - 1) / T;      // 16-byte chunks of quants per thread
@@ -128,6 +122,25 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1(const MatvecJobs jobs, c
     }
 }
 
+// One weight: everything the first loads need is a plain leading argument (12 dwords, preloaded into registers
+// when the wavefront starts), so the activation and weight requests go out without waiting for a scalar load
+// of the argument block.
+template <class UT, int ITER, int R, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec1(const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs,
+                                                        const uint8_t *__restrict__ W, float *y, const float *res, int K,
+                                                        int N) {
+    matvec1_body<UT, ITER, R, WAVES>(W, y, res, N, (int)blockIdx.x, xq, xs, K);
+}
+
+// Up to three weights that share the activation (q / k / v): the workgroup finds its weight in the job table.
+template <class UT, int ITER, int R, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec1_jobs(const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs,
+                                                             int K, const MatvecJobs jobs) {
+    const int ji = (int)(blockIdx.x >= (unsigned)jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)jobs.j[1].wg_end);
+    const int wg = blockIdx.x - (ji > 0 ? jobs.j[ji - 1].wg_end : 0);
+    matvec1_body<UT, ITER, R, WAVES>(jobs.j[ji].W, jobs.j[ji].y, jobs.j[ji].res, jobs.j[ji].N, wg, xq, xs, K);
+}
+
 // Batch-1 kernel for the formats whose blocks are not 16-byte aligned (34, 18, 210 bytes).  Loading
 // block by block makes every wavefront load straddle twice the cache lines it uses and touch each
 // line from three instructions (measured on the Q8_0 pattern alone: 3.8 TB/s against 5.6 TB/s for
@@ -136,14 +149,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1(const MatvecJobs jobs, c
 // to the wavefront, and each lane then picks its own block from the slice.  Needs rows that start
 // and end on 16-byte boundaries.
 template <class U, int ITER, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_matvec1_span(const MatvecJobs jobs, const int8_t *__restrict__ xq,
-                                                             const Q8Scale *__restrict__ xs, int K) {
-    const int ji = (int)(blockIdx.x >= (unsigned)jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)jobs.j[1].wg_end);
-    const int wg = blockIdx.x - (ji > 0 ? jobs.j[ji - 1].wg_end : 0);
-    const uint8_t *__restrict__ W = jobs.j[ji].W;
-    float *y = jobs.j[ji].y;  // may alias res (h += W.x)
-    const float *res = jobs.j[ji].res;
-    const int N = jobs.j[ji].N;
+__device__ __forceinline__ void matvec1_span_body(const uint8_t *__restrict__ W, float *y, const float *res, int N, int wg,
+                                                  const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs, int K) {
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;
     constexpr int AQ = (CAP / 16 + T - 1) / T;
@@ -205,6 +212,22 @@ __global__ __launch_bounds__(WAVES * 64) void k_matvec1_span(const MatvecJobs jo
     }
     const float v = wave_sum(acc);
     if (lane == 0 && row < N) y[row] = res ? res[row] + v : v;
+}
+
+template <class U, int ITER, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec1_span(const int8_t *__restrict__ xq, const Q8Scale *__restrict__ xs,
+                                                             const uint8_t *__restrict__ W, float *y, const float *res,
+                                                             int K, int N) {
+    matvec1_span_body<U, ITER, WAVES>(W, y, res, N, (int)blockIdx.x, xq, xs, K);
+}
+
+template <class U, int ITER, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_matvec1_span_jobs(const int8_t *__restrict__ xq,
+                                                                  const Q8Scale *__restrict__ xs, int K,
+                                                                  const MatvecJobs jobs) {
+    const int ji = (int)(blockIdx.x >= (unsigned)jobs.j[0].wg_end) + (int)(blockIdx.x >= (unsigned)jobs.j[1].wg_end);
+    const int wg = blockIdx.x - (ji > 0 ? jobs.j[ji - 1].wg_end : 0);
+    matvec1_span_body<U, ITER, WAVES>(jobs.j[ji].W, jobs.j[ji].y, jobs.j[ji].res, jobs.j[ji].N, wg, xq, xs, K);
 }
 
 // General kernel: NB activation rows (small batch) and any contraction length; each wavefront
@@ -276,8 +299,12 @@ static int launch1(candy_hip_device *dev, MatvecJobs jobs, int K, const int8_t *
         if (i < jobs.n) total += (jobs.j[i].N + rows_per_wg - 1) / rows_per_wg;
         jobs.j[i].wg_end = total;  // unused slots end where the last real one does
     }
-    hipLaunchKernelGGL((k_matvec1<U, ITER, R, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), smem, dev->stream, jobs,
-                       qs, scales, K);
+    if (jobs.n == 1)
+        hipLaunchKernelGGL((k_matvec1<U, ITER, R, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), smem, dev->stream, qs,
+                           scales, jobs.j[0].W, jobs.j[0].y, jobs.j[0].res, K, jobs.j[0].N);
+    else
+        hipLaunchKernelGGL((k_matvec1_jobs<U, ITER, R, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), smem, dev->stream,
+                           qs, scales, K, jobs);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
@@ -295,8 +322,12 @@ static int launch1_span(candy_hip_device *dev, MatvecJobs jobs, int K, const int
         if (i < jobs.n) total += (jobs.j[i].N + WAVES - 1) / WAVES;
         jobs.j[i].wg_end = total;
     }
-    hipLaunchKernelGGL((k_matvec1_span<U, ITER, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), smem, dev->stream,
-                       jobs, qs, scales, K);
+    if (jobs.n == 1)
+        hipLaunchKernelGGL((k_matvec1_span<U, ITER, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), smem, dev->stream, qs,
+                           scales, jobs.j[0].W, jobs.j[0].y, jobs.j[0].res, K, jobs.j[0].N);
+    else
+        hipLaunchKernelGGL((k_matvec1_span_jobs<U, ITER, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), smem,
+                           dev->stream, qs, scales, K, jobs);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }

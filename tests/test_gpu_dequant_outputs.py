@@ -66,6 +66,54 @@ def test_dequantize_f64_bit_exact(dev, fmt, n_blocks):
     assert got.dtype == np.float64 and np.array_equal(got.view(np.uint64), want.view(np.uint64))
 
 
+NONFINITE = [0x7C00, 0xFC00, 0x7E00, 0x7D00, 0xFE01, 0x7FFF]  # +inf, -inf, quiet NaN, signalling NaN, NaNs with payload
+
+
+def nonfinite_blocks(fmt, seed):
+    """Random blocks whose fp16 scale fields run through infinities and NaNs, one field at a time and together."""
+    dt = synth.BLOCK_DTYPES[fmt]
+    fields = [f for f in ("d", "m", "dmin") if f in dt.names]
+    n = len(NONFINITE) * (len(fields) + 1) + 2
+    b = synth.random_blocks(fmt, n, seed=seed).view(dt).copy()
+    if fmt == synth.Q8_K:  # an f32 scale
+        b["d"][: len(NONFINITE)] = np.array([0x7F800000, 0xFF800000, 0x7FC00000, 0x7FA00000, 0xFFC00001, 0x7FFFFFFF],
+                                            np.uint32).view(np.float32)
+        return b
+    i = 0
+    for f in fields:
+        for s in NONFINITE:
+            b[f][i] = s
+            i += 1
+    for k, s in enumerate(NONFINITE):  # every scale field of the block non-finite, with different patterns
+        for j, f in enumerate(fields):
+            b[f][i] = NONFINITE[(k + j) % len(NONFINITE)]
+        i += 1
+    return b
+
+
+@pytest.mark.parametrize("fmt", ALL, ids=name)
+def test_dequantize_with_infinite_and_nan_scales(dev, fmt):
+    # fp16ToFloat32 (quantized.go:149-173) widens an infinite scale to an infinity and a NaN scale to a NaN that
+    # keeps its payload (:156); the products then follow IEEE: inf * 0 and anything with a NaN are NaNs, the rest
+    # signed infinities.  Which NaN comes out (sign, payload, quiet bit) is not fixed by the arithmetic - the CPU's
+    # default NaN has the sign bit set, the GPU's does not, and each keeps the payload of a different operand - so
+    # NaN positions are compared as NaNs and every other element bit for bit, in each output type.
+    b = nonfinite_blocks(fmt, 5000 + fmt)
+    outputs = [(np.float32, np.uint32, o.dequantize), (np.float16, np.uint16, o.dequantize_f16)]
+    if fmt in (synth.Q4_0, synth.Q4_1, synth.Q8_0):
+        outputs.append((np.float64, np.uint64, o.dequantize_f64))
+    for dtype, bits, ref in outputs:
+        with np.errstate(all="ignore"):
+            want = np.asarray(ref(fmt, b))
+        got = dev.dequantize_blocks(fmt, b) if dtype is np.float32 else dev.dequantize_blocks_as(fmt, b, dtype)
+        got = np.asarray(got).reshape(want.shape)
+        nan = np.isnan(want)
+        # the cases are really there (the ggml-order Q4_0 is d * q + (-8 d), quantized.cu:857-866: inf - inf, all NaNs)
+        assert nan.any() and (fmt == synth.Q4_0_GGML or np.isinf(want).any()), name(fmt)
+        assert np.array_equal(np.isnan(got), nan), (name(fmt), dtype)
+        assert np.array_equal(got.view(bits)[~nan], want.view(bits)[~nan]), (name(fmt), dtype)
+
+
 def test_dequantize_outputs_errors_and_empty(dev):
     assert dev.dequantize_blocks_as(synth.Q4_K, np.zeros(0, np.uint8), np.float16).size == 0
     assert dev.dequantize_blocks_as(synth.Q8_0, np.zeros(0, np.uint8), np.float64).size == 0
