@@ -6,6 +6,14 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// Kernel attributes: threads per workgroup, and the fewest / most wavefronts per SIMD the kernel is meant to run with.
+// The fewest caps the registers (512 / MINW per lane).  The most matters as much: without it the instruction
+// scheduler works towards the highest occupancy the hardware has, and to save registers it sinks the last loads of a
+// wavefront below the first wait for memory, where they start a whole memory round trip late.  With the intended
+// occupancy stated, every load of a wavefront is issued before its first wait.
+#define CANDY_KERNEL(T, MINW, MAXW) \
+    __global__ __attribute__((amdgpu_flat_work_group_size(1, T), amdgpu_waves_per_eu(MINW, MAXW)))
+
 namespace candy {
 
 struct __attribute__((packed)) BlockQ4_0 {

@@ -52,7 +52,7 @@ struct FusedArgs {
 __device__ __forceinline__ float silu_exact(float x) { return x / (1.0f + expf(-x)); }
 
 template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
-__global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1) void k_matvec_fused(
+CANDY_KERNEL(WAVES * 64, ((EPI == EPI_PAIR && ITER == 1) ? 4 : 1), 4) void k_matvec_fused(
     const void *__restrict__ in0, const void *__restrict__ in1, const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
     const uint8_t *__restrict__ W2, int K, int e0, int e1, int e2, const FusedRest a) {
     constexpr int T = WAVES * 64;
@@ -119,6 +119,24 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
                                                  : (job[r] <= 0 ? W0 : job[r] == 1 ? W1 : W2) + (size_t)jrow[r] * rb;
 #pragma unroll
             for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
+        }
+    }
+
+    // PLAIN: where each row goes, and the residual it is added to, requested now: asked for after the reduction it
+    // would be a memory round trip (two, with the output pointer picked out of the argument block by a vector
+    // index) at the very end of every wavefront.  Rows without a residual read their own output slot (valid
+    // memory, value unused), so that nothing branches around a load.
+    float *yp[R];
+    float rv[R];
+    bool has_res[R];
+    if (EPI == EPI_PLAIN) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int j = job[r];
+            yp[r] = (j <= 0 ? a.y[0] : j == 1 ? a.y[1] : a.y[2]) + jrow[r];  // may alias the residual (h += W.x)
+            const float *rp = j <= 0 ? a.res[0] : j == 1 ? a.res[1] : a.res[2];
+            has_res[r] = rp != nullptr;
+            rv[r] = *(has_res[r] ? rp + jrow[r] : yp[r]);
         }
     }
 
@@ -191,11 +209,7 @@ __global__ __launch_bounds__(WAVES * 64, (EPI == EPI_PAIR && ITER == 1) ? 4 : 1)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float v = wave_sum(acc[0][r]);
-            if (lane == 0 && job[r] >= 0) {
-                float *y = a.y[job[r]];  // may alias res (h += W.x)
-                const float *res = a.res[job[r]];
-                y[jrow[r]] = res ? res[jrow[r]] + v : v;
-            }
+            if (lane == 0 && job[r] >= 0) *yp[r] = has_res[r] ? rv[r] + v : v;
         }
     } else {
         // A PAIR workgroup owns S = 32, 16 or 8 consecutive outputs: a whole Q8_0 block, or a part of one.  Parts

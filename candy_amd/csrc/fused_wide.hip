@@ -31,7 +31,7 @@ enum { WEPI_PLAIN = 0, WEPI_PAIR = 1 };
 struct WideHead {
     const float *x, *alpha;  // prologue input and (RMS) the norm weight
     const uint8_t *W[3];     // PLAIN: up to 3 weights as one run of rows; PAIR: W[0] gate, W[1] up
-    int total;               // rows of the run (PLAIN) or row pairs (PAIR)
+    int per_rem;             // rows of the run (PLAIN) or row pairs (PAIR) per workgroup | (the remainder << 16)
     int K;
     int e0, e1;              // PLAIN: END ROW of the first and second weight in the run
 };
@@ -52,19 +52,33 @@ struct WideArgs {
 
 __device__ __forceinline__ float wide_silu(float x) { return x / (1.0f + expf(-x)); }
 
-// First item of workgroup g when `total` items are dealt to G workgroups as evenly as they go.
-__device__ __forceinline__ int wide_start(int g, int total, int G) { return (int)(((long long)g * total) / G); }
-// The workgroup that item p falls to under wide_start.
-__device__ __forceinline__ int wide_owner(int p, int total, int G) { return (int)((((long long)p + 1) * G - 1) / total); }
+// `total` items dealt to G workgroups as evenly as they go: the first `rem` = total % G workgroups take `per` + 1 =
+// total / G + 1 items, the others `per`.  The host passes per and rem (packed: per | rem << 16), so that a workgroup
+// finds its share with a multiply and an add - a 64-bit division here was 350 scalar instructions in front of the
+// first load of every wavefront.
+__device__ __forceinline__ int wide_start(int g, int per, int rem) { return g * per + min(g, rem); }
+// How many workgroups hold a part of the 32-item block that starts at `first`, seen from workgroup g, which holds
+// one (shares are at least 8 items, so at most four boundaries between workgroups fall inside the block, none
+// further than three workgroups from g).
+__device__ __forceinline__ int wide_sharers(int first, int g, int G, int per, int rem) {
+    int n = 1;
+#pragma unroll
+    for (int d = -3; d <= 4; ++d) {
+        const int b = g + d;  // the boundary between workgroups b - 1 and b
+        const int at = wide_start(b, per, rem);
+        n += (b >= 1 && b <= G - 1 && at > first && at < first + 32) ? 1 : 0;
+    }
+    return n;
+}
 
 // Two workgroups of 8 wavefronts (or one of 16) per CU are four wavefronts per SIMD: 128 registers each.  The shapes
 // that hold up to eight rows of weights per lane are held to that (gate / up with four pairs per wavefront came to
 // 130 registers without it, one workgroup per CU at a time and two rounds: 22.5 us per launch on a 2 x 14336 x 4096
 // pair); the one-workgroup-per-CU shape with sixteen rows per lane keeps its 226.
 template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
-__global__ __launch_bounds__(WAVES * 64, ((EPI == WEPI_PAIR ? 2 : 1) * R * ITER <= 8 ? 4 : 2))
+CANDY_KERNEL(WAVES * 64, ((EPI == WEPI_PAIR ? 2 : 1) * R * ITER <= 8 ? 4 : 2), 4)
 void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha, const uint8_t *__restrict__ W0,
-                   const uint8_t *__restrict__ W1, const uint8_t *__restrict__ W2, int total, int K, int e0, int e1,
+                   const uint8_t *__restrict__ W1, const uint8_t *__restrict__ W2, int per_rem, int K, int e0, int e1,
                    const WideRest a) {
     constexpr int T = WAVES * 64;
     constexpr int CAP = ITER * 64 * U::ELEMS;   // activation values the LDS image is sized for
@@ -81,7 +95,8 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
     const int units = K / U::ELEMS;
     const size_t rb = U::row_bytes(K);
     const int G = gridDim.x;
-    const int start = wide_start(blockIdx.x, total, G), end = wide_start(blockIdx.x + 1, total, G);
+    const int per = per_rem & 0xFFFF, rem = per_rem >> 16;
+    const int start = wide_start(blockIdx.x, per, rem), end = wide_start(blockIdx.x + 1, per, rem);
     const int n4 = K >> 2;
 
     // ---- prologue inputs first (they return first)
@@ -119,6 +134,22 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
 #pragma unroll
             for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
         }
+
+    // PLAIN: where each row goes, and the residual it is added to, requested now rather than as a memory round
+    // trip after the reduction (rows without one read their own output slot: valid memory, value unused).
+    float *yp[R];
+    float rv[R];
+    bool has_res[R];
+    if (EPI == WEPI_PLAIN) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int j = job[r];
+            yp[r] = (j == 0 ? a.y[0] : j == 1 ? a.y[1] : a.y[2]) + jrow[r];  // may alias the residual (h += W.x)
+            const float *rp = j == 0 ? a.res[0] : j == 1 ? a.res[1] : a.res[2];
+            has_res[r] = rp != nullptr;
+            rv[r] = *(has_res[r] ? rp + jrow[r] : yp[r]);
+        }
+    }
 
     // ---- the activation row: normalised (or merged) and quantized into LDS, once per workgroup
     float4 val[XF];
@@ -187,11 +218,7 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float v = wave_sum(acc[0][r]);
-            if (lane == 0 && start + wave + WAVES * r < end) {
-                float *y = a.y[job[r]];  // may alias res (h += W.x)
-                const float *res = a.res[job[r]];
-                y[jrow[r]] = res ? res[jrow[r]] + v : v;
-            }
+            if (lane == 0 && start + wave + WAVES * r < end) *yp[r] = has_res[r] ? rv[r] + v : v;
         }
         return;
     }
@@ -221,7 +248,7 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
             if (lane < 32 && first + lane >= lo && first + lane < hi)
                 __hip_atomic_store(a.pair_act + first + lane, s_act[first + lane - start], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            const unsigned expected = (unsigned)(wide_owner(first + 31, total, G) - wide_owner(first, total, G) + 1);
+            const unsigned expected = (unsigned)wide_sharers(first, blockIdx.x, G, per, rem);
             unsigned old = 0;
             if (lane == 0) old = __hip_atomic_fetch_add(a.pair_tickets + blk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
@@ -244,14 +271,17 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
 }
 
 template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
-static int launch_wide_cfg(candy_hip_device *dev, const WideArgs &a, int grid) {
+static int launch_wide_cfg(candy_hip_device *dev, WideArgs a, int total, int grid) {
+    if ((EPI == WEPI_PAIR && total / grid < 8) || total / grid > 0xFFFF || grid > 0x7FFF)
+        return CANDY_HIP_ERR_UNSUPPORTED;  // what wide_sharers and the packing assume
+    a.h.per_rem = (total / grid) | ((total % grid) << 16);
     constexpr int T = WAVES * 64, CAP = ITER * 64 * U::ELEMS;
     constexpr int XF = (CAP / 4 + T - 1) / T;
     constexpr size_t QBYTES = (size_t)XF * T * 4;
     constexpr size_t smem = QBYTES + ((QBYTES >> 8) << 4) + ((size_t)XF * T / 8 + 1) * 8;
     static_assert(smem <= 48 * 1024, "LDS image too large");
     hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a.h.x,
-                       a.h.alpha, a.h.W[0], a.h.W[1], a.h.W[2], a.h.total, a.h.K, a.h.e0, a.h.e1, a.r);
+                       a.h.alpha, a.h.W[0], a.h.W[1], a.h.W[2], a.h.per_rem, a.h.K, a.h.e0, a.h.e1, a.r);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
@@ -290,53 +320,53 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
     const int cus = dev->num_cus;
     if (L.pair) {
         if (n != 2 || L.w[0]->rows != L.w[1]->rows || w0->rows % 32 != 0 || !L.pair_act || !L.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
-        a.h.total = (int)w0->rows;
-        a.h.e0 = a.h.e1 = a.h.total;
-        if (a.h.total < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
+        const int total = (int)w0->rows;
+        a.h.e0 = a.h.e1 = total;
+        if (total < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
         // one workgroup per CU; 16 wavefronts x 3 pairs while a CU's share fits, else 8 wavefronts x up to 8 pairs
         // (the weights of a wavefront's pairs stay in registers: 24 per pair and round of units)
-        const int per = (a.h.total + cus - 1) / cus;
+        const int per = (total + cus - 1) / cus;
         if (iter == 1 && dev->opt.wide_waves == 8) {  // two workgroups of eight wavefronts per CU
-            const int per2 = (a.h.total + 2 * cus - 1) / (2 * cus);
-            if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
-            if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+            const int per2 = (total + 2 * cus - 1) / (2 * cus);
+            if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
+            if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
             // four pairs per wavefront need every register: three workgroups of three pairs per CU instead, the third
             // starting when the first is done (2 x 14336 x 4096: 508 against 502 tokens/s on the Llama-3-8B shape; the
             // same step from three pairs to two loses, 509 against 539 on the 7B shape: more blocks are shared)
-            if (per2 <= 32 && (a.h.total + 3 * cus - 1) / (3 * cus) <= 24)
-                return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 3 * cus);
-            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+            if (per2 <= 32 && (total + 3 * cus - 1) / (3 * cus) <= 24)
+                return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 3 * cus);
+            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
         }
         if (iter == 1) {
-            if (per <= 32) return launch_wide_cfg<UnitQ4K, 1, 2, 16, WPRO_RMS, WEPI_PAIR>(dev, a, cus);
-            if (per <= 48) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PAIR>(dev, a, cus);
-            if (per <= 64) return launch_wide_cfg<UnitQ4K, 1, 8, 8, WPRO_RMS, WEPI_PAIR>(dev, a, cus);
-            if (per <= 96) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PAIR>(dev, a, 2 * cus);
+            if (per <= 32) return launch_wide_cfg<UnitQ4K, 1, 2, 16, WPRO_RMS, WEPI_PAIR>(dev, a, total, cus);
+            if (per <= 48) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PAIR>(dev, a, total, cus);
+            if (per <= 64) return launch_wide_cfg<UnitQ4K, 1, 8, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, cus);
+            if (per <= 96) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
         }
         return CANDY_HIP_ERR_UNSUPPORTED;
     }
-    a.h.total = rows;
+    const int total = rows;
     if (rows < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
     const int per = (rows + cus - 1) / cus;
     if (quant) {
         // the whole f32-in -> f32-out contraction of one row as one launch: measured ahead of quantize + matvec only
         // for short rows and one row per wavefront (4096 x 4096: 5.0 against 5.8 us; 11008 x 4096: 9.5 against 8.2;
         // 4096 x 11008: 9.0 against 8.9), where the prologue's 16 KB do not hold the weight stream up
-        if (iter == 1 && per <= 16) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_QUANT, WEPI_PLAIN>(dev, a, cus);
+        if (iter == 1 && per <= 16) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_QUANT, WEPI_PLAIN>(dev, a, total, cus);
         return CANDY_HIP_ERR_UNSUPPORTED;
     }
     if (iter == 1) {
         if (dev->opt.wide_waves == 8) {
             const int per2 = (rows + 2 * cus - 1) / (2 * cus);
-            if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
-            if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
-            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
+            if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, total, 2 * cus);
+            if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, total, 2 * cus);
+            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PLAIN>(dev, a, total, 2 * cus);
         }
-        if (per <= 16) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
-        if (per <= 32) return launch_wide_cfg<UnitQ4K, 1, 2, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
-        if (per <= 48) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
-        if (per <= 64) return launch_wide_cfg<UnitQ4K, 1, 4, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, cus);
-        if (per <= 128) return launch_wide_cfg<UnitQ4K, 1, 4, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, 2 * cus);
+        if (per <= 16) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, total, cus);
+        if (per <= 32) return launch_wide_cfg<UnitQ4K, 1, 2, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, total, cus);
+        if (per <= 48) return launch_wide_cfg<UnitQ4K, 1, 3, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, total, cus);
+        if (per <= 64) return launch_wide_cfg<UnitQ4K, 1, 4, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, total, cus);
+        if (per <= 128) return launch_wide_cfg<UnitQ4K, 1, 4, 16, WPRO_RMS, WEPI_PLAIN>(dev, a, total, 2 * cus);
     }
     return CANDY_HIP_ERR_UNSUPPORTED;
 }

@@ -524,7 +524,7 @@ static int launch_mb(candy_hip_device *dev, const candy_hip_qtensor *w, const in
 template <class U, int ITER, int R, int NB>
 __global__ __launch_bounds__(512, 4) void k_matvec_even(const uint8_t *__restrict__ W, const int8_t *__restrict__ xq,
                                                      const Q8Scale *__restrict__ xs, float *__restrict__ y, int N, int K,
-                                                     int m) {
+                                                     int m, int per, int rem) {
     constexpr int WAVES = 8;
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -533,8 +533,10 @@ __global__ __launch_bounds__(512, 4) void k_matvec_even(const uint8_t *__restric
     const int q_bytes = skewed(K), blocks_per_row = K >> 5;
     int8_t *sq = (int8_t *)smem;
     Q8Scale *ss = (Q8Scale *)(smem + NB * q_bytes);
-    const int G = gridDim.x;
-    const int start = (int)(((long long)blockIdx.x * N) / G), end = (int)(((long long)(blockIdx.x + 1) * N) / G);
+    // the first `rem` = N % grid workgroups take per + 1 = N / grid + 1 rows, the others per (both from the host: a
+    // 64-bit division here is some 350 scalar instructions in front of the first load)
+    const int g = blockIdx.x;
+    const int start = g * per + min(g, rem), end = (g + 1) * per + min(g + 1, rem);
 
     typename U::W w[R][ITER];
 #pragma unroll
@@ -598,7 +600,7 @@ static int launch_even_cfg(candy_hip_device *dev, const candy_hip_qtensor *w, co
     if (smem > 48 * 1024)
         CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, dev->stream, (const uint8_t *)w->data, qs, scales, y, N,
-                       K, m);
+                       K, m, N / grid, N % grid);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
