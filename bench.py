@@ -10,9 +10,16 @@ device, then the matvec.  Steps rotate over enough distinct copies of the weight
 that none of it is still in the 256 MB last-level cache when it is read again, so `value` is
 an HBM figure.  Inputs are resident in HBM before the timed region starts.
 
+A timed "step" is ONE such call.  So that a short `--steps` still gives a steady figure, every step is
+repeated `config.inner_reps` times back to back inside the timed region (at least 1000 timed calls in all) and
+`ms_per_step` / `value` are per single call; `steps` and `warmup` echo the command line.
+
 Extra objects on the same line:
   roofline     the matvec kernel alone (activations quantized before the timed region), timed
-               with HIP events on the library's stream over the same rotation.
+               with HIP events on the library's stream over the same rotation; with `fit`: launch time against
+               bytes over six weight sizes for this kernel and for a kernel that only reads (fixed_us,
+               marginal_GBps), `launch_split`: empty kernels and one-load kernels, and `sustained`: the same kernel
+               with the fixed part amortised (2 or 3 weights per launch) or hidden (two streams).
   cpu_baseline candy's literal CPU composition (dequantize, then the naive f32 matmul loops)
                restated in C, single thread, on a bounded sample of the same workload.
   sweep        the other shapes / formats of the batch-1 sweep (GB/s of the matvec kernel).
@@ -126,6 +133,68 @@ def time_matvec(dev, fmt, rows, cols, steps, warmup, quantize_each, seed=1, m=1)
     return ms / steps, len(ws)
 
 
+def linear_fit(xs, ys):
+    """Least squares y = a + b x."""
+    n = len(xs)
+    mx, my = sum(xs) / n, sum(ys) / n
+    b = sum((x - mx) * (y - my) for x, y in zip(xs, ys)) / sum((x - mx) ** 2 for x in xs)
+    return my - b * mx, b
+
+
+def launch_fit(dev, fmt, cols, launches):
+    """Launch time against bytes for the batch-1 kernel and for a kernel that only reads the same bytes, over six
+    weight sizes (rows 1024 .. 32768 at `cols` columns, 6 .. 203 MB of Q4_K), every launch on weights not in any
+    cache: time = fixed_us + bytes / marginal_GBps."""
+    from candy_amd import synth
+    pts = []
+    for rows in (1024, 2048, 4096, 8192, 16384, 32768):
+        nb = synth.weight_nbytes(fmt, rows, cols)
+        ms, _ = time_matvec(dev, fmt, rows, cols, launches, max(20, launches // 10), quantize_each=False, seed=rows)
+        span = max(2, -(-ROTATE_BYTES // nb)) * nb
+        us_read = dev.stream_probe(nb, span, launches) / launches * 1e3
+        pts.append({"rows": rows, "weight_bytes": nb, "matvec_us": round(ms * 1e3, 3), "read_only_us": round(us_read, 3)})
+        log(f"  fit {rows}x{cols}: {nb / 1e6:.1f} MB, matvec {ms * 1e3:.2f} us, read-only {us_read:.2f} us")
+    out = {"points": pts}
+    for key, name in (("matvec_us", "matvec"), ("read_only_us", "read_only")):
+        a, b = linear_fit([p["weight_bytes"] for p in pts], [p[key] for p in pts])
+        worst = max(abs(a + b * p["weight_bytes"] - p[key]) / p[key] for p in pts)
+        out[name] = {"fixed_us": round(a, 3), "marginal_GBps": round(1e-3 / b, 1), "max_rel_residual": round(worst, 4)}
+    return out
+
+
+def launch_split(dev, n=2000):
+    """Where the fixed part goes: microseconds per launch of empty kernels and of kernels whose wavefronts issue
+    exactly one load."""
+    names = ("empty_1_wavefront_us", "empty_1024x256_us", "one_load_per_wavefront_warm_us", "one_load_per_wavefront_cold_us")
+    return {name: round(dev.launch_probe(kind, n) / n * 1e3, 3) for kind, name in enumerate(names)}
+
+
+def sustained(dev, fmt, rows, cols, launches):
+    """The batch-1 kernel at the headline shape with the fixed part of a launch amortised (2 or 3 independent weights
+    sharing x in one launch: the q / k / v mechanism) or hidden (launches alternating over two streams).  Independent
+    contractions only - not the headline."""
+    from candy_amd import synth
+    ws, nbytes = make_rotation(dev, fmt, rows, cols, seed=31)
+    x = dev.from_numpy(synth.random_activations(1, cols, seed=32))
+    y = dev.alloc(4 * rows * 6)
+    out = {"note": "independent contractions (no launch waits for the previous one's result); bytes = weights + x + y "
+                   "per contraction; NOT the headline: a single serialized launch is roofline.us_per_launch"}
+    per = algorithmic_bytes(fmt, rows, cols)
+    for key, group, streams in (("weights_per_launch_2", 2, 1), ("weights_per_launch_3", 3, 1), ("two_streams", 1, 2),
+                                ("two_streams_weights_per_launch_3", 3, 2)):
+        dev.qmatmul_sustained_sweep(ws, group, streams, x, y, max(20, launches // 10))
+        ms = dev.qmatmul_sustained_sweep(ws, group, streams, x, y, launches) / launches
+        gb = per * group / (ms * 1e-3) / 1e9
+        out[key] = {"us_per_launch": round(ms * 1e3, 3), "us_per_contraction": round(ms * 1e3 / group, 3),
+                    "GBps": round(gb, 1), "frac": round(gb / HBM_PEAK_GBPS, 4)}
+        log(f"  sustained {key}: {ms * 1e3:.2f} us per launch, {gb:.0f} GB/s ({gb / HBM_PEAK_GBPS:.1%})")
+    for w in ws:
+        w.free()
+    x.free()
+    y.free()
+    return out
+
+
 def cpu_baseline(rows, cols, budget_s=12.0):
     """candy's CPU path (dequantize + naive f32 loops), C restatement, one thread."""
     from candy_amd import synth
@@ -215,7 +284,7 @@ def build_8b(dev, max_pos, seed=8000):
     return cfg, model, nbytes + synth.weight_nbytes(synth.Q6_K, 128256, 4096)
 
 
-def llama3_leg(dev, n_prompt=512, n_decode=128):
+def llama3_leg(dev, n_prompt=512, n_decode=128, not_eager=True):
     """Prefill a seeded random prompt in one batched pass, then decode greedily at batch 1."""
     log("building random-init Llama-3-8B shape (Q4_K / Q6_K down+head / Q8_0 embedding) ...")
     cfg, model, weight_bytes = build_8b(dev, max_pos=n_prompt + n_decode + 8)
@@ -241,6 +310,12 @@ def llama3_leg(dev, n_prompt=512, n_decode=128):
     dev.synchronize()
     pre_s = (time.perf_counter() - t0) / reps
     pos = n_prompt
+    # the first decoded token twice: as a replay of the captured graph and as one-by-one launches (same kernels, same
+    # cache slot rewritten with the same rows) - they must agree
+    first_graph, _ = model.decode(tok, pos, want_logits=False)
+    model.set_graph(False)
+    first_eager, _ = model.decode(tok, pos, want_logits=False)
+    model.set_graph(not_eager)
     for _ in range(4):
         tok, _ = model.decode(tok, pos, want_logits=False)
         pos += 1
@@ -263,7 +338,7 @@ def llama3_leg(dev, n_prompt=512, n_decode=128):
             "prefill_linear_TFLOPs": round(lin_flops / pre_s / 1e12, 1),
             "decode_tokens": n_decode - 4, "decode_ms_per_token": round(dec_s * 1e3, 4), "decode_tok_s": round(1 / dec_s, 2),
             "decode_bytes_per_token": bpt, "decode_hbm_frac": round(bpt / dec_s / 1e9 / HBM_PEAK_GBPS, 4),
-            "tokens": toks[:8]}
+            "tokens": toks[:8], "first_token": first_graph, "first_token_graph_equals_eager": first_graph == first_eager}
 
 
 def prefill_kv(dev, model, cfg, n_pos, seed=9):
@@ -331,6 +406,8 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-fit", action="store_true", help="skip the launch-time fit, launch split and sustained figures")
+    ap.add_argument("--fit-only", action="store_true", help="stop after the headline, fit, launch split and sustained figures")
     ap.add_argument("--no-sweep", action="store_true", help="skip the other shapes of the batch-1 sweep")
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the batched-prefill (MFMA) leg")
@@ -370,11 +447,14 @@ def main():
         a.free()
         b.free()
 
-    # headline: whole f32-in -> f32-out path
-    ms_step, n_copies = time_matvec(dev, fmt, rows, cols, args.steps, args.warmup, quantize_each=True)
+    # headline: whole f32-in -> f32-out path.  Every step is inner_reps calls back to back (>= 1000 timed calls whatever
+    # --steps is: twenty calls are 0.2 ms, one short sample); figures are per single call.
+    inner = max(1, -(-1000 // max(args.steps, 1)))
+    n_timed, n_warm = args.steps * inner, max(args.warmup * inner, 50)
+    ms_step, n_copies = time_matvec(dev, fmt, rows, cols, n_timed, n_warm, quantize_each=True)
     value = alg / (ms_step * 1e-3) / 1e9
     # dominant kernel alone
-    ms_kernel, _ = time_matvec(dev, fmt, rows, cols, args.steps, args.warmup, quantize_each=False)
+    ms_kernel, _ = time_matvec(dev, fmt, rows, cols, n_timed, n_warm, quantize_each=False)
     achieved = alg / (ms_kernel * 1e-3) / 1e9
     log(f"Q4_K {rows}x{cols}: path {ms_step * 1e3:.2f} us/step = {value:.0f} GB/s; "
         f"matvec kernel {ms_kernel * 1e3:.2f} us = {achieved:.0f} GB/s ({achieved / HBM_PEAK_GBPS:.1%} of 8 TB/s)")
@@ -391,7 +471,7 @@ def main():
         "config": {"workload": "configs[1]: Q4_K 4096x11008 (N x K) batch-1 matvec, activation quantized to Q8_0 "
                                "on device each step", "weight_bytes": synth.weight_nbytes(fmt, rows, cols),
                    "algorithmic_bytes_per_step": alg, "distinct_weight_copies": n_copies,
-                   "device": dev.name,
+                   "inner_reps": inner, "timed_calls": n_timed, "device": dev.name,
                    "decode_model": "random-init 7B: one N(0, 0.02) draw per weight shape quantized on the device by "
                                    "candy_hip_quantize (Q4_K / Q6_K quantizers restate ggml's published reference "
                                    "quantizers; parity unpinned against ggml itself), each layer taking the draw "
@@ -402,6 +482,15 @@ def main():
                      "achievable_GBps_25MB": round(floor_small, 1), "achievable_GBps_stream": round(floor_big, 1),
                      "empty_launch_us": round(us_empty, 3), "frac_of_achievable": round(achieved / floor_small, 4)},
     }
+    if not args.no_fit:
+        log("launch time against bytes (six sizes), launch split, sustained figures ...")
+        out["roofline"]["fit"] = launch_fit(dev, fmt, cols, 400)
+        out["roofline"]["launch_split"] = launch_split(dev)
+        out["roofline"]["sustained"] = sustained(dev, fmt, rows, cols, 1000)
+    if args.fit_only:
+        dev.close()
+        print(json.dumps(out))
+        return
 
     if not args.no_sweep:
         sweep = []
@@ -477,32 +566,45 @@ def main():
         out["weight_quantizers"] = wq
 
     if not args.no_sweep:
-        # the two conversions, both HBM-bound: dequantize writes 4 B per weight, quantize reads 4 B per value
+        # the two conversions, both HBM-bound: dequantize writes 4 B per weight, quantize reads 4 B per value.  Inputs AND
+        # outputs rotate over more than ROTATE_BYTES each, so neither side is served from the 256 MB last-level cache.
         conv = []
         for f, name in ((synth.Q4_K, "q4_k"), (synth.Q6_K, "q6_k"), (synth.Q8_0, "q8_0"), (synth.Q4_0, "q4_0")):
             r, k = 4096, 11008
             nb = synth.weight_nbytes(f, r, k)
-            base = synth.random_weight(f, r, k, seed=500 + f)
-            ws = [dev.qtensor(f, r, k, base) for _ in range(3)]
-            outb = dev.alloc(4 * r * k)
-            dev.dequantize_sweep(ws, outb, 5)
-            ms = dev.dequantize_sweep(ws, outb, 30) / 30
+            ws, _ = make_rotation(dev, f, r, k, seed=500 + f)
+            n_out = -(-ROTATE_BYTES // (4 * r * k))
+            outb = dev.alloc(4 * r * k * n_out)
+            dev.dequantize_sweep(ws, outb, 10, n_out)
+            ms = dev.dequantize_sweep(ws, outb, 60, n_out) / 60
             byts = nb + 4 * r * k
             conv.append({"op": "dequantize", "fmt": name, "rows": r, "cols": k, "us": round(ms * 1e3, 2),
-                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                         "rotation": f"{len(ws)} inputs, {n_out} outputs ({(nb * len(ws) + 4 * r * k * n_out) >> 20} MiB)"})
             log(f"  dequantize {name} {r}x{k}: {ms * 1e3:.1f} us, {conv[-1]['GBps']} GB/s")
             for w in ws:
                 w.free()
             outb.free()
-        for r, k, copies in ((1, 4096, 1), (512, 4096, 32)):
-            x = dev.from_numpy(synth.random_activations(r * copies, k, seed=9))
-            outb = dev.alloc(r * k // 32 * 34 + 64)
-            dev.quantize_sweep(x, r * k, copies, r, k, outb, 20)
-            ms = dev.quantize_sweep(x, r * k, copies, r, k, outb, 200) / 200
-            byts = 4 * r * k + r * k // 32 * 34
+        for r, k in ((1, 4096), (512, 4096)):
+            in_bytes, out_bytes = 4 * r * k, r * k // 32 * 34
+            copies = max(1, min(4096, -(-ROTATE_BYTES // in_bytes)))
+            n_out = max(1, min(4096, -(-ROTATE_BYTES // out_bytes)))
+            x = dev.alloc(in_bytes * copies)
+            x.zero()
+            one = synth.random_activations(r, k, seed=9)
+            for c in range(min(copies, 64)):  # N(0, 1) in the first copies, zeros in the rest (the time is the same)
+                hip._check(hip.lib().candy_hip_h2d(dev.handle, x.ptr + c * in_bytes, one.ctypes.data, in_bytes))
+            outb = dev.alloc(out_bytes * n_out + 64)
+            dev.quantize_sweep(x, r * k, copies, r, k, outb, 20, n_out)
+            ms = dev.quantize_sweep(x, r * k, copies, r, k, outb, 400, n_out) / 400
+            byts = in_bytes + out_bytes
+            label = "HBM" if in_bytes * copies >= ROTATE_BYTES else "cache-resident (launch-bound: the rotation is %d MiB)" % ((in_bytes * copies) >> 20)
             conv.append({"op": "quantize_q8_0", "rows": r, "cols": k, "us": round(ms * 1e3, 2),
-                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
-            log(f"  quantize_q8_0 {r}x{k}: {ms * 1e3:.2f} us, {conv[-1]['GBps']} GB/s")
+                         "GBps": round(byts / (ms * 1e-3) / 1e9, 1), "frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                         "memory": label})
+            log(f"  quantize_q8_0 {r}x{k}: {ms * 1e3:.2f} us, {conv[-1]['GBps']} GB/s ({label})")
+            x.free()
+            outb.free()
         out["conversions"] = conv
 
     if not args.no_prefill:
@@ -537,7 +639,7 @@ def main():
         log("decode:", out["decode"])
 
     if not args.no_llama3:
-        out["llama3_8b"] = llama3_leg(dev)
+        out["llama3_8b"] = llama3_leg(dev, not_eager=not args.eager)
         log("llama3-8b shape:", out["llama3_8b"])
 
     if not args.no_cpu:

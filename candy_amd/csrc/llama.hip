@@ -234,6 +234,12 @@ int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, s
     return CANDY_HIP_OK;
 }
 
+int candy_hip_llama_hidden(candy_hip_llama *m, const float **dev_hidden) {
+    CANDY_REQUIRE(m && dev_hidden, "nil argument");
+    *dev_hidden = m->h;
+    return CANDY_HIP_OK;
+}
+
 int candy_hip_llama_set_kv_f16(candy_hip_llama *m, int enable) {
     CANDY_REQUIRE(m, "model is nil");
     if (int rc = use_device(m->dev)) return rc;

@@ -1013,4 +1013,67 @@ int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *cons
     return CANDY_HIP_OK;
 }
 
+
+// Batch-1 contractions with the fixed part of a launch amortised or hidden: `group` weights of the rotation that share
+// the quantized activation row go out as ONE launch (the q / k / v mechanism), and with n_streams = 2 the launches
+// alternate between the handle's stream and a second one, so that one launch's start overlaps the other's tail.
+// A figure for independent contractions; the serialized single launch is what candy_hip_qmatmul_sweep times.
+int candy_hip_qmatmul_sustained_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws, int group,
+                                      int n_streams, const float *dev_x, float *dev_y, int iters, float *elapsed_ms) {
+    CANDY_REQUIRE(dev && ws && n_ws > 0 && dev_x && dev_y && elapsed_ms, "nil argument");
+    CANDY_REQUIRE(group >= 1 && group <= 3 && n_ws >= group, "1 .. 3 weights per launch, no more than the rotation holds");
+    CANDY_REQUIRE(n_streams == 1 || n_streams == 2, "one or two streams");
+    CANDY_REQUIRE(iters > 0, "invalid iteration count");
+    for (int i = 0; i < n_ws; ++i) {
+        CANDY_REQUIRE(ws[i] && ws[i]->dev == dev, "weight %d is nil or on another device", i);
+        CANDY_REQUIRE(ws[i]->cols == ws[0]->cols && ws[i]->rows == ws[0]->rows && ws[i]->fmt == ws[0]->fmt,
+                      "weights must share one shape and format");
+    }
+    CANDY_REQUIRE(format_has_batch1_kernel(ws[0]->fmt), "format has no batch-1 kernel");
+    CANDY_REQUIRE(((uintptr_t)dev_x & 15) == 0, "lhs must be 16-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    const int64_t K = ws[0]->cols, N = ws[0]->rows;
+    ActWorkspace a;
+    if (int rc = act_workspace(dev, 1, K, true, &a)) return rc;
+    if (int rc = launch_quantize_q8(dev, dev_x, 1, K, a.qs, a.scales, nullptr)) return rc;
+    hipStream_t main_stream = dev->stream, second = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    int rc = CANDY_HIP_OK;
+    hipError_t e = hipSuccess;
+    if (n_streams == 2) {
+        e = hipStreamCreateWithFlags(&second, hipStreamNonBlocking);  // default priority
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&fork, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&join, hipEventDisableTiming);
+    }
+    const int groups = n_ws / group;  // whole groups of the rotation
+    if (e == hipSuccess) e = hipEventRecord(dev->ev_start, main_stream);
+    if (e == hipSuccess && second) {
+        e = hipEventRecord(fork, main_stream);
+        if (e == hipSuccess) e = hipStreamWaitEvent(second, fork, 0);
+    }
+    for (int i = 0; i < iters && e == hipSuccess && rc == CANDY_HIP_OK; ++i) {
+        const int lane = second ? (i & 1) : 0;
+        const candy_hip_qtensor *const *w = ws + (size_t)(i % groups) * group;
+        float *ys[3];
+        for (int j = 0; j < group; ++j) ys[j] = dev_y + ((size_t)lane * group + j) * N;  // each stream its own outputs
+        dev->stream = lane ? second : main_stream;
+        rc = launch_matvec_multi(dev, w, ys, nullptr, group, a.qs, a.scales);
+    }
+    dev->stream = main_stream;
+    if (e == hipSuccess && second) {
+        e = hipEventRecord(join, second);
+        if (e == hipSuccess) e = hipStreamWaitEvent(main_stream, join, 0);
+    }
+    if (e == hipSuccess) e = hipEventRecord(dev->ev_stop, main_stream);
+    if (e == hipSuccess) e = hipEventSynchronize(dev->ev_stop);
+    if (second) (void)hipStreamSynchronize(second);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, dev->ev_start, dev->ev_stop);
+    if (fork) (void)hipEventDestroy(fork);
+    if (join) (void)hipEventDestroy(join);
+    if (second) (void)hipStreamDestroy(second);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail(CANDY_HIP_ERR_HIP, "sustained sweep failed: %s", hipGetErrorString(e));
+    return CANDY_HIP_OK;
+}
+
 }  // extern "C"

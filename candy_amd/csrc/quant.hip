@@ -336,12 +336,15 @@ int candy_hip_quantize_q8_0(candy_hip_device *dev, const float *dev_x, int64_t r
 }
 
 int candy_hip_dequantize_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws, float *dev_out,
-                               int iters, float *elapsed_ms) {
-    CANDY_REQUIRE(dev && ws && n_ws > 0 && dev_out && elapsed_ms && iters > 0, "nil argument");
+                               int n_out, int iters, float *elapsed_ms) {
+    CANDY_REQUIRE(dev && ws && n_ws > 0 && n_out > 0 && dev_out && elapsed_ms && iters > 0, "nil argument");
     if (int rc = use_device(dev)) return rc;
     CANDY_HIP_TRY(hipEventRecord(dev->ev_start, dev->stream));
-    for (int i = 0; i < iters; ++i)
-        if (int rc = candy_hip_dequantize(dev, ws[i % n_ws], dev_out)) return rc;
+    for (int i = 0; i < iters; ++i) {
+        const candy_hip_qtensor *w = ws[i % n_ws];
+        CANDY_REQUIRE(w, "weight %d is nil", i % n_ws);
+        if (int rc = candy_hip_dequantize(dev, w, dev_out + (size_t)(i % n_out) * (size_t)(w->rows * w->cols))) return rc;
+    }
     CANDY_HIP_TRY(hipEventRecord(dev->ev_stop, dev->stream));
     CANDY_HIP_TRY(hipEventSynchronize(dev->ev_stop));
     CANDY_HIP_TRY(hipEventElapsedTime(elapsed_ms, dev->ev_start, dev->ev_stop));
@@ -349,12 +352,15 @@ int candy_hip_dequantize_sweep(candy_hip_device *dev, const candy_hip_qtensor *c
 }
 
 int candy_hip_quantize_sweep(candy_hip_device *dev, const float *dev_x, int64_t x_stride, int n_x, int64_t rows,
-                             int64_t cols, void *dev_out_blocks, int iters, float *elapsed_ms) {
-    CANDY_REQUIRE(dev && dev_x && dev_out_blocks && elapsed_ms && iters > 0 && n_x > 0, "nil argument");
+                             int64_t cols, void *dev_out_blocks, int n_out, int iters, float *elapsed_ms) {
+    CANDY_REQUIRE(dev && dev_x && dev_out_blocks && elapsed_ms && iters > 0 && n_x > 0 && n_out > 0, "nil argument");
     if (int rc = use_device(dev)) return rc;
+    const size_t out_bytes = (size_t)(rows * (cols >> 5)) * sizeof(BlockQ8_0);
     CANDY_HIP_TRY(hipEventRecord(dev->ev_start, dev->stream));
     for (int i = 0; i < iters; ++i)
-        if (int rc = candy_hip_quantize_q8_0(dev, dev_x + (int64_t)(i % n_x) * x_stride, rows, cols, dev_out_blocks)) return rc;
+        if (int rc = candy_hip_quantize_q8_0(dev, dev_x + (int64_t)(i % n_x) * x_stride, rows, cols,
+                                             (uint8_t *)dev_out_blocks + (size_t)(i % n_out) * out_bytes))
+            return rc;
     CANDY_HIP_TRY(hipEventRecord(dev->ev_stop, dev->stream));
     CANDY_HIP_TRY(hipEventSynchronize(dev->ev_stop));
     CANDY_HIP_TRY(hipEventElapsedTime(elapsed_ms, dev->ev_start, dev->ev_stop));

@@ -96,16 +96,20 @@ SIGNATURES = {
     "candy_hip_llama_set_graph": (c_int, [c_void_p, c_int]),
     "candy_hip_llama_set_kv_f16": (c_int, [c_void_p, c_int]),
     "candy_hip_llama_kv_cache": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_size_t)]),
+    "candy_hip_llama_hidden": (c_int, [c_void_p, POINTER(c_void_p)]),
     "candy_hip_llama_decode": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_llama_decode_hidden": (c_int, [c_void_p, c_void_p, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_llama_prefill": (c_int, [c_void_p, POINTER(c_int32), c_int32, c_int32, POINTER(c_void_p),
                                         POINTER(c_int32)]),
     "candy_hip_qmatmul_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int64, c_void_p, c_int, c_int,
                                         POINTER(c_float)]),
-    "candy_hip_dequantize_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int, POINTER(c_float)]),
-    "candy_hip_quantize_sweep": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p, c_int,
+    "candy_hip_qmatmul_sustained_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_int, c_int, c_void_p, c_void_p, c_int,
+                                                  POINTER(c_float)]),
+    "candy_hip_dequantize_sweep": (c_int, [c_void_p, POINTER(c_void_p), c_int, c_void_p, c_int, c_int, POINTER(c_float)]),
+    "candy_hip_quantize_sweep": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p, c_int, c_int,
                                          POINTER(c_float)]),
     "candy_hip_stream_probe": (c_int, [c_void_p, c_size_t, c_size_t, c_int, POINTER(c_float)]),
+    "candy_hip_launch_probe": (c_int, [c_void_p, c_int, c_int, POINTER(c_float)]),
     "candy_hip_timer_start": (c_int, [c_void_p]),
     "candy_hip_timer_stop": (c_int, [c_void_p, POINTER(c_float)]),
 }
@@ -440,23 +444,41 @@ class Device:
                                              int(quantize_each), byref(ms)))
         return ms.value
 
-    def dequantize_sweep(self, weights: list, out_buf: "Buffer", iters: int) -> float:
+    def qmatmul_sustained_sweep(self, weights: list, group: int, n_streams: int, x_buf: "Buffer", y_buf: "Buffer",
+                                iters: int) -> float:
+        """Elapsed milliseconds of `iters` batch-1 launches of `group` weights each, alternating over `n_streams`
+        streams (y_buf: n_streams * group * rows floats)."""
         arr = (c_void_p * len(weights))(*[w.handle for w in weights])
         ms = c_float(0)
-        _check(lib().candy_hip_dequantize_sweep(self.handle, arr, len(weights), out_buf.ptr, iters, byref(ms)))
+        _check(lib().candy_hip_qmatmul_sustained_sweep(self.handle, arr, len(weights), group, n_streams, x_buf.ptr,
+                                                       y_buf.ptr, iters, byref(ms)))
+        return ms.value
+
+    def dequantize_sweep(self, weights: list, out_buf: "Buffer", iters: int, n_out: int = 1) -> float:
+        """out_buf holds n_out outputs of rows*cols f32 end to end; iteration i writes output i % n_out."""
+        arr = (c_void_p * len(weights))(*[w.handle for w in weights])
+        ms = c_float(0)
+        _check(lib().candy_hip_dequantize_sweep(self.handle, arr, len(weights), out_buf.ptr, n_out, iters, byref(ms)))
         return ms.value
 
     def quantize_sweep(self, x_buf: "Buffer", x_stride: int, n_x: int, rows: int, cols: int, out_buf: "Buffer",
-                       iters: int) -> float:
+                       iters: int, n_out: int = 1) -> float:
         ms = c_float(0)
-        _check(lib().candy_hip_quantize_sweep(self.handle, x_buf.ptr, x_stride, n_x, rows, cols, out_buf.ptr, iters,
-                                              byref(ms)))
+        _check(lib().candy_hip_quantize_sweep(self.handle, x_buf.ptr, x_stride, n_x, rows, cols, out_buf.ptr, n_out,
+                                              iters, byref(ms)))
         return ms.value
 
     def stream_probe(self, bytes_per_launch: int, span_bytes: int, iters: int) -> float:
         """Elapsed milliseconds of `iters` read-only launches (0 bytes: empty kernels)."""
         ms = c_float(0)
         _check(lib().candy_hip_stream_probe(self.handle, bytes_per_launch, span_bytes, iters, byref(ms)))
+        return ms.value
+
+    def launch_probe(self, kind: int, iters: int) -> float:
+        """Elapsed milliseconds of `iters` launches of an empty kernel (kind 0: one wavefront, 1: 1024 workgroups) or
+        of a kernel whose wavefronts issue one load each (2: cache-warm, 3: cold)."""
+        ms = c_float(0)
+        _check(lib().candy_hip_launch_probe(self.handle, kind, iters, byref(ms)))
         return ms.value
 
     def timer_start(self):
@@ -510,6 +532,14 @@ class Llama:
         k, v, n = c_void_p(), c_void_p(), c_size_t()
         _check(lib().candy_hip_llama_kv_cache(self.handle, byref(k), byref(v), byref(n)))
         return k.value, v.value, n.value
+
+    def hidden(self) -> np.ndarray:
+        """The residual stream as the last decode step left it behind the last layer (before the final norm)."""
+        p = c_void_p()
+        _check(lib().candy_hip_llama_hidden(self.handle, byref(p)))
+        out = np.empty(self.cfg.d_model, np.float32)
+        _check(lib().candy_hip_d2h(self.dev.handle, out.ctypes.data, p.value, out.nbytes))
+        return out
 
     def decode(self, token: int, pos: int, want_logits: bool = True):
         lg, nt = c_void_p(), c_int32(-1)

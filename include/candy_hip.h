@@ -310,6 +310,11 @@ int candy_hip_llama_set_kv_f16(candy_hip_llama *m, int enable);
 /* KV cache, [n_layers][n_kv_heads][max_pos][head_dim] for K and the same for V: f32, or fp16 after
  * candy_hip_llama_set_kv_f16(m, 1) (bytes_each tells which). */
 int candy_hip_llama_kv_cache(candy_hip_llama *m, float **dev_k, float **dev_v, size_t *bytes_each);
+/* The residual stream [d_model] as the last decode step left it behind its last layer (before the final norm): a
+ * device pointer owned by the model, valid until the next step.  What a candy model holds in its hidden-state tensor
+ * between blocks; lets a caller run a model one block at a time (a one-layer model per block, its input through
+ * candy_hip_llama_decode_hidden). */
+int candy_hip_llama_hidden(candy_hip_llama *m, const float **dev_hidden);
 /* One decode step: token id at position pos -> logits [vocab] (device pointer owned by the
  * model, valid until the next step) and the greedy next token.  Either output may be NULL. */
 int candy_hip_llama_decode(candy_hip_llama *m, int32_t token, int32_t pos, const float **dev_logits,
@@ -335,13 +340,22 @@ int candy_hip_llama_prefill(candy_hip_llama *m, const int32_t *tokens, int32_t n
 int candy_hip_qmatmul_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws,
                             const float *dev_x, int64_t m, float *dev_y, int iters, int quantize_each,
                             float *elapsed_ms);
-/* Same for the two bandwidth-bound conversions: `iters` dequantizations rotating over ws[]
- * (dev_out holds rows*cols f32), and `iters` Q8_0 quantizations of x[rows, cols] rotating over
- * n_x inputs spaced x_stride elements apart (dev_out_blocks holds rows*cols/32 blocks). */
+/* The two conversions timed the same way: `iters` dequantizations rotating over n_ws weights and over n_out
+ * outputs laid end to end in dev_out (n_out * rows*cols f32), and `iters` Q8_0 quantizations of x[rows, cols] rotating
+ * over n_x inputs spaced x_stride elements apart and n_out outputs end to end (each rows*cols/32 blocks).  Rotating
+ * inputs AND outputs over more bytes than the last-level cache holds makes both sides HBM traffic. */
 int candy_hip_dequantize_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws,
-                               float *dev_out, int iters, float *elapsed_ms);
+                               float *dev_out, int n_out, int iters, float *elapsed_ms);
 int candy_hip_quantize_sweep(candy_hip_device *dev, const float *dev_x, int64_t x_stride, int n_x, int64_t rows,
-                             int64_t cols, void *dev_out_blocks, int iters, float *elapsed_ms);
+                             int64_t cols, void *dev_out_blocks, int n_out, int iters, float *elapsed_ms);
+/* The same batch-1 contraction with the fixed part of a launch amortised or hidden (timing only; no counterpart in
+ * the reference): every launch contracts `group` (1 .. 3) weights of the rotation that share the one quantized
+ * activation row - the mechanism q / k / v use, after mul_mat_vec_q's one weight per launch (quantized.cu:2787-2871)
+ * - and with n_streams = 2 the launches alternate between the handle's stream and a second stream the call creates,
+ * so that one launch starts while the other drains.  dev_y holds n_streams * group * rows floats.  A figure for
+ * independent contractions: a caller whose next contraction needs this one's result gets candy_hip_qmatmul_sweep's. */
+int candy_hip_qmatmul_sustained_sweep(candy_hip_device *dev, const candy_hip_qtensor *const *ws, int n_ws, int group,
+                                      int n_streams, const float *dev_x, float *dev_y, int iters, float *elapsed_ms);
 /* What the device delivers to a kernel that only reads (no counterpart in the reference; the matvec's bytes per
  * second are quoted against it beside the published peak).  `iters` launches back to back, launch i reading
  * bytes_per_launch bytes (a multiple of 16) with 16-byte loads from region i of a scratch buffer of span_bytes
@@ -350,6 +364,12 @@ int candy_hip_quantize_sweep(candy_hip_device *dev, const float *dev_x, int64_t 
  * on the handle's stream around the loop. */
 int candy_hip_stream_probe(candy_hip_device *dev, size_t bytes_per_launch, size_t span_bytes, int iters,
                            float *elapsed_ms);
+/* Where the fixed part of a launch goes (no counterpart in the reference; bench.py reports it beside the headline
+ * kernel).  `iters` launches back to back of: kind 0 an empty kernel of one wavefront; 1 an empty kernel of 1024
+ * workgroups x 256 threads (the grid of a 4096-row batch-1 contraction); 2 that grid with every wavefront issuing
+ * one 16-byte load per lane, rows 6192 bytes apart, the same lines every launch (cache-warm); 3 the same with every
+ * launch in a region of its own out of 640 MiB (cold).  Returns the time between HIP events around the loop. */
+int candy_hip_launch_probe(candy_hip_device *dev, int kind, int iters, float *elapsed_ms);
 int candy_hip_timer_start(candy_hip_device *dev);
 int candy_hip_timer_stop(candy_hip_device *dev, float *elapsed_ms);   /* synchronises */
 

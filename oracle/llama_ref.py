@@ -77,11 +77,15 @@ class LlamaRef:
         rb = o.block_bytes(fmt) * (self.c["d_model"] // o.block_elems(fmt))
         return o.dequantize(fmt, blocks[token * rb:(token + 1) * rb])
 
-    def step(self, h: np.ndarray, pos: int):
+    def step(self, h: np.ndarray, pos: int, trace: list | None = None):
+        """trace (optional): receives, per layer, the hidden state in front of the layer and the one between its
+        attention and feed-forward halves, then the one behind the last layer (2 * n_layers + 1 arrays)."""
         c = self.c
         d, hd, nh, nkv, ffn = c["d_model"], c["head_dim"], c["n_heads"], c["n_kv_heads"], c["d_ffn"]
         h = np.ascontiguousarray(h, np.float32).copy()
         for l in range(c["n_layers"]):
+            if trace is not None:
+                trace.append(h.copy())
             xn = o.fast_rms_norm(h, d, c["rms_eps"], self.w[("attn_norm", l)])
             q = self._lin("q", l, xn, nh * hd, d)
             k = self._lin("k", l, xn, nkv * hd, d)
@@ -95,11 +99,15 @@ class LlamaRef:
             att = o.attention_decode(q, self.k_cache[l], self.v_cache[l], nh, nkv, hd, pos + 1,
                                      c["max_pos"] * hd, 1.0 / math.sqrt(hd))
             h = o.add(h, self._lin("o", l, att, d, nh * hd))
+            if trace is not None:
+                trace.append(h.copy())
             xn = o.fast_rms_norm(h, d, c["rms_eps"], self.w[("ffn_norm", l)])
             g = self._lin("gate", l, xn, ffn, d)
             u = self._lin("up", l, xn, ffn, d)
             act = o.mul(o.silu(g), u)
             h = o.add(h, self._lin("down", l, act, d, ffn))
+        if trace is not None:
+            trace.append(h.copy())
         xn = o.fast_rms_norm(h, d, c["rms_eps"], self.w[("out_norm", -1)])
         logits = self._lin("head", -1, xn, c["vocab"], d)
         return int(o.fast_argmax(logits, c["vocab"])[0]), logits, h

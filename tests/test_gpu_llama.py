@@ -245,6 +245,143 @@ def test_full_depth_7b_step_within_activation_noise(dev):
     model.free()
 
 
+def test_full_depth_7b_half_layers_teacher_forced(dev):
+    # The benchmark's model again (32 layers 4096 / 11008, every matrix N(0, 0.02) quantized on the device, 2048 cached
+    # positions of N(0, 1)), held to the per-op bar at every layer.  The CPU composition runs the whole step once and
+    # records the hidden state in front of every layer and between its two halves.  The device then runs each HALF
+    # layer on its own from the CPU's input for it - a one-layer model with that layer's weights and cache rows whose
+    # other half is switched off with all-zero weights (zero FFN: the output is h + Wo.att; zero Wo: the attention
+    # adds nothing and the output is h + Wdown.act) - and its k / v rows and output must match the CPU's to 1e-3.
+    # A half layer is the longest stretch this bar can be asked of: it re-quantizes twice (norm output, then the
+    # attention output or SiLU*Mul), a last-place difference may flip a rounding at the second quantizer, and with no
+    # third quantizer behind it that moves the output by a few 1e-4 at most.  A whole layer has a third and fourth, where such a
+    # flip is amplified to several 1e-3 (CPU evaluations in another summation order differ as much): the drift the
+    # end-to-end test allows for.  Here it cannot hide a wrong layer.
+    n_layers, n_pos = 32, 2048
+    cfg = dict(n_layers=n_layers, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=11008, vocab=256,
+               max_pos=n_pos + 8, rms_eps=1e-5, rope_base=10000.0)
+    shapes = {"q": (4096, 4096), "k": (4096, 4096), "v": (4096, 4096), "o": (4096, 4096), "gate": (11008, 4096),
+              "up": (11008, 4096), "down": (4096, 11008)}
+
+    def drawn(fmt, r, k, seed):
+        x = np.random.Generator(np.random.Philox(seed)).standard_normal((r, k), dtype=np.float32) * np.float32(0.02)
+        return dev.quantize(fmt, x)
+
+    base = {rk: drawn(synth.Q4_K, rk[0], rk[1], 300 + rk[0] + rk[1]).reshape(-1, 144) for rk in set(shapes.values())}
+    rng = np.random.default_rng(17)
+    host, qts, shift = {}, {}, 0
+    for l in range(n_layers):
+        for kind, (r, k) in shapes.items():
+            shift += 1
+            b = np.roll(base[(r, k)], 977 * shift, axis=0).reshape(-1)
+            host[(kind, l)] = (synth.Q4_K, b)
+            qts[(kind, l)] = dev.qtensor(synth.Q4_K, r, k, b)
+        for kind in ("attn_norm", "ffn_norm"):
+            host[(kind, l)] = (1 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
+    zero = {kind: dev.qtensor(synth.Q4_K, r, k, np.zeros(synth.weight_nbytes(synth.Q4_K, r, k), np.uint8))
+            for kind, (r, k) in shapes.items() if kind in ("o", "gate", "up", "down")}
+    host[("out_norm", -1)] = np.ones(4096, np.float32)
+    for kind, fmt, seed in (("head", synth.Q6_K, 7), ("embed", synth.Q8_0, 8)):
+        host[(kind, -1)] = (fmt, drawn(fmt, cfg["vocab"], 4096, seed))
+    # CPU: one full step with a trace
+    crng = np.random.Generator(np.random.Philox(19))
+    ref = llama_ref.LlamaRef(dict(cfg, max_pos=1), host)
+    ref.c = cfg
+    ref.k_cache = np.zeros((n_layers, 32, cfg["max_pos"], 128), np.float32)
+    ref.v_cache = np.zeros_like(ref.k_cache)
+    ref.k_cache[:, :, :n_pos] = crng.standard_normal((n_layers, 32, n_pos, 128), dtype=np.float32)
+    ref.v_cache[:, :, :n_pos] = crng.standard_normal((n_layers, 32, n_pos, 128), dtype=np.float32)
+    ref.cos, ref.sin = llama_ref.rope_tables(cfg["max_pos"], 128, cfg["rope_base"])
+    trace = []
+    ref.step(ref.embed(77), n_pos, trace=trace)
+    assert len(trace) == 2 * n_layers + 1
+    # device: half a layer at a time from the CPU's inputs
+    one = hip.Llama(dev, **dict(cfg, n_layers=1))
+    one.set_norm(hip.W_OUT_NORM, -1, host[("out_norm", -1)])
+    for kind in ("head", "embed"):
+        fmt, b = host[(kind, -1)]
+        one.set_qweight(KINDS[kind], -1, dev.qtensor(fmt, cfg["vocab"], 4096, b))
+    kptr, vptr, nbytes = one.kv_cache()
+    worst = {"k": 0.0, "v": 0.0, "attention half": 0.0, "ffn half": 0.0}
+    for l in range(n_layers):
+        for kind in ("attn_norm", "ffn_norm"):
+            one.set_norm(KINDS[kind], 0, host[(kind, l)])
+        for ptr, cache in ((kptr, ref.k_cache), (vptr, ref.v_cache)):
+            rows = cache[l].copy()
+            rows[:, n_pos] = 0  # the row this step writes
+            hip._check(hip.lib().candy_hip_h2d(dev.handle, ptr, rows.ctypes.data, rows.nbytes))
+        # attention half: the feed-forward weights are zero
+        for kind in shapes:
+            one.set_qweight(KINDS[kind], 0, zero[kind] if kind in ("gate", "up", "down") else qts[(kind, l)])
+        one.decode_hidden(trace[2 * l], n_pos, want_logits=False)
+        h_mid = one.hidden()
+        kc, vc = read_cache(dev, one, (1, 32, cfg["max_pos"], 128))
+        errs = {"k": rel(kc[0, :, n_pos], ref.k_cache[l, :, n_pos].astype(np.float64)),
+                "v": rel(vc[0, :, n_pos], ref.v_cache[l, :, n_pos].astype(np.float64)),
+                "attention half": rel(h_mid, trace[2 * l + 1].astype(np.float64))}
+        assert np.array_equal(kc[0, :, :n_pos], ref.k_cache[l, :, :n_pos])  # nothing but the new row was touched
+        # feed-forward half: Wo is zero, so the hidden state reaches the FFN as it was given
+        for kind in shapes:
+            one.set_qweight(KINDS[kind], 0, zero[kind] if kind == "o" else qts[(kind, l)])
+        one.decode_hidden(trace[2 * l + 1], n_pos, want_logits=False)
+        errs["ffn half"] = rel(one.hidden(), trace[2 * l + 2].astype(np.float64))
+        for key, e in errs.items():
+            worst[key] = max(worst[key], e)
+            assert e <= 1e-3, (l, key, e)
+    print("teacher-forced half layers, worst over 32 layers: " + ", ".join(f"{k} {v:.2e}" for k, v in worst.items()))
+    one.free()
+    for q in list(qts.values()) + list(zero.values()):
+        q.free()
+
+
+def test_full_depth_llama3_8b_shape_step(dev):
+    # The Llama-3-8B-shaped model of the benchmark at full depth: 32 layers, 32 query / 8 kv heads x 128, d_ffn 14336,
+    # vocab 128256, Q4_K attention and gate / up, Q6_K down (K = 14336 on the batch-1 kernel of its own) and head (the
+    # norm launch + batch-1 path of a vocabulary-sized Q6_K head), Q8_0 embedding rows; 512 cached positions of
+    # N(0, 1), one decode step from an embedding row.  The bar is the one the 7B step has: no further from the CPU
+    # composition than 1.5 times the distance between CPU evaluations that add each row's blocks in another order
+    # (or 1e-3 where that is larger), and the same token picked by all of them.
+    n_layers, n_pos = 32, 512
+    cfg = dict(n_layers=n_layers, d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, d_ffn=14336, vocab=128256,
+               max_pos=n_pos + 8, rms_eps=1e-5, rope_base=500000.0)
+    fmts = {"default": synth.Q4_K, "down": synth.Q6_K, "head": synth.Q6_K, "embed": synth.Q8_0}
+    host, model = build(dev, cfg, fmts, seed=88)
+    rng = np.random.Generator(np.random.Philox(89))
+    kptr, vptr, _ = model.kv_cache()
+    caches = []
+    for ptr in (kptr, vptr):
+        full = np.zeros((n_layers, 8, cfg["max_pos"], 128), np.float32)
+        full[:, :, :n_pos] = rng.standard_normal((n_layers, 8, n_pos, 128), dtype=np.float32)
+        hip._check(hip.lib().candy_hip_h2d(dev.handle, ptr, full.ctypes.data, full.nbytes))
+        caches.append(full)
+    tok, pos = 100000, n_pos
+    nt, logits = model.decode(tok, pos)
+
+    def cpu(**kw):
+        ref = llama_ref.LlamaRef(dict(cfg, max_pos=1), host, **kw)
+        ref.c = cfg
+        ref.k_cache, ref.v_cache = caches
+        ref.cos, ref.sin = llama_ref.rope_tables(cfg["max_pos"], 128, cfg["rope_base"])
+        t, lg, _ = ref.step(ref.embed(tok), pos)
+        return t, lg.astype(np.float64)
+
+    rt, rlogits = cpu()
+    alts = [cpu(block_order=k) for k in (1, 2)]
+    drift = max(rel(a[1], rlogits) for a in alts)
+    err = rel(logits, rlogits)
+    print(f"8B shape: device vs CPU {err:.2e}; CPU vs CPU in another summation order {[float('%.2e' % rel(a[1], rlogits)) for a in alts]}")
+    assert err <= max(1e-3, 1.5 * drift), (err, drift)
+    assert nt == int(np.argmax(logits))
+    top2 = np.sort(rlogits)[-2:]
+    if top2[1] - top2[0] > 2 * max(err, drift) * np.max(np.abs(rlogits)):
+        assert nt == rt and all(a[0] == rt for a in alts)
+    # the new k / v rows of the first layer (one quantizer upstream) hold the per-op bar
+    kc, vc = read_cache(dev, model, (n_layers, 8, cfg["max_pos"], 128))
+    assert rel(kc[0, :, pos], caches[0][0, :, pos].astype(np.float64)) <= 1e-3
+    assert rel(vc[0, :, pos], caches[1][0, :, pos].astype(np.float64)) <= 1e-3
+    model.free()
+
+
 @pytest.mark.parametrize("d_ffn", [11008, 14336])
 def test_long_cache_step_on_the_even_split_kernels(dev, d_ffn):
     # One full-width 7B layer over a cache of 600 positions with q/k/v and gate/up on the kernels that deal the rows
