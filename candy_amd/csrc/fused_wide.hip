@@ -224,11 +224,22 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
     }
 
     // ---- PAIR: silu(gate) * up of this workgroup's pairs, then the 32-value blocks they belong to
+    // Without a quantized output (oq null) the f32 values go to pair_act as they are and the consumer quantizes them in
+    // its own prologue (the down projection, QUANT prologue): no block is shared between workgroups then, no tickets.
+    const bool f32_out = a.oq == nullptr;  // uniform
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const float g = wave_sum(acc[0][r]), u = wave_sum(acc[1][r]);
-        if (lane == 0) s_act[wave + WAVES * r] = wide_silu(g) * u;  // slots past `end` hold a clamped row: never read
+        const float act = wide_silu(g) * u;
+        if (lane == 0) {
+            if (f32_out) {
+                if (start + wave + WAVES * r < end) a.pair_act[jrow[r]] = act;
+            } else {
+                s_act[wave + WAVES * r] = act;  // slots past `end` hold a clamped row: never read
+            }
+        }
     }
+    if (f32_out) return;
     __syncthreads();
     const int b0 = start >> 5, b1 = (end - 1) >> 5;
     for (int blk = b0 + wave; blk <= b1; blk += WAVES) {  // wavefront-uniform: one block per wavefront
@@ -289,6 +300,16 @@ static int launch_wide_cfg(candy_hip_device *dev, WideArgs a, int total, int gri
 // The shapes these kernels exist for: Q4_K weights, rows up to 8192 values (two rounds of units), at least a
 // few rows per wavefront.  Anything else: CANDY_HIP_ERR_UNSUPPORTED without error text (the caller takes the
 // narrower kernels).
+// One Q4_K weight with rows of 4097 .. 16384 values and at most eight rows per workgroup at two workgroups per CU, f32
+// input quantized in the prologue: what the decode step's down projection asks for.
+bool wide_quant_long_covers(const candy_hip_device *dev, const WideLaunch &L) {
+    if (!dev->opt.fused_wide || !dev->opt.down_quant || L.n != 1 || L.alpha || L.pair || !L.x || ((uintptr_t)L.x & 15) != 0) return false;
+    const candy_hip_qtensor *w = L.w[0];
+    if (w->fmt != CANDY_HIP_Q4_K || ((uintptr_t)w->data & 15) != 0 || w->cols % 256 != 0) return false;
+    const int iter = (int)((w->cols / 64 + 63) / 64);
+    return iter >= 2 && iter <= 4 && w->rows >= 4 * (int64_t)dev->num_cus && w->rows <= 16 * (int64_t)dev->num_cus;
+}
+
 int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
     const int n = L.n;
     if (n < 1 || n > 3 || !dev->opt.fused_wide) return CANDY_HIP_ERR_UNSUPPORTED;
@@ -298,9 +319,9 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
         if (L.w[i]->rows > 0x3FFFFFFF) return CANDY_HIP_ERR_UNSUPPORTED;
     }
     const int64_t K = w0->cols;
-    if (K % 256 != 0 || K > 8192) return CANDY_HIP_ERR_UNSUPPORTED;
-    const int iter = (int)((K / 64 + 63) / 64);
     const bool quant = L.alpha == nullptr;
+    if (K % 256 != 0 || K > (quant ? 16384 : 8192)) return CANDY_HIP_ERR_UNSUPPORTED;
+    const int iter = (int)((K / 64 + 63) / 64);
     if (!L.x || ((uintptr_t)L.x & 15) != 0) return CANDY_HIP_ERR_UNSUPPORTED;
     if (quant && L.pair) return CANDY_HIP_ERR_UNSUPPORTED;
     WideArgs a{};
@@ -320,6 +341,7 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
     const int cus = dev->num_cus;
     if (L.pair) {
         if (n != 2 || L.w[0]->rows != L.w[1]->rows || w0->rows % 32 != 0 || !L.pair_act || !L.pair_tickets) return CANDY_HIP_ERR_UNSUPPORTED;
+        if (iter != 1) return CANDY_HIP_ERR_UNSUPPORTED;
         const int total = (int)w0->rows;
         a.h.e0 = a.h.e1 = total;
         if (total < 16 * cus) return CANDY_HIP_ERR_UNSUPPORTED;
@@ -352,7 +374,16 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
         // the whole f32-in -> f32-out contraction of one row as one launch: measured ahead of quantize + matvec only
         // for short rows and one row per wavefront (4096 x 4096: 5.0 against 5.8 us; 11008 x 4096: 9.5 against 8.2;
         // 4096 x 11008: 9.0 against 8.9), where the prologue's 16 KB do not hold the weight stream up
-        if (iter == 1 && per <= 16) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_QUANT, WEPI_PLAIN>(dev, a, total, cus);
+        if (iter == 1 && per <= 16 && !L.res[0]) return launch_wide_cfg<UnitQ4K, 1, 1, 16, WPRO_QUANT, WEPI_PLAIN>(dev, a, total, cus);
+        // long rows, one row per wavefront, two workgroups of eight per CU: the down projection of a decode step taking
+        // the f32 SiLU*Mul values as they come (the gate / up launch then has no 32-value blocks to hand between
+        // workgroups)
+        if (wide_quant_long_covers(dev, L)) switch (iter) {
+            case 2: return launch_wide_cfg<UnitQ4K, 2, 1, 8, WPRO_QUANT, WEPI_PLAIN>(dev, a, total, 2 * cus);
+            case 3: return launch_wide_cfg<UnitQ4K, 3, 1, 8, WPRO_QUANT, WEPI_PLAIN>(dev, a, total, 2 * cus);
+            case 4: return launch_wide_cfg<UnitQ4K, 4, 1, 8, WPRO_QUANT, WEPI_PLAIN>(dev, a, total, 2 * cus);
+            default: break;
+            }
         return CANDY_HIP_ERR_UNSUPPORTED;
     }
     if (iter == 1) {

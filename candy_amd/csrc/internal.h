@@ -72,6 +72,7 @@ struct Options {
     int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
     int fused_wide = 1;          // decode step: one-workgroup-per-CU kernels for the big Q4_K shapes (0: the narrower ones)
     int wide_waves = 8;          // wavefronts per workgroup of those kernels: 8 (two workgroups per CU) or 16 (one)
+    int down_quant = 0;          // decode step: 1 = gate / up leaves f32 SiLU*Mul values and the down projection quantizes them in its prologue (measured slower: 561 against 583 tok/s on the 7B shape); 0 = gate / up quantizes, blocks shared between workgroups through tickets
 };
 
 }  // namespace candy
@@ -90,6 +91,7 @@ struct SplitPending {
 struct candy_hip_device {
     int ordinal = 0;
     candy::Options opt;
+    unsigned opt_epoch = 0;  // counts candy_hip_set_option calls: a decoder's captured graph is stale when it moved
     hipStream_t stream = nullptr;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int num_cus = 0;
@@ -262,6 +264,8 @@ struct WideLaunch {
     unsigned *pair_tickets = nullptr;
 };
 int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &launch);
+// whether launch_matvec_wide takes this launch on its long-row QUANT shape (the decode step's down projection)
+bool wide_quant_long_covers(const candy_hip_device *dev, const WideLaunch &launch);
 // attention.hip
 struct AttnLaunch {
     const float *q = nullptr;      // [n_heads, head_dim]; pre-Rope when k_new is set

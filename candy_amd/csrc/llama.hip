@@ -40,6 +40,7 @@ struct candy_hip_llama {
     hipGraphExec_t graph_exec = nullptr;
     bool graph_dirty = true;
     bool use_graph = true;
+    unsigned graph_epoch = 0;                     // the device's option epoch the graph was captured under
     std::vector<void *> owned;
     // prompt buffers, grown on demand to the longest prompt seen: [n][width] activations
     struct Prompt {
@@ -345,11 +346,22 @@ static int llama_enqueue_step(candy_hip_llama *m) {
             Wd.n = 2; Wd.w[0] = L.gate; Wd.w[1] = L.up; Wd.pair = true;
             Wd.x = m->h; Wd.alpha = L.ffn_norm; Wd.eps = c.rms_eps; Wd.oq = m->xq; Wd.os = m->xs;
             Wd.pair_act = m->gate_o; Wd.pair_tickets = m->pair_tickets;
+            // Where the down projection can quantize its input itself, gate / up leaves the f32 values: the same 32
+            // values per block quantized by the same code, so the same bits, without blocks shared between workgroups.
+            WideLaunch Dn;
+            Dn.n = 1; Dn.w[0] = L.down; Dn.y[0] = m->h; Dn.res[0] = m->h; Dn.x = m->gate_o;
+            const bool down_quant = wide_quant_long_covers(dev, Dn);
+            if (down_quant) { Wd.oq = nullptr; Wd.os = nullptr; }
             rc = launch_matvec_wide(dev, Wd);
             if (rc == CANDY_HIP_OK) {
+                if (down_quant) {
+                    if ((rc = launch_matvec_wide(dev, Dn))) return rc;  // h += Wdown . q8(act)
+                    continue;
+                }
                 if ((rc = linear_residual(m, L.down))) return rc;  // h += Wdown . act
                 continue;
             }
+            if (down_quant && rc == CANDY_HIP_ERR_UNSUPPORTED) return fail(CANDY_HIP_ERR_HIP, "internal: gate / up launch refused");
             if (rc != CANDY_HIP_ERR_UNSUPPORTED) return rc;
             FusedLaunch F;
             F.n = 2; F.w[0] = L.gate; F.w[1] = L.up; F.pair = true;
@@ -386,6 +398,7 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
         if ((rc = candy_hip_qindex_select(dev, m->embed, m->tok_id, 1, m->h))) return rc;
     }
     if (m->use_graph) {
+        if (m->graph_epoch != dev->opt_epoch) m->graph_dirty = true;  // an option changed: other kernels may be due
         if (m->graph_dirty) {
             // a replay of the old graph may still be in flight (a caller that did not ask for the token): drain first
             if (m->graph_exec) CANDY_HIP_TRY(hipStreamSynchronize(dev->stream));
@@ -403,6 +416,7 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
             CANDY_HIP_TRY(e);
             CANDY_HIP_TRY(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
             m->graph_dirty = false;
+            m->graph_epoch = dev->opt_epoch;
         }
         CANDY_HIP_TRY(hipGraphLaunch(m->graph_exec, dev->stream));
     } else if ((rc = llama_enqueue_step(m))) {

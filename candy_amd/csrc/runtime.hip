@@ -364,6 +364,7 @@ const OptionKey OPTION_KEYS[] = {
     {"llama.graph", &candy::Options::llama_graph, 0, 1},
     {"fused.wide", &candy::Options::fused_wide, 0, 1},
     {"fused.wide_waves", &candy::Options::wide_waves, 8, 16},
+    {"fused.down_quant", &candy::Options::down_quant, 0, 1},
 };
 const OptionKey *find_option(const char *key) {
     for (const OptionKey &k : OPTION_KEYS)
@@ -378,11 +379,15 @@ int candy_hip_set_option(candy_hip_device *dev, const char *key, int64_t value) 
     CANDY_REQUIRE(k, "unknown option \"%s\"", key);
     CANDY_REQUIRE(value >= k->lo && value <= k->hi, "option %s takes %d .. %d, got %lld", key, k->lo, k->hi, (long long)value);
     dev->opt.*(k->field) = (int)value;
+    ++dev->opt_epoch;  // decoders notice and capture their step again under the new options
     return CANDY_HIP_OK;
 }
 
 int candy_hip_get_option(const candy_hip_device *dev, const char *key, int64_t *value) {
     CANDY_REQUIRE(dev && key && value, "nil argument");
+    // read-only: what the handle's grow-only workspaces hold at the moment
+    if (strcmp(key, "runtime.workspace_bytes") == 0) { *value = (int64_t)dev->ws_bytes; return CANDY_HIP_OK; }
+    if (strcmp(key, "runtime.split_workspace_bytes") == 0) { *value = (int64_t)dev->ws_split_bytes; return CANDY_HIP_OK; }
     const OptionKey *k = find_option(key);
     CANDY_REQUIRE(k, "unknown option \"%s\"", key);
     *value = dev->opt.*(k->field);

@@ -108,12 +108,20 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *   "fused.rms_rows"             0        fused RMSNorm prologue: rows per workgroup 16 / 24 (0: most even split)
  *   "fused.wide"                 1        decode step: kernels that deal the rows of the big Q4_K shapes evenly over the CUs
  *   "fused.wide_waves"           8        wavefronts per workgroup of those kernels: 8 (two workgroups per CU) or 16 (one)
+ *   "fused.down_quant"           0        decode step, comparison runs and tests: 1 = the gate / up launch leaves its f32
+ *                                         SiLU*Mul values and the down projection quantizes them in its own prologue (0: gate /
+ *                                         up quantizes them, handing 32-value blocks that two workgroups share through
+ *                                         per-block tickets); same bits, measured slower
  *   "prefill.qkv_group"          1        prompt pass: projections that share their input (q / k / v; gate / up) as one
  *                                         grid each where all of them run on the fp16 tiles (0: one launch each)
  *   "prefill.fold_split_sums"    1        prompt pass: the partial copies a projection split along K leaves are summed by the
  *                                         launch that follows (RMSNorm + quantize behind o / down, rope behind q / k / v;
  *                                         0: a launch of its own sums them)
- *   "prefill.attention_valu"     0        prompt attention for head_dim 128 on the vector ALU */
+ *   "prefill.attention_valu"     0        prompt attention for head_dim 128 on the vector ALU
+ * A decoder whose step has been captured into a graph notices a later candy_hip_set_option on its device and captures
+ * the step again at its next decode call.
+ * Read-only keys (candy_hip_get_option): "runtime.workspace_bytes", "runtime.split_workspace_bytes" - what the
+ * handle's two grow-only workspaces hold at the moment (0 until a call needs them). */
 int candy_hip_set_option(candy_hip_device *dev, const char *key, int64_t value);
 int candy_hip_get_option(const candy_hip_device *dev, const char *key, int64_t *value);
 

@@ -54,6 +54,82 @@ def tiny_model(seed=1, tied=False, fmts=None):
     return cfg, meta, tensors, orig
 
 
+@pytest.mark.parametrize("version", [2, 3])
+def test_reader_on_bytes_assembled_by_hand_from_the_published_layout(tmp_path, version):
+    # Every other test here reads files that write_gguf wrote: a misreading of the format shared by reader and writer
+    # would pass them all.  This file is put together byte by byte from the constants of the published GGUF
+    # specification (ggml docs/gguf.md), with struct.pack and literal numbers only - nothing from candy_amd.gguf:
+    #   header   magic "GGUF" = 0x46554747 little endian, u32 version, u64 tensor count, u64 metadata count
+    #   string   u64 length + UTF-8 bytes, no terminator
+    #   value    u32 type, then the value; types UINT8 0, INT8 1, UINT16 2, INT16 3, UINT32 4, INT32 5, FLOAT32 6,
+    #            BOOL 7 (one byte), STRING 8, ARRAY 9 (u32 element type, u64 count, elements), UINT64 10, INT64 11,
+    #            FLOAT64 12
+    #   tensor   name string, u32 n_dims, u64 dims[n_dims] (dims[0] the contiguous one), u32 ggml type (F32 0, F16 1,
+    #            Q4_0 2, Q8_0 8, Q4_K 12, Q6_K 14, ...), u64 offset from the start of the data section
+    #   data     starts at the next multiple of general.alignment (default 32) after the last tensor info; every
+    #            tensor offset is a multiple of it
+    def gstr(t):
+        b = t.encode("utf-8")
+        return struct.pack("<Q", len(b)) + b
+
+    kv = [
+        gstr("general.architecture") + struct.pack("<I", 8) + gstr("llama"),
+        gstr("general.alignment") + struct.pack("<II", 4, 64),
+        gstr("t.u8") + struct.pack("<IB", 0, 200),
+        gstr("t.i8") + struct.pack("<Ib", 1, -100),
+        gstr("t.u16") + struct.pack("<IH", 2, 60000),
+        gstr("t.i16") + struct.pack("<Ih", 3, -30000),
+        gstr("t.i32") + struct.pack("<Ii", 5, -2000000000),
+        gstr("t.f32") + struct.pack("<If", 6, 0.15625),
+        gstr("t.bool") + struct.pack("<IB", 7, 1),
+        gstr("t.u64") + struct.pack("<IQ", 10, 2 ** 63 + 5),
+        gstr("t.i64") + struct.pack("<Iq", 11, -(2 ** 62)),
+        gstr("t.f64") + struct.pack("<Id", 12, 1.0 / 3.0),
+        gstr("t.strs") + struct.pack("<IIQ", 9, 8, 3) + gstr("a") + gstr("") + gstr("h\u00e9llo"),
+        gstr("t.ints") + struct.pack("<IIQ", 9, 5, 4) + struct.pack("<4i", 7, -8, 9, -10),
+        gstr("t.floats") + struct.pack("<IIQ", 9, 6, 2) + struct.pack("<2f", 0.5, -2.0),
+    ]
+    # tensor 0: F32 vector of 8 values (32 bytes) at offset 0; tensor 1: Q8_0 matrix, 64 columns x 2 rows = 4 blocks of
+    # 34 bytes, at the next multiple of 64; tensor 2: Q4_K 256 columns x 1 row = 144 bytes, after 136 -> offset 256
+    vec = struct.pack("<8f", *[0.25 * i for i in range(8)])
+    q8 = bytes((37 * i + 11) % 256 for i in range(4 * 34))
+    q4k = bytes((91 * i + 3) % 256 for i in range(144))
+    infos = [
+        gstr("vec.weight") + struct.pack("<I", 1) + struct.pack("<Q", 8) + struct.pack("<IQ", 0, 0),
+        gstr("blk.0.q8.weight") + struct.pack("<I", 2) + struct.pack("<QQ", 64, 2) + struct.pack("<IQ", 8, 64),
+        gstr("blk.0.q4k.weight") + struct.pack("<I", 2) + struct.pack("<QQ", 256, 1) + struct.pack("<IQ", 12, 256),
+    ]
+    head = b"GGUF" + struct.pack("<IQQ", version, len(infos), len(kv)) + b"".join(kv) + b"".join(infos)
+    assert head[:4] == struct.pack("<I", 0x46554747)
+    pad = (-len(head)) % 64
+    data = vec + b"\x00" * 32 + q8 + b"\x00" * (256 - 64 - len(q8)) + q4k
+    path = tmp_path / "hand.gguf"
+    path.write_bytes(head + b"\x00" * pad + data)
+
+    g = gguf.GGUFFile(str(path))
+    assert g.version == version and g.alignment == 64 and g.data_start == len(head) + pad
+    m = g.metadata
+    assert m["general.architecture"] == "llama"
+    assert (m["t.u8"], m["t.i8"], m["t.u16"], m["t.i16"], m["t.i32"]) == (200, -100, 60000, -30000, -2000000000)
+    assert m["t.f32"] == 0.15625 and m["t.bool"] is True and m["t.f64"] == 1.0 / 3.0
+    assert m["t.u64"] == 2 ** 63 + 5 and m["t.i64"] == -(2 ** 62)
+    assert list(m["t.strs"]) == ["a", "", "h\u00e9llo"]
+    assert list(m["t.ints"]) == [7, -8, 9, -10] and list(m["t.floats"]) == [0.5, -2.0]
+    assert set(g.tensors) == {"vec.weight", "blk.0.q8.weight", "blk.0.q4k.weight"}
+    t = g.tensors["blk.0.q8.weight"]
+    assert (t.shape, t.ggml_type, t.offset, t.nbytes, t.rows, t.cols) == ((64, 2), 8, 64, 136, 2, 64)
+    assert bytes(g.raw("blk.0.q8.weight")) == q8 and bytes(g.raw("blk.0.q4k.weight")) == q4k
+    assert np.array_equal(g.f32("vec.weight"), np.arange(8, dtype=np.float32) * 0.25)
+    fmt, rows, cols, blocks = g.blocks("blk.0.q8.weight")
+    assert (fmt, rows, cols) == (synth.Q8_0, 2, 64)
+    # the block bytes mean what the format says: fp16 scale first, then 32 int8 quants (quantized.go:34-37)
+    d = np.frombuffer(q8[:2], "<f2")[0].astype(np.float32)
+    want = d * np.frombuffer(q8[2:34], np.int8).astype(np.float32)
+    assert np.array_equal(o.dequantize(fmt, np.frombuffer(bytes(blocks), np.uint8))[:32], want)
+    fmt, rows, cols, blocks = g.blocks("blk.0.q4k.weight")
+    assert (fmt, rows, cols, len(blocks)) == (synth.Q4_K, 1, 256, 144)
+
+
 @pytest.mark.parametrize("alignment", [32, 64, 4096])
 def test_round_trip_keeps_every_byte(tmp_path, alignment):
     cfg, meta, tensors, _ = tiny_model()

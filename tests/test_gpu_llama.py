@@ -739,10 +739,11 @@ def test_prompt_chunks_on_either_side_of_the_fp16_threshold(dev):
 
 
 @pytest.mark.parametrize("d_ffn", [11008, 14336, 1024 + 256])
-def test_gate_up_block_parts_give_the_same_bits(dev, monkeypatch, d_ffn):
-    # the fused gate/up kernel lets a workgroup own a whole 32-value block of the FFN activation or a half / quarter
-    # of one (whichever divides the rows evenly over the CUs); the block is quantized from the same 32 f32 values
-    # either way, so the logits are the same bits, step after step (the per-block counters return to zero)
+def test_gate_up_block_parts_give_the_same_bits(dev, d_ffn):
+    # The narrower fused gate/up kernel (fused.wide = 0) lets a workgroup own a whole 32-value block of the FFN
+    # activation or a half / quarter of one (whichever divides the rows evenly over the CUs); the block is quantized
+    # from the same 32 f32 values either way, so the logits are the same bits, step after step (the per-block
+    # counters return to zero).
     cfg = dict(n_layers=2, d_model=4096 if d_ffn > 4096 else 512, n_heads=8, n_kv_heads=8,
                head_dim=512 // 8 if d_ffn <= 4096 else 128, d_ffn=d_ffn, vocab=512, max_pos=16, rms_eps=1e-5, rope_base=10000.0)
     if d_ffn > 4096:
@@ -750,17 +751,48 @@ def test_gate_up_block_parts_give_the_same_bits(dev, monkeypatch, d_ffn):
     fmts = {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}
     tokens = [int(t) for t in np.random.default_rng(31).integers(0, cfg["vocab"], 5)]
     runs = {}
-    for rows in ("32", "16", "8"):
-        dev.set_option("fused.pair_rows", int(rows))
-        try:
+    dev.set_option("fused.wide", 0)
+    try:
+        for rows in ("32", "16", "8"):
+            dev.set_option("fused.pair_rows", int(rows))
             _, model = build(dev, cfg, fmts, seed=30)
             runs[rows] = [model.decode(t, pos)[1].copy() for pos, t in enumerate(tokens)]
             model.free()
-        finally:
-            dev.set_option("fused.pair_rows", 0)
+    finally:
+        dev.set_option("fused.pair_rows", 0)
+        dev.set_option("fused.wide", 1)
     for rows in ("16", "8"):
         for a, b in zip(runs["32"], runs[rows]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), rows
+
+
+@pytest.mark.parametrize("d_ffn", [11008, 14336])
+def test_even_split_gate_up_hand_over_and_quantizing_down_projection_give_the_same_bits(dev, d_ffn):
+    # The even-split gate/up kernel (fused.wide = 1) deals the row pairs to two or three workgroups per CU wherever
+    # they fall, so most 32-value blocks of the FFN activation belong to two workgroups (d_ffn 11008: 512 workgroups
+    # of 21.5 pairs) or to two or three (14336: 768 of 18.7).  Two ways to get them quantized, same bits asked:
+    #   fused.down_quant = 0  the parts of a block meet through write-through stores and a per-block ticket, the
+    #                         workgroup that draws the last ticket quantizes (this rests on gfx950's memory behaviour,
+    #                         not on the HIP memory model: this test is what covers it);
+    #   fused.down_quant = 1  gate/up stores its f32 values and the down projection quantizes them in its prologue.
+    # Twenty steps each, captured graph replayed, against each other and against one-by-one launches.
+    cfg = dict(n_layers=2, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=d_ffn, vocab=512, max_pos=24,
+               rms_eps=1e-5, rope_base=10000.0)
+    fmts = {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}
+    tokens = [int(t) for t in np.random.default_rng(33).integers(0, cfg["vocab"], 20)]
+    runs = {}
+    try:
+        for key, down_quant, graph in (("tickets", 0, True), ("quantizing down", 1, True), ("tickets, eager", 0, False)):
+            dev.set_option("fused.down_quant", down_quant)
+            _, model = build(dev, cfg, fmts, seed=34)
+            model.set_graph(graph)
+            runs[key] = [model.decode(t, pos)[1].copy() for pos, t in enumerate(tokens)]
+            model.free()
+    finally:
+        dev.set_option("fused.down_quant", 0)
+    for key in ("quantizing down", "tickets, eager"):
+        for pos, (a, b) in enumerate(zip(runs["tickets"], runs[key])):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (key, pos)
 
 
 def test_graph_replay_equals_eager_launches(dev):

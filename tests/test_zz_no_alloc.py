@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from candy_amd import hip, synth
+from oracle import oracle as o
 
 pytestmark = pytest.mark.gpu
 
@@ -36,7 +37,10 @@ def both(dev, w, x):
 def test_two_calls_in_a_row_second_smaller(dev, fmt):
     big = dev.qtensor(fmt, 512, 4096, synth.random_weight(fmt, 512, 4096, seed=900 + fmt))
     small = dev.qtensor(fmt, 200, 1024, synth.random_weight(fmt, 200, 1024, seed=901 + fmt))
-    for (w, m) in ((big, 8), (small, 3), (big, 1), (small, 1), (big, 15), (small, 4)):
+    shapes = [(big, 8), (small, 3), (big, 1), (small, 1), (big, 15), (small, 4)]
+    if fmt == synth.Q4_K:  # one row against 4096 x 4096: candy_hip_qmatmul quantizes inside the contraction's launch there
+        shapes.append((dev.qtensor(fmt, 4096, 4096, synth.random_weight(fmt, 4096, 4096, seed=902)), 1))
+    for (w, m) in shapes:
         x = synth.random_activations(m, w.cols, seed=17 * m + w.cols)
         ref, got = both(dev, w, x)
         assert np.abs(ref).max() > 0
@@ -46,8 +50,35 @@ def test_two_calls_in_a_row_second_smaller(dev, fmt):
         else:
             # candy_hip_qmatmul may take the int8 tile kernel here: the same integer dots in another f32 summation order
             err = float(np.max(np.abs(got.astype(np.float64) - ref)) / np.max(np.abs(ref)))
-            assert err <= 1e-3, (fmt, m, err)
-            assert err <= 2e-6, (fmt, m, err)
+            assert err <= 2e-6, (fmt, m, err)  # the bar is 1e-3; two evaluations of the same exact dots stay far inside it
+
+
+@pytest.mark.parametrize("fmt", [synth.Q4_K, synth.Q8_0, synth.Q6_K, synth.Q4_0])
+def test_against_the_cpu_oracle_on_a_handle_that_never_allocated(fmt):
+    # A fresh device handle whose FIRST contraction is the allocation-free one: the handle's grow-only workspaces
+    # (the only device memory candy_hip_qmatmul allocates on the way) must still be empty afterwards, and the
+    # result is held to the CPU oracle, not to another device path: 1e-3 asked, 2e-5 expected of exact integer dots.
+    d = hip.Device(0)
+    try:
+        L = hip.lib()
+        for rows, cols, m in ((4096, 4096, 1), (512, 4096, 8), (200, 1024, 3)):
+            blocks = synth.random_weight(fmt, rows, cols, seed=950 + fmt + m)
+            w = d.qtensor(fmt, rows, cols, blocks)
+            x = synth.random_activations(m, cols, seed=951 + m)
+            src, dst = d.from_numpy(x), d.alloc(m * rows * 4)
+            hip._check(L.candy_hip_qmatmul_noalloc(d.handle, w.handle, src.ptr, m, dst.ptr))
+            got = dst.download(np.float32, m * rows).reshape(m, rows)
+            assert d.get_option("runtime.workspace_bytes") == 0 and d.get_option("runtime.split_workspace_bytes") == 0
+            want = o.qmatmul(fmt, blocks, rows, cols, x)
+            err = float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want)))
+            assert err <= 1e-3 and err <= 2e-5, (fmt, rows, cols, m, err)
+        # the allocating entry point on the same handle does grow the workspace (the key reports it), same result
+        hip._check(L.candy_hip_qmatmul(d.handle, w.handle, src.ptr, m, dst.ptr))
+        assert d.get_option("runtime.workspace_bytes") > 0
+        again = dst.download(np.float32, m * rows).reshape(m, rows)
+        assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    finally:
+        d.close()
 
 
 def test_sizes_beyond_the_scratch_are_refused(dev):
