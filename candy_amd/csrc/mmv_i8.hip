@@ -49,7 +49,11 @@ __device__ __forceinline__ size_t mmv_frag_offset(int r, int k) {
 
 // f32 [m, K] -> Q8_0 (quantize_q8_1 without its sum, quantized.cu:3521-3558; the same lane code as the quantize
 // kernel, hence the same quants and scales) written in operand order for 16 rows.
-__global__ __launch_bounds__(256) void k_mmv_quantize_pack(const float4 *__restrict__ x, int m, int K, MmvOperands o) {
+// (plain leading arguments: they arrive in registers with the wavefront, no scalar load of the argument block first)
+__global__ __launch_bounds__(256) void k_mmv_quantize_pack(const float4 *__restrict__ x, int m, int K, uint8_t *xfrag_,
+                                                          float *xd_, float *xm_, size_t frag_stride_,
+                                                          size_t scale_stride_) {
+    const MmvOperands o = {xfrag_, xd_, xm_, frag_stride_, scale_stride_};
     const int per_row = K >> 2;
     const int i = blockIdx.x * 256 + threadIdx.x;  // 16 * tiles * per_row lanes in all (a multiple of 256)
     const int row = i / per_row, k = (i - row * per_row) * 4;
@@ -120,8 +124,12 @@ struct MmvShape {
 // contracted while strip s+1 is still arriving, and the B operands and activation scales, which depend on the slice
 // only, stay in registers for all strips.  MT tiles of 16 activation rows share every A operand.
 template <int MT, int STRIPS, int SBW, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restrict__ W, MmvOperands o,
-                                                        float *__restrict__ y, int N, int M, int K) {
+__global__ __launch_bounds__(WAVES * 64) void k_mmv_q4k(const uint8_t *__restrict__ W, const uint8_t *xfrag_,
+                                                        const float *xd_, const float *xm_, float *__restrict__ y, int N,
+                                                        int M, int K, size_t frag_stride_, size_t scale_stride_) {
+    // plain leading arguments (13 dwords up to K arrive in registers with the wavefront; the two strides matter to
+    // the second activation tile only)
+    const MmvOperands o = {(uint8_t *)xfrag_, (float *)xd_, (float *)xm_, frag_stride_, scale_stride_};
     using S = MmvShape<MT, STRIPS, SBW, WAVES>;
     static_assert(S::ROWS_LD >= 1, "a row's slice must fit one load instruction");
     extern __shared__ __align__(16) uint8_t smem[];
@@ -285,7 +293,8 @@ static int launch_mmv_cfg(candy_hip_device *dev, const candy_hip_qtensor *w, con
         CANDY_HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::SMEM));
     const int N = (int)w->rows, K = (int)w->cols;
     hipLaunchKernelGGL(kern, dim3((unsigned)(N / (16 * STRIPS))), dim3(WAVES * 64), S::SMEM, dev->stream,
-                       (const uint8_t *)w->data, o, y, N, M, K);
+                       (const uint8_t *)w->data, (const uint8_t *)o.xfrag, (const float *)o.xd, (const float *)o.xm, y, N, M, K,
+                       o.frag_stride, o.scale_stride);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
@@ -316,7 +325,7 @@ int launch_mmv(candy_hip_device *dev, const candy_hip_qtensor *w, const float *x
     o.xm = o.xd + 2 * o.scale_stride;
     if (x)
         hipLaunchKernelGGL(k_mmv_quantize_pack, dim3((unsigned)(16 * tiles * (K >> 2) / 256)), dim3(256), 0, dev->stream,
-                           (const float4 *)x, (int)m, K, o);
+                           (const float4 *)x, (int)m, K, o.xfrag, o.xd, o.xm, o.frag_stride, o.scale_stride);
     else
         hipLaunchKernelGGL(k_mmv_pack_blocks, dim3((unsigned)((16 * tiles * (K >> 5) + 255) / 256)), dim3(256), 0,
                            dev->stream, (const BlockQ8_0 *)q8_blocks, (int)m, tiles, K, o);

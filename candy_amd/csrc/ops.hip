@@ -56,6 +56,38 @@ __global__ __launch_bounds__(256) void k_rope(const float *__restrict__ src, con
     dst[i2] = a * s + b * c;
 }
 
+// reduce.go:3825-3838 (rope_i): adjacent pairs (2i, 2i + 1)
+__global__ __launch_bounds__(256) void k_rope_i(const float2 *__restrict__ src, const float *__restrict__ cos_t,
+                                                const float *__restrict__ sin_t, int64_t num_pairs, int64_t half_td,
+                                                int64_t stride_b, float2 *__restrict__ dst) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= num_pairs) return;
+    int64_t rope_idx = idx % half_td;
+    if (stride_b > 0) rope_idx += ((2 * idx) / stride_b) * half_td;
+    const float c = cos_t[rope_idx], s = sin_t[rope_idx];
+    const float2 v = src[idx];
+    dst[idx] = make_float2(v.x * c - v.y * s, v.x * s + v.y * c);
+}
+
+// reduce.go:4178-4196 (rope_thd): [b, t, h, d], pairs (i, i + d/2), cos / sin rows by the token index
+__global__ __launch_bounds__(256) void k_rope_thd(const float *__restrict__ src, const float *__restrict__ cos_t,
+                                                  const float *__restrict__ sin_t, int64_t num_pairs, int64_t t, int64_t h,
+                                                  int64_t d, int64_t stride_b, float *__restrict__ dst) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= num_pairs) return;
+    const int64_t half_d = d / 2;
+    const int64_t i_bth = idx / half_d;
+    const int64_t i_d = idx - half_d * i_bth;
+    const int64_t i_t = (i_bth / h) % t;
+    const int64_t i1 = i_bth * d + i_d, i2 = i1 + half_d;
+    int64_t i_cs = i_t * half_d + i_d;
+    if (stride_b > 0) i_cs += ((2 * idx) / stride_b) * ((t * d) / 2);
+    const float c = cos_t[i_cs], s = sin_t[i_cs];
+    const float a = src[i1], b = src[i2];
+    dst[i1] = a * c - b * s;
+    dst[i2] = a * s + b * c;
+}
+
 // reduce.go:2855-2879: max, exp(x - max), multiply by 1/sum.
 __global__ __launch_bounds__(256) void k_softmax(const float *__restrict__ src, int cols, float *__restrict__ dst) {
     __shared__ float red[16];
@@ -454,6 +486,35 @@ int candy_hip_rope(candy_hip_device *dev, const float *src, const float *cos_t, 
     CANDY_REQUIRE(src && cos_t && sin_t && dst, "nil pointer");
     if (int rc = use_device(dev)) return rc;
     hipLaunchKernelGGL(k_rope, dim3(blocks_for(pairs)), dim3(256), 0, dev->stream, src, cos_t, sin_t, pairs, td, d,
+                       stride_b, dst);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_rope_i(candy_hip_device *dev, const float *src, const float *cos_t, const float *sin_t, int64_t bh,
+                     int64_t td, int64_t stride_b, float *dst) {
+    CANDY_REQUIRE(bh >= 0 && td >= 0 && stride_b >= 0, "invalid dimensions");
+    const int64_t pairs = bh * td / 2;
+    if (pairs == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(td % 2 == 0, "rope_i needs an even t*d");
+    CANDY_REQUIRE(src && cos_t && sin_t && dst, "nil pointer");
+    CANDY_REQUIRE((((uintptr_t)src | (uintptr_t)dst) & 7) == 0, "rope_i operands must be 8-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    hipLaunchKernelGGL(k_rope_i, dim3(blocks_for(pairs)), dim3(256), 0, dev->stream, (const float2 *)src, cos_t, sin_t,
+                       pairs, td / 2, stride_b, (float2 *)dst);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
+int candy_hip_rope_thd(candy_hip_device *dev, const float *src, const float *cos_t, const float *sin_t, int64_t b,
+                       int64_t t, int64_t h, int64_t d, int64_t stride_b, float *dst) {
+    CANDY_REQUIRE(b >= 0 && t >= 0 && h >= 0 && d >= 0 && stride_b >= 0, "invalid dimensions");
+    const int64_t pairs = b * t * h * d / 2;
+    if (pairs == 0) return CANDY_HIP_OK;
+    CANDY_REQUIRE(d >= 2 && d % 2 == 0, "rope_thd needs an even head dim");
+    CANDY_REQUIRE(src && cos_t && sin_t && dst, "nil pointer");
+    if (int rc = use_device(dev)) return rc;
+    hipLaunchKernelGGL(k_rope_thd, dim3(blocks_for(pairs)), dim3(256), 0, dev->stream, src, cos_t, sin_t, pairs, t, h, d,
                        stride_b, dst);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;

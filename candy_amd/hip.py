@@ -79,6 +79,9 @@ SIGNATURES = {
                                              c_int64, c_int64, c_int64]),
     "candy_hip_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p]),
     "candy_hip_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]),
+    "candy_hip_rope_i": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    "candy_hip_rope_thd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                   c_void_p]),
     "candy_hip_softmax": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "candy_hip_silu": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "candy_hip_add": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
@@ -371,6 +374,26 @@ class Device:
         ds, dc, dn = self._f32(src), self._f32(cos), self._f32(sin)
         out = self.from_numpy(src)
         _check(lib().candy_hip_rope(self.handle, ds.ptr, dc.ptr, dn.ptr, bh, td, d, stride_b, out.ptr))
+        return out.download(np.float32, src.size)
+
+    def rope_i(self, src, cos, sin, bh, td, stride_b=0) -> np.ndarray:
+        """RopeI (backend.go:156): adjacent pairs."""
+        src = np.ascontiguousarray(src, np.float32).reshape(-1)
+        if src.size == 0:
+            return src.copy()
+        ds, dc, dn = self._f32(src), self._f32(cos), self._f32(sin)
+        out = self.from_numpy(src)
+        _check(lib().candy_hip_rope_i(self.handle, ds.ptr, dc.ptr, dn.ptr, bh, td, stride_b, out.ptr))
+        return out.download(np.float32, src.size)
+
+    def rope_thd(self, src, cos, sin, b, t, h, d, stride_b=0) -> np.ndarray:
+        """RopeThd (backend.go:162): [b, t, h, d] layout."""
+        src = np.ascontiguousarray(src, np.float32).reshape(-1)
+        if src.size == 0:
+            return src.copy()
+        ds, dc, dn = self._f32(src), self._f32(cos), self._f32(sin)
+        out = self.from_numpy(src)
+        _check(lib().candy_hip_rope_thd(self.handle, ds.ptr, dc.ptr, dn.ptr, b, t, h, d, stride_b, out.ptr))
         return out.download(np.float32, src.size)
 
     def softmax(self, src, cols: int) -> np.ndarray:

@@ -195,6 +195,20 @@ public:
 
     // backend.go:159; checks of cpu/storage.go:2502-2546. cos/sin are [t, d/2] or [b, t, d/2].
     Result<Ptr> Rope(const Layout *layout, const Ptr &cos, const Layout *cosLayout, const Ptr &sin, const Layout *sinLayout) const {
+        return rope_variant(0, layout, cos, cosLayout, sin, sinLayout);
+    }
+    // backend.go:156 (adjacent pairs; input [b, h, t, d]); checks of cpu/storage.go:2428-2470
+    Result<Ptr> RopeI(const Layout *layout, const Ptr &cos, const Layout *cosLayout, const Ptr &sin, const Layout *sinLayout) const {
+        return rope_variant(1, layout, cos, cosLayout, sin, sinLayout);
+    }
+    // backend.go:162 (input [b, t, h, d]); checks of cpu/storage.go:2577-2620
+    Result<Ptr> RopeThd(const Layout *layout, const Ptr &cos, const Layout *cosLayout, const Ptr &sin, const Layout *sinLayout) const {
+        return rope_variant(2, layout, cos, cosLayout, sin, sinLayout);
+    }
+
+  private:
+    Result<Ptr> rope_variant(int variant, const Layout *layout, const Ptr &cos, const Layout *cosLayout, const Ptr &sin,
+                             const Layout *sinLayout) const {
         if (!layout) return {nullptr, Errorf("layout cannot be nil")};
         if (!cosLayout) return {nullptr, Errorf("cos layout cannot be nil")};
         if (!sinLayout) return {nullptr, Errorf("sin layout cannot be nil")};
@@ -205,7 +219,8 @@ public:
         if (!cos) return {nullptr, Errorf("cos must be HIP storage")};
         if (!sin) return {nullptr, Errorf("sin must be HIP storage")};
         if (layout->Rank() != 4) return {nullptr, Errorf("input must be 4D for RoPE")};
-        const int b = layout->Dims()[0], h = layout->Dims()[1], t = layout->Dims()[2], d = layout->Dims()[3];
+        const int b = layout->Dims()[0];
+        const int h = layout->Dims()[variant == 2 ? 2 : 1], t = layout->Dims()[variant == 2 ? 1 : 2], d = layout->Dims()[3];
         const int per_batch = t * d / 2;
         int64_t stride_b = 0;
         if (cosLayout->Numel() == b * per_batch && b > 1) stride_b = (int64_t)h * t * d;  // one table per batch entry
@@ -215,11 +230,17 @@ public:
             return {nullptr, Errorf("sin size mismatch: expected " + std::to_string(cosLayout->Numel()) + ", got " + std::to_string(sinLayout->Numel()))};
         auto out = Alloc(dev_, n_);
         if (!out.ok()) return out;
-        if (Error e = last_error(candy_hip_rope(dev_->handle(), (const float *)ptr_, (const float *)cos->ptr_, (const float *)sin->ptr_,
-                                                (int64_t)b * h, (int64_t)t * d, d, stride_b, (float *)out.value->ptr_), "rope"))
-            return {nullptr, e};
+        const float *x = (const float *)ptr_, *c = (const float *)cos->ptr_, *sn = (const float *)sin->ptr_;
+        float *y = (float *)out.value->ptr_;
+        int rc;
+        if (variant == 0) rc = candy_hip_rope(dev_->handle(), x, c, sn, (int64_t)b * h, (int64_t)t * d, d, stride_b, y);
+        else if (variant == 1) rc = candy_hip_rope_i(dev_->handle(), x, c, sn, (int64_t)b * h, (int64_t)t * d, stride_b, y);
+        else rc = candy_hip_rope_thd(dev_->handle(), x, c, sn, b, t, h, d, stride_b, y);
+        if (Error e = last_error(rc, "rope")) return {nullptr, e};
         return out;
     }
+
+  public:
 
     // backend.go:147; cpu/storage.go:2304-2325
     Result<Ptr> FastSoftmax(const Layout *layout) const {

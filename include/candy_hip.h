@@ -248,6 +248,14 @@ int candy_hip_rms_norm(candy_hip_device *dev, const float *x, const float *alpha
 /* backend.go:159 Rope; reduce.go:3987-4006 (pairs (i, i+d/2)). */
 int candy_hip_rope(candy_hip_device *dev, const float *src, const float *cos_t, const float *sin_t,
                    int64_t bh, int64_t td, int64_t d, int64_t stride_b, float *dst);
+/* backend.go:156 RopeI; reduce.go:3825-3838: adjacent pairs (2i, 2i + 1) of rows of td = t*d values, cos / sin
+ * [t*d/2] per row of the tables (stride_b > 0: one table row per stride_b source elements, as in Rope). */
+int candy_hip_rope_i(candy_hip_device *dev, const float *src, const float *cos_t, const float *sin_t,
+                     int64_t bh, int64_t td, int64_t stride_b, float *dst);
+/* backend.go:162 RopeThd; reduce.go:4178-4196: src [b, t, h, d], pairs (i, i + d/2), cos / sin [t, d/2] picked by
+ * the token index. */
+int candy_hip_rope_thd(candy_hip_device *dev, const float *src, const float *cos_t, const float *sin_t,
+                       int64_t b, int64_t t, int64_t h, int64_t d, int64_t stride_b, float *dst);
 /* backend.go:147 FastSoftmax; reduce.go:2855-2879. */
 int candy_hip_softmax(candy_hip_device *dev, const float *src, int64_t rows, int64_t cols, float *dst);
 /* backend.go:228 Silu; unary.go:3353-3366. */

@@ -70,6 +70,8 @@
  *                         conv_test.go:11-65.
  *   co_fast_rms_norm_f32  RED:3071-3092. Pinned: reduce_test.go:1909-1971 fixtures.
  *   co_rope_f32           RED:3987-4006. Pinned: reduce_test.go:2775-2832 fixtures.
+ *   co_rope_i_f32         RED:3825-3838. Pinned: reduce_test.go:2507-2560 fixtures; a rotation of adjacent pairs (float64).
+ *   co_rope_thd_f32       RED:4178-4196. Pinned: reduce_test.go:3033-3094 fixtures; equals co_rope_f32 on the transposed layout.
  *   co_fast_softmax_f32   RED:2855-2879. Pinned: reduce_test.go:1665-1717 fixtures.
  *   co_silu_f32           UNA:3353-3366. Pinned: unary_test.go:4199-4241 closed form.
  *   co_fast_argmax_f32    RED:846-862. Pinned: reduce_test.go:1063-1113 fixtures.
@@ -1046,6 +1048,39 @@ void co_rope_f32(int64_t bh, int64_t td, int64_t d, int64_t stride_b, const floa
         float a = src[i1], b = src[i2];
         dst[i1] = a * c - b * s;
         dst[i2] = a * s + b * c;
+    }
+}
+
+/* RED:3825-3838: adjacent pairs (2i, 2i + 1), cos / sin indexed by the pair within the row of td values */
+void co_rope_i_f32(int64_t bh, int64_t td, int64_t stride_b, const float *src, const float *cos_t,
+                   const float *sin_t, float *dst) {
+    int64_t num_pairs = bh * td / 2;
+    for (int64_t idx = 0; idx < num_pairs; ++idx) {
+        int64_t rope_idx = idx % (td / 2);
+        if (stride_b > 0) rope_idx += ((2 * idx) / stride_b) * (td / 2);
+        float c = cos_t[rope_idx], s = sin_t[rope_idx];
+        float a = src[2 * idx], b = src[2 * idx + 1];
+        dst[2 * idx] = a * c - b * s;
+        dst[2 * idx + 1] = a * s + b * c;
+    }
+}
+
+/* RED:4178-4196: [b, t, h, d] layout, pairs (i, i + d/2), cos / sin rows picked by the token index t */
+void co_rope_thd_f32(int64_t b, int64_t t, int64_t h, int64_t d, int64_t stride_b, const float *src,
+                     const float *cos_t, const float *sin_t, float *dst) {
+    int64_t num_pairs = b * t * h * d / 2;
+    for (int64_t idx = 0; idx < num_pairs; ++idx) {
+        int64_t i_bth = idx / (d / 2);
+        int64_t i_d = idx - (d / 2) * i_bth;
+        int64_t i_t = (i_bth / h) % t;
+        int64_t i1 = i_bth * d + i_d;
+        int64_t i2 = i1 + d / 2;
+        int64_t i_cs = i_t * (d / 2) + i_d;
+        if (stride_b > 0) i_cs += ((2 * idx) / stride_b) * ((t * d) / 2);
+        float c = cos_t[i_cs], s = sin_t[i_cs];
+        float a = src[i1], bb = src[i2];
+        dst[i1] = a * c - bb * s;
+        dst[i2] = a * s + bb * c;
     }
 }
 

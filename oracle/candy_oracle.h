@@ -92,6 +92,10 @@ void co_fast_rms_norm_f32(int64_t numel, int64_t ncols, float eps, const float *
                           const float *x, float *dst);
 void co_rope_f32(int64_t bh, int64_t td, int64_t d, int64_t stride_b, const float *src,
                  const float *cos_t, const float *sin_t, float *dst);
+void co_rope_i_f32(int64_t bh, int64_t td, int64_t stride_b, const float *src, const float *cos_t,
+                   const float *sin_t, float *dst);
+void co_rope_thd_f32(int64_t b, int64_t t, int64_t h, int64_t d, int64_t stride_b, const float *src,
+                     const float *cos_t, const float *sin_t, float *dst);
 void co_fast_softmax_f32(int64_t numel, int64_t ncols, const float *src, float *dst);
 void co_silu_f32(int64_t numel, const float *inp, float *out);
 void co_fast_argmax_f32(int64_t numel, int64_t ncols, const float *src, uint32_t *dst);

@@ -65,6 +65,10 @@ def lib() -> ctypes.CDLL:
         L.co_fast_rms_norm_f32.restype = None
         L.co_rope_f32.argtypes = [i64, i64, i64, i64, vp, vp, vp, vp]
         L.co_rope_f32.restype = None
+        L.co_rope_i_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp]
+        L.co_rope_i_f32.restype = None
+        L.co_rope_thd_f32.argtypes = [i64, i64, i64, i64, i64, vp, vp, vp, vp]
+        L.co_rope_thd_f32.restype = None
         L.co_fast_softmax_f32.argtypes = [i64, i64, vp, vp]
         L.co_fast_softmax_f32.restype = None
         L.co_silu_f32.argtypes = [i64, vp, vp]
@@ -266,6 +270,22 @@ def rope(src, cos, sin, bh: int, td: int, d: int, stride_b: int = 0) -> np.ndarr
     src, cos, sin = _f32(src).reshape(-1), _f32(cos).reshape(-1), _f32(sin).reshape(-1)
     dst = src.copy()
     lib().co_rope_f32(bh, td, d, stride_b, _p(src), _p(cos), _p(sin), _p(dst))
+    return dst
+
+
+def rope_i(src, cos, sin, bh: int, td: int, stride_b: int = 0) -> np.ndarray:
+    """RopeIF32 (reduce.go:3825-3838): adjacent pairs."""
+    src, cos, sin = _f32(src).reshape(-1), _f32(cos).reshape(-1), _f32(sin).reshape(-1)
+    dst = src.copy()
+    lib().co_rope_i_f32(bh, td, stride_b, _p(src), _p(cos), _p(sin), _p(dst))
+    return dst
+
+
+def rope_thd(src, cos, sin, b: int, t: int, h: int, d: int, stride_b: int = 0) -> np.ndarray:
+    """RopeThdF32 (reduce.go:4178-4196): [b, t, h, d] layout, half-split pairs."""
+    src, cos, sin = _f32(src).reshape(-1), _f32(cos).reshape(-1), _f32(sin).reshape(-1)
+    dst = src.copy()
+    lib().co_rope_thd_f32(b, t, h, d, stride_b, _p(src), _p(cos), _p(sin), _p(dst))
     return dst
 
 

@@ -135,6 +135,21 @@ int main() {
         auto c3 = F::FromSlice(dev, {1, 0, 1}).value;
         CHECK(x->Rope(&l, c3, &lbad, s, &lc).err.msg.rfind("cos size mismatch", 0) == 0, "rope cos size");
     }
+    // ---- RopeI / RopeThd: reduce_test.go:2507-2560 and 3033-3094 (first and second cases)
+    {
+        auto c = F::FromSlice(dev, {1, 0}).value, s = F::FromSlice(dev, {0, 1}).value;
+        Layout l = Layout::Contiguous({1, 1, 1, 4}), lc = Layout::Contiguous({1, 2});
+        auto xi = F::FromSlice(dev, {1, 3, 2, 4}).value;
+        auto ri = xi->RopeI(&l, c, &lc, s, &lc);
+        CHECK(ri.ok() && close_vec(ri.value->Data(), {1, 3, -4, 2}, 1e-6), "RopeI");
+        auto xt = F::FromSlice(dev, {1, 2, 3, 4, 5, 6, 7, 8}).value;
+        auto c2 = F::FromSlice(dev, {1, 0, 0.5f, 0.5f}).value, s2 = F::FromSlice(dev, {0, 1, 0.5f, 0.5f}).value;
+        Layout lt = Layout::Contiguous({1, 2, 1, 4}), lc2 = Layout::Contiguous({2, 2});
+        auto rt = xt->RopeThd(&lt, c2, &lc2, s2, &lc2);
+        CHECK(rt.ok() && close_vec(rt.value->Data(), {1, -4, 3, 2, -1, -1, 6, 7}, 1e-6), "RopeThd");
+        Layout l3 = Layout::Contiguous({1, 1, 4});
+        CHECK(xi->RopeI(&l3, c, &lc, s, &lc).err.msg == "input must be 4D for RoPE", "rope_i rank");
+    }
     // ---- FastSoftmax / Silu / Add / Mul / FastArgmax
     {
         auto x = F::FromSlice(dev, {1, 2, 3, 4, 5, 6}).value;

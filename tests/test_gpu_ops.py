@@ -29,6 +29,10 @@ def test_reference_vectors(dev, golden):
         assert close(dev.rms_norm(c["src"], c["dims"][-1], c["eps"], c["alpha"]), c["want"], 0, 1e-6), c["name"]
     for c in golden["rope_f32"]:
         assert close(dev.rope(c["src"], c["cos"], c["sin"], c["bh"], c["td"], c["d"], c["stride_b"]), c["want"], 0, 1e-6), c["name"]
+    for c in golden["rope_i_f32"]:
+        assert close(dev.rope_i(c["src"], c["cos"], c["sin"], c["bh"], c["td"], c["stride_b"]), c["want"], 0, 1e-6), c["name"]
+    for c in golden["rope_thd_f32"]:
+        assert close(dev.rope_thd(c["src"], c["cos"], c["sin"], c["b"], c["t"], c["h"], c["d"], c["stride_b"]), c["want"], 0, 1e-6), c["name"]
     for c in golden["fast_softmax_f32"]:
         assert close(dev.softmax(c["src"], c["dims"][-1]), c["want"], 0, 1e-6), c["name"]
     for c in golden["fast_argmax_f32"]:
@@ -120,6 +124,22 @@ def test_rope_decode_and_prefill_shapes(dev):
         cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
         got = dev.rope(src, cos, sin, bh, t * d, d)
         assert np.array_equal(got, o.rope(src, cos, sin, bh, t * d, d)) or close(got, o.rope(src, cos, sin, bh, t * d, d))
+
+
+def test_rope_i_and_rope_thd_match_oracle(dev):
+    # RopeI (adjacent pairs) and RopeThd ([b, t, h, d] layout) against the CPU loops, with one table for all batch
+    # entries and with one per entry; the device may fuse the multiply and the add, so a last-place difference is allowed
+    rng = np.random.default_rng(3)
+    for b, h, t, d in [(1, 32, 1, 128), (2, 8, 7, 64), (3, 4, 33, 128)]:
+        src = rng.standard_normal(b * h * t * d).astype(np.float32)
+        for per_batch in (False, True):
+            ang = rng.standard_normal((b if per_batch else 1, t, d // 2))
+            cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+            sb = h * t * d if per_batch else 0
+            assert close(dev.rope_i(src, cos, sin, b * h, t * d, sb), o.rope_i(src, cos, sin, b * h, t * d, sb))
+            assert close(dev.rope_thd(src, cos, sin, b, t, h, d, sb), o.rope_thd(src, cos, sin, b, t, h, d, sb))
+    with pytest.raises(hip.CandyHipError, match="even"):
+        dev.rope_thd(np.zeros(6, np.float32), np.zeros(3, np.float32), np.zeros(3, np.float32), 1, 2, 1, 3)
 
 
 @pytest.mark.parametrize("rows,cols", [(32, 2049), (1, 32000), (5, 17)])

@@ -58,6 +58,43 @@ def test_rope_is_a_rotation_of_half_split_pairs():
     assert _close(np.sum(got ** 2, -1), np.sum(src.astype(np.float64) ** 2, -1), 1e-4)  # norm preserved
 
 
+def test_rope_i_and_rope_thd_reference_vectors(golden):
+    for c in golden["rope_i_f32"]:
+        got = o.rope_i(c["src"], c["cos"], c["sin"], c["bh"], c["td"], c["stride_b"])
+        assert _close(got, c["want"], golden["tolerance"]), c["name"]
+    for c in golden["rope_thd_f32"]:
+        got = o.rope_thd(c["src"], c["cos"], c["sin"], c["b"], c["t"], c["h"], c["d"], c["stride_b"])
+        assert _close(got, c["want"], golden["tolerance"]), c["name"]
+
+
+def test_rope_i_rotates_adjacent_pairs_and_rope_thd_is_rope_on_the_transposed_layout():
+    rng = np.random.default_rng(2)
+    b, h, t, d = 2, 3, 5, 8
+    ang = rng.standard_normal((t, d // 2))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    # rope_i: pair (2i, 2i + 1) of every row of t*d values turns by the angle of pair i (float64 closed form)
+    src = rng.standard_normal((b * h, t, d // 2, 2)).astype(np.float32)
+    got = o.rope_i(src, cos, sin, b * h, t * d).reshape(b * h, t, d // 2, 2).astype(np.float64)
+    x, y = src[..., 0].astype(np.float64), src[..., 1].astype(np.float64)
+    assert _close(got[..., 0], x * np.cos(ang) - y * np.sin(ang), 1e-5)
+    assert _close(got[..., 1], x * np.sin(ang) + y * np.cos(ang), 1e-5)
+    # per-batch tables (stride_b = elements per batch entry): batch entry i takes table i
+    ang2 = rng.standard_normal((b, t, d // 2))
+    cos2, sin2 = np.cos(ang2).astype(np.float32), np.sin(ang2).astype(np.float32)
+    got2 = o.rope_i(src, cos2, sin2, b * h, t * d, stride_b=h * t * d).reshape(b, h, t, d // 2, 2)
+    for i in range(b):
+        want = o.rope_i(src.reshape(b, h, t, d // 2, 2)[i], cos2[i], sin2[i], h, t * d).reshape(h, t, d // 2, 2)
+        assert np.array_equal(got2[i], want)
+    # rope_thd on [b, t, h, d] is rope on [b, h, t, d] with the two middle axes swapped: same products, same bits
+    src4 = rng.standard_normal((b, t, h, d)).astype(np.float32)
+    thd = o.rope_thd(src4, cos, sin, b, t, h, d).reshape(b, t, h, d)
+    bhtd = o.rope(np.ascontiguousarray(src4.transpose(0, 2, 1, 3)), cos, sin, b * h, t * d, d).reshape(b, h, t, d)
+    assert np.array_equal(thd, bhtd.transpose(0, 2, 1, 3))
+    thd2 = o.rope_thd(src4, cos2, sin2, b, t, h, d, stride_b=t * h * d).reshape(b, t, h, d)
+    for i in range(b):
+        assert np.array_equal(thd2[i], o.rope_thd(src4[i], cos2[i], sin2[i], 1, t, h, d).reshape(t, h, d))
+
+
 def test_softmax_reference_vectors(golden):
     for c in golden["fast_softmax_f32"]:
         got = o.fast_softmax(c["src"], c["dims"][-1])
