@@ -74,12 +74,28 @@ __global__ __launch_bounds__(256) void k_attn_decode(const int *__restrict__ pos
     const int hw = lane >> 5, hl = lane & 31;
     const int kvh = blockIdx.x, split = blockIdx.y;
     const bool fresh = fresh_arg != 0;                        // new token's k/v arrive in registers
-    const int pos = pos_ptr ? *pos_ptr : n_pos - 1;           // position of the new token
-    const int n_cached = fresh ? pos : pos + 1;               // rows to read from the cache
-    const int per = (n_cached + n_splits - 1) / n_splits;
-    const int p0 = split * per, p1 = min(n_cached, p0 + per);
     KV *kh = (KV *)k_cache + (size_t)kvh * cache_stride;
     KV *vh = (KV *)v_cache + (size_t)kvh * cache_stride;
+    // Groups of 32 cached positions (one batch of rows per wavefront of the workgroup) are dealt to the splits round
+    // robin: split s takes groups s, s + n_splits, ...  Which rows a split reads first therefore does not depend on
+    // the position, and its first batch is requested before the position (a scalar load from device memory, a
+    // memory round trip of its own) is known; rows at or past the position are masked afterwards.  With the position
+    // in device memory the cache is the decoder's own and every row below cache_stride / HD is memory of this head;
+    // with the position as an argument only the rows up to it are known to exist.
+    constexpr int GROUP_POS = 4 * 2 * UNR;
+    const int max_row = pos_ptr ? (int)(cache_stride / HD) - 1 : n_pos - 1;
+    vecf kv0[UNR], vv0[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        const int p = split * GROUP_POS + wave * 2 * UNR + 2 * u + hw;
+        const size_t off = (size_t)min(p, max_row) * HD + hl * VEC;
+        kv0[u] = __builtin_convertvector(__builtin_nontemporal_load((const veckv *)(kh + off)), vecf);
+        vv0[u] = __builtin_convertvector(__builtin_nontemporal_load((const veckv *)(vh + off)), vecf);
+    }
+    const int pos = pos_ptr ? *pos_ptr : n_pos - 1;           // position of the new token
+    const int n_cached = fresh ? pos : pos + 1;               // rows to read from the cache
+    const int n_groups = (n_cached + GROUP_POS - 1) / GROUP_POS;
+    const int p1 = n_cached;
 
     // Rope pairs (i, i + HD/2) sit 16 lanes apart inside the half-wavefront
     vecf cs, sn;
@@ -144,9 +160,9 @@ __global__ __launch_bounds__(256) void k_attn_decode(const int *__restrict__ pos
         }
     };
 
-    // cached positions: wavefront w, half hw, slot u takes position base + 2u + hw.  The next
-    // batch of rows is requested before the current one is absorbed, so two batches (up to
-    // 16 KB) are in flight per wavefront.
+    // cached positions: in group g wavefront w, half hw, slot u takes position 32 g + 8 w + 2u + hw.  The next
+    // group's rows are requested before the current ones are absorbed, so two batches (up to 16 KB) are in flight
+    // per wavefront.
     auto fetch = [&](int base, vecf (&kv)[UNR], vecf (&vv)[UNR], bool (&valid)[UNR]) {
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
@@ -159,23 +175,27 @@ __global__ __launch_bounds__(256) void k_attn_decode(const int *__restrict__ pos
         }
     };
     {
-        constexpr int STEP = 4 * 2 * UNR;
-        int base = p0 + wave * 2 * UNR;
+        int g = split;
         vecf kv[UNR], vv[UNR], kn[UNR], vn[UNR];
         bool valid[UNR], vnext[UNR];
-        if (base < p1) fetch(base, kv, vv, valid);
-        while (base < p1) {
-            const int nb = base + STEP;
-            if (nb < p1) fetch(nb, kn, vn, vnext);
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {  // the first group: requested above
+            kv[u] = kv0[u];
+            vv[u] = vv0[u];
+            valid[u] = split * GROUP_POS + wave * 2 * UNR + 2 * u + hw < p1;
+        }
+        while (g < n_groups) {
+            const int gn = g + n_splits;
+            if (gn < n_groups) fetch(gn * GROUP_POS + wave * 2 * UNR, kn, vn, vnext);
             absorb(kv, vv, valid);
-            if (nb >= p1) break;
+            if (gn >= n_groups) break;
 #pragma unroll
             for (int u = 0; u < UNR; ++u) {
                 kv[u] = kn[u];
                 vv[u] = vn[u];
                 valid[u] = vnext[u];
             }
-            base = nb;
+            g = gn;
         }
     }
 
