@@ -256,39 +256,48 @@ __global__ __launch_bounds__(256) void k_attn_decode(const int *__restrict__ pos
 
 }
 
-// Merges the splits of one head (one workgroup of HD threads per head) and, if asked, quantizes
-// the head output to planar Q8_0 for the output projection.  Everything it needs is requested
-// up front: lane s of every wavefront reads split s's (max, sum), thread c reads column c of
-// every split's partial output.
+// Merges the splits of one head (one workgroup per head) and, if asked, quantizes the head output to planar Q8_0 for
+// the output projection.  Everything it needs is requested up front: lane s of every wavefront reads split s's
+// (max, sum); the 256 threads share the head's partial outputs as 16-byte loads, thread (sg, c4) taking columns
+// 4 c4 .. 4 c4 + 3 of splits sg, sg + SG, ...; the SG partial sums per column meet in LDS.
 template <int HD>
-__global__ __launch_bounds__(HD) void k_attn_merge(const float *__restrict__ part_o, const float *__restrict__ part_ml,
-                                                   int n_splits, float *__restrict__ out, int8_t *__restrict__ oq,
-                                                   Q8Scale *__restrict__ os) {
-    constexpr int MAX_SPLITS = 64;
-    const int h = blockIdx.x, c = threadIdx.x, lane = c & 63;
+__global__ __launch_bounds__(256) void k_attn_merge(const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                                                    int n_splits, float *__restrict__ out, int8_t *__restrict__ oq,
+                                                    Q8Scale *__restrict__ os) {
+    constexpr int MAX_SPLITS = 64, C4 = HD / 4, SG = 256 / C4, PER = MAX_SPLITS / SG;
+    const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const int c4 = tid % C4, sg = tid / C4;
     const float2 *ml = (const float2 *)(part_ml + (size_t)h * n_splits * 2);
-    const float *po = part_o + (size_t)h * n_splits * HD + c;
+    const float4 *po = (const float4 *)(part_o + (size_t)h * n_splits * HD) + c4;
     const float2 mine = lane < n_splits ? ml[lane] : make_float2(NEG_BIG, 0.0f);
-    float acc[MAX_SPLITS / 8][8];
+    float4 acc[PER];
 #pragma unroll
-    for (int s8 = 0; s8 < MAX_SPLITS / 8; ++s8)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int s = s8 * 8 + j;
-            acc[s8][j] = (s8 * 8 < n_splits) ? po[(size_t)min(s, n_splits - 1) * HD] : 0.0f;
-        }
+    for (int j = 0; j < PER; ++j) {
+        // splits at and past n_splits re-read the last one (finite values) and get weight zero below: no branch
+        // around a load, every load in flight before the first wait
+        acc[j] = po[(size_t)min(sg + SG * j, n_splits - 1) * C4];
+    }
+    __builtin_amdgcn_sched_barrier(0);  // keep the reductions below from being scheduled between the loads
     const float m = wave_max(mine.x);
     const float f = lane < n_splits ? expf(mine.x - m) : 0.0f;
     const float l = wave_sum(mine.y * f);
+    float4 o4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const float fs = __shfl(f, sg + SG * j, 64);  // zero for lanes at and past n_splits
+        o4.x += acc[j].x * fs;
+        o4.y += acc[j].y * fs;
+        o4.z += acc[j].z * fs;
+        o4.w += acc[j].w * fs;
+    }
+    __shared__ float4 red[SG][C4];
+    red[sg][c4] = o4;
+    __syncthreads();
+    if (tid >= HD) return;
+    const int c = tid;
     float o = 0.0f;
 #pragma unroll
-    for (int s8 = 0; s8 < MAX_SPLITS / 8; ++s8)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int s = s8 * 8 + j;
-            const float fs = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), s));
-            o += s < n_splits ? acc[s8][j] * fs : 0.0f;
-        }
+    for (int g = 0; g < SG; ++g) o += ((const float *)&red[g][0])[c];
     o *= 1.0f / l;
     if (out) out[(size_t)h * HD + c] = o;
     if (oq) {
@@ -333,14 +342,14 @@ static int launch_group(candy_hip_device *dev, const AttnArgs &a, int n_kv_heads
         hipLaunchKernelGGL((k_attn_decode<GROUP, 2, KV>), grid, dim3(256), 0, dev->stream, h.pos_ptr, h.k_cache, h.v_cache,
                            h.q, h.cache_stride, h.n_pos, h.n_splits, h.scale, h.fresh, a.r);
         CANDY_LAUNCH_CHECK();
-        hipLaunchKernelGGL((k_attn_merge<64>), dim3(n_heads), dim3(64), 0, dev->stream, a.r.part_o, a.r.part_ml, h.n_splits,
+        hipLaunchKernelGGL((k_attn_merge<64>), dim3(n_heads), dim3(256), 0, dev->stream, a.r.part_o, a.r.part_ml, h.n_splits,
                            a.r.out, a.r.oq, a.r.os);
         break;
     case 128:
         hipLaunchKernelGGL((k_attn_decode<GROUP, 4, KV>), grid, dim3(256), 0, dev->stream, h.pos_ptr, h.k_cache, h.v_cache,
                            h.q, h.cache_stride, h.n_pos, h.n_splits, h.scale, h.fresh, a.r);
         CANDY_LAUNCH_CHECK();
-        hipLaunchKernelGGL((k_attn_merge<128>), dim3(n_heads), dim3(128), 0, dev->stream, a.r.part_o, a.r.part_ml,
+        hipLaunchKernelGGL((k_attn_merge<128>), dim3(n_heads), dim3(256), 0, dev->stream, a.r.part_o, a.r.part_ml,
                            h.n_splits, a.r.out, a.r.oq, a.r.os);
         break;
     default: return fail(CANDY_HIP_ERR_UNSUPPORTED, "head_dim %d unsupported (64 or 128)", head_dim);
