@@ -421,6 +421,8 @@ def main():
                     help="decoders launch their kernels one by one instead of replaying a captured HIP graph (for "
                          "profiler runs: each launch is then a dispatch the tool sees on its own)")
     ap.add_argument("--no-fp16-kv", action="store_true", help="skip the decode leg's second figure (fp16 KV cache)")
+    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
+                    help="set a library option (candy_hip_set_option) before anything runs; comparison runs only")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for counter runs)")
     ap.add_argument("--write-traffic", metavar="DIR",
@@ -435,6 +437,9 @@ def main():
     from candy_amd import hip, synth
     dev = hip.Device(0)
     log("device:", dev.name)
+    for kv in args.option:
+        key, _, val = kv.partition("=")
+        dev.set_option(key, int(val))
     if args.eager:
         dev.set_option("llama.graph", 0)
     fmt, rows, cols = synth.Q4_K, 4096, 11008

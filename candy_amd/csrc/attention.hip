@@ -322,6 +322,7 @@ int attention_splits(const candy_hip_device *dev, int64_t n_kv_heads, int64_t ma
     // gives each split a lane)
     int n_splits = (int)((4 * (int64_t)dev->num_cus + n_kv_heads - 1) / n_kv_heads);
     const int max_splits = (int)((max_pos + 31) / 32);
+    if (dev->opt.attn_splits > 0) n_splits = dev->opt.attn_splits;  // comparison runs
     if (n_splits > max_splits) n_splits = max_splits;
     if (n_splits > 64) n_splits = 64;
     return n_splits < 1 ? 1 : n_splits;

@@ -75,7 +75,7 @@ __device__ __forceinline__ int wide_sharers(int first, int g, int G, int per, in
 // that hold up to eight rows of weights per lane are held to that (gate / up with four pairs per wavefront came to
 // 130 registers without it, one workgroup per CU at a time and two rounds: 22.5 us per launch on a 2 x 14336 x 4096
 // pair); the one-workgroup-per-CU shape with sixteen rows per lane keeps its 226.
-template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI, int MID = 0>
 CANDY_KERNEL(WAVES * 64, ((EPI == WEPI_PAIR ? 2 : 1) * R * ITER <= 8 ? 4 : 2), 4)
 void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha, const uint8_t *__restrict__ W0,
                    const uint8_t *__restrict__ W1, const uint8_t *__restrict__ W2, int per_rem, int K, int e0, int e1,
@@ -125,31 +125,27 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
             jrow[r] = g - (ji == 0 ? 0 : ji == 1 ? e0 : e1);
         }
     }
+    // Only the loads of the wavefront's FIRST item go out in front of the prologue; MID more between its two barriers,
+    // the rest behind it.  With every item requested up front (as the batch-1 kernel does, which has no barrier) the
+    // step of the 7B shape measured 614 tokens/s against 637 this way.  What fits that: a CU accepts a bounded number
+    // of bytes in flight, so wavefronts that request all their rows sit in their load instructions for most of the
+    // stream, the prologue's barrier - behind those instructions in program order - is reached when the stream is
+    // nearly over, and normalising and quantizing the activation row then runs after the weights have arrived instead
+    // of under them.  One item per wavefront (37 KB per workgroup of a 4096-wide pair) is accepted at once and keeps the
+    // memory busy for as long as the prologue takes.  Two plain rows up front instead of one: 630 against 637.
+    auto load_item = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
-    for (int m = 0; m < NW; ++m)
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
+        for (int m = 0; m < NW; ++m) {
             const uint8_t *Wj = EPI == WEPI_PAIR ? (m == 0 ? W0 : W1) : (job[r] == 0 ? W0 : job[r] == 1 ? W1 : W2);
             const uint8_t *row = Wj + (size_t)jrow[r] * rb;
 #pragma unroll
             for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
         }
-
-    // PLAIN: where each row goes, and the residual it is added to, requested now rather than as a memory round
-    // trip after the reduction (rows without one read their own output slot: valid memory, value unused).
-    float *yp[R];
-    float rv[R];
-    bool has_res[R];
-    if (EPI == WEPI_PLAIN) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int j = job[r];
-            yp[r] = (j == 0 ? a.y[0] : j == 1 ? a.y[1] : a.y[2]) + jrow[r];  // may alias the residual (h += W.x)
-            const float *rp = j == 0 ? a.res[0] : j == 1 ? a.res[1] : a.res[2];
-            has_res[r] = rp != nullptr;
-            rv[r] = *(has_res[r] ? rp + jrow[r] : yp[r]);
-        }
-    }
+    };
+    constexpr int FIRST = 1, SECOND = FIRST + MID;
+    static_assert(SECOND <= R && (MID == 0 || PRO == WPRO_RMS), "items between the prologue's barriers");
+    load_item(0);
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- the activation row: normalised (or merged) and quantized into LDS, once per workgroup
     float4 val[XF];
@@ -167,6 +163,10 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
         s = wave_sum(s);
         if (lane == 0) s_red[wave] = s;
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = FIRST; r < SECOND; ++r) load_item(r);  // the second item goes out between the two barriers
+        __builtin_amdgcn_sched_barrier(0);
         float tot = 0.0f;
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) tot += s_red[i];
@@ -193,6 +193,27 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
         }
     }
     __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- the other items' loads
+#pragma unroll
+    for (int r = SECOND; r < R; ++r) load_item(r);
+    // PLAIN: where each row goes, and the residual it is added to, requested now rather than as a memory round
+    // trip after the reduction (rows without one read their own output slot: valid memory, value unused).
+    float *yp[R];
+    float rv[R];
+    bool has_res[R];
+    if (EPI == WEPI_PLAIN) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int j = job[r];
+            yp[r] = (j == 0 ? a.y[0] : j == 1 ? a.y[1] : a.y[2]) + jrow[r];  // may alias the residual (h += W.x)
+            const float *rp = j == 0 ? a.res[0] : j == 1 ? a.res[1] : a.res[2];
+            has_res[r] = rp != nullptr;
+            rv[r] = *(has_res[r] ? rp + jrow[r] : yp[r]);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- contraction
     float acc[NW][R];
@@ -281,7 +302,7 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
     }
 }
 
-template <class U, int ITER, int R, int WAVES, int PRO, int EPI>
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI, int MID = 0>
 static int launch_wide_cfg(candy_hip_device *dev, WideArgs a, int total, int grid) {
     if ((EPI == WEPI_PAIR && total / grid < 8) || total / grid > 0xFFFF || grid > 0x7FFF)
         return CANDY_HIP_ERR_UNSUPPORTED;  // what wide_sharers and the packing assume
@@ -291,7 +312,7 @@ static int launch_wide_cfg(candy_hip_device *dev, WideArgs a, int total, int gri
     constexpr size_t QBYTES = (size_t)XF * T * 4;
     constexpr size_t smem = QBYTES + ((QBYTES >> 8) << 4) + ((size_t)XF * T / 8 + 1) * 8;
     static_assert(smem <= 48 * 1024, "LDS image too large");
-    hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a.h.x,
+    hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI, MID>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a.h.x,
                        a.h.alpha, a.h.W[0], a.h.W[1], a.h.W[2], a.h.per_rem, a.h.K, a.h.e0, a.h.e1, a.r);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
@@ -355,8 +376,12 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
             // four pairs per wavefront need every register: three workgroups of three pairs per CU instead, the third
             // starting when the first is done (2 x 14336 x 4096: 508 against 502 tokens/s on the Llama-3-8B shape; the
             // same step from three pairs to two loses, 509 against 539 on the 7B shape: more blocks are shared)
+            // (there the second pair's loads go out between the prologue's two barriers: the third workgroup of a CU
+            // starts on a memory pipeline that has room, and waiting for the end of the prologue with a third of its
+            // bytes requested costs it a round trip: 585 against 575 tokens/s on the Llama-3-8B shape; with two
+            // workgroups per CU the same loses, 635 against 637.5 on the 7B shape)
             if (per2 <= 32 && (total + 3 * cus - 1) / (3 * cus) <= 24)
-                return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 3 * cus);
+                return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR, 1>(dev, a, total, 3 * cus);
             if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
         }
         if (iter == 1) {

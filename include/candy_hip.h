@@ -112,6 +112,8 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *                                         SiLU*Mul values and the down projection quantizes them in its own prologue (0: gate /
  *                                         up quantizes them, handing 32-value blocks that two workgroups share through
  *                                         per-block tickets); same bits, measured slower
+ *   "attention.splits"           0        comparison runs: decode attention deals the cached positions to this many
+ *                                         workgroups per kv head, 1..64 (0: by shape); read when a decoder is created
  *   "prefill.qkv_group"          1        prompt pass: projections that share their input (q / k / v; gate / up) as one
  *                                         grid each where all of them run on the fp16 tiles (0: one launch each)
  *   "prefill.fold_split_sums"    1        prompt pass: the partial copies a projection split along K leaves are summed by the
