@@ -75,8 +75,8 @@ __device__ __forceinline__ int wide_sharers(int first, int g, int G, int per, in
 // that hold up to eight rows of weights per lane are held to that (gate / up with four pairs per wavefront came to
 // 130 registers without it, one workgroup per CU at a time and two rounds: 22.5 us per launch on a 2 x 14336 x 4096
 // pair); the one-workgroup-per-CU shape with sixteen rows per lane keeps its 226.
-template <class U, int ITER, int R, int WAVES, int PRO, int EPI, int MID = 0>
-CANDY_KERNEL(WAVES * 64, ((EPI == WEPI_PAIR ? 2 : 1) * R * ITER <= 8 ? 4 : 2), 4)
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI, int SLOTS = R>
+CANDY_KERNEL(WAVES * 64, ((EPI == WEPI_PAIR ? 2 : 1) * SLOTS * ITER <= 8 ? 4 : 2), 4)
 void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha, const uint8_t *__restrict__ W0,
                    const uint8_t *__restrict__ W1, const uint8_t *__restrict__ W2, int per_rem, int K, int e0, int e1,
                    const WideRest a) {
@@ -109,7 +109,7 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
     }
 
     // ---- every weight load of the wavefront: items start + wave + WAVES * r
-    typename U::W w[NW][R][ITER];
+    typename U::W w[NW][SLOTS][ITER];  // item r sits in slot r % SLOTS
     int job[R], jrow[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -125,25 +125,25 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
             jrow[r] = g - (ji == 0 ? 0 : ji == 1 ? e0 : e1);
         }
     }
-    // Only the loads of the wavefront's FIRST item go out in front of the prologue; MID more between its two barriers,
-    // the rest behind it.  With every item requested up front (as the batch-1 kernel does, which has no barrier) the
-    // step of the 7B shape measured 614 tokens/s against 637 this way.  What fits that: a CU accepts a bounded number
-    // of bytes in flight, so wavefronts that request all their rows sit in their load instructions for most of the
-    // stream, the prologue's barrier - behind those instructions in program order - is reached when the stream is
-    // nearly over, and normalising and quantizing the activation row then runs after the weights have arrived instead
-    // of under them.  One item per wavefront (37 KB per workgroup of a 4096-wide pair) is accepted at once and keeps the
-    // memory busy for as long as the prologue takes.  Two plain rows up front instead of one: 630 against 637.
+    // Only the loads of the wavefront's FIRST item go out in front of the prologue, the rest behind it.  With every
+    // item requested up front (as the batch-1 kernel does, which has no barrier) the step of the 7B shape measured 614
+    // tokens/s against 637 this way.  What fits that: a CU accepts a bounded number of bytes in flight, so wavefronts
+    // that request all their rows sit in their load instructions for most of the stream, the prologue's barrier -
+    // behind those instructions in program order - is reached when the stream is nearly over, and normalising and
+    // quantizing the activation row then runs after the weights have arrived instead of under them.  One item per
+    // wavefront (37 KB per workgroup of a 4096-wide pair) is accepted at once and keeps the memory busy for as long
+    // as the prologue takes.  Two plain rows up front instead of one: 630 against 637.
+    // Items beyond the SLOTS whose weights fit the registers are requested as items in front of them are contracted.
     auto load_item = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
         for (int m = 0; m < NW; ++m) {
             const uint8_t *Wj = EPI == WEPI_PAIR ? (m == 0 ? W0 : W1) : (job[r] == 0 ? W0 : job[r] == 1 ? W1 : W2);
             const uint8_t *row = Wj + (size_t)jrow[r] * rb;
 #pragma unroll
-            for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r][it]);
+            for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r % SLOTS][it]);
         }
     };
-    constexpr int FIRST = 1, SECOND = FIRST + MID;
-    static_assert(SECOND <= R && (MID == 0 || PRO == WPRO_RMS), "items between the prologue's barriers");
+    static_assert(SLOTS >= 1 && SLOTS <= R, "register slots for the items' weights");
     load_item(0);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -163,10 +163,6 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
         s = wave_sum(s);
         if (lane == 0) s_red[wave] = s;
         __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int r = FIRST; r < SECOND; ++r) load_item(r);  // the second item goes out between the two barriers
-        __builtin_amdgcn_sched_barrier(0);
         float tot = 0.0f;
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) tot += s_red[i];
@@ -197,7 +193,7 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
 
     // ---- the other items' loads
 #pragma unroll
-    for (int r = SECOND; r < R; ++r) load_item(r);
+    for (int r = 1; r < SLOTS; ++r) load_item(r);
     // PLAIN: where each row goes, and the residual it is added to, requested now rather than as a memory round
     // trip after the reduction (rows without one read their own output slot: valid memory, value unused).
     float *yp[R];
@@ -221,18 +217,42 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
     for (int m = 0; m < NW; ++m)
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+    if constexpr (SLOTS == R) {
 #pragma unroll
-    for (int it = 0; it < ITER; ++it) {
-        const int u = it * 64 + lane;
-        const bool live = u < units;
-        const int uc = live ? u : units - 1;
+        for (int it = 0; it < ITER; ++it) {
+            const int u = it * 64 + lane;
+            const bool live = u < units;
+            const int uc = live ? u : units - 1;
 #pragma unroll
-        for (int m = 0; m < NW; ++m)
+            for (int m = 0; m < NW; ++m)
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const float v = U::dot(w[m][r][it], uc, sq, ss);
-                acc[m][r] += live ? v : 0.0f;
+                for (int r = 0; r < R; ++r) {
+                    const float v = U::dot(w[m][r][it], uc, sq, ss);
+                    acc[m][r] += live ? v : 0.0f;
+                }
+        }
+    } else {
+        // more items than register slots: an item is contracted (units in the same order as above) and the item
+        // SLOTS further on is requested into the registers it leaves
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                const int u = it * 64 + lane;
+                const bool live = u < units;
+                const int uc = live ? u : units - 1;
+#pragma unroll
+                for (int m = 0; m < NW; ++m) {
+                    const float v = U::dot(w[m][r % SLOTS][it], uc, sq, ss);
+                    acc[m][r] += live ? v : 0.0f;
+                }
             }
+            if (r + SLOTS < R) {
+                __builtin_amdgcn_sched_barrier(0);
+                load_item(r + SLOTS);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
     }
 
     if (EPI == WEPI_PLAIN) {
@@ -302,7 +322,7 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
     }
 }
 
-template <class U, int ITER, int R, int WAVES, int PRO, int EPI, int MID = 0>
+template <class U, int ITER, int R, int WAVES, int PRO, int EPI, int SLOTS = R>
 static int launch_wide_cfg(candy_hip_device *dev, WideArgs a, int total, int grid) {
     if ((EPI == WEPI_PAIR && total / grid < 8) || total / grid > 0xFFFF || grid > 0x7FFF)
         return CANDY_HIP_ERR_UNSUPPORTED;  // what wide_sharers and the packing assume
@@ -312,7 +332,7 @@ static int launch_wide_cfg(candy_hip_device *dev, WideArgs a, int total, int gri
     constexpr size_t QBYTES = (size_t)XF * T * 4;
     constexpr size_t smem = QBYTES + ((QBYTES >> 8) << 4) + ((size_t)XF * T / 8 + 1) * 8;
     static_assert(smem <= 48 * 1024, "LDS image too large");
-    hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI, MID>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a.h.x,
+    hipLaunchKernelGGL((k_matvec_wide<U, ITER, R, WAVES, PRO, EPI, SLOTS>), dim3((unsigned)grid), dim3(T), smem, dev->stream, a.h.x,
                        a.h.alpha, a.h.W[0], a.h.W[1], a.h.W[2], a.h.per_rem, a.h.K, a.h.e0, a.h.e1, a.r);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
@@ -373,16 +393,13 @@ int launch_matvec_wide(candy_hip_device *dev, const WideLaunch &L) {
             const int per2 = (total + 2 * cus - 1) / (2 * cus);
             if (per2 <= 16) return launch_wide_cfg<UnitQ4K, 1, 2, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
             if (per2 <= 24) return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
-            // four pairs per wavefront need every register: three workgroups of three pairs per CU instead, the third
-            // starting when the first is done (2 x 14336 x 4096: 508 against 502 tokens/s on the Llama-3-8B shape; the
-            // same step from three pairs to two loses, 509 against 539 on the 7B shape: more blocks are shared)
-            // (there the second pair's loads go out between the prologue's two barriers: the third workgroup of a CU
-            // starts on a memory pipeline that has room, and waiting for the end of the prologue with a third of its
-            // bytes requested costs it a round trip: 585 against 575 tokens/s on the Llama-3-8B shape; with two
-            // workgroups per CU the same loses, 635 against 637.5 on the 7B shape)
-            if (per2 <= 32 && (total + 3 * cus - 1) / (3 * cus) <= 24)
-                return launch_wide_cfg<UnitQ4K, 1, 3, 8, WPRO_RMS, WEPI_PAIR, 1>(dev, a, total, 3 * cus);
-            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR>(dev, a, total, 2 * cus);
+            // More pairs per wavefront than three: their weights would need more than the 128 registers that let two
+            // workgroups share a CU, so the fourth .. sixth pair is requested into the registers of the first .. third
+            // once that is contracted (2 x 14336 x 4096, four pairs: 605 tokens/s on the Llama-3-8B shape against 585
+            // for three workgroups of three pairs per CU, the third starting when the first is done).
+            if (per2 <= 32) return launch_wide_cfg<UnitQ4K, 1, 4, 8, WPRO_RMS, WEPI_PAIR, 3>(dev, a, total, 2 * cus);
+            if (per2 <= 40) return launch_wide_cfg<UnitQ4K, 1, 5, 8, WPRO_RMS, WEPI_PAIR, 3>(dev, a, total, 2 * cus);
+            if (per2 <= 48) return launch_wide_cfg<UnitQ4K, 1, 6, 8, WPRO_RMS, WEPI_PAIR, 3>(dev, a, total, 2 * cus);
         }
         if (iter == 1) {
             if (per <= 32) return launch_wide_cfg<UnitQ4K, 1, 2, 16, WPRO_RMS, WEPI_PAIR>(dev, a, total, cus);

@@ -382,12 +382,13 @@ def test_full_depth_llama3_8b_shape_step(dev):
     model.free()
 
 
-@pytest.mark.parametrize("d_ffn", [11008, 14336])
+@pytest.mark.parametrize("d_ffn", [11008, 14336, 18432, 22016])
 def test_long_cache_step_on_the_even_split_kernels(dev, d_ffn):
     # One full-width 7B layer over a cache of 600 positions with q/k/v and gate/up on the kernels that deal the rows
-    # evenly over the CUs (two workgroups of eight wavefronts per CU, or one of sixteen; three of eight for the 14336
-    # pairs of the wider FFN, where a 32-value block can belong to three workgroups), against the CPU composition
-    # and against the same step on the narrower kernels (the RMS sum runs in another order, so not the same bits).
+    # evenly over the CUs (two workgroups of eight wavefronts per CU, or one of sixteen; the wider FFNs give a
+    # wavefront four, five and six row pairs, the fourth and later ones loaded into the registers of pairs already
+    # contracted), against the CPU composition and against the same step on the narrower kernels (the RMS sum runs
+    # in another order, so not the same bits).
     n_pos = 600
     cfg = dict(n_layers=1, d_model=4096, n_heads=32, n_kv_heads=32, head_dim=128, d_ffn=d_ffn, vocab=512,
                max_pos=n_pos + 8, rms_eps=1e-5, rope_base=10000.0)
@@ -770,7 +771,7 @@ def test_gate_up_block_parts_give_the_same_bits(dev, d_ffn):
 def test_even_split_gate_up_hand_over_and_quantizing_down_projection_give_the_same_bits(dev, d_ffn):
     # The even-split gate/up kernel (fused.wide = 1) deals the row pairs to two or three workgroups per CU wherever
     # they fall, so most 32-value blocks of the FFN activation belong to two workgroups (d_ffn 11008: 512 workgroups
-    # of 21.5 pairs) or to two or three (14336: 768 of 18.7).  Two ways to get them quantized, same bits asked:
+    # of 21.5 pairs; 14336: 512 of 28).  Two ways to get them quantized, same bits asked:
     #   fused.down_quant = 0  the parts of a block meet through write-through stores and a per-block ticket, the
     #                         workgroup that draws the last ticket quantizes (this rests on gfx950's memory behaviour,
     #                         not on the HIP memory model: this test is what covers it);
