@@ -125,26 +125,27 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
             jrow[r] = g - (ji == 0 ? 0 : ji == 1 ? e0 : e1);
         }
     }
-    // Only the loads of the wavefront's FIRST item go out in front of the prologue, the rest behind it.  With every
-    // item requested up front (as the batch-1 kernel does, which has no barrier) the step of the 7B shape measured 614
-    // tokens/s against 637 this way.  What fits that: a CU accepts a bounded number of bytes in flight, so wavefronts
-    // that request all their rows sit in their load instructions for most of the stream, the prologue's barrier -
-    // behind those instructions in program order - is reached when the stream is nearly over, and normalising and
-    // quantizing the activation row then runs after the weights have arrived instead of under them.  One item per
-    // wavefront (37 KB per workgroup of a 4096-wide pair) is accepted at once and keeps the memory busy for as long
-    // as the prologue takes.  Two plain rows up front instead of one: 630 against 637.
+    // Only ONE row's loads (the gate row of the wavefront's first pair) go out in front of the prologue, the rest
+    // behind it.  With every row requested up front (as the batch-1 kernel does, which has no barrier) the step of the
+    // 7B shape measured 614 tokens/s; with the first pair (or two plain rows) in front 637 (630); with one row 645; with
+    // none 628.  What fits that: a CU accepts a bounded number of bytes in flight, so wavefronts that request all their
+    // rows sit in their load instructions for most of the stream, the prologue's barrier - behind those instructions in
+    // program order - is reached when the stream is nearly over, and normalising and quantizing the activation row
+    // then runs after the weights have arrived instead of under them.  One row per wavefront (18 KB per workgroup at
+    // 4096 columns) is taken at once and keeps the memory busy while the prologue runs.
     // Items beyond the SLOTS whose weights fit the registers are requested as items in front of them are contracted.
+    auto load_row = [&](int r, int m) __attribute__((always_inline)) {
+        const uint8_t *Wj = EPI == WEPI_PAIR ? (m == 0 ? W0 : W1) : (job[r] == 0 ? W0 : job[r] == 1 ? W1 : W2);
+        const uint8_t *row = Wj + (size_t)jrow[r] * rb;
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r % SLOTS][it]);
+    };
     auto load_item = [&](int r) __attribute__((always_inline)) {
 #pragma unroll
-        for (int m = 0; m < NW; ++m) {
-            const uint8_t *Wj = EPI == WEPI_PAIR ? (m == 0 ? W0 : W1) : (job[r] == 0 ? W0 : job[r] == 1 ? W1 : W2);
-            const uint8_t *row = Wj + (size_t)jrow[r] * rb;
-#pragma unroll
-            for (int it = 0; it < ITER; ++it) U::load(row, min(it * 64 + lane, units - 1), w[m][r % SLOTS][it]);
-        }
+        for (int m = 0; m < NW; ++m) load_row(r, m);
     };
     static_assert(SLOTS >= 1 && SLOTS <= R, "register slots for the items' weights");
-    load_item(0);
+    load_row(0, 0);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- the activation row: normalised (or merged) and quantized into LDS, once per workgroup
@@ -192,6 +193,7 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- the other items' loads
+    if (NW == 2) load_row(0, 1);
 #pragma unroll
     for (int r = 1; r < SLOTS; ++r) load_item(r);
     // PLAIN: where each row goes, and the residual it is added to, requested now rather than as a memory round
