@@ -320,12 +320,10 @@ def llama3_leg(dev, n_prompt=512, n_decode=128, not_eager=True):
         tok, _ = model.decode(tok, pos, want_logits=False)
         pos += 1
     dev.synchronize()
+    # greedy generation, the chosen token handed to the next step on the device (candy_hip_llama_generate): one
+    # copy of the token list at the end instead of a device round trip per token
     t0 = time.perf_counter()
-    toks = []
-    for _ in range(n_decode - 4):
-        tok, _ = model.decode(tok, pos, want_logits=False)
-        toks.append(tok)
-        pos += 1
+    toks = model.generate(tok, pos, n_decode - 4)
     dev.synchronize()
     dec_s = (time.perf_counter() - t0) / (n_decode - 4)
     kv_mid = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * (n_prompt + n_decode // 2) * cfg["head_dim"] * 4
@@ -375,20 +373,26 @@ def decode_leg(dev, steps, warmup, fp16_kv=True):
             tok, _ = model.decode(tok, pos, want_logits=False)
             pos += 1
         dev.synchronize()
+        # the timed region: `steps` greedy steps, each step's token handed to the next on the device
+        # (candy_hip_llama_generate), the token list copied out once at the end
         t0 = time.perf_counter()
-        toks = []
-        for _ in range(steps):
-            tok, _ = model.decode(tok, pos, want_logits=False)
-            toks.append(tok)
-            pos += 1
+        toks = model.generate(tok, pos, steps)
         dev.synchronize()
         dt = time.perf_counter() - t0
+        # beside it: the same steps with the host fetching every token (candy_hip_llama_decode in a loop)
+        tok2, pos2 = toks[-1], pos + steps
+        t1 = time.perf_counter()
+        for _ in range(min(steps, 16)):
+            tok2, _ = model.decode(tok2, pos2 - 1, want_logits=False)
+        dev.synchronize()
+        fetched = (time.perf_counter() - t1) / min(steps, 16)
         kv_bytes = 2 * cfg["n_layers"] * cfg["n_kv_heads"] * n_pos * cfg["head_dim"] * kv_elem_bytes
         bpt = weight_bytes + kv_bytes
         ms = dt / steps * 1e3
         return {"tok_s": round(steps / dt, 2), "ms_per_token": round(ms, 4), "steps": steps, "kv_positions": n_pos,
                 "bytes_per_token": bpt, "hbm_GBps": round(bpt / (ms * 1e-3) / 1e9, 1),
-                "hbm_frac": round(bpt / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "tokens": toks[:8]}
+                "hbm_frac": round(bpt / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "tokens": toks[:8],
+                "tok_s_token_fetched_every_step": round(1 / fetched, 2)}
 
     out = run(4)  # candy's cache is f32: this is the figure quoted
     # the optional half-size cache, beside it (k and v rounded to fp16 on entry; not what the reference computes)

@@ -63,6 +63,15 @@ __global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok)
     if (tok >= 0) *tok_dst = tok;
 }
 
+// Greedy generation without the host in the loop: the token the last step chose becomes the next step's input and
+// is written to the list the caller gets at the end.
+__global__ void k_chain_step(int *pos_dst, int pos, int64_t *tok_dst, const uint32_t *chosen, int32_t *list) {
+    *pos_dst = pos;
+    const uint32_t t = *chosen;
+    *tok_dst = (int64_t)t;
+    *list = (int32_t)t;
+}
+
 }  // namespace candy
 
 using namespace candy;
@@ -386,11 +395,15 @@ static int llama_enqueue_step(candy_hip_llama *m) {
     return candy_hip_argmax(dev, m->logits, 1, c.vocab, m->next_tok);
 }
 
+// chain_to: null, or where the token chosen by the previous step is recorded while it becomes this step's input
 static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const float *dev_hidden,
-                      const float **dev_logits, int32_t *next_token) {
+                      const float **dev_logits, int32_t *next_token, int32_t *chain_to = nullptr) {
     candy_hip_device *dev = m->dev;
     int rc;
-    hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token);
+    if (chain_to)
+        hipLaunchKernelGGL(k_chain_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, m->next_tok, chain_to);
+    else
+        hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token);
     CANDY_LAUNCH_CHECK();
     if (dev_hidden) {
         if ((rc = candy_hip_d2d(dev, m->h, dev_hidden, (size_t)m->cfg.d_model * sizeof(float)))) return rc;
@@ -597,6 +610,31 @@ int candy_hip_llama_decode(candy_hip_llama *m, int32_t token, int32_t pos, const
     if (int rc = llama_check_complete(m)) return rc;
     if (int rc = use_device(m->dev)) return rc;
     return llama_step(m, pos, token, nullptr, dev_logits, next_token);
+}
+
+int candy_hip_llama_generate(candy_hip_llama *m, int32_t token, int32_t pos, int32_t n_steps, int32_t *tokens) {
+    CANDY_REQUIRE(m && tokens, "nil argument");
+    CANDY_REQUIRE(m->embed, "embedding table not set");
+    CANDY_REQUIRE(token >= 0 && token < m->cfg.vocab, "token %d outside the vocabulary", token);
+    CANDY_REQUIRE(n_steps >= 1, "invalid number of steps %d", n_steps);
+    CANDY_REQUIRE(pos >= 0 && (int64_t)pos + n_steps <= m->cfg.max_pos, "positions %d .. %lld outside the cache (max_pos %d)",
+                  pos, (long long)pos + n_steps - 1, m->cfg.max_pos);
+    if (int rc = llama_check_complete(m)) return rc;
+    if (int rc = use_device(m->dev)) return rc;
+    int32_t *list = nullptr;  // one slot per step; slot i takes the token step i chose
+    if (int rc = candy_hip_alloc(m->dev, (size_t)(n_steps + 1) * sizeof(int32_t), (void **)&list)) return rc;
+    int rc = llama_step(m, pos, token, nullptr, nullptr, nullptr);
+    for (int i = 1; i < n_steps && !rc; ++i) rc = llama_step(m, pos + i, -1, nullptr, nullptr, nullptr, list + i - 1);
+    if (!rc) {
+        // the last step's choice: recorded by the same kernel, into a step that is not run (position and token
+        // registers are rewritten by whatever step comes next)
+        hipLaunchKernelGGL(k_chain_step, dim3(1), dim3(1), 0, m->dev->stream, m->d_pos, (int)(pos + n_steps - 1), m->tok_id,
+                           m->next_tok, list + n_steps - 1);
+        if (hipGetLastError() != hipSuccess) rc = fail(CANDY_HIP_ERR_HIP, "launch failed");
+    }
+    if (!rc) rc = candy_hip_d2h(m->dev, tokens, list, (size_t)n_steps * sizeof(int32_t));
+    const int rc2 = candy_hip_free(m->dev, list);
+    return rc ? rc : rc2;
 }
 
 }  // extern "C"

@@ -101,6 +101,7 @@ SIGNATURES = {
     "candy_hip_llama_kv_cache": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_size_t)]),
     "candy_hip_llama_hidden": (c_int, [c_void_p, POINTER(c_void_p)]),
     "candy_hip_llama_decode": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
+    "candy_hip_llama_generate": (c_int, [c_void_p, c_int32, c_int32, c_int32, POINTER(c_int32)]),
     "candy_hip_llama_decode_hidden": (c_int, [c_void_p, c_void_p, c_int32, POINTER(c_void_p), POINTER(c_int32)]),
     "candy_hip_llama_prefill": (c_int, [c_void_p, POINTER(c_int32), c_int32, c_int32, POINTER(c_void_p),
                                         POINTER(c_int32)]),
@@ -568,6 +569,12 @@ class Llama:
         lg, nt = c_void_p(), c_int32(-1)
         _check(lib().candy_hip_llama_decode(self.handle, token, pos, byref(lg), byref(nt)))
         return self._result(lg, nt, want_logits)
+
+    def generate(self, token: int, pos: int, n_steps: int):
+        """n_steps greedy steps without a host round trip between them; returns the chosen tokens."""
+        out = (c_int32 * n_steps)()
+        _check(lib().candy_hip_llama_generate(self.handle, token, pos, n_steps, out))
+        return [int(t) for t in out]
 
     def decode_hidden(self, hidden: np.ndarray, pos: int, want_logits: bool = True):
         buf = self.dev.from_numpy(np.ascontiguousarray(hidden, np.float32))

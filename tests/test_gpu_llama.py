@@ -816,6 +816,38 @@ def test_graph_replay_equals_eager_launches(dev):
         dev.synchronize()
 
 
+def test_generate_chains_the_same_tokens_as_step_by_step_decoding(dev):
+    # candy_hip_llama_generate hands each step's greedy token to the next step in device memory and copies the list
+    # out once; the tokens are those of candy_hip_llama_decode called step by step (graph replay and one-by-one
+    # launches), and the cache ends up the same.
+    cfg = dict(n_layers=2, d_model=1024, n_heads=8, n_kv_heads=4, head_dim=128, d_ffn=2816, vocab=1024, max_pos=24,
+               rms_eps=1e-5, rope_base=10000.0)
+    fmts = {"default": synth.Q4_K, "head": synth.Q6_K, "embed": synth.Q8_0}
+    _, model = build(dev, cfg, fmts, seed=77, from_normal=True)  # such weights do not settle on one token at once
+    n = 12
+    for graph in (True, False):
+        model.set_graph(graph)
+        tok, steps = 3, []
+        for pos in range(n):
+            tok, _ = model.decode(tok, pos, want_logits=False)
+            steps.append(tok)
+        k_steps, v_steps = read_cache(dev, model, (cfg["n_layers"], cfg["n_kv_heads"], cfg["max_pos"], cfg["head_dim"]))
+        chained = model.generate(3, 0, n)
+        assert chained == steps, (graph, chained, steps)
+        k_gen, v_gen = read_cache(dev, model, (cfg["n_layers"], cfg["n_kv_heads"], cfg["max_pos"], cfg["head_dim"]))
+        assert np.array_equal(k_steps[:, :, :n], k_gen[:, :, :n]) and np.array_equal(v_steps[:, :, :n], v_gen[:, :, :n])
+        assert len(set(steps)) > 1  # the chain is not a fixed point from the first token on
+    # a single step, and one more from where the list ended
+    assert model.generate(3, 0, 1) == steps[:1]
+    with pytest.raises(hip.CandyHipError):
+        model.generate(3, cfg["max_pos"] - 2, 3)
+    with pytest.raises(hip.CandyHipError):
+        model.generate(cfg["vocab"], 0, 2)
+    with pytest.raises(hip.CandyHipError):
+        model.generate(3, 0, 0)
+    model.free()
+
+
 def test_decode_errors(dev):
     cfg = dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, head_dim=128, d_ffn=256, vocab=64, max_pos=4,
                rms_eps=1e-5, rope_base=10000.0)
