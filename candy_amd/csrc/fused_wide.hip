@@ -145,6 +145,14 @@ void k_matvec_wide(const float *__restrict__ x, const float *__restrict__ alpha,
         for (int m = 0; m < NW; ++m) load_row(r, m);
     };
     static_assert(SLOTS >= 1 && SLOTS <= R, "register slots for the items' weights");
+    if (PRO == WPRO_RMS) {
+        // every wavefront's prologue inputs are in the CU's memory pipeline before any weight request of this
+        // workgroup (the pipeline returns data in the order it took the requests, whichever wavefront they belong
+        // to).  The bare barrier instruction: __syncthreads() would wait for the loads themselves first.
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
     load_row(0, 0);
     __builtin_amdgcn_sched_barrier(0);
 
