@@ -281,6 +281,58 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant(const float *__restrict_
     }
 }
 
+// The same for rows of up to 1024 * ITER values: row and norm weight requested together and held in registers, one
+// memory round trip where the kernel above makes two (the decode step's final norm, one row of 4096: 6.9 -> about 4 us).
+// Same additions in the same order, same bits.
+template <int ITER>
+__global__ __launch_bounds__(256) void k_rms_norm_quant_row(const float *__restrict__ x, const float *__restrict__ alpha,
+                                                            float eps, int cols, float *__restrict__ xn_out,
+                                                            uint32_t *__restrict__ qs, Q8Scale *__restrict__ scales,
+                                                            half4v *__restrict__ xh) {
+    __shared__ float red[16];
+    const float4 *xr = (const float4 *)(x + (size_t)blockIdx.x * cols);
+    const int n4 = cols >> 2;
+    float4 v[ITER], al[ITER];
+#pragma unroll
+    for (int i = 0; i < ITER; ++i) {
+        const int c = min((int)threadIdx.x + 256 * i, n4 - 1);
+        v[i] = xr[c];
+        if (alpha) al[i] = ((const float4 *)alpha)[c];
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITER; ++i)
+        if ((int)threadIdx.x + 256 * i < n4) s += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    s = block_reduce<false>(s, red);
+    const float mean = s / (float)cols;
+    const float scale = rms_inv_sqrt(mean + eps);
+#pragma unroll
+    for (int i = 0; i < ITER; ++i) {
+        const int c = (int)threadIdx.x + 256 * i;
+        if (c >= ((n4 + 255) & ~255)) break;  // whole wavefronts take part in the cross-lane steps
+        const bool live = c < n4;
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) {
+            if (alpha) o = make_float4(scale * v[i].x * al[i].x, scale * v[i].y * al[i].y, scale * v[i].z * al[i].z, scale * v[i].w * al[i].w);
+            else o = make_float4(scale * v[i].x, scale * v[i].y, scale * v[i].z, scale * v[i].w);
+        }
+        __half h;
+        int bsum;
+        const uint32_t packed = quantize_q8_lane4(o, h, bsum);
+        if (!live) continue;
+        const size_t at = (size_t)blockIdx.x * n4 + c;
+        if (xn_out) ((float4 *)xn_out)[at] = o;
+        qs[at] = packed;
+        if (xh) xh[xh_index4(blockIdx.x, c, cols)] = q8_lane4_to_half(packed, h);
+        if ((c & 7) == 0) {
+            Q8Scale sc;
+            sc.d = __half2float(h);
+            sc.bsum = bsum;
+            scales[at >> 3] = sc;
+        }
+    }
+}
+
 // The same for rows of up to 1024 * ITER values, the row held in registers between the two passes, and with the row
 // optionally assembled first from the partial copies a contraction split along K has left: x = res + (part[0] +
 // part[1] + ...), the additions in the order of the separate split sum, written back to x_out (res may alias x_out:
@@ -384,8 +436,9 @@ __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
                           int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales, _Float16 *xh) {
     CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0 && cols <= 0x7FFFFFFF, "rms_norm_quant needs cols %% 32 == 0");
-    hipLaunchKernelGGL(k_rms_norm_quant, dim3((unsigned)rows), dim3(256), 0, dev->stream, x, alpha, eps, (int)cols,
-                       xn_out, (uint32_t *)qs, scales, (half4v *)xh);
+    auto kern = cols <= 4096 ? k_rms_norm_quant_row<4> : cols <= 8192 ? k_rms_norm_quant_row<8> : k_rms_norm_quant;
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(256), 0, dev->stream, x, alpha, eps, (int)cols, xn_out, (uint32_t *)qs,
+                       scales, (half4v *)xh);
     CANDY_LAUNCH_CHECK();
     return CANDY_HIP_OK;
 }
