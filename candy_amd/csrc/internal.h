@@ -287,6 +287,12 @@ struct AttnLaunch {
     int8_t *oq = nullptr;          // optional planar Q8_0 output
     Q8Scale *os = nullptr;
 };
+// ops.hip: FastArgmax of one long row over many workgroups into a 64-bit word (zero before the launch), and the index
+// the word stands for
+int launch_argmax_key(candy_hip_device *dev, const float *logits, int64_t cols, unsigned long long *key);
+__host__ __device__ inline uint32_t argmax_key_index(unsigned long long key) {
+    return key ? 0xFFFFFFFFu - (uint32_t)(key & 0xFFFFFFFFull) : 0u;
+}
 int attention_splits(const candy_hip_device *dev, int64_t n_kv_heads, int64_t max_pos);
 size_t attention_scratch_bytes(int n_heads, int n_kv_heads, int head_dim, int n_splits);
 int launch_attention(candy_hip_device *dev, const AttnLaunch &launch);

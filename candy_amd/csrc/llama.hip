@@ -31,7 +31,7 @@ struct candy_hip_llama {
     float *proj = nullptr;  // [d_model]: a projection's output before the residual add, for formats without that epilogue
     int8_t *xq = nullptr;           // planar Q8_0 quants of the current activation
     candy::Q8Scale *xs = nullptr;
-    uint32_t *next_tok = nullptr;   // greedy token of the last step
+    unsigned long long *next_key = nullptr;  // greedy token of the last step as k_argmax_key leaves it; zero before a step
     int64_t *tok_id = nullptr;
     int *d_pos = nullptr;                         // position of the token being decoded (device copy)
     void *attn_scratch = nullptr;                 // attention split partials
@@ -58,16 +58,18 @@ struct candy_hip_llama {
 namespace candy {
 
 // Parks the step's position and token id in device memory (read by the captured kernels).
-__global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok) {
+__global__ void k_set_step(int *pos_dst, int pos, int64_t *tok_dst, int64_t tok, unsigned long long *key) {
     *pos_dst = pos;
     if (tok >= 0) *tok_dst = tok;
+    *key = 0;  // the step's argmax folds into it
 }
 
 // Greedy generation without the host in the loop: the token the last step chose becomes the next step's input and
 // is written to the list the caller gets at the end.
-__global__ void k_chain_step(int *pos_dst, int pos, int64_t *tok_dst, const uint32_t *chosen, int32_t *list) {
+__global__ void k_chain_step(int *pos_dst, int pos, int64_t *tok_dst, unsigned long long *key, int32_t *list) {
     *pos_dst = pos;
-    const uint32_t t = *chosen;
+    const uint32_t t = argmax_key_index(*key);
+    *key = 0;
     *tok_dst = (int64_t)t;
     *list = (int32_t)t;
 }
@@ -132,11 +134,11 @@ int candy_hip_llama_create(candy_hip_device *dev, const candy_hip_llama_config *
     if (!rc) rc = candy_hip_zero(dev, m->pair_tickets, ((size_t)cfg->d_ffn / 32 + 1) * sizeof(unsigned));
     if (!rc) rc = dev_alloc(m, &m->proj, (size_t)cfg->d_model);
     if (!rc) rc = dev_alloc(m, &m->up_o, (size_t)cfg->d_ffn);
-    if (!rc) rc = dev_alloc(m, &m->logits, (size_t)cfg->vocab);
+    if (!rc) rc = dev_alloc(m, &m->logits, (size_t)cfg->vocab + 4);  // the argmax kernel reads whole 16-byte pieces
     if (!rc) rc = dev_alloc(m, &m->xq, widest);
     if (!rc) rc = dev_alloc(m, &m->xs, widest / 32);
-    if (!rc) rc = dev_alloc(m, &m->next_tok, 1);
-    if (!rc) rc = candy_hip_zero(dev, m->next_tok, sizeof(uint32_t));
+    if (!rc) rc = dev_alloc(m, &m->next_key, 1);
+    if (!rc) rc = candy_hip_zero(dev, m->next_key, sizeof(unsigned long long));
     if (!rc) rc = dev_alloc(m, &m->tok_id, 1);
     if (!rc) rc = dev_alloc(m, &m->d_pos, 1);
     m->n_splits = attention_splits(dev, cfg->n_kv_heads, cfg->max_pos);
@@ -392,7 +394,7 @@ static int llama_enqueue_step(candy_hip_llama *m) {
         float *ys[1] = {m->logits};
         if ((rc = norm_linear(m, m->out_norm, ws, ys, 1))) return rc;
     }
-    return candy_hip_argmax(dev, m->logits, 1, c.vocab, m->next_tok);
+    return launch_argmax_key(dev, m->logits, c.vocab, m->next_key);
 }
 
 // chain_to: null, or where the token chosen by the previous step is recorded while it becomes this step's input
@@ -401,9 +403,9 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
     candy_hip_device *dev = m->dev;
     int rc;
     if (chain_to)
-        hipLaunchKernelGGL(k_chain_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, m->next_tok, chain_to);
+        hipLaunchKernelGGL(k_chain_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, m->next_key, chain_to);
     else
-        hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token);
+        hipLaunchKernelGGL(k_set_step, dim3(1), dim3(1), 0, dev->stream, m->d_pos, (int)pos, m->tok_id, token, m->next_key);
     CANDY_LAUNCH_CHECK();
     if (dev_hidden) {
         if ((rc = candy_hip_d2d(dev, m->h, dev_hidden, (size_t)m->cfg.d_model * sizeof(float)))) return rc;
@@ -438,9 +440,9 @@ static int llama_step(candy_hip_llama *m, int32_t pos, int64_t token, const floa
     }
     if (dev_logits) *dev_logits = m->logits;
     if (next_token) {
-        uint32_t t = 0;
-        if ((rc = candy_hip_d2h(dev, &t, m->next_tok, sizeof(t)))) return rc;
-        *next_token = (int32_t)t;
+        unsigned long long key = 0;
+        if ((rc = candy_hip_d2h(dev, &key, m->next_key, sizeof(key)))) return rc;
+        *next_token = (int32_t)argmax_key_index(key);
     }
     return CANDY_HIP_OK;
 }
@@ -562,7 +564,8 @@ static int llama_enqueue_prompt(candy_hip_llama *m, int n, int pos0) {
     const candy_hip_qtensor *ws[1] = {m->head};
     float *ys[1] = {m->logits};
     if ((rc = norm_linear(m, m->out_norm, ws, ys, 1))) return rc;
-    return candy_hip_argmax(dev, m->logits, 1, c.vocab, m->next_tok);
+    if ((rc = launch_zero(dev, m->next_key, sizeof(unsigned long long)))) return rc;  // no step kernel in front here
+    return launch_argmax_key(dev, m->logits, c.vocab, m->next_key);
 }
 
 int candy_hip_llama_prefill(candy_hip_llama *m, const int32_t *tokens, int32_t n_tokens, int32_t pos0,
@@ -585,9 +588,9 @@ int candy_hip_llama_prefill(candy_hip_llama *m, const int32_t *tokens, int32_t n
     if (int rc = llama_enqueue_prompt(m, n_tokens, pos0)) return rc;
     if (dev_logits) *dev_logits = m->logits;
     if (next_token) {
-        uint32_t t = 0;
-        if (int rc = candy_hip_d2h(m->dev, &t, m->next_tok, sizeof(t))) return rc;
-        *next_token = (int32_t)t;
+        unsigned long long key = 0;
+        if (int rc = candy_hip_d2h(m->dev, &key, m->next_key, sizeof(key))) return rc;
+        *next_token = (int32_t)argmax_key_index(key);
     }
     return CANDY_HIP_OK;
 }
@@ -629,7 +632,7 @@ int candy_hip_llama_generate(candy_hip_llama *m, int32_t token, int32_t pos, int
         // the last step's choice: recorded by the same kernel, into a step that is not run (position and token
         // registers are rewritten by whatever step comes next)
         hipLaunchKernelGGL(k_chain_step, dim3(1), dim3(1), 0, m->dev->stream, m->d_pos, (int)(pos + n_steps - 1), m->tok_id,
-                           m->next_tok, list + n_steps - 1);
+                           m->next_key, list + n_steps - 1);
         if (hipGetLastError() != hipSuccess) rc = fail(CANDY_HIP_ERR_HIP, "launch failed");
     }
     if (!rc) rc = candy_hip_d2h(m->dev, tokens, list, (size_t)n_steps * sizeof(int32_t));

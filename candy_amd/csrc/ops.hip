@@ -176,6 +176,58 @@ __global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ src, 
     }
 }
 
+// The same choice over many workgroups, for one long row (the decode step's vocabulary): every workgroup reduces
+// its part to (value, index) and folds it into one 64-bit word with an atomic maximum - the value's bits made
+// monotonic in the upper half, 0xFFFFFFFF - index in the lower, so that the larger value wins and among equal values
+// the smaller index, whatever order the workgroups arrive in.  Values that the CPU loop's strict > against
+// -MaxFloat32 never selects (NaN, -inf, -MaxFloat32) fold in nothing; a word still zero means index 0
+// (argmax_key_index).  The word must be zero before the launch.  One workgroup pulls 128 KB of logits in 6.8 us; this
+// takes about 3.
+__global__ __launch_bounds__(256) void k_argmax_key(const float *__restrict__ src, int cols, unsigned long long *key) {
+    constexpr int U = 2;
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    const int n4 = cols >> 2;  // a 16-byte aligned row (launcher); the last cols % 4 values go to workgroup 0
+    const float4 *x4 = (const float4 *)src;
+    const int c0 = blockIdx.x * (256 * U) + threadIdx.x;
+    float4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = x4[max(min(c0 + 256 * u, n4 - 1), 0)];  // a row shorter than 4: one piece past it (allocated)
+    float best = -3.402823466e+38f;
+    uint32_t bi = 0xFFFFFFFFu;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int c = c0 + 256 * u;
+        const bool in = c < n4;
+        if (in && v[u].x > best) { best = v[u].x; bi = (uint32_t)(4 * c); }
+        if (in && v[u].y > best) { best = v[u].y; bi = (uint32_t)(4 * c + 1); }
+        if (in && v[u].z > best) { best = v[u].z; bi = (uint32_t)(4 * c + 2); }
+        if (in && v[u].w > best) { best = v[u].w; bi = (uint32_t)(4 * c + 3); }
+    }
+    if (blockIdx.x == 0 && (int)threadIdx.x < (cols & 3)) {  // indices past every float4 of this thread
+        const float t = src[4 * n4 + threadIdx.x];
+        if (t > best) { best = t; bi = (uint32_t)(4 * n4 + threadIdx.x); }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, 64);
+        const uint32_t oi = __shfl_xor(bi, off, 64);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { sv[wave] = best; si[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 4; ++i)
+            if (sv[i] > best || (sv[i] == best && si[i] < bi)) { best = sv[i]; bi = si[i]; }
+        if (bi != 0xFFFFFFFFu) {
+            const uint32_t b = __float_as_uint(best);
+            const uint32_t ordered = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+            atomicMax(key, ((unsigned long long)ordered << 32) | (unsigned long long)(0xFFFFFFFFu - bi));
+        }
+    }
+}
+
 // indexing.go:8-26 along dim 0 of a [n_src, width] table; id == MaxInt64 selects zeros.
 // indexing.go:8-26: the MaxInt64 id selects a row of zeros.  Any other id outside [0, n_src) makes the CPU loop
 // panic on its bounds check; a kernel cannot, so the row is written as zeros, nothing is read, and the device
@@ -433,6 +485,15 @@ __global__ __launch_bounds__(256) void k_silu_mul_quant(const float4 *__restrict
 }
 
 // ------------------------------------------------------------------ launchers shared with llama.hip
+int launch_argmax_key(candy_hip_device *dev, const float *logits, int64_t cols, unsigned long long *key) {
+    CANDY_REQUIRE(cols > 0 && cols <= 0x7FFFFFFF && ((uintptr_t)logits & 15) == 0, "argmax over a row of another shape");
+    const int64_t n4 = cols >> 2;
+    hipLaunchKernelGGL(k_argmax_key, dim3((unsigned)std::max<int64_t>(1, (n4 + 511) / 512)), dim3(256), 0, dev->stream, logits,
+                       (int)cols, key);
+    CANDY_LAUNCH_CHECK();
+    return CANDY_HIP_OK;
+}
+
 int launch_rms_norm_quant(candy_hip_device *dev, const float *x, const float *alpha, float eps, int64_t rows,
                           int64_t cols, float *xn_out, int8_t *qs, Q8Scale *scales, _Float16 *xh) {
     CANDY_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0 && cols <= 0x7FFFFFFF, "rms_norm_quant needs cols %% 32 == 0");

@@ -848,6 +848,41 @@ def test_generate_chains_the_same_tokens_as_step_by_step_decoding(dev):
     model.free()
 
 
+def test_greedy_token_over_several_workgroups_ties_and_an_odd_vocabulary(dev):
+    # The decoder's argmax folds the logits of a long row into one word from several workgroups.  A vocabulary of 4099
+    # (two workgroups of 16-byte pieces + three trailing values) whose head rows are all the same block bytes gives 4099
+    # bit-identical logits: the first index must win whichever workgroup arrives first.  With the last row's scales
+    # negated (a value in the trailing part) and with a row in the second workgroup's part negated, the token is
+    # numpy's argmax of the logits (first maximum) step after step, over replayed graphs and one-by-one launches.
+    cfg = dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, head_dim=128, d_ffn=512, vocab=4099, max_pos=8,
+               rms_eps=1e-5, rope_base=10000.0)
+    fmts = {"default": synth.Q4_K, "head": synth.Q8_0, "embed": synth.Q8_0}
+    host, model = build(dev, cfg, fmts, seed=88)
+    fmt, blocks = host[("head", -1)]
+    bb = synth.BLOCK_BYTES[fmt]
+    rows = np.array(blocks, copy=True).reshape(cfg["vocab"], -1)
+    rows[:] = rows[0]
+    keep = []
+    for variant in ("all equal", "last row negated", "a row of the second part negated"):
+        r = rows.copy()
+        if variant != "all equal":
+            at = cfg["vocab"] - 1 if variant == "last row negated" else 3000
+            r[at].reshape(-1, bb)[:, 1] ^= 0x80  # sign bit of every block's fp16 scale
+        head = dev.qtensor(fmt, cfg["vocab"], cfg["d_model"], r.reshape(-1))
+        keep.append(head)
+        model.set_qweight(hip.W_HEAD, -1, head)
+        for graph in (True, False):
+            model.set_graph(graph)
+            for pos, tok in enumerate([5, 4098, 77]):
+                nt, logits = model.decode(tok, pos)
+                assert nt == int(np.argmax(logits)), (variant, graph, pos, nt, int(np.argmax(logits)))
+                if variant == "all equal":
+                    assert np.all(logits.view(np.uint32) == logits.view(np.uint32)[0]) and nt == 0
+            chained = model.generate(5, 0, 3)
+            assert len(chained) == 3 and all(0 <= t < cfg["vocab"] for t in chained)
+    model.free()
+
+
 def test_decode_errors(dev):
     cfg = dict(n_layers=1, d_model=256, n_heads=2, n_kv_heads=2, head_dim=128, d_ffn=256, vocab=64, max_pos=4,
                rms_eps=1e-5, rope_base=10000.0)
