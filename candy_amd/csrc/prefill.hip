@@ -318,7 +318,10 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
         }
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
-            const int e = tid + it * 256, kp = e >> 5, d4 = e & 31;
+            // a wavefront's lanes: 16 key pairs x 4 neighbouring d4.  With the 32 d4 of one key pair per half wavefront
+            // the transposed stores below put 32 lanes on two LDS banks (a row of V^T is 80 bytes: 4 rows are 320,
+            // a multiple of 64) - 16-way conflicts on every one of them: 512 prompt tokens 48 -> 42.5 us per launch
+            const int e = tid + it * 256, kp = e & 15, d4 = e >> 4;
             vreg[it][0] = kv_load4(vh + (size_t)min(p0 + 2 * kp, n_keys - 1) * HD + 4 * d4);
             vreg[it][1] = kv_load4(vh + (size_t)min(p0 + 2 * kp + 1, n_keys - 1) * HD + 4 * d4);
         }
@@ -344,7 +347,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
         // V transposed: two keys of one d share a 32-bit store
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
-            const int e = tid + it * 256, kp = e >> 5, d4 = e & 31;
+            const int e = tid + it * 256, kp = e & 15, d4 = e >> 4;
             const float4 v0 = vreg[it][0], v1 = vreg[it][1];
             const float a[4] = {v0.x, v0.y, v0.z, v0.w}, b[4] = {v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
