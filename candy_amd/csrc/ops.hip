@@ -389,7 +389,10 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant_row(const float *__restr
 // optionally assembled first from the partial copies a contraction split along K has left: x = res + (part[0] +
 // part[1] + ...), the additions in the order of the separate split sum, written back to x_out (res may alias x_out:
 // a thread reads what it overwrites).  With n_split == 0 the row is read from res.
-template <int ITER>
+// NS: the number of partial copies when it is 2 or 4 (what the prompt pass's o and down projections leave) - every
+// load of the thread, norm weight included, is then requested before the first is used; 0: any number, read one after
+// the other.
+template <int ITER, int NS = 0>
 __global__ __launch_bounds__(256) void k_rms_norm_quant_regs(const float *res, const float *__restrict__ part, int n_split,
                                                              size_t stride, float *x_out,
                                                              const float *__restrict__ alpha, float eps, int cols,
@@ -398,7 +401,29 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant_regs(const float *res, c
     __shared__ float red[16];
     const int n4 = cols >> 2;
     const size_t row4 = (size_t)blockIdx.x * n4;
-    float4 v[ITER];
+    float4 v[ITER], al[ITER];
+    if constexpr (NS > 0) {
+        // rows of n4 = 256 * ITER float4 or fewer: chunks past the row re-read its last one and are dropped below
+        float4 pv[ITER][NS], rv[ITER];
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int c = min((int)threadIdx.x + 256 * it, n4 - 1);
+#pragma unroll
+            for (int k = 0; k < NS; ++k) pv[it][k] = ((const float4 *)(part + (size_t)k * stride))[row4 + c];
+            if (res) rv[it] = ((const float4 *)res)[row4 + c];
+            if (alpha) al[it] = ((const float4 *)alpha)[c];
+        }
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int c = threadIdx.x + 256 * it;
+            float4 t = pv[it][0];
+#pragma unroll
+            for (int k = 1; k < NS; ++k) { t.x += pv[it][k].x; t.y += pv[it][k].y; t.z += pv[it][k].z; t.w += pv[it][k].w; }
+            if (res) t = make_float4(rv[it].x + t.x, rv[it].y + t.y, rv[it].z + t.z, rv[it].w + t.w);
+            v[it] = c < n4 ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (c < n4) ((float4 *)x_out)[row4 + c] = t;
+        }
+    } else
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {
         const int c = threadIdx.x + 256 * it;
@@ -435,7 +460,7 @@ __global__ __launch_bounds__(256) void k_rms_norm_quant_regs(const float *res, c
         float4 w = v[it];
         if (live) {
             if (alpha) {
-                const float4 a = ((const float4 *)alpha)[c];
+                const float4 a = NS > 0 ? al[it] : ((const float4 *)alpha)[c];
                 w = make_float4(scale * w.x * a.x, scale * w.y * a.y, scale * w.z * a.z, scale * w.w * a.w);
             } else {
                 w = make_float4(scale * w.x, scale * w.y, scale * w.z, scale * w.w);
@@ -515,7 +540,9 @@ int launch_split_rms_norm_quant(candy_hip_device *dev, const SplitPending &sp, c
         if (int rc = launch_splitk_sum(dev, sp.part, sp.y, sp.res, sp.count, sp.n_split, sp.stride)) return rc;
         return launch_rms_norm_quant(dev, sp.y, alpha, eps, rows, cols, nullptr, qs, scales, xh);
     }
-    auto kern = cols <= 4096 ? k_rms_norm_quant_regs<4> : k_rms_norm_quant_regs<8>;
+    auto kern = cols <= 4096 ? (sp.n_split == 2 ? k_rms_norm_quant_regs<4, 2> : sp.n_split == 4 ? k_rms_norm_quant_regs<4, 4>
+                                                                                                 : k_rms_norm_quant_regs<4>)
+                             : k_rms_norm_quant_regs<8>;
     hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(256), 0, dev->stream, sp.res, sp.part, sp.n_split, sp.stride, sp.y,
                        alpha, eps, (int)cols, (uint32_t *)qs, scales, (half4v *)xh);
     CANDY_LAUNCH_CHECK();
