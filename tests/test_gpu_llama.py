@@ -880,6 +880,37 @@ def test_greedy_token_over_several_workgroups_ties_and_an_odd_vocabulary(dev):
                     assert np.all(logits.view(np.uint32) == logits.view(np.uint32)[0]) and nt == 0
             chained = model.generate(5, 0, 3)
             assert len(chained) == 3 and all(0 <= t < cfg["vocab"] for t in chained)
+    # Logits that are NaN or -inf are never chosen (reduce.go:846-862 compares with a strict > against -MaxFloat32,
+    # so a row of nothing else yields 0); +inf is.  Head rows with a NaN scale give NaN logits, rows with an infinite
+    # scale +inf, -inf or NaN.
+    def reference_choice(logits):
+        best, at = np.float32(-3.4028234663852886e38), 0
+        for i, v in enumerate(logits):
+            if v > best:
+                best, at = v, i
+        return at
+    _, plain = host[("head", -1)]
+    base = np.array(plain, copy=True).reshape(cfg["vocab"], -1)
+    for variant in ("every logit NaN", "NaN in front, finite behind", "infinite scales"):
+        r = base.copy()
+        blk = r.reshape(cfg["vocab"], -1, bb)
+        if variant == "every logit NaN":
+            blk[:, :, 0], blk[:, :, 1] = 0x00, 0x7E
+        elif variant == "NaN in front, finite behind":
+            blk[:700, :, 0], blk[:700, :, 1] = 0x00, 0x7E
+        else:
+            blk[1000:1100, :, 0], blk[1000:1100, :, 1] = 0x00, 0x7C
+        head = dev.qtensor(fmt, cfg["vocab"], cfg["d_model"], r.reshape(-1))
+        keep.append(head)
+        model.set_qweight(hip.W_HEAD, -1, head)
+        model.set_graph(True)
+        for pos, tok in enumerate([5, 4098, 77]):
+            nt, logits = model.decode(tok, pos)
+            assert nt == reference_choice(logits), (variant, pos, nt, reference_choice(logits))
+            if variant == "every logit NaN":
+                assert np.all(np.isnan(logits)) and nt == 0
+            if variant == "NaN in front, finite behind":
+                assert np.all(np.isnan(logits[:700])) and nt >= 700
     model.free()
 
 
