@@ -72,6 +72,7 @@ struct Options {
     int llama_graph = 1;         // decoders created afterwards replay a captured HIP graph (0: eager launches)
     int fused_wide = 1;          // decode step: one-workgroup-per-CU kernels for the big Q4_K shapes (0: the narrower ones)
     int wide_waves = 8;          // wavefronts per workgroup of those kernels: 8 (two workgroups per CU) or 16 (one)
+    int prefill_attention_groups = 0;  // comparison runs: key-tile groups per workgroup in matrix-core prompt attention, 1 or 2 (0: by shape)
     int attn_splits = 0;         // comparison runs: splits of the cached positions in decode attention, 1..64 (0: by shape)
     int down_quant = 0;          // decode step: 1 = gate / up leaves f32 SiLU*Mul values and the down projection quantizes them in its prologue (measured slower: 561 against 583 tok/s on the 7B shape); 0 = gate / up quantizes, blocks shared between workgroups through tickets
 };

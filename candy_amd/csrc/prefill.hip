@@ -261,20 +261,30 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-template <class KV>
-__global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restrict__ q, const KV *__restrict__ k_cache,
-                                                           const KV *__restrict__ v_cache, float *__restrict__ out,
-                                                           int n, int pos0, int n_heads, int n_kv_heads,
-                                                           int64_t cache_stride, float scale,
-                                                           _Float16 *__restrict__ xh_out) {
+// GROUPS = 2: two groups of four wavefronts share the workgroup's 64 queries and take alternate key tiles, each with
+// tile buffers of its own, and merge their (max, sum, output) per row at the end: a short prompt has about one
+// workgroup per CU and the launch lasts as long as the last query tile's walk over all the keys, which this halves.
+template <class KV, int GROUPS>
+__global__ __launch_bounds__(256 * GROUPS) void k_attn_prefill_mfma(const float *__restrict__ q, const KV *__restrict__ k_cache,
+                                                                    const KV *__restrict__ v_cache, float *__restrict__ out,
+                                                                    int n, int pos0, int n_heads, int n_kv_heads,
+                                                                    int64_t cache_stride, float scale,
+                                                                    _Float16 *__restrict__ xh_out) {
     constexpr int HD = 128, QT = 64, KT = 32;
     constexpr int KP = HD + 8;   // K tile pitch in halves (272 bytes: the 16 rows of an operand read hit distinct banks)
     constexpr int VP = KT + 8;   // V^T tile pitch in halves (80 bytes, same property)
     constexpr int PP = KT + 8;   // P tile pitch
-    __shared__ __align__(16) _Float16 s_k[2][KT * KP];        // [hi/lo][key][d]
-    __shared__ __align__(16) _Float16 s_vt[2][HD * VP];       // [hi/lo][d][key]
-    __shared__ __align__(16) _Float16 s_p[4][2][16 * PP];     // per wavefront [hi/lo][row][key]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int K_HALVES = 2 * KT * KP, VT_HALVES = 2 * HD * VP, P_HALVES = 4 * 2 * 16 * PP;
+    constexpr int GROUP_HALVES = K_HALVES + VT_HALVES + P_HALVES;
+    static_assert(GROUP_HALVES * 2 >= 40 * 256 * 4, "a group's buffers hold the other group's state at the merge");
+    __shared__ __align__(16) _Float16 s_all[GROUPS * GROUP_HALVES];
+    const int grp = GROUPS == 1 ? 0 : (int)(threadIdx.x >> 8);
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+    _Float16 *const s_kb = s_all + grp * GROUP_HALVES;   // [hi/lo][key][d]
+    _Float16 *const s_vtb = s_kb + K_HALVES;              // [hi/lo][d][key]
+    _Float16 *const s_pb = s_vtb + VT_HALVES;             // per wavefront [hi/lo][row][key]
+    _Float16 *const s_k[2] = {s_kb, s_kb + KT * KP};
+    _Float16 *const s_vt[2] = {s_vtb, s_vtb + HD * VP};
     const int r16 = lane & 15, c4 = lane >> 4;
     const int head = blockIdx.x, i0 = blockIdx.y * QT;
     const int kvh = head / (n_heads / n_kv_heads);
@@ -282,7 +292,8 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
     const int n_keys = pos0 + min(i0 + QT, n);   // positions the tile's last query may see
     const int wave_last = pos0 + i0 + 16 * wave + 15;  // last position any row of this wavefront may see
 
-    // Q as the A operand (row = query r16, 8 consecutive d per k-step), pre-scaled, split hi / lo
+    // Q as the A operand (row = query r16, 8 consecutive d per k-step), pre-scaled by scale * log2(e) (the softmax
+    // runs on powers of two: one v_exp_f32 per value), split hi / lo
     half8 qh[4], ql[4];
     {
         const int i = min(i0 + 16 * wave + r16, n - 1);
@@ -293,7 +304,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
             const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const HiLo t = split_half(v[e] * scale);
+                const HiLo t = split_half(v[e] * (scale * 1.44269504088896341f));
                 qh[ks][e] = t.hi;
                 ql[ks][e] = t.lo;
             }
@@ -326,9 +337,17 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
             vreg[it][1] = kv_load4(vh + (size_t)min(p0 + 2 * kp + 1, n_keys - 1) * HD + 4 * d4);
         }
     };
-    request(0);
-    for (int p0 = 0; p0 < n_keys; p0 += KT) {
+    // every group runs the same number of rounds (the barriers are the workgroup's); a group without a tile in the
+    // last round sits it out
+    const int n_rounds = ((n_keys + KT - 1) / KT + GROUPS - 1) / GROUPS;
+    if (grp * KT < n_keys) request(grp * KT);
+    for (int round = 0; round < n_rounds; ++round) {
+        const int p0 = (round * GROUPS + grp) * KT;
         __syncthreads();  // previous tile fully consumed
+        if (GROUPS > 1 && p0 >= n_keys) {
+            __syncthreads();
+            continue;
+        }
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
             const int e = tid + it * 256, key = e >> 5, d4 = e & 31;
@@ -360,7 +379,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
                 *(half2h *)&s_vt[1][(4 * d4 + c) * VP + 2 * kp] = lo;
             }
         }
-        if (p0 + KT < n_keys) request(p0 + KT);
+        if (p0 + GROUPS * KT < n_keys) request(p0 + GROUPS * KT);
         __syncthreads();
         if (p0 > wave_last) continue;  // every key of the tile is in the future of all 16 rows (the barriers above stay uniform)
 
@@ -381,7 +400,7 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
         }
         // ---- online softmax per row
         float corr[4];
-        _Float16 *ph = &s_p[wave][0][0], *pl = &s_p[wave][1][0];
+        _Float16 *ph = s_pb + wave * 2 * 16 * PP, *pl = ph + 16 * PP;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int qpos = pos0 + i0 + 16 * wave + 4 * c4 + j;
@@ -394,12 +413,15 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
                 mx = fmaxf(mx, sv[nt]);
             }
             mx = row16_max(mx);
-            const float m_new = fmaxf(m_run[j], mx);  // position 0 is visible to every row: finite from the first tile on
-            corr[j] = expf(m_run[j] - m_new);
+            // position 0 is visible to every row: with one group finite from the first tile on; a second group's first
+            // tile may lie in a row's future altogether
+            const float m_new = fmaxf(m_run[j], mx);
+            const bool seen = GROUPS == 1 || m_new != -INFINITY;
+            corr[j] = seen ? __builtin_amdgcn_exp2f(m_run[j] - m_new) : 1.0f;
             float ps = 0.0f;
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt) {
-                const float pw = expf(sv[nt] - m_new);  // exp(-inf) = 0 for masked keys
+                const float pw = seen ? __builtin_amdgcn_exp2f(sv[nt] - m_new) : 0.0f;  // 2^-inf = 0 for masked keys
                 ps += pw;
                 const HiLo t = split_half(pw);
                 ph[(4 * c4 + j) * PP + nt * 16 + r16] = t.hi;
@@ -409,10 +431,13 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
             l_run[j] = l_run[j] * corr[j] + ps;
             m_run[j] = m_new;
         }
+        // the running maxima settle after the first tiles: most rounds have nothing to rescale
+        if (__any(corr[0] != 1.0f || corr[1] != 1.0f || corr[2] != 1.0f || corr[3] != 1.0f)) {
 #pragma unroll
-        for (int dt = 0; dt < 8; ++dt)
+            for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) o[dt][j] *= corr[j];
+                for (int j = 0; j < 4; ++j) o[dt][j] *= corr[j];
+        }
         // the wavefront's own P tile: its LDS operations complete in order, no workgroup barrier needed
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -430,6 +455,34 @@ __global__ __launch_bounds__(256) void k_attn_prefill_mfma(const float *__restri
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if constexpr (GROUPS == 2) {
+        // the second group's state goes through its own tile buffers (value k of thread t at k * 256 + t); the first
+        // group, whose tiles hold position 0, always has a finite maximum
+        float *st = (float *)(s_all + GROUP_HALVES);
+        __syncthreads();
+        if (grp == 1) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                st[j * 256 + tid] = m_run[j];
+                st[(4 + j) * 256 + tid] = l_run[j];
+            }
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) st[(8 + 4 * dt + j) * 256 + tid] = o[dt][j];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float m1 = st[j * 256 + tid], l1 = st[(4 + j) * 256 + tid];
+            const float m = fmaxf(m_run[j], m1);
+            const float f0 = __builtin_amdgcn_exp2f(m_run[j] - m), f1 = __builtin_amdgcn_exp2f(m1 - m);
+            l_run[j] = l_run[j] * f0 + l1 * f1;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) o[dt][j] = o[dt][j] * f0 + st[(8 + 4 * dt + j) * 256 + tid] * f1;
+        }
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -504,10 +557,21 @@ static void launch_attn_prefill_kv(candy_hip_device *dev, const float *q, const 
                                    float scale, _Float16 *xh_out) {
     const dim3 grid((unsigned)n_heads, (unsigned)((n + 31) / 32));
     const bool valu_only = dev->opt.prefill_attention_valu != 0;  // comparison runs
-    if (head_dim == 128 && !valu_only)
-        hipLaunchKernelGGL(k_attn_prefill_mfma<KV>, dim3((unsigned)n_heads, (unsigned)((n + 63) / 64)), dim3(256), 0,
-                           dev->stream, q, k_cache, v_cache, out, n, pos0, n_heads, n_kv_heads, cache_stride, scale, xh_out);
-    else if (head_dim == 128)
+    if (head_dim == 128 && !valu_only) {
+        // Two key-tile groups per workgroup where the launch lasts as long as its longest workgroup: a grid of about one
+        // workgroup per CU and a walk of more than four key tiles.  A larger grid fills the CUs with several of the
+        // smaller workgroups, a shorter walk does not pay for the merge.
+        const dim3 tiles((unsigned)n_heads, (unsigned)((n + 63) / 64));
+        const int64_t wgs = (int64_t)tiles.x * tiles.y;
+        const int groups = dev->opt.prefill_attention_groups ? dev->opt.prefill_attention_groups
+                                                             : (n > 128 && 2 * wgs <= 3 * (int64_t)dev->num_cus ? 2 : 1);
+        if (groups == 2)
+            hipLaunchKernelGGL((k_attn_prefill_mfma<KV, 2>), tiles, dim3(512), 0, dev->stream, q, k_cache, v_cache, out, n,
+                               pos0, n_heads, n_kv_heads, cache_stride, scale, xh_out);
+        else
+            hipLaunchKernelGGL((k_attn_prefill_mfma<KV, 1>), tiles, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n,
+                               pos0, n_heads, n_kv_heads, cache_stride, scale, xh_out);
+    } else if (head_dim == 128)
         hipLaunchKernelGGL((k_attn_prefill<128, KV>), grid, dim3(256), 0, dev->stream, q, k_cache, v_cache, out, n, pos0,
                            n_heads, n_kv_heads, cache_stride, scale);
     else

@@ -365,6 +365,7 @@ const OptionKey OPTION_KEYS[] = {
     {"fused.wide", &candy::Options::fused_wide, 0, 1},
     {"fused.wide_waves", &candy::Options::wide_waves, 8, 16},
     {"fused.down_quant", &candy::Options::down_quant, 0, 1},
+    {"prefill.attention_groups", &candy::Options::prefill_attention_groups, 0, 2},
     {"attention.splits", &candy::Options::attn_splits, 0, 64},
 };
 const OptionKey *find_option(const char *key) {

@@ -120,6 +120,9 @@ int candy_hip_synchronize(candy_hip_device *dev);       /* device.go:81 Synchron
  *                                         launch that follows (RMSNorm + quantize behind o / down, rope behind q / k / v;
  *                                         0: a launch of its own sums them)
  *   "prefill.attention_valu"     0        prompt attention for head_dim 128 on the vector ALU
+ *   "prefill.attention_groups"   0        comparison runs: matrix-core prompt attention with one (1) or two (2) groups of
+ *                                         wavefronts per query tile that take alternate key tiles (0: two for prompts of
+ *                                         more than 128 tokens whose grid is at most 1.5 workgroups per CU)
  * A decoder whose step has been captured into a graph notices a later candy_hip_set_option on its device and captures
  * the step again at its next decode call.
  * Read-only keys (candy_hip_get_option): "runtime.workspace_bytes", "runtime.split_workspace_bytes" - what the

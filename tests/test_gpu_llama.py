@@ -714,6 +714,30 @@ def test_prompt_in_two_chunks_equals_one_pass(dev, case, n, cut):
         a.prefill([], 0)
 
 
+@pytest.mark.parametrize("cut", [20, 77, 128])
+def test_prompt_attention_with_one_and_two_key_tile_groups(dev, cut):
+    # The matrix-core kernel's two forms (one group of wavefronts per query tile walking every key tile; two groups
+    # taking alternate tiles and merging at the end) agree on a whole prompt and on a chunk continued off the tile
+    # boundaries: at pos0 = 20 the second group's first tile (keys 32..63) lies wholly in the future of some rows of a
+    # wavefront that others of its rows can see.
+    name, cfg, fmts, n, _ = PROMPT_CASES[2]
+    tokens = [int(t) for t in np.random.default_rng(31).integers(0, cfg["vocab"], n)]
+    got = {}
+    try:
+        for groups in (1, 2):
+            dev.set_option("prefill.attention_groups", groups)
+            _, a = build(dev, cfg, fmts, seed=30)
+            _, b = build(dev, cfg, fmts, seed=30)
+            _, whole = a.prefill(tokens, 0)
+            b.prefill(tokens[:cut], 0)
+            _, chunked = b.prefill(tokens[cut:], cut)
+            assert rel(chunked, whole.astype(np.float64)) <= 1e-4, groups
+            got[groups] = whole
+    finally:
+        dev.set_option("prefill.attention_groups", 0)
+    assert rel(got[2], got[1].astype(np.float64)) <= 1e-5
+
+
 def test_prompt_chunks_on_either_side_of_the_fp16_threshold(dev):
     # Results are not invariant under batching: a 300-token prompt fed whole contracts fp16 operands (256 rows or
     # more), the same prompt fed as 150 + 150 runs every Linear on the exact int8 kernels.  The two agree within
