@@ -271,6 +271,7 @@ __global__ __launch_bounds__(256 * GROUPS) void k_attn_prefill_mfma(const float 
                                                                     int64_t cache_stride, float scale,
                                                                     _Float16 *__restrict__ xh_out) {
     constexpr int HD = 128, QT = 64, KT = 32;
+    constexpr bool HALF_KV = std::is_same<KV, _Float16>::value;  // cache values are their own fp16 head: no tail tiles
     constexpr int KP = HD + 8;   // K tile pitch in halves (272 bytes: the 16 rows of an operand read hit distinct banks)
     constexpr int VP = KT + 8;   // V^T tile pitch in halves (80 bytes, same property)
     constexpr int PP = KT + 8;   // P tile pitch
@@ -361,7 +362,7 @@ __global__ __launch_bounds__(256 * GROUPS) void k_attn_prefill_mfma(const float 
                 lo[c] = t.lo;
             }
             *(half4h *)&s_k[0][key * KP + 4 * d4] = hi;
-            *(half4h *)&s_k[1][key * KP + 4 * d4] = lo;
+            if (!HALF_KV) *(half4h *)&s_k[1][key * KP + 4 * d4] = lo;
         }
         // V transposed: two keys of one d share a 32-bit store
 #pragma unroll
@@ -376,7 +377,7 @@ __global__ __launch_bounds__(256 * GROUPS) void k_attn_prefill_mfma(const float 
                 hi[0] = ta.hi; lo[0] = ta.lo;
                 hi[1] = tb.hi; lo[1] = tb.lo;
                 *(half2h *)&s_vt[0][(4 * d4 + c) * VP + 2 * kp] = hi;
-                *(half2h *)&s_vt[1][(4 * d4 + c) * VP + 2 * kp] = lo;
+                if (!HALF_KV) *(half2h *)&s_vt[1][(4 * d4 + c) * VP + 2 * kp] = lo;
             }
         }
         if (p0 + GROUPS * KT < n_keys) request(p0 + GROUPS * KT);
@@ -391,9 +392,9 @@ __global__ __launch_bounds__(256 * GROUPS) void k_attn_prefill_mfma(const float 
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 const int off = (nt * 16 + r16) * KP + ks * 32 + c4 * 8;
-                const half8 kh8 = *(const half8 *)&s_k[0][off], kl8 = *(const half8 *)&s_k[1][off];
+                const half8 kh8 = *(const half8 *)&s_k[0][off];
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql[ks], kh8, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[ks], kl8, acc, 0, 0, 0);
+                if (!HALF_KV) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[ks], *(const half8 *)&s_k[1][off], acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[ks], kh8, acc, 0, 0, 0);
             }
             s_acc[nt] = acc;
@@ -447,9 +448,9 @@ __global__ __launch_bounds__(256 * GROUPS) void k_attn_prefill_mfma(const float 
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) {
             const int off = (dt * 16 + r16) * VP + c4 * 8;
-            const half8 vh8 = *(const half8 *)&s_vt[0][off], vl8 = *(const half8 *)&s_vt[1][off];
+            const half8 vh8 = *(const half8 *)&s_vt[0][off];
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_l, vh8, o[dt], 0, 0, 0);
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_h, vl8, o[dt], 0, 0, 0);
+            if (!HALF_KV) o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_h, *(const half8 *)&s_vt[1][off], o[dt], 0, 0, 0);
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_h, vh8, o[dt], 0, 0, 0);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
